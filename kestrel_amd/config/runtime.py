@@ -1,0 +1,77 @@
+"""Knobs of the engine, as one typed object.
+
+Reference: ``kestrel/config.py:155-202`` (``RuntimeConfig``: ``model_path``, ``device``,
+``dtype``, ``max_batch_size``, ``page_size``, ``kv_cache_pages``, ``enable_cuda_graphs``,
+``model``) with its checks (``:181-197``); names are kept where the meaning is the same.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+from pathlib import Path
+from typing import Optional, Union
+
+import torch
+
+_DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.float32, "fp32": torch.float32,
+           "float": torch.float32}
+
+
+def parse_dtype(value) -> torch.dtype:
+    if isinstance(value, torch.dtype):
+        if value not in (torch.bfloat16, torch.float32):
+            raise ValueError(f"dtype must be bfloat16 or float32, got {value}")
+        return value
+    try:
+        return _DTYPES[str(value).lower()]
+    except KeyError:
+        raise ValueError(f"dtype must be bfloat16 or float32, got {value!r}") from None
+
+
+@dataclass
+class RuntimeConfig:
+    """``model_path``: folder with ``config.json`` and ``model.safetensors``.
+
+    ``model``: architecture name; ``None`` takes it from ``config.json``.
+    ``max_batch_size``: most requests decoded together. ``page_size``: tokens per cache
+    page. ``kv_cache_pages``: pages of the pool; ``None`` sizes it from
+    ``kv_cache_tokens`` or, failing that, for ``max_batch_size`` full contexts.
+    ``max_num_batched_tokens``: token budget of one step (prompt portions are cut to it).
+    ``enable_graphs``: replay decode-only steps as captured HIP graphs.
+    ``seed``: base of the sampling generator.
+    """
+
+    model_path: Union[str, Path, None] = None
+    device: str = "cuda"
+    dtype: Union[torch.dtype, str] = torch.bfloat16
+    max_batch_size: int = 4
+    page_size: int = 16
+    kv_cache_pages: Optional[int] = None
+    kv_cache_tokens: Optional[int] = None
+    max_num_batched_tokens: int = 2048
+    enable_graphs: bool = True
+    model: Optional[str] = None
+    seed: int = 0
+    max_seq_len: Optional[int] = None
+
+    def __post_init__(self) -> None:
+        self.dtype = parse_dtype(self.dtype)
+        if self.max_batch_size <= 0:
+            raise ValueError("max_batch_size must be a positive integer")
+        if self.page_size <= 0:
+            raise ValueError("page_size must be a positive integer")
+        if self.kv_cache_pages is not None and self.kv_cache_pages <= 0:
+            raise ValueError("kv_cache_pages must be a positive integer")
+        if self.kv_cache_tokens is not None and self.kv_cache_tokens <= 0:
+            raise ValueError("kv_cache_tokens must be a positive integer")
+        if self.max_num_batched_tokens <= 0:
+            raise ValueError("max_num_batched_tokens must be a positive integer")
+        if self.max_seq_len is not None and self.max_seq_len <= 0:
+            raise ValueError("max_seq_len must be a positive integer")
+        device = torch.device(self.device)
+        if device.type != "cuda":
+            raise ValueError(f"device must be a GPU ('cuda' or 'cuda:N'), got {self.device!r}: there is no CPU path")
+
+    def resolved_device(self) -> torch.device:
+        device = torch.device(self.device)
+        return torch.device("cuda", device.index if device.index is not None else 0)

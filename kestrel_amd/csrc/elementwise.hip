@@ -1,0 +1,213 @@
+// Embedding gather, LayerNorm and rotary + paged cache write.
+//
+// The residual stream is fp32 in every precision mode; these kernels read and write
+// it as fp32 and convert only at the boundary to the model's storage type.
+#include "ka_common.h"
+
+#include <stdarg.h>
+#include <stdio.h>
+
+static thread_local char g_error[512];
+
+void ka_set_error(const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_error, sizeof(g_error), fmt, ap);
+    va_end(ap);
+}
+
+KA_API const char* ka_last_error() { return g_error; }
+
+KA_API int ka_version() { return 1; }
+
+// ----------------------------------------------------------------------------
+// Embedding: out[t, :] = table[ids[t], :] as fp32; rows with ids[t] < 0 are left
+// as they are (their embedding was given by the caller).
+// ----------------------------------------------------------------------------
+template <typename T>
+__global__ void embed_kernel(const T* __restrict__ table, const int* __restrict__ ids,
+                             float* __restrict__ out, int dim) {
+    int t = blockIdx.x;
+    int id = ids[t];
+    if (id < 0) return;
+    const T* src = table + (size_t)id * dim;
+    float* dst = out + (size_t)t * dim;
+    for (int d = threadIdx.x; d < dim; d += blockDim.x) dst[d] = ka_to_float(src[d]);
+}
+
+KA_API int ka_embed(const void* table, int table_dtype, const int* ids, float* out, int n,
+                    int dim, hipStream_t stream) {
+    KA_CHECK(n >= 0 && dim > 0, "ka_embed: bad sizes n=%d dim=%d", n, dim);
+    if (n == 0) return 0;
+    dim3 grid(n), block(256);
+    if (table_dtype == KA_F32)
+        hipLaunchKernelGGL(embed_kernel<float>, grid, block, 0, stream, (const float*)table, ids, out, dim);
+    else if (table_dtype == KA_BF16)
+        hipLaunchKernelGGL(embed_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)table, ids, out, dim);
+    else
+        KA_CHECK(false, "ka_embed: unsupported table dtype %d", table_dtype);
+    KA_LAUNCH_CHECK();
+    return 0;
+}
+
+// out[rows[i], :] = src[i, :] (given embeddings spliced into the stream).
+template <typename T>
+__global__ void scatter_rows_kernel(const T* __restrict__ src, const int* __restrict__ rows,
+                                    float* __restrict__ out, int dim) {
+    int i = blockIdx.x;
+    const T* s = src + (size_t)i * dim;
+    float* dst = out + (size_t)rows[i] * dim;
+    for (int d = threadIdx.x; d < dim; d += blockDim.x) dst[d] = ka_to_float(s[d]);
+}
+
+KA_API int ka_scatter_rows(const void* src, int src_dtype, const int* rows, float* out, int m,
+                           int dim, hipStream_t stream) {
+    KA_CHECK(m >= 0 && dim > 0, "ka_scatter_rows: bad sizes m=%d dim=%d", m, dim);
+    if (m == 0) return 0;
+    dim3 grid(m), block(256);
+    if (src_dtype == KA_F32)
+        hipLaunchKernelGGL(scatter_rows_kernel<float>, grid, block, 0, stream, (const float*)src, rows, out, dim);
+    else if (src_dtype == KA_BF16)
+        hipLaunchKernelGGL(scatter_rows_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)src, rows, out, dim);
+    else
+        KA_CHECK(false, "ka_scatter_rows: unsupported dtype %d", src_dtype);
+    KA_LAUNCH_CHECK();
+    return 0;
+}
+
+// ----------------------------------------------------------------------------
+// LayerNorm over the last axis, statistics in fp32, two passes (mean, then the
+// variance of the centred values). `rows` (optional) selects input rows, which
+// fuses the gather of the wanted positions into the final norm.
+// ----------------------------------------------------------------------------
+constexpr int LN_THREADS = 256;
+
+__device__ __forceinline__ float block_sum_256(float v, float* smem) {
+    v = ka_wave_sum(v);
+    int wave = threadIdx.x / KA_WAVE, lane = threadIdx.x % KA_WAVE;
+    __syncthreads();
+    if (lane == 0) smem[wave] = v;
+    __syncthreads();
+    float total = 0.f;
+#pragma unroll
+    for (int w = 0; w < LN_THREADS / KA_WAVE; ++w) total += smem[w];
+    return total;
+}
+
+template <typename TOut>
+__global__ void __launch_bounds__(LN_THREADS)
+layernorm_kernel(const float* __restrict__ x, const int* __restrict__ rows,
+                 const float* __restrict__ gamma, const float* __restrict__ beta, float eps,
+                 TOut* __restrict__ out, int dim) {
+    __shared__ float smem[LN_THREADS / KA_WAVE];
+    int i = blockIdx.x;
+    const float* src = x + (size_t)(rows ? rows[i] : i) * dim;
+    TOut* dst = out + (size_t)i * dim;
+    float s = 0.f;
+    for (int d = threadIdx.x; d < dim; d += LN_THREADS) s += src[d];
+    float mean = block_sum_256(s, smem) / (float)dim;
+    float v = 0.f;
+    for (int d = threadIdx.x; d < dim; d += LN_THREADS) {
+        float c = src[d] - mean;
+        v += c * c;
+    }
+    float var = block_sum_256(v, smem) / (float)dim;
+    float rstd = 1.0f / sqrtf(var + eps);
+    for (int d = threadIdx.x; d < dim; d += LN_THREADS) {
+        float y = (src[d] - mean) * rstd * gamma[d];
+        if (beta) y += beta[d];
+        dst[d] = ka_from_float<TOut>(y);
+    }
+}
+
+KA_API int ka_layernorm(const float* x, const int* rows, const float* gamma, const float* beta,
+                        float eps, void* out, int out_dtype, int n, int dim, hipStream_t stream) {
+    KA_CHECK(n >= 0 && dim > 0, "ka_layernorm: bad sizes n=%d dim=%d", n, dim);
+    KA_CHECK(eps >= 0.f, "ka_layernorm: negative eps");
+    if (n == 0) return 0;
+    dim3 grid(n), block(LN_THREADS);
+    if (out_dtype == KA_F32)
+        hipLaunchKernelGGL(layernorm_kernel<float>, grid, block, 0, stream, x, rows, gamma, beta, eps, (float*)out, dim);
+    else if (out_dtype == KA_BF16)
+        hipLaunchKernelGGL(layernorm_kernel<bf16_t>, grid, block, 0, stream, x, rows, gamma, beta, eps, (bf16_t*)out, dim);
+    else
+        KA_CHECK(false, "ka_layernorm: unsupported out dtype %d", out_dtype);
+    KA_LAUNCH_CHECK();
+    return 0;
+}
+
+// ----------------------------------------------------------------------------
+// Rotary position encoding (non-interleaved halves of the first `rot` channels of
+// each head) applied in place to the q heads of a fused qkv row, and to the k heads
+// on their way into the paged cache together with v. The table row of position p is
+// [cos(p f_0..f_{rot/2-1}), sin(...)] in fp32; the rotation is computed in fp32.
+//
+// qkv row: [H*hd q | Hkv*hd k | Hkv*hd v]. Cache: [pages, Hkv, page_size, hd].
+// slots[t] = page * page_size + offset, or < 0 for "do not write" (a layer that
+// reads another layer's cache).
+// ----------------------------------------------------------------------------
+template <typename T>
+__global__ void rope_cache_kernel(T* __restrict__ qkv, long row_stride,
+                                  const int* __restrict__ positions, const int* __restrict__ slots,
+                                  const float* __restrict__ table, T* __restrict__ k_cache,
+                                  T* __restrict__ v_cache, int H, int Hkv, int hd, int rot,
+                                  int page_size, int rotate) {
+    int t = blockIdx.x;
+    T* row = qkv + (size_t)t * row_stride;
+    int pos = positions[t];
+    const float* cs = table + (size_t)pos * rot;
+    int half = rot / 2;
+    // q heads: rotate in place. One thread per (head, pair).
+    if (rotate) {
+        for (int idx = threadIdx.x; idx < H * half; idx += blockDim.x) {
+            int h = idx / half, i = idx % half;
+            T* p = row + h * hd;
+            float a = ka_to_float(p[i]), b = ka_to_float(p[i + half]);
+            float c = cs[i], s = cs[half + i];
+            p[i] = ka_from_float<T>(a * c - b * s);
+            p[i + half] = ka_from_float<T>(b * c + a * s);
+        }
+    }
+    long slot = slots ? slots[t] : -1;
+    if (slot < 0) return;
+    long page = slot / page_size, off = slot % page_size;
+    const T* krow = row + (size_t)H * hd;
+    const T* vrow = krow + (size_t)Hkv * hd;
+    for (int idx = threadIdx.x; idx < Hkv * hd; idx += blockDim.x) {
+        int h = idx / hd, d = idx % hd;
+        size_t dst = (((size_t)page * Hkv + h) * page_size + off) * hd + d;
+        float kv = ka_to_float(krow[idx]);
+        if (rotate && d < rot) {
+            int i = d < half ? d : d - half;
+            float a = ka_to_float(krow[h * hd + i]), b = ka_to_float(krow[h * hd + i + half]);
+            float c = cs[i], s = cs[half + i];
+            kv = d < half ? a * c - b * s : b * c + a * s;
+        }
+        k_cache[dst] = ka_from_float<T>(kv);
+        v_cache[dst] = vrow[idx];
+    }
+}
+
+KA_API int ka_rope_cache(void* qkv, int dtype, long row_stride, const int* positions,
+                         const int* slots, const float* table, int table_rows, void* k_cache,
+                         void* v_cache, int n, int H, int Hkv, int hd, int rot, int page_size,
+                         hipStream_t stream) {
+    KA_CHECK(n >= 0 && H > 0 && Hkv > 0 && hd > 0, "ka_rope_cache: bad sizes");
+    KA_CHECK(rot >= 0 && rot <= hd && rot % 2 == 0, "ka_rope_cache: rotary dim %d must be even and <= head dim %d", rot, hd);
+    KA_CHECK(row_stride >= (long)(H + 2 * Hkv) * hd, "ka_rope_cache: row stride %ld too small", row_stride);
+    KA_CHECK(page_size > 0, "ka_rope_cache: page size %d", page_size);
+    KA_CHECK(rot == 0 || (table != nullptr && table_rows > 0), "ka_rope_cache: rotary table missing");
+    if (n == 0) return 0;
+    dim3 grid(n), block(256);
+    int rotate = rot > 0;
+    if (dtype == KA_F32)
+        hipLaunchKernelGGL(rope_cache_kernel<float>, grid, block, 0, stream, (float*)qkv, row_stride, positions, slots,
+                           table, (float*)k_cache, (float*)v_cache, H, Hkv, hd, rot, page_size, rotate);
+    else if (dtype == KA_BF16)
+        hipLaunchKernelGGL(rope_cache_kernel<bf16_t>, grid, block, 0, stream, (bf16_t*)qkv, row_stride, positions, slots,
+                           table, (bf16_t*)k_cache, (bf16_t*)v_cache, H, Hkv, hd, rot, page_size, rotate);
+    else
+        KA_CHECK(false, "ka_rope_cache: unsupported dtype %d", dtype);
+    KA_LAUNCH_CHECK();
+    return 0;
+}

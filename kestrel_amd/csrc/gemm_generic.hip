@@ -1,0 +1,101 @@
+// Generic linear layer: out = act(A W^T + bias) or out += A W^T + bias.
+//
+// Plain FMA in fp32 with an LDS-tiled 64x64x16 block, any M, N, K, any mix of fp32
+// and bf16 operands. Every output element is the sum over k = 0..K-1 in that order,
+// whatever M and N are, so a row's result does not depend on what else is in the
+// batch. This is the true 32-bit path and the fallback of the bf16 path.
+#include "ka_common.h"
+
+constexpr int GT = 64;   // tile edge in M and N
+constexpr int GK = 16;   // tile depth
+
+template <typename TA, typename TW, typename TOut>
+__global__ void __launch_bounds__(256)
+gemm_generic_kernel(const TA* __restrict__ A, long lda, const TW* __restrict__ W, long ldw,
+                    const float* __restrict__ bias, TOut* __restrict__ out, long ldo, int M, int N,
+                    int K, int act, int accumulate) {
+    __shared__ float As[GK][GT + 4];
+    __shared__ float Ws[GK][GT + 4];
+    int tx = threadIdx.x % 16, ty = threadIdx.x / 16;
+    int m0 = blockIdx.y * GT, n0 = blockIdx.x * GT;
+    float acc[4][4] = {};
+    // Each thread loads 4 elements of each operand tile: row = tid / 4, k = (tid % 4) * 4 .. +4.
+    int lr = threadIdx.x / 4, lk = (threadIdx.x % 4) * 4;
+    for (int k0 = 0; k0 < K; k0 += GK) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            int k = k0 + lk + j;
+            int m = m0 + lr, n = n0 + lr;
+            As[lk + j][lr] = (m < M && k < K) ? ka_to_float(A[(size_t)m * lda + k]) : 0.f;
+            Ws[lk + j][lr] = (n < N && k < K) ? ka_to_float(W[(size_t)n * ldw + k]) : 0.f;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < GK; ++k) {
+            float a[4], w[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) a[i] = As[k][ty * 4 + i];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) w[j] = Ws[k][tx * 4 + j];
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], w[j], acc[i][j]);
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        int m = m0 + ty * 4 + i;
+        if (m >= M) continue;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            int n = n0 + tx * 4 + j;
+            if (n >= N) continue;
+            float v = acc[i][j] + (bias ? bias[n] : 0.f);
+            if (act == 1) v = ka_gelu_tanh(v);
+            size_t o = (size_t)m * ldo + n;
+            if (accumulate) v += ka_to_float(out[o]);
+            out[o] = ka_from_float<TOut>(v);
+        }
+    }
+}
+
+template <typename TA, typename TW, typename TOut>
+static void launch(const void* A, long lda, const void* W, long ldw, const float* bias, void* out,
+                   long ldo, int M, int N, int K, int act, int accumulate, hipStream_t stream) {
+    dim3 grid(ka_cdiv(N, GT), ka_cdiv(M, GT)), block(256);
+    hipLaunchKernelGGL((gemm_generic_kernel<TA, TW, TOut>), grid, block, 0, stream, (const TA*)A, lda,
+                       (const TW*)W, ldw, bias, (TOut*)out, ldo, M, N, K, act, accumulate);
+}
+
+// A: [M, K] rows lda apart; W: [N, K] rows ldw apart; bias: fp32 [N] or null;
+// out: [M, N] rows ldo apart. act: 0 none, 1 GELU-tanh. accumulate: out += result
+// (only into fp32 out).
+KA_API int ka_linear_generic(const void* A, int a_dtype, long lda, const void* W, int w_dtype,
+                             long ldw, const float* bias, void* out, int out_dtype, long ldo,
+                             int M, int N, int K, int act, int accumulate, hipStream_t stream) {
+    KA_CHECK(M >= 0 && N > 0 && K > 0, "ka_linear_generic: bad sizes M=%d N=%d K=%d", M, N, K);
+    KA_CHECK(lda >= K && ldw >= K && ldo >= N, "ka_linear_generic: strides too small");
+    KA_CHECK(act == 0 || act == 1, "ka_linear_generic: unknown activation %d", act);
+    KA_CHECK(!(accumulate && out_dtype != KA_F32), "ka_linear_generic: accumulate needs an fp32 output");
+    KA_CHECK(ka_cdiv(M, GT) <= 65535, "ka_linear_generic: M=%d too large for one launch", M);
+    if (M == 0) return 0;
+    int key = a_dtype * 4 + w_dtype * 2 + out_dtype;
+#define KA_CASE(k, TA, TW, TO) \
+    case k: launch<TA, TW, TO>(A, lda, W, ldw, bias, out, ldo, M, N, K, act, accumulate, stream); break;
+    switch (key) {
+        KA_CASE(0, float, float, float)
+        KA_CASE(1, float, float, bf16_t)
+        KA_CASE(2, float, bf16_t, float)
+        KA_CASE(3, float, bf16_t, bf16_t)
+        KA_CASE(4, bf16_t, float, float)
+        KA_CASE(5, bf16_t, float, bf16_t)
+        KA_CASE(6, bf16_t, bf16_t, float)
+        KA_CASE(7, bf16_t, bf16_t, bf16_t)
+        default: KA_CHECK(false, "ka_linear_generic: unsupported dtypes a=%d w=%d out=%d", a_dtype, w_dtype, out_dtype);
+    }
+#undef KA_CASE
+    KA_LAUNCH_CHECK();
+    return 0;
+}

@@ -1,0 +1,72 @@
+// Shared declarations of the kestrel_amd HIP kernels (gfx950 / CDNA4).
+//
+// Every entry point is `extern "C"`, takes raw device pointers, plain integers and
+// a hipStream_t, validates its sizes on the host and returns 0 on success or a
+// negative code; `ka_last_error()` then gives the reason as text. Entry points
+// never allocate and never synchronise.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#define KA_API extern "C" __attribute__((visibility("default")))
+
+// Element types of tensors crossing the C boundary.
+enum KaDType : int { KA_F32 = 0, KA_BF16 = 1 };
+
+typedef __bf16 bf16_t;
+
+constexpr int KA_WAVE = 64;
+
+// Error text of the last failed call in this thread (defined in elementwise.hip
+// for the core library; each library has its own copy).
+void ka_set_error(const char* fmt, ...);
+
+#define KA_CHECK(cond, ...)            \
+    do {                               \
+        if (!(cond)) {                 \
+            ka_set_error(__VA_ARGS__); \
+            return -1;                 \
+        }                              \
+    } while (0)
+
+#define KA_LAUNCH_CHECK()                                                        \
+    do {                                                                         \
+        hipError_t e__ = hipGetLastError();                                      \
+        if (e__ != hipSuccess) {                                                 \
+            ka_set_error("%s: launch failed: %s", __func__, hipGetErrorString(e__)); \
+            return -2;                                                           \
+        }                                                                        \
+    } while (0)
+
+__device__ __forceinline__ float ka_to_float(float v) { return v; }
+__device__ __forceinline__ float ka_to_float(bf16_t v) { return (float)v; }
+
+template <typename T>
+__device__ __forceinline__ T ka_from_float(float v);
+template <>
+__device__ __forceinline__ float ka_from_float<float>(float v) { return v; }
+template <>
+__device__ __forceinline__ bf16_t ka_from_float<bf16_t>(float v) { return (bf16_t)v; }
+
+__device__ __forceinline__ float ka_wave_sum(float v) {
+#pragma unroll
+    for (int off = KA_WAVE / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, KA_WAVE);
+    return v;
+}
+
+__device__ __forceinline__ float ka_wave_max(float v) {
+#pragma unroll
+    for (int off = KA_WAVE / 2; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, KA_WAVE));
+    return v;
+}
+
+// GELU with the tanh approximation: 0.5 x (1 + tanh(sqrt(2/pi) (x + 0.044715 x^3))).
+__device__ __forceinline__ float ka_gelu_tanh(float x) {
+    const float k0 = 0.7978845608028654f;
+    const float k1 = 0.044715f;
+    float inner = k0 * (x + k1 * x * x * x);
+    return 0.5f * x * (1.0f + tanhf(inner));
+}
+
+static inline int ka_cdiv(long a, long b) { return (int)((a + b - 1) / b); }

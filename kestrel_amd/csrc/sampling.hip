@@ -1,0 +1,186 @@
+// Token selection from fp32 logits: argmax, and temperature + top-p sampling.
+//
+// One workgroup of 1024 threads per row. A row with temperature <= 1e-6 is greedy
+// (the first index of the maximum). Otherwise the distribution is
+// softmax(logits / T) restricted to the smallest set of most probable tokens whose
+// mass reaches top_p, found by bisection on the probability threshold; the token is
+// drawn by inversion with a uniform number from a counter-based generator keyed by
+// (rng_key[row], rng_counter[row]), so a request's draws do not depend on what else
+// is in the batch. Logits of value -inf are never chosen.
+#include "ka_common.h"
+
+constexpr int SM_THREADS = 1024;
+constexpr int SM_WAVES = SM_THREADS / KA_WAVE;
+constexpr float SM_GREEDY_EPS = 1e-6f;
+
+__device__ __forceinline__ float block_reduce_sum(float v, float* smem) {
+    v = ka_wave_sum(v);
+    __syncthreads();
+    if (threadIdx.x % KA_WAVE == 0) smem[threadIdx.x / KA_WAVE] = v;
+    __syncthreads();
+    float t = 0.f;
+#pragma unroll
+    for (int w = 0; w < SM_WAVES; ++w) t += smem[w];
+    return t;
+}
+
+__device__ __forceinline__ float block_reduce_max(float v, float* smem) {
+    v = ka_wave_max(v);
+    __syncthreads();
+    if (threadIdx.x % KA_WAVE == 0) smem[threadIdx.x / KA_WAVE] = v;
+    __syncthreads();
+    float t = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < SM_WAVES; ++w) t = fmaxf(t, smem[w]);
+    return t;
+}
+
+// splitmix64 of (key + counter * odd constant): uniform in [0, 1) with 24 bits.
+__host__ __device__ inline float ka_uniform(unsigned long long key, unsigned long long counter) {
+    unsigned long long z = key + 0x9E3779B97F4A7C15ull * (counter + 1ull);
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    z = z ^ (z >> 31);
+    return (float)(z >> 40) * (1.0f / 16777216.0f);
+}
+
+// Index of the maximum (lowest index on ties) of one row, by all threads.
+__device__ int block_argmax(const float* __restrict__ row, int V, float* smem_f, int* smem_i) {
+    float best = -INFINITY;
+    int best_i = 0x7fffffff;
+    for (int i = threadIdx.x; i < V; i += SM_THREADS) {
+        float v = row[i];
+        if (v > best || (v == best && i < best_i)) { best = v; best_i = i; }
+    }
+#pragma unroll
+    for (int off = KA_WAVE / 2; off > 0; off >>= 1) {
+        float ov = __shfl_xor(best, off, KA_WAVE);
+        int oi = __shfl_xor(best_i, off, KA_WAVE);
+        if (ov > best || (ov == best && oi < best_i)) { best = ov; best_i = oi; }
+    }
+    __syncthreads();
+    if (threadIdx.x % KA_WAVE == 0) { smem_f[threadIdx.x / KA_WAVE] = best; smem_i[threadIdx.x / KA_WAVE] = best_i; }
+    __syncthreads();
+    best = smem_f[0]; best_i = smem_i[0];
+    for (int w = 1; w < SM_WAVES; ++w) {
+        float ov = smem_f[w]; int oi = smem_i[w];
+        if (ov > best || (ov == best && oi < best_i)) { best = ov; best_i = oi; }
+    }
+    if (best_i == 0x7fffffff) best_i = 0;
+    return best_i;
+}
+
+__global__ void __launch_bounds__(SM_THREADS)
+argmax_kernel(const float* __restrict__ logits, long ld, int* __restrict__ out, int V) {
+    __shared__ float sf[SM_WAVES];
+    __shared__ int si[SM_WAVES];
+    int r = blockIdx.x;
+    int idx = block_argmax(logits + (size_t)r * ld, V, sf, si);
+    if (threadIdx.x == 0) out[r] = idx;
+}
+
+__global__ void __launch_bounds__(SM_THREADS)
+sample_kernel(const float* __restrict__ logits, long ld, const float* __restrict__ temps,
+              const float* __restrict__ top_ps, const unsigned long long* __restrict__ rng_key,
+              const int* __restrict__ rng_counter, int* __restrict__ out, int V) {
+    __shared__ float sf[SM_WAVES];
+    __shared__ int si[SM_WAVES];
+    __shared__ float wave_tot[SM_WAVES];
+    __shared__ int found_idx;
+    int r = blockIdx.x;
+    const float* row = logits + (size_t)r * ld;
+    float T = temps[r];
+    int greedy = block_argmax(row, V, sf, si);
+    if (!(T > SM_GREEDY_EPS)) {
+        if (threadIdx.x == 0) out[r] = greedy;
+        return;
+    }
+    float inv_t = 1.0f / T;
+    float mx = row[greedy];
+    float z = 0.f;
+    for (int i = threadIdx.x; i < V; i += SM_THREADS) z += expf((row[i] - mx) * inv_t);
+    z = block_reduce_sum(z, sf);
+    float inv_z = 1.0f / z;
+    float top_p = top_ps ? top_ps[r] : 1.0f;
+    float thresh = 0.f, mass = 1.0f;
+    if (top_p < 1.0f) {
+        // f(t) = mass of {p >= t} falls with t; keep the largest t with f(t) >= top_p.
+        float lo = 0.f, hi = 1.0f + 1e-6f;
+        for (int it = 0; it < 30; ++it) {
+            float mid = 0.5f * (lo + hi);
+            float f = 0.f;
+            for (int i = threadIdx.x; i < V; i += SM_THREADS) {
+                float p = expf((row[i] - mx) * inv_t) * inv_z;
+                if (p >= mid) f += p;
+            }
+            f = block_reduce_sum(f, sf);
+            if (f >= top_p) lo = mid; else hi = mid;
+        }
+        thresh = lo;
+        float f = 0.f;
+        for (int i = threadIdx.x; i < V; i += SM_THREADS) {
+            float p = expf((row[i] - mx) * inv_t) * inv_z;
+            if (p >= thresh) f += p;
+        }
+        mass = block_reduce_sum(f, sf);
+    }
+    float u = ka_uniform(rng_key[r], (unsigned long long)(unsigned)rng_counter[r]);
+    float target = u * mass;
+    // Inversion in index order: first i with cumulative mass > target.
+    if (threadIdx.x == 0) found_idx = -1;
+    __syncthreads();
+    float running = 0.f;
+    int lane = threadIdx.x % KA_WAVE, wave = threadIdx.x / KA_WAVE;
+    for (int base = 0; base < V; base += SM_THREADS) {
+        int i = base + threadIdx.x;
+        float p = 0.f;
+        if (i < V) {
+            p = expf((row[i] - mx) * inv_t) * inv_z;
+            if (p < thresh || p <= 0.f) p = 0.f;
+        }
+        // inclusive scan inside the wave
+        float scan = p;
+#pragma unroll
+        for (int off = 1; off < KA_WAVE; off <<= 1) {
+            float o = __shfl_up(scan, off, KA_WAVE);
+            if (lane >= off) scan += o;
+        }
+        __syncthreads();
+        if (lane == KA_WAVE - 1) wave_tot[wave] = scan;
+        __syncthreads();
+        float before = running;
+        for (int w = 0; w < wave; ++w) before += wave_tot[w];
+        float chunk = 0.f;
+#pragma unroll
+        for (int w = 0; w < SM_WAVES; ++w) chunk += wave_tot[w];
+        float incl = before + scan;
+        if (p > 0.f && incl > target && incl - p <= target) atomicMax(&found_idx, i);
+        running += chunk;
+        __syncthreads();
+        if (found_idx >= 0) break;
+    }
+    if (threadIdx.x == 0) out[r] = found_idx >= 0 ? found_idx : greedy;
+}
+
+KA_API int ka_argmax(const float* logits, long ld, int* out, int rows, int V, hipStream_t stream) {
+    KA_CHECK(rows >= 0 && V > 0 && ld >= V, "ka_argmax: bad sizes rows=%d V=%d ld=%ld", rows, V, ld);
+    if (rows == 0) return 0;
+    hipLaunchKernelGGL(argmax_kernel, dim3(rows), dim3(SM_THREADS), 0, stream, logits, ld, out, V);
+    KA_LAUNCH_CHECK();
+    return 0;
+}
+
+KA_API int ka_sample(const float* logits, long ld, const float* temps, const float* top_ps,
+                     const unsigned long long* rng_key, const int* rng_counter, int* out, int rows,
+                     int V, hipStream_t stream) {
+    KA_CHECK(rows >= 0 && V > 0 && ld >= V, "ka_sample: bad sizes rows=%d V=%d ld=%ld", rows, V, ld);
+    KA_CHECK(temps && rng_key && rng_counter, "ka_sample: temperatures and generator state are required");
+    if (rows == 0) return 0;
+    hipLaunchKernelGGL(sample_kernel, dim3(rows), dim3(SM_THREADS), 0, stream, logits, ld, temps, top_ps, rng_key,
+                       rng_counter, out, V);
+    KA_LAUNCH_CHECK();
+    return 0;
+}
+
+// The uniform number the kernel draws, for tests and host-side replay.
+KA_API float ka_uniform_host(unsigned long long key, unsigned long long counter) { return ka_uniform(key, counter); }

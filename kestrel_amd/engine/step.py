@@ -1,0 +1,245 @@
+"""The step function: one batch of (request, its next tokens) through the model.
+
+A step takes, for any number of live requests, the next tokens of each: a portion of
+a prompt (cut anywhere) or one decoded token, all packed into one token stream. It
+runs only these tokens, reading what earlier steps left in the cache, and returns the
+logits at the places asked for. The reference runs either padded whole prompts
+(``kestrel/models/moondream/runtime.py:1999-2157``) or one token per row
+(``runtime.py:2479-2586``); its metadata (slot mapping ``kv_cache.py:524-551``, per-row
+block table and key counts ``runtime.py:2283-2290``) is what is built here per token.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import torch
+
+from ..cache.manager import CacheManager
+from ..models.decoder import DecoderModel
+from .batch import GroupBatch, StepBatch, Workspace
+
+
+@dataclass
+class StepEntry:
+    """The next tokens of one request.
+
+    ``tokens``: ids; ``-1`` marks a place whose embedding is given in ``embeds`` (rows in
+    order of the ``-1`` places). ``want``: indices into ``tokens`` whose logits are returned.
+    ``bidirectional``: position ranges ``[lo, hi)`` whose tokens see each other both ways
+    (an image block); each must lie wholly inside this portion. ``start``: position of the
+    first token; ``None`` means right after what the request already holds.
+    """
+
+    slot: int
+    tokens: Sequence[int]
+    want: Sequence[int] = ()
+    embeds: Optional[torch.Tensor] = None
+    bidirectional: Sequence[Tuple[int, int]] = ()
+    start: Optional[int] = None
+
+
+def _align(n: int) -> int:
+    return (n + 3) & ~3
+
+
+class ModelRunner:
+    """Owns the model, its cache and the scratch memory; ``step`` is the only way in."""
+
+    STAGING_RING = 4
+
+    def __init__(self, model: DecoderModel, cache: CacheManager, device: torch.device,
+                 max_tokens_per_step: int = 4096) -> None:
+        self.model, self.cache, self.device = model, cache, device
+        self.max_tokens_per_step = max_tokens_per_step
+        self.workspace = Workspace(device)
+        self.layer_caches = cache.layer_caches()
+        self.held: Dict[int, int] = {}            # slot -> tokens the request holds in the cache
+        self._staging: List[Optional[torch.Tensor]] = [None] * self.STAGING_RING
+        self._staging_events: List[Optional[torch.cuda.Event]] = [None] * self.STAGING_RING
+        self._staging_next = 0
+        self._meta_device: Optional[torch.Tensor] = None
+
+    # ------------------------------------------------------------------ requests
+    def admit(self, reserve_length: int = 0, portion: int = 1) -> int:
+        slot = self.cache.admit(reserve_length, portion)
+        self.held[slot] = 0
+        return slot
+
+    def release(self, slot: int) -> None:
+        self.cache.release(slot)
+        del self.held[slot]
+
+    # ------------------------------------------------------------------ metadata
+    def _stage(self, count: int) -> Tuple[torch.Tensor, int]:
+        index = self._staging_next
+        self._staging_next = (index + 1) % self.STAGING_RING
+        event = self._staging_events[index]
+        if event is not None:
+            event.synchronize()
+        buf = self._staging[index]
+        if buf is None or buf.numel() < count:
+            buf = torch.empty(max(count, 4096), dtype=torch.int32, pin_memory=True)
+            self._staging[index] = buf
+        return buf, index
+
+    def build_batch(self, entries: Sequence[StepEntry]) -> StepBatch:
+        """Checks the entries, backs their positions with pages and lays the metadata out."""
+        cache, plan = self.cache, self.model.plan
+        ps = cache.page_size
+        if not entries:
+            raise ValueError("a step needs at least one entry")
+        seen = set()
+        starts: List[int] = []
+        n_tokens = 0
+        for e in entries:
+            if e.slot in seen:
+                raise ValueError(f"slot {e.slot} appears twice in one step")
+            seen.add(e.slot)
+            if e.slot not in self.held:
+                raise ValueError(f"slot {e.slot} is not live")
+            if len(e.tokens) == 0:
+                raise ValueError(f"slot {e.slot}: an entry needs at least one token")
+            start = self.held[e.slot] if e.start is None else int(e.start)
+            if start != self.held[e.slot]:
+                raise ValueError(f"slot {e.slot}: portion starts at {start} but the request holds {self.held[e.slot]} tokens")
+            if start + len(e.tokens) > plan.max_positions:
+                raise ValueError(f"slot {e.slot}: {start + len(e.tokens)} tokens exceed the model's {plan.max_positions} positions")
+            starts.append(start)
+            n_tokens += len(e.tokens)
+        if n_tokens > self.max_tokens_per_step:
+            raise ValueError(f"{n_tokens} tokens in one step exceed the limit of {self.max_tokens_per_step}")
+        for e, start in zip(entries, starts):
+            cache.ensure(e.slot, start + len(e.tokens))
+
+        n_rows = len(entries)
+        n_groups = len(cache.groups)
+        ids: List[int] = []
+        positions: List[int] = []
+        token_row: List[int] = []
+        kv_hi: List[int] = []
+        logit_rows: List[int] = []
+        given_rows: List[int] = []
+        given: List[torch.Tensor] = []
+        cu_q = [0]
+        kv_len: List[int] = []
+        slots: List[List[int]] = [[] for _ in range(n_groups)]
+        kv_lo: List[Optional[List[int]]] = [[] if g.spec.window is not None else None for g in cache.groups]
+        max_pages = 1
+        max_q = max_kv = 1
+        causal_only = True
+        for r, (e, start) in enumerate(zip(entries, starts)):
+            q = len(e.tokens)
+            base = len(ids)
+            hi = [start + i + 1 for i in range(q)]
+            for lo_b, hi_b in e.bidirectional:
+                if not (start <= lo_b < hi_b <= start + q):
+                    raise ValueError(f"slot {e.slot}: the bidirectional block [{lo_b}, {hi_b}) must lie inside one "
+                                     f"portion, this one covers [{start}, {start + q})")
+                for p in range(lo_b, hi_b):
+                    hi[p - start] = max(hi[p - start], hi_b)
+                causal_only = False
+            n_given = 0
+            for i, tok in enumerate(e.tokens):
+                tok = int(tok)
+                if tok < 0:
+                    given_rows.append(base + i)
+                    n_given += 1
+                    tok = -1
+                elif tok >= plan.vocab_size:
+                    raise ValueError(f"slot {e.slot}: token id {tok} outside the vocabulary of {plan.vocab_size}")
+                ids.append(tok)
+            if n_given:
+                if e.embeds is None or e.embeds.dim() != 2 or tuple(e.embeds.shape) != (n_given, plan.dim):
+                    raise ValueError(f"slot {e.slot}: {n_given} places need embeddings of shape [{n_given}, {plan.dim}]")
+                given.append(e.embeds)
+            elif e.embeds is not None and e.embeds.numel():
+                raise ValueError(f"slot {e.slot}: embeddings given but no token id is -1")
+            positions.extend(range(start, start + q))
+            token_row.extend([r] * q)
+            kv_hi.extend(hi)
+            for w in e.want:
+                if not 0 <= int(w) < q:
+                    raise ValueError(f"slot {e.slot}: wanted place {w} outside its {q} tokens")
+                logit_rows.append(base + int(w))
+            cu_q.append(base + q)
+            kv_len.append(start + q)
+            max_q, max_kv = max(max_q, q), max(max_kv, start + q)
+            for g in range(n_groups):
+                table = cache.block_table(g, e.slot)
+                max_pages = max(max_pages, len(table))
+                slots[g].extend(table[p // ps] * ps + p % ps for p in range(start, start + q))
+                if kv_lo[g] is not None:
+                    kv_lo[g].extend(cache.window_start(g, p) for p in range(start, start + q))
+
+        # one packed int32 buffer: [ids | positions | token_row | kv_hi | row_slot | cu_q | kv_len | logit_rows |
+        #                           given_rows | per group: slots, kv_lo, block_table]
+        sections: List[Tuple[str, List[int]]] = [
+            ("ids", ids), ("positions", positions), ("token_row", token_row), ("kv_hi", kv_hi),
+            ("row_slot", [e.slot for e in entries]), ("cu_q", cu_q), ("kv_len", kv_len), ("logit_rows", logit_rows),
+            ("given_rows", given_rows),
+        ]
+        for g in range(n_groups):
+            sections.append((f"slots{g}", slots[g]))
+            if kv_lo[g] is not None:
+                sections.append((f"kv_lo{g}", kv_lo[g]))
+            flat: List[int] = []
+            for e in entries:
+                table = cache.block_table(g, e.slot)
+                flat.extend(table)
+                flat.extend([-1] * (max_pages - len(table)))
+            sections.append((f"table{g}", flat))
+        offsets: Dict[str, Tuple[int, int]] = {}
+        total = 0
+        for name, values in sections:
+            offsets[name] = (total, len(values))
+            total += _align(len(values))
+        staging, ring = self._stage(total)
+        host = staging.numpy()
+        for name, values in sections:
+            off, count = offsets[name]
+            if count:
+                host[off:off + count] = values
+        if self._meta_device is None or self._meta_device.numel() < total:
+            self._meta_device = torch.empty(max(total, 4096), dtype=torch.int32, device=self.device)
+        meta = self._meta_device
+        meta[:total].copy_(staging[:total], non_blocking=True)
+        event = self._staging_events[ring] or torch.cuda.Event()
+        event.record()
+        self._staging_events[ring] = event
+
+        def view(name: str) -> torch.Tensor:
+            off, count = offsets[name]
+            return meta[off:off + count]
+
+        groups: Dict[int, GroupBatch] = {}
+        for g in range(n_groups):
+            groups[g] = GroupBatch(block_table=view(f"table{g}").view(n_rows, max_pages), slots=view(f"slots{g}"),
+                                   kv_lo=view(f"kv_lo{g}") if kv_lo[g] is not None else None, page_size=ps)
+        given_embeds = None
+        if given:
+            given_embeds = torch.cat([t.to(self.device) for t in given], dim=0).contiguous()
+            if given_embeds.dtype not in (torch.float32, torch.bfloat16):
+                given_embeds = given_embeds.float()
+        return StepBatch(
+            n_tokens=n_tokens, n_rows=n_rows, token_ids=view("ids"), positions=view("positions"),
+            token_row=view("token_row"), kv_hi=view("kv_hi"), row_slot=view("row_slot"), cu_q=view("cu_q"),
+            kv_len=view("kv_len"), logit_rows=view("logit_rows"), groups=groups, workspace=self.workspace,
+            given_embeds=given_embeds, given_rows=view("given_rows") if given else None, max_q=max_q, max_kv=max_kv,
+            decode_only=max_q == 1, causal_only=causal_only,
+            host={"starts": starts, "q_lens": [len(e.tokens) for e in entries], "kv_len": kv_len},
+        )
+
+    # ------------------------------------------------------------------ the step
+    @torch.inference_mode()
+    def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
+        """Run the entries as one batch. Returns fp32 logits ``[wanted, vocab]`` in the order of
+        the entries and of their ``want``; the tensor is scratch memory and is overwritten by
+        the next step."""
+        batch = self.build_batch(entries)
+        logits = self.model.forward(batch, self.layer_caches)
+        for e, start in zip(entries, batch.host["starts"]):
+            self.held[e.slot] = start + len(e.tokens)
+            self.cache.trim(e.slot, self.held[e.slot])
+        return logits

@@ -1,0 +1,94 @@
+"""The generic decoder: embedding, the scheduled blocks, final norm and head.
+
+It is put together from a ``ModelPlan`` alone and knows no architecture. The order of
+execution is the plan's ``schedule``: a list of runs, each naming a layer (a layer may be
+named twice and then shares its weights) and optionally an earlier run whose cache it
+reads instead of keeping one.
+"""
+
+from __future__ import annotations
+
+from typing import Dict, List, Optional
+
+import torch
+
+from ..ops import core
+from ..ops.linear import linear
+from ..parts.base import LayerCache, build_part
+from ..parts.block import Block
+from ..parts.specs import ModelPlan, ParamSpec
+
+
+class DecoderModel:
+    def __init__(self, plan: ModelPlan) -> None:
+        self.plan = plan
+        self.blocks: List[Block] = [Block(layer) for layer in plan.layers]
+        self.final_norm = build_part("norm", plan.final_norm)
+        for index, entry in enumerate(plan.schedule):
+            if not 0 <= entry.layer < len(self.blocks):
+                raise ValueError(f"schedule entry {index} names layer {entry.layer}, the plan has {len(self.blocks)}")
+            if entry.reads_cache_of is not None:
+                if not 0 <= entry.reads_cache_of < index:
+                    raise ValueError(f"schedule entry {index} must read the cache of an earlier entry")
+                if plan.schedule[entry.reads_cache_of].reads_cache_of is not None:
+                    raise ValueError(f"schedule entry {index} reads the cache of an entry that keeps none")
+        self.embedding: Optional[torch.Tensor] = None
+        self.head_weight: Optional[torch.Tensor] = None
+        self.head_bias: Optional[torch.Tensor] = None
+        self.dtype: Optional[torch.dtype] = None
+        self.device: Optional[torch.device] = None
+
+    # ------------------------------------------------------------------ tensors
+    def params(self) -> Dict[str, ParamSpec]:
+        """Checkpoint tensor name -> shape and role of every tensor the model owns."""
+        plan = self.plan
+        out = {plan.names["embedding"]: ParamSpec((plan.vocab_size, plan.dim), "matrix", "normal")}
+        for block in self.blocks:
+            out.update(block.params())
+        for local, pspec in self.final_norm.params().items():
+            out[plan.names[f"final_norm.{local}"]] = pspec
+        if not plan.tied_head:
+            out[plan.names["head.weight"]] = ParamSpec((plan.vocab_size, plan.dim), "matrix", "normal")
+        if plan.head_bias:
+            out[plan.names["head.bias"]] = ParamSpec((plan.vocab_size,), "vector", "bias")
+        return out
+
+    def bind(self, tensors: Dict[str, torch.Tensor], dtype: torch.dtype, device: torch.device) -> None:
+        plan = self.plan
+        self.dtype, self.device = dtype, device
+        self.embedding = tensors[plan.names["embedding"]].to(device).contiguous()
+        for block in self.blocks:
+            block.bind(tensors, dtype, device)
+        self.final_norm.bind({k: tensors[plan.names[f"final_norm.{k}"]] for k in self.final_norm.params()}, dtype,
+                             device)
+        self.head_weight = self.embedding if plan.tied_head else tensors[plan.names["head.weight"]].to(device).contiguous()
+        if plan.head_bias:
+            self.head_bias = tensors[plan.names["head.bias"]].to(device=device, dtype=torch.float32).contiguous()
+
+    # ------------------------------------------------------------------ cache needs
+    def cache_needs(self):
+        """Per schedule entry: ``(cache_spec or None, state_spec or None, reads_cache_of)``."""
+        needs = []
+        for entry in self.plan.schedule:
+            mixer = self.blocks[entry.layer].mixer
+            needs.append((mixer.cache_spec(), mixer.state_spec(), entry.reads_cache_of))
+        return needs
+
+    # ------------------------------------------------------------------ forward
+    def forward(self, batch, caches: List[LayerCache]) -> torch.Tensor:
+        """Run the packed tokens of ``batch``; returns fp32 logits ``[wanted, vocab]``."""
+        plan = self.plan
+        ws = batch.workspace
+        x = ws.get("model.x", (batch.n_tokens, plan.dim), torch.float32)
+        core.embed(self.embedding, batch.token_ids, x)
+        if batch.given_embeds is not None:
+            core.scatter_rows(batch.given_embeds, batch.given_rows, x)
+        for index, entry in enumerate(plan.schedule):
+            self.blocks[entry.layer].forward(x, batch, caches[index])
+        wanted = int(batch.logit_rows.numel())
+        logits = ws.get("model.logits", (wanted, plan.vocab_size), torch.float32)
+        if wanted:
+            normed = ws.get("model.head_in", (wanted, plan.dim), self.dtype)
+            self.final_norm.forward(x, normed, rows=batch.logit_rows)
+            linear(normed, self.head_weight, self.head_bias, logits)
+        return logits

@@ -1,0 +1,232 @@
+"""Python faces of the generic HIP kernels (library ``core``).
+
+Each function checks what the kernel assumes about its operands (device, type,
+contiguity, sizes), then passes raw pointers and the current HIP stream to the C
+entry point. Nothing here computes on the CPU and nothing falls back to a library.
+"""
+
+from __future__ import annotations
+
+import ctypes
+from typing import Optional
+
+import torch
+
+from ..csrc import build as _build
+
+KA_F32, KA_BF16 = 0, 1
+_DTYPE_CODE = {torch.float32: KA_F32, torch.bfloat16: KA_BF16}
+
+_c_void_p, _c_int, _c_long, _c_float = ctypes.c_void_p, ctypes.c_int, ctypes.c_long, ctypes.c_float
+
+_SIGNATURES = {
+    "ka_embed": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_void_p],
+    "ka_scatter_rows": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_void_p],
+    "ka_layernorm": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_float, _c_void_p, _c_int, _c_int, _c_int,
+                     _c_void_p],
+    "ka_rope_cache": [_c_void_p, _c_int, _c_long, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p,
+                      _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
+    "ka_linear_generic": [_c_void_p, _c_int, _c_long, _c_void_p, _c_int, _c_long, _c_void_p, _c_void_p, _c_int,
+                          _c_long, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
+    "ka_attention_generic": [_c_void_p, _c_int, _c_long, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p,
+                             _c_void_p, _c_void_p, _c_void_p, _c_long, _c_float, _c_int, _c_int, _c_int, _c_int,
+                             _c_int, _c_void_p],
+    "ka_argmax": [_c_void_p, _c_long, _c_void_p, _c_int, _c_int, _c_void_p],
+    "ka_sample": [_c_void_p, _c_long, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int,
+                  _c_void_p],
+}
+
+_lib = None
+
+
+class KernelError(RuntimeError):
+    """A HIP entry point refused its arguments or failed to launch."""
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        handle = _build.load("core")
+        for name, argtypes in _SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.argtypes = argtypes
+            fn.restype = _c_int
+        handle.ka_last_error.restype = ctypes.c_char_p
+        handle.ka_uniform_host.argtypes = [ctypes.c_ulonglong, ctypes.c_ulonglong]
+        handle.ka_uniform_host.restype = _c_float
+        _lib = handle
+    return _lib
+
+
+def _check(status: int, handle=None) -> None:
+    if status != 0:
+        handle = handle or lib()
+        raise KernelError(handle.ka_last_error().decode())
+
+
+def stream_ptr() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def code_of(dtype: torch.dtype) -> int:
+    try:
+        return _DTYPE_CODE[dtype]
+    except KeyError:
+        raise KernelError(f"unsupported tensor type {dtype}: the kernels take float32 and bfloat16") from None
+
+
+def _need(cond: bool, message: str) -> None:
+    if not cond:
+        raise KernelError(message)
+
+
+def _dev(*tensors) -> None:
+    for t in tensors:
+        if t is not None:
+            _need(t.is_cuda, "kernel operand is not on the GPU")
+
+
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def uniform(key: int, counter: int) -> float:
+    """The uniform number the sampling kernel draws for (key, counter)."""
+    return float(lib().ka_uniform_host(key & (2 ** 64 - 1), counter))
+
+
+def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor) -> None:
+    """``out[t] = table[ids[t]]`` in fp32; rows with a negative id are left untouched."""
+    _dev(table, ids, out)
+    n, dim = out.shape
+    _need(table.dim() == 2 and table.shape[1] == dim and table.is_contiguous(), "embed: table must be [vocab, dim]")
+    _need(ids.dtype == torch.int32 and ids.numel() == n and ids.is_contiguous(), "embed: ids must be int32 [n]")
+    _need(out.dtype == torch.float32 and out.is_contiguous(), "embed: out must be contiguous fp32")
+    _check(lib().ka_embed(table.data_ptr(), code_of(table.dtype), ids.data_ptr(), out.data_ptr(), n, dim,
+                          stream_ptr()))
+
+
+def scatter_rows(src: torch.Tensor, rows: torch.Tensor, out: torch.Tensor) -> None:
+    """``out[rows[i]] = src[i]`` in fp32 (given embeddings spliced into the stream)."""
+    _dev(src, rows, out)
+    m, dim = src.shape
+    _need(out.dim() == 2 and out.shape[1] == dim and out.dtype == torch.float32 and out.is_contiguous(),
+          "scatter_rows: out must be contiguous fp32 [n, dim]")
+    _need(src.is_contiguous(), "scatter_rows: src must be contiguous")
+    _need(rows.dtype == torch.int32 and rows.numel() == m and rows.is_contiguous(), "scatter_rows: rows int32 [m]")
+    _check(lib().ka_scatter_rows(src.data_ptr(), code_of(src.dtype), rows.data_ptr(), out.data_ptr(), m, dim,
+                                 stream_ptr()))
+
+
+def layernorm(x: torch.Tensor, gamma: torch.Tensor, beta: Optional[torch.Tensor], eps: float, out: torch.Tensor,
+              rows: Optional[torch.Tensor] = None) -> None:
+    """LayerNorm of fp32 rows of ``x`` (all, or those named by ``rows``) into ``out``."""
+    _dev(x, gamma, beta, out, rows)
+    n, dim = out.shape
+    _need(x.dtype == torch.float32 and x.dim() == 2 and x.shape[1] == dim and x.is_contiguous(),
+          "layernorm: x must be contiguous fp32 [*, dim]")
+    _need(gamma.dtype == torch.float32 and gamma.numel() == dim, "layernorm: gamma must be fp32 [dim]")
+    _need(beta is None or (beta.dtype == torch.float32 and beta.numel() == dim), "layernorm: beta must be fp32 [dim]")
+    _need(out.is_contiguous(), "layernorm: out must be contiguous")
+    if rows is None:
+        _need(x.shape[0] == n, "layernorm: row counts differ")
+    else:
+        _need(rows.dtype == torch.int32 and rows.numel() == n and rows.is_contiguous(), "layernorm: rows int32 [n]")
+    _check(lib().ka_layernorm(x.data_ptr(), _ptr(rows), gamma.data_ptr(), _ptr(beta), float(eps), out.data_ptr(),
+                              code_of(out.dtype), n, dim, stream_ptr()))
+
+
+def rope_cache(qkv: torch.Tensor, positions: torch.Tensor, slots: Optional[torch.Tensor],
+               table: Optional[torch.Tensor], k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor],
+               n_heads: int, n_kv_heads: int, head_dim: int, page_size: int) -> None:
+    """Rotate q in place and write rotated k and v into the paged cache.
+
+    ``qkv``: ``[n, (H + 2 Hkv) hd]``; ``table``: fp32 ``[positions, R]`` or ``None`` for no
+    rotation; caches ``[pages, Hkv, page_size, hd]``; ``slots`` ``None`` writes nothing.
+    """
+    _dev(qkv, positions, slots, table, k_cache, v_cache)
+    n = qkv.shape[0]
+    _need(qkv.dim() == 2 and qkv.stride(1) == 1 and qkv.shape[1] == (n_heads + 2 * n_kv_heads) * head_dim,
+          "rope_cache: qkv must be [n, (H + 2 Hkv) hd]")
+    _need(positions.dtype == torch.int32 and positions.numel() == n and positions.is_contiguous(),
+          "rope_cache: positions int32 [n]")
+    rot, rows = 0, 0
+    if table is not None:
+        _need(table.dtype == torch.float32 and table.dim() == 2 and table.is_contiguous(),
+              "rope_cache: table must be contiguous fp32 [positions, R]")
+        rows, rot = table.shape
+    if slots is not None:
+        _need(slots.dtype == torch.int32 and slots.numel() == n and slots.is_contiguous(), "rope_cache: slots int32 [n]")
+        _need(k_cache is not None and v_cache is not None, "rope_cache: cache tensors missing")
+        for c in (k_cache, v_cache):
+            _need(c.dtype == qkv.dtype and c.is_contiguous() and c.dim() == 4
+                  and tuple(c.shape[1:]) == (n_kv_heads, page_size, head_dim),
+                  "rope_cache: cache must be [pages, Hkv, page_size, hd] of the qkv type")
+    _check(lib().ka_rope_cache(qkv.data_ptr(), code_of(qkv.dtype), qkv.stride(0), positions.data_ptr(), _ptr(slots),
+                               _ptr(table), rows, _ptr(k_cache), _ptr(v_cache), n, n_heads, n_kv_heads, head_dim,
+                               rot, page_size, stream_ptr()))
+
+
+def linear_generic(a: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,
+                   act: int = 0, accumulate: bool = False) -> None:
+    """``out = act(a @ weight.T + bias)`` or ``out += ...``; plain fp32 FMA, any sizes and type mix."""
+    _dev(a, weight, bias, out)
+    m, k = a.shape
+    n = weight.shape[0]
+    _need(weight.dim() == 2 and weight.shape[1] == k, f"linear: weight {tuple(weight.shape)} does not match K={k}")
+    _need(out.dim() == 2 and tuple(out.shape) == (m, n), f"linear: out {tuple(out.shape)} is not [{m}, {n}]")
+    _need(a.stride(1) == 1 and weight.stride(1) == 1 and out.stride(1) == 1, "linear: rows must be contiguous")
+    _need(bias is None or (bias.dtype == torch.float32 and bias.numel() == n and bias.is_contiguous()),
+          "linear: bias must be fp32 [N]")
+    _check(lib().ka_linear_generic(a.data_ptr(), code_of(a.dtype), a.stride(0), weight.data_ptr(),
+                                   code_of(weight.dtype), weight.stride(0), _ptr(bias), out.data_ptr(),
+                                   code_of(out.dtype), out.stride(0), m, n, k, act, int(accumulate), stream_ptr()))
+
+
+def attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
+                      token_row: torch.Tensor, kv_lo: Optional[torch.Tensor], kv_hi: torch.Tensor,
+                      out: torch.Tensor, scale: float, n_heads: int, n_kv_heads: int, head_dim: int) -> None:
+    """Paged attention of ``n`` packed tokens; ``q`` may be a strided view into a qkv buffer."""
+    _dev(q, k_cache, v_cache, block_table, token_row, kv_lo, kv_hi, out)
+    n = q.shape[0]
+    _need(q.dim() == 2 and q.stride(1) == 1 and q.shape[1] >= n_heads * head_dim, "attention: q must be [n, >= H hd]")
+    _need(out.dim() == 2 and out.stride(1) == 1 and tuple(out.shape) == (n, n_heads * head_dim) and out.dtype == q.dtype,
+          "attention: out must be [n, H hd] of the q type")
+    page_size = k_cache.shape[2]
+    for c in (k_cache, v_cache):
+        _need(c.dtype == q.dtype and c.is_contiguous() and c.dim() == 4
+              and tuple(c.shape[1:]) == (n_kv_heads, page_size, head_dim),
+              "attention: cache must be [pages, Hkv, page_size, hd] of the q type")
+    _need(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.is_contiguous(),
+          "attention: block table must be contiguous int32 [rows, pages]")
+    for t in (token_row, kv_hi) + ((kv_lo,) if kv_lo is not None else ()):
+        _need(t.dtype == torch.int32 and t.numel() == n and t.is_contiguous(), "attention: per-token int32 [n] expected")
+    _check(lib().ka_attention_generic(q.data_ptr(), code_of(q.dtype), q.stride(0), k_cache.data_ptr(),
+                                      v_cache.data_ptr(), block_table.data_ptr(), block_table.shape[1],
+                                      token_row.data_ptr(), _ptr(kv_lo), kv_hi.data_ptr(), out.data_ptr(),
+                                      out.stride(0), float(scale), n, n_heads, n_kv_heads, head_dim, page_size,
+                                      stream_ptr()))
+
+
+def argmax(logits: torch.Tensor, out: torch.Tensor) -> None:
+    """Index of the largest logit of every fp32 row into int32 ``out``."""
+    _dev(logits, out)
+    rows, vocab = logits.shape
+    _need(logits.dtype == torch.float32 and logits.stride(1) == 1, "argmax: logits must be fp32 rows")
+    _need(out.dtype == torch.int32 and out.numel() == rows and out.is_contiguous(), "argmax: out int32 [rows]")
+    _check(lib().ka_argmax(logits.data_ptr(), logits.stride(0), out.data_ptr(), rows, vocab, stream_ptr()))
+
+
+def sample(logits: torch.Tensor, temps: torch.Tensor, top_ps: Optional[torch.Tensor], rng_key: torch.Tensor,
+           rng_counter: torch.Tensor, out: torch.Tensor) -> None:
+    """Temperature and top-p sampling of every row (greedy where temperature <= 1e-6)."""
+    _dev(logits, temps, top_ps, rng_key, rng_counter, out)
+    rows, vocab = logits.shape
+    _need(logits.dtype == torch.float32 and logits.stride(1) == 1, "sample: logits must be fp32 rows")
+    _need(temps.dtype == torch.float32 and temps.numel() == rows, "sample: temps fp32 [rows]")
+    _need(top_ps is None or (top_ps.dtype == torch.float32 and top_ps.numel() == rows), "sample: top_ps fp32 [rows]")
+    _need(rng_key.dtype == torch.int64 and rng_key.numel() == rows, "sample: rng_key int64 [rows]")
+    _need(rng_counter.dtype == torch.int32 and rng_counter.numel() == rows, "sample: rng_counter int32 [rows]")
+    _need(out.dtype == torch.int32 and out.numel() == rows and out.is_contiguous(), "sample: out int32 [rows]")
+    _check(lib().ka_sample(logits.data_ptr(), logits.stride(0), temps.data_ptr(), _ptr(top_ps), rng_key.data_ptr(),
+                           rng_counter.data_ptr(), out.data_ptr(), rows, vocab, stream_ptr()))

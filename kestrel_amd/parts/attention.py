@@ -1,0 +1,76 @@
+"""Attention over the paged cache with a fused q|k|v projection."""
+
+from __future__ import annotations
+
+from typing import Dict, Optional
+
+import torch
+
+from ..ops import core
+from ..ops.attention import paged_attention
+from ..ops.linear import linear
+from .base import LayerCache, Mixer, build_part, register_mixer
+from .specs import AttentionSpec, CacheSpec, ParamSpec
+
+
+class PagedAttention(Mixer):
+    """``proj(softmax(q k^T scale + mask) v)`` with grouped kv heads.
+
+    One linear gives ``[q (H hd) | k (Hkv hd) | v (Hkv hd)]`` per token
+    (``kestrel/models/moondream/text.py:101-121``); the position encoding is applied to
+    q and k, k and v go into the paged cache first and attention then reads the cache
+    (``text.py:123-135``); query head ``h`` reads kv head ``h // (H / Hkv)``; the scale is
+    ``hd ** -0.5`` unless given (``text.py:158-185``); the output projection adds into the
+    residual (``text.py:187-193``). Which keys a token sees comes with the batch
+    (``kv_hi``, and the group's ``kv_lo`` for a window).
+    """
+
+    def __init__(self, spec: AttentionSpec) -> None:
+        super().__init__(spec)
+        if spec.n_heads % spec.n_kv_heads:
+            raise ValueError(f"{spec.n_heads} query heads cannot share {spec.n_kv_heads} kv heads")
+        self.position = build_part("position", spec.position)
+        self.scale = float(spec.scale) if spec.scale is not None else float(spec.head_dim) ** -0.5
+        self.q_dim = spec.n_heads * spec.head_dim
+        self.kv_dim = spec.n_kv_heads * spec.head_dim
+        self.qkv_dim = self.q_dim + 2 * self.kv_dim
+        self.qkv_weight = self.qkv_bias = self.proj_weight = self.proj_bias = None
+        self.dtype: Optional[torch.dtype] = None
+        self._table = None
+
+    def params(self) -> Dict[str, ParamSpec]:
+        spec = self.spec
+        out = {"qkv.weight": ParamSpec((self.qkv_dim, spec.dim)), "proj.weight": ParamSpec((spec.dim, self.q_dim))}
+        if spec.bias:
+            out["qkv.bias"] = ParamSpec((self.qkv_dim,), "vector", "bias")
+            out["proj.bias"] = ParamSpec((spec.dim,), "vector", "bias")
+        return out
+
+    def cache_spec(self) -> CacheSpec:
+        return CacheSpec(self.spec.n_kv_heads, self.spec.head_dim, self.spec.window)
+
+    def bind(self, tensors, dtype, device) -> None:
+        self.dtype = dtype
+        self.qkv_weight = tensors["qkv.weight"].to(device).contiguous()
+        self.proj_weight = tensors["proj.weight"].to(device).contiguous()
+        if self.spec.bias:
+            self.qkv_bias = tensors["qkv.bias"].to(device=device, dtype=torch.float32).contiguous()
+            self.proj_bias = tensors["proj.bias"].to(device=device, dtype=torch.float32).contiguous()
+        self._table = self.position.table(device)
+
+    def forward(self, h, batch, cache: LayerCache, residual) -> None:
+        spec = self.spec
+        n = h.shape[0]
+        ws = batch.workspace
+        qkv = ws.get("attn.qkv", (n, self.qkv_dim), self.dtype)
+        linear(h, self.qkv_weight, self.qkv_bias, qkv)
+        group = batch.groups[cache.group]
+        core.rope_cache(qkv, batch.positions, group.slots if cache.writes else None, self._table, cache.k, cache.v,
+                        spec.n_heads, spec.n_kv_heads, spec.head_dim, group.page_size)
+        out = ws.get("attn.out", (n, self.q_dim), self.dtype)
+        paged_attention(qkv, cache.k, cache.v, group.block_table, batch.token_row, group.kv_lo, batch.kv_hi, out,
+                        self.scale, spec.n_heads, spec.n_kv_heads, spec.head_dim, batch)
+        linear(out, self.proj_weight, self.proj_bias, residual, accumulate=True)
+
+
+register_mixer("attention", PagedAttention)

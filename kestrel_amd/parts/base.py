@@ -1,0 +1,119 @@
+"""Interfaces of the parts and the registries they are built through.
+
+A part is built from its specification alone, says which tensors it owns
+(``params``), takes them (``bind``) and runs on the packed tokens of one step
+(``forward``). It never sees the model or the architecture it is used in.
+
+Adding a part of a new kind: subclass the interface, and call ``register_mixer`` /
+``register_feed_forward`` / ``register_norm`` / ``register_position`` with the kind
+name that its specification carries.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Callable, Dict, Optional
+
+import torch
+
+from .specs import CacheSpec, ParamSpec, StateSpec
+
+
+class Part:
+    """Common face of every part."""
+
+    def __init__(self, spec) -> None:
+        self.spec = spec
+
+    def params(self) -> Dict[str, ParamSpec]:
+        """Local tensor name -> its shape and role."""
+        return {}
+
+    def bind(self, tensors: Dict[str, torch.Tensor], dtype: torch.dtype, device: torch.device) -> None:
+        """Take the loaded tensors (on ``device``); ``dtype`` is the precision of activations."""
+
+
+class Norm(Part):
+    def forward(self, x: torch.Tensor, out: torch.Tensor, rows: Optional[torch.Tensor] = None) -> None:
+        """Normalise fp32 rows of ``x`` (all, or those in ``rows``) into ``out``."""
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    """Holds what a mixer needs to encode positions (for rotary: the angle table)."""
+
+    def table(self, device: torch.device) -> Optional[torch.Tensor]:
+        return None
+
+
+@dataclass
+class LayerCache:
+    """What one run of a layer may touch of the cache manager's memory.
+
+    ``group``: key into ``StepBatch.groups`` (block table, slots, window start) or ``None``
+    if the mixer keeps no keys and values; ``k``/``v``: ``[pages, Hkv, page_size, hd]``;
+    ``writes``: ``False`` when this run reads the cache of another run; ``state``:
+    ``[slots, *shape]`` per-request state, indexed by ``StepBatch.row_slot``.
+    """
+
+    group: Optional[int] = None
+    k: Optional[torch.Tensor] = None
+    v: Optional[torch.Tensor] = None
+    writes: bool = True
+    state: Optional[torch.Tensor] = None
+
+
+class Mixer(Part):
+    def cache_spec(self) -> Optional[CacheSpec]:
+        """Keys and values kept per token, or ``None``."""
+        return None
+
+    def state_spec(self) -> Optional[StateSpec]:
+        """Fixed-size state kept per request, or ``None``."""
+        return None
+
+    def forward(self, h: torch.Tensor, batch, cache: LayerCache, residual: torch.Tensor) -> None:
+        """Add the mixer's output for the normalised input ``h`` into fp32 ``residual``."""
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, h: torch.Tensor, batch, residual: torch.Tensor) -> None:
+        """Add the feed-forward output for ``h`` into fp32 ``residual``."""
+        raise NotImplementedError
+
+
+_REGISTRIES: Dict[str, Dict[str, Callable]] = {"mixer": {}, "feed_forward": {}, "norm": {}, "position": {}}
+
+
+def _register(family: str, kind: str, cls: Callable) -> None:
+    _REGISTRIES[family][kind] = cls
+
+
+def register_mixer(kind: str, cls: Callable) -> None:
+    _register("mixer", kind, cls)
+
+
+def register_feed_forward(kind: str, cls: Callable) -> None:
+    _register("feed_forward", kind, cls)
+
+
+def register_norm(kind: str, cls: Callable) -> None:
+    _register("norm", kind, cls)
+
+
+def register_position(kind: str, cls: Callable) -> None:
+    _register("position", kind, cls)
+
+
+def build_part(family: str, spec) -> Part:
+    """The part registered for ``spec.kind`` in ``family``."""
+    kinds = _REGISTRIES[family]
+    kind = getattr(spec, "kind", None)
+    if kind not in kinds:
+        raise ValueError(f"no {family} of kind {kind!r} is registered; known: {', '.join(sorted(kinds)) or 'none'}")
+    return kinds[kind](spec)
+
+
+def known_kinds(family: str):
+    return sorted(_REGISTRIES[family])
