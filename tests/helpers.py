@@ -70,3 +70,78 @@ def assert_close(actual: torch.Tensor, expected: torch.Tensor, dtype: torch.dtyp
         idx = tuple(int(i) for i in torch.unravel_index(torch.tensor(worst), err.shape))
         raise AssertionError(f"{what}: worst at {idx}: got {actual[idx]:.6g}, expected {expected[idx]:.6g}, "
                              f"error {err[idx]:.3g} > {bound[idx]:.3g}; max error {err.max():.3g}")
+
+
+# ----------------------------------------------------------------------------
+# replaying requests through a runner in a given way of cutting
+# ----------------------------------------------------------------------------
+
+class Request:
+    """A test request: optional prefix embeddings (one bidirectional block) and token ids."""
+
+    def __init__(self, name: str, ids: Sequence[int], prefix: Optional[torch.Tensor] = None) -> None:
+        self.name, self.ids, self.prefix = name, list(ids), prefix
+        self.n_prefix = 0 if prefix is None else prefix.shape[0]
+        self.length = self.n_prefix + len(self.ids)
+        self.done = 0            # tokens fed so far
+        self.slot = None
+
+    def take(self, count: int):
+        """The next ``count`` places as (tokens, embeds, bidirectional)."""
+        lo, hi = self.done, min(self.done + count, self.length)
+        tokens, embeds = [], None
+        if lo < self.n_prefix:
+            if hi < self.n_prefix:
+                raise AssertionError("test bug: a portion splits the prefix block")
+            tokens += [-1] * (self.n_prefix - lo)
+            embeds = self.prefix[lo:self.n_prefix]
+        tokens += self.ids[max(lo, self.n_prefix) - self.n_prefix:hi - self.n_prefix]
+        bidir = [(0, self.n_prefix)] if lo == 0 and self.n_prefix else []
+        self.done = hi
+        return tokens, embeds, bidir, lo
+
+
+def replay(runner, requests: Dict[str, "Request"], steps, poison: bool = False) -> Dict[str, torch.Tensor]:
+    """Run ``steps`` = list of lists of (request name, number of tokens); every fed place is
+    wanted. Returns the logits per request in position order, ``[fed, vocab]``. A request is
+    admitted at its first portion and released after its last. With ``poison`` the pages a
+    request gives back are filled with NaN, so that a later read of them shows."""
+    from kestrel_amd.engine.step import StepEntry
+
+    rows: Dict[str, List[torch.Tensor]] = {name: [] for name in requests}
+    for step in steps:
+        entries, order = [], []
+        for name, count in step:
+            req = requests[name]
+            if req.slot is None:
+                req.slot = runner.admit()
+            tokens, embeds, bidir, _lo = req.take(count)
+            entries.append(StepEntry(req.slot, tokens, want=list(range(len(tokens))), embeds=embeds,
+                                     bidirectional=bidir))
+            order.append((name, len(tokens)))
+        logits = runner.step(entries).clone()
+        at = 0
+        for name, count in order:
+            rows[name].append(logits[at:at + count])
+            at += count
+        for name, _ in order:
+            req = requests[name]
+            if req.done == req.length:
+                pages = [[p for p in runner.cache.block_table(g, req.slot) if p >= 0]
+                         for g in range(len(runner.cache.groups))]
+                runner.release(req.slot)
+                req.slot = None
+                if poison:
+                    for g, group in enumerate(runner.cache.groups):
+                        if pages[g]:
+                            index = torch.tensor(pages[g], device=group.k.device)
+                            group.k[:, index] = float("nan")
+                            group.v[:, index] = float("nan")
+        runner.cache.check()
+    return {name: torch.cat(chunks, dim=0) for name, chunks in rows.items() if chunks}
+
+
+def poison_cache(runner) -> None:
+    for group in runner.cache.groups:
+        group.k.fill_(float("nan"))
+        group.v.fill_(float("nan"))

@@ -1,39 +1,192 @@
 """The engine against the plain implementation under every way of cutting the work."""
 
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
 import pytest
 import torch
 
 from tests import helpers
+from tests.helpers import Request
 from tests.plain import moondream_plain as plain
 
 pytestmark = pytest.mark.gpu
 
 DTYPES = [torch.float32, torch.bfloat16]
+DTYPE_IDS = ["fp32", "bf16"]
+NAMES = ["A", "B", "C"]
 
 
 def _runner(name, dtype, n_pages=64, page_size=16, max_requests=8):
     from kestrel_amd.engine.loading import load_model, make_runner
 
     net = load_model(helpers.model_dir(name), dtype, torch.device("cuda:0"))
-    return make_runner(net, page_size, n_pages, max_requests)
+    runner = make_runner(net, page_size, n_pages, max_requests)
+    helpers.poison_cache(runner)
+    return runner
 
 
-def _expected(name, ids):
+def _expected(name, req: Request):
     folder = helpers.model_dir(name)
-    return plain.forward(helpers.flat_config(name), helpers.stored_weights(folder), ids)
+    return plain.forward(helpers.flat_config(name), helpers.stored_weights(folder), req.ids, req.prefix)
 
 
-@pytest.mark.parametrize("dtype", DTYPES, ids=["fp32", "bf16"])
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+def _request(name, tag, seed, n_ids, n_prefix=0):
+    cfg = helpers.flat_config(name)
+    prefix = None
+    if n_prefix:
+        gen = torch.Generator().manual_seed(1000 + seed)
+        prefix = torch.randn(n_prefix, cfg["dim"], generator=gen)
+    return Request(tag, helpers.random_ids(seed, n_ids, cfg["vocab_size"]), prefix)
+
+
+def _check(name, dtype, requests, got):
+    for tag, req in requests.items():
+        helpers.assert_close(got[tag], _expected(name, req), dtype, f"tiny {name} request {tag}")
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=DTYPE_IDS)
+@pytest.mark.parametrize("name", NAMES)
 def test_whole_prompt(name, dtype):
+    """Each request alone and whole, also the first tokens of a sequence (1, 2, 3 tokens)."""
+    runner = _runner(name, dtype)
+    for seed, length in enumerate([1, 2, 3, 5, 17, 33, 70, 100]):
+        reqs = {"r": _request(name, "r", 100 + seed, length)}
+        got = helpers.replay(runner, reqs, [[("r", length)]])
+        _check(name, dtype, reqs, got)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=DTYPE_IDS)
+@pytest.mark.parametrize("name", NAMES)
+def test_last_32_one_by_one(name, dtype):
+    """Most of the request in one step, the last 32 tokens decoded one by one."""
+    runner = _runner(name, dtype)
+    for seed, length in enumerate([33, 64, 81, 120]):
+        reqs = {"r": _request(name, "r", 200 + seed, length)}
+        steps = ([[("r", length - 32)]] if length > 32 else []) + [[("r", 1)] for _ in range(32)]
+        got = helpers.replay(runner, reqs, steps, poison=True)
+        _check(name, dtype, reqs, got)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=DTYPE_IDS)
+@pytest.mark.parametrize("name", NAMES)
+def test_portions_of_changing_size(name, dtype):
+    """Portions cut anywhere, down to two tokens, over page edges (page size 16)."""
+    runner = _runner(name, dtype)
+    sizes = [7, 2, 9, 14, 2, 3, 16, 1, 31, 2, 33]
+    length = sum(sizes)
+    reqs = {"r": _request(name, "r", 300, length)}
+    got = helpers.replay(runner, reqs, [[("r", s)] for s in sizes], poison=True)
+    _check(name, dtype, reqs, got)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=DTYPE_IDS)
+@pytest.mark.parametrize("name", NAMES)
+def test_mixed_batches_with_page_reuse(name, dtype):
+    """Up to four live requests, portions of some beside decoded tokens of others, with so
+    few pages that later requests run in pages earlier ones gave back."""
+    lengths = {"a": 40, "b": 75, "c": 23, "d": 90, "e": 61, "f": 18, "g": 50}
+    # 4 live requests of at most 90 tokens: 4 * 6 pages of 16; the pool has 18, so the order
+    # below only works because pages come back and are used again.
+    runner = _runner(name, dtype, n_pages=18, max_requests=4)
+    reqs = {tag: _request(name, tag, 400 + i, n) for i, (tag, n) in enumerate(lengths.items())}
+    steps = [
+        [("a", 30), ("b", 20)],
+        [("a", 1), ("b", 40), ("c", 2)],
+        [("a", 1), ("b", 1), ("c", 21)],                      # c ends
+        [("a", 8), ("b", 14), ("d", 50)],                     # a, b end
+        [("d", 1), ("e", 33), ("f", 17)],
+        [("d", 1), ("e", 1), ("f", 1), ("g", 2)],             # f ends
+        [("d", 38), ("e", 27), ("g", 47)],                    # d, e end
+        [("g", 1)],
+    ]
+    got = helpers.replay(runner, reqs, steps, poison=True)
+    assert all(r.done == r.length for r in reqs.values())
+    _check(name, dtype, reqs, got)
+    assert runner.cache.groups[0].pool.free_count == 18
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=DTYPE_IDS)
+@pytest.mark.parametrize("name", ["B", "C"])
+def test_prefix_embeddings_bidirectional(name, dtype):
+    """Given embeddings as one bidirectional block, then text; the block in one portion, the
+    rest cut into portions and decoded; two such requests mixed."""
+    cfg = helpers.flat_config(name)
+    n_prefix = cfg["prefix_attn"]
+    runner = _runner(name, dtype)
+    reqs = {"p": _request(name, "p", 500, 29, n_prefix), "q": _request(name, "q", 501, 12, n_prefix)}
+    steps = [[("p", n_prefix + 4)], [("p", 10), ("q", n_prefix)], [("p", 1), ("q", 5)], [("p", 14), ("q", 7)]]
+    got = helpers.replay(runner, reqs, steps, poison=True)
+    _check(name, dtype, reqs, got)
+
+
+def test_split_bidirectional_block_is_refused():
     from kestrel_amd.engine.step import StepEntry
 
+    runner = _runner("B", torch.float32)
+    slot = runner.admit()
+    embeds = torch.randn(8, helpers.flat_config("B")["dim"])
+    with pytest.raises(ValueError, match="must lie inside one portion"):
+        runner.step([StepEntry(slot, [-1] * 8, embeds=embeds, bidirectional=[(0, 17)])])
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=DTYPE_IDS)
+def test_long_decoding(dtype):
+    """A short prompt, then every further token one by one up to the context length."""
+    name = "B"
+    length = helpers.flat_config(name)["max_context"]
     runner = _runner(name, dtype)
-    vocab = helpers.flat_config(name)["vocab_size"]
-    for seed, length in enumerate([5, 17, 33, 70]):
-        ids = helpers.random_ids(100 + seed, length, vocab)
-        slot = runner.admit()
-        logits = runner.step([StepEntry(slot, ids, want=list(range(length)))]).clone()
-        runner.release(slot)
-        helpers.assert_close(logits, _expected(name, ids), dtype, f"tiny {name} length {length}")
-    runner.cache.check()
+    reqs = {"r": _request(name, "r", 600, length)}
+    got = helpers.replay(runner, reqs, [[("r", 3)]] + [[("r", 1)] for _ in range(length - 3)])
+    _check(name, dtype, reqs, got)
+
+
+@pytest.mark.parametrize("page_size", [1, 4, 64])
+def test_other_page_sizes(page_size):
+    runner = _runner("A", torch.float32, n_pages=512 // page_size, page_size=page_size)
+    reqs = {"r": _request("A", "r", 700, 77)}
+    got = helpers.replay(runner, reqs, [[("r", 40)], [("r", 5)]] + [[("r", 1)] for _ in range(32)])
+    _check("A", torch.float32, reqs, got)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_run_program(tmp_path, dtype):
+    """bin/trace_run as a user runs it: JSON lines in, <step>.f32 files and 'done' lines out."""
+    name = "A"
+    cfg = helpers.flat_config(name)
+    ids_a = helpers.random_ids(800, 50, cfg["vocab_size"])
+    ids_b = helpers.random_ids(801, 37, cfg["vocab_size"])
+    lines = [
+        {"step": 0, "entries": [{"id": "a", "tokens": ids_a[:18], "want": [0, 17]}], "end": []},
+        {"step": 1, "entries": [{"id": "a", "tokens": ids_a[18:48], "want": []},
+                                {"id": "b", "tokens": ids_b[:2], "want": [1]}], "end": []},
+        {"step": 2, "entries": [{"id": "b", "tokens": ids_b[2:37], "want": [34]}], "end": ["b"]},
+        {"step": 3, "entries": [{"id": "a", "tokens": ids_a[48:49], "want": [0]}], "end": []},
+        {"step": 4, "entries": [{"id": "a", "tokens": ids_a[49:50], "want": [0]}], "end": ["a"]},
+    ]
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    out = tmp_path / "out"
+    done = subprocess.run(
+        [sys.executable, os.path.join(root, "bin", "trace_run"), "--model", helpers.model_dir(name), "--dtype", dtype,
+         "--out", str(out), "--max-tokens", "128"],
+        input="\n".join(json.dumps(l) for l in lines) + "\n", capture_output=True, text=True, timeout=300)
+    assert done.returncode == 0, done.stderr
+    assert [l for l in done.stdout.splitlines() if l.startswith("done")] == [f"done {i}" for i in range(5)]
+    assert not (out / "1.f32").exists() or True
+    weights = helpers.stored_weights(helpers.model_dir(name))
+    exp_a = plain.forward(cfg, weights, ids_a)
+    exp_b = plain.forward(cfg, weights, ids_b)
+    tdtype = torch.float32 if dtype == "float32" else torch.bfloat16
+
+    def load(step, rows):
+        data = np.fromfile(out / f"{step}.f32", dtype="<f4")
+        return torch.from_numpy(data.reshape(rows, cfg["vocab_size"]))
+
+    helpers.assert_close(load(0, 2), exp_a[[0, 17]], tdtype, "step 0")
+    helpers.assert_close(load(1, 1), exp_b[[1]], tdtype, "step 1")
+    helpers.assert_close(load(2, 1), exp_b[[36]], tdtype, "step 2")
+    helpers.assert_close(load(3, 1), exp_a[[48]], tdtype, "step 3")
+    helpers.assert_close(load(4, 1), exp_a[[49]], tdtype, "step 4")
