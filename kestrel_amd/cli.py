@@ -1,0 +1,140 @@
+"""Command line: ``python -m kestrel_amd <generate | random-weights | replay>``.
+
+Option names follow the reference's ``RuntimeConfig`` fields (``kestrel/config.py:155-179``:
+``--model-path --dtype --max-batch-size --page-size --kv-cache-pages``) and its request
+settings (``temperature``, ``top_p``, ``max_tokens``; ``kestrel/engine/core.py:1161-1174``).
+Prompts are token ids: the tokenizer is outside this engine.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import sys
+import time
+from typing import List
+
+
+def _add_runtime_options(parser: argparse.ArgumentParser) -> None:
+    parser.add_argument("--model-path", required=True, help="folder with config.json and model.safetensors")
+    parser.add_argument("--model", default=None, help="architecture name (default: taken from config.json)")
+    parser.add_argument("--device", default="cuda")
+    parser.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    parser.add_argument("--max-batch-size", type=int, default=4)
+    parser.add_argument("--page-size", type=int, default=16)
+    parser.add_argument("--kv-cache-pages", type=int, default=None)
+    parser.add_argument("--max-num-batched-tokens", type=int, default=2048)
+    parser.add_argument("--seed", type=int, default=0)
+    parser.add_argument("--disable-graphs", action="store_true", help="do not replay decode steps as HIP graphs")
+
+
+def _parse_ids(text: str) -> List[int]:
+    return [int(t) for t in text.replace(",", " ").split()]
+
+
+def _generate(args) -> int:
+    import torch
+
+    from .config import RuntimeConfig
+    from .engine import InferenceEngine
+
+    prompts: List[List[int]] = []
+    for text in args.prompt_ids or []:
+        prompts.append(_parse_ids(text))
+    if args.prompt_file:
+        with open(args.prompt_file) as handle:
+            data = json.load(handle)
+        prompts.extend([list(map(int, p)) for p in data])
+    cfg = RuntimeConfig(model_path=args.model_path, model=args.model, device=args.device, dtype=args.dtype,
+                        max_batch_size=args.max_batch_size, page_size=args.page_size,
+                        kv_cache_pages=args.kv_cache_pages, max_num_batched_tokens=args.max_num_batched_tokens,
+                        seed=args.seed, enable_graphs=not args.disable_graphs)
+    engine = InferenceEngine.create_sync(cfg)
+    try:
+        if args.random_prompts:
+            gen = torch.Generator().manual_seed(args.seed)
+            vocab = engine.plan.vocab_size
+            prompts.extend(torch.randint(0, vocab, (args.prompt_len,), generator=gen).tolist()
+                           for _ in range(args.random_prompts))
+        if not prompts:
+            print("generate: give --prompt-ids, --prompt-file or --random-prompts", file=sys.stderr)
+            return 2
+        started = time.perf_counter()
+        results = engine.generate_batch_sync(prompts, max_new_tokens=args.max_tokens, temperature=args.temperature,
+                                             top_p=args.top_p)
+        elapsed = time.perf_counter() - started
+        for result in results:
+            print(json.dumps({"request_id": result.request_id, "tokens": result.tokens,
+                              "finish_reason": result.finish_reason, "input_tokens": result.metrics.input_tokens,
+                              "output_tokens": result.metrics.output_tokens,
+                              "ttft_ms": round(result.metrics.ttft_ms, 3),
+                              "decode_time_ms": round(result.metrics.decode_time_ms, 3)}))
+        total = sum(r.metrics.output_tokens for r in results)
+        print(f"# {len(results)} requests, {total} tokens in {elapsed:.3f} s", file=sys.stderr)
+    finally:
+        engine.shutdown_sync()
+    return 0
+
+
+def _random_weights(args) -> int:
+    from .config import get_spec
+    from .weights import InitRecipe, write_random_model
+
+    if args.config:
+        with open(args.config) as handle:
+            config = json.load(handle)
+    else:
+        spec = get_spec(args.preset)
+        if spec.default_config is None:
+            print(f"random-weights: {args.preset} has no preset configuration; give --config", file=sys.stderr)
+            return 2
+        config = dict(spec.default_config())
+        config.setdefault("model", spec.name)
+    recipe = InitRecipe(std=args.std, bias_std=args.bias_std, gain_std=args.gain_std, shift_std=args.shift_std)
+    folder = write_random_model(args.out, config, args.seed, recipe, store_dtype=args.store_dtype, model=args.model)
+    print(folder)
+    return 0
+
+
+def main(argv=None) -> int:
+    parser = argparse.ArgumentParser(prog="kestrel_amd", description="MI355X inference engine")
+    sub = parser.add_subparsers(dest="command", required=True)
+
+    gen = sub.add_parser("generate", help="generate tokens for prompts given as token ids")
+    _add_runtime_options(gen)
+    gen.add_argument("--prompt-ids", action="append", help="token ids of one prompt, e.g. '5,17,3' (repeatable)")
+    gen.add_argument("--prompt-file", help="JSON file with a list of prompts, each a list of token ids")
+    gen.add_argument("--random-prompts", type=int, default=0, help="this many random prompts")
+    gen.add_argument("--prompt-len", type=int, default=32, help="length of the random prompts")
+    gen.add_argument("--max-tokens", type=int, default=16, help="tokens to generate per prompt")
+    gen.add_argument("--temperature", type=float, default=0.0)
+    gen.add_argument("--top-p", type=float, default=1.0)
+    gen.set_defaults(run=_generate)
+
+    rw = sub.add_parser("random-weights", help="write a model folder with seeded random weights")
+    rw.add_argument("--out", required=True)
+    rw.add_argument("--config", help="config.json to build the model from")
+    rw.add_argument("--preset", default="moondream2", help="registered model whose preset sizes are used without --config")
+    rw.add_argument("--model", default=None)
+    rw.add_argument("--seed", type=int, default=0)
+    rw.add_argument("--std", type=float, default=0.02)
+    rw.add_argument("--bias-std", type=float, default=None)
+    rw.add_argument("--gain-std", type=float, default=0.0)
+    rw.add_argument("--shift-std", type=float, default=0.0)
+    rw.add_argument("--store-dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    rw.set_defaults(run=_random_weights)
+
+    rp = sub.add_parser("replay", help="trace replay (the same program as bin/trace_run)", add_help=False)
+    rp.set_defaults(run=None)
+
+    if argv is None:
+        argv = sys.argv[1:]
+    if argv and argv[0] == "replay":
+        from .engine.replay import main as replay_main
+        return replay_main(argv[1:])
+    args = parser.parse_args(argv)
+    return args.run(args)
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -1,0 +1,280 @@
+"""The Python entry point: ``InferenceEngine.create(cfg)`` and its ways to generate.
+
+In the reference's manner (``kestrel/engine/core.py:262-319`` ``create``, ``:556,767``
+``submit`` / ``submit_streaming``, ``:486`` ``shutdown``; results
+``kestrel/engine/_types.py:35-56``): an asynchronous facade over one scheduler thread that
+owns the GPU. Request options keep the reference's names and meanings: ``temperature``
+(>= 0, ``None`` -> 0.0), ``top_p`` (in (0, 1], ``None`` -> 1.0), ``max_tokens`` / ``max_new_tokens``
+(``core.py:1161-1174``). The reference's skills, tokenizer and image encoder are outside
+this engine: prompts are token ids, an image is a block of given embeddings.
+"""
+
+from __future__ import annotations
+
+import asyncio
+import queue
+import threading
+import time
+from concurrent.futures import Future
+from dataclasses import dataclass
+from typing import AsyncIterator, Dict, List, Optional, Sequence
+
+import torch
+
+from ..config.runtime import RuntimeConfig
+from ..sampling.sampler import Sampler
+from .loading import load_model, make_runner
+from .scheduler import GenerationScheduler
+from .types import GenerationRequest, SchedulerResult
+
+
+@dataclass
+class EngineMetrics:
+    """Token counts and timing of one request (``kestrel/engine/_types.py:35-44``)."""
+
+    input_tokens: int
+    output_tokens: int
+    prefill_time_ms: float
+    decode_time_ms: float
+    ttft_ms: float
+
+
+@dataclass
+class EngineResult:
+    """What a caller gets back (``kestrel/engine/_types.py:47-56``)."""
+
+    request_id: int
+    tokens: List[int]
+    finish_reason: str
+    metrics: EngineMetrics
+    output: Dict[str, object]
+
+
+@dataclass
+class StreamUpdate:
+    request_id: int
+    token: int
+    token_index: int
+
+
+class _Pending:
+    def __init__(self, request: GenerationRequest, future: Future, stream: Optional["queue.Queue"]) -> None:
+        self.request, self.future, self.stream = request, future, stream
+
+
+def _normalise(temperature, top_p):
+    temperature = 0.0 if temperature is None else float(temperature)
+    top_p = 1.0 if top_p is None else float(top_p)
+    if temperature < 0.0:
+        raise ValueError("temperature must be non-negative")
+    if not 0.0 < top_p <= 1.0:
+        raise ValueError("top_p must be in the range (0, 1]")
+    return temperature, top_p
+
+
+class InferenceEngine:
+    """Loads a model folder, keeps the cache and runs the scheduler on a thread of its own."""
+
+    def __init__(self, cfg: RuntimeConfig) -> None:
+        self.cfg = cfg
+        self._inbox: "queue.Queue" = queue.Queue()
+        self._thread: Optional[threading.Thread] = None
+        self._started = threading.Event()
+        self._startup_error: Optional[BaseException] = None
+        self._fatal: Optional[BaseException] = None
+        self._stop = False
+        self._next_id = 0
+        self._id_lock = threading.Lock()
+        self.runner = None
+        self.scheduler: Optional[GenerationScheduler] = None
+        self.plan = None
+
+    # ------------------------------------------------------------------ life cycle
+    @classmethod
+    async def create(cls, cfg: RuntimeConfig) -> "InferenceEngine":
+        engine = cls(cfg)
+        await asyncio.get_running_loop().run_in_executor(None, engine.start)
+        return engine
+
+    @classmethod
+    def create_sync(cls, cfg: RuntimeConfig) -> "InferenceEngine":
+        engine = cls(cfg)
+        engine.start()
+        return engine
+
+    def start(self) -> None:
+        if self._thread is not None:
+            return
+        self._thread = threading.Thread(target=self._scheduler_loop, name="kestrel-scheduler", daemon=True)
+        self._thread.start()
+        self._started.wait()
+        if self._startup_error is not None:
+            raise self._startup_error
+
+    def _build(self) -> None:
+        cfg = self.cfg
+        if cfg.model_path is None:
+            raise ValueError("RuntimeConfig.model_path must name a folder with config.json and model.safetensors")
+        device = cfg.resolved_device()
+        torch.cuda.set_device(device)
+        net = load_model(cfg.model_path, cfg.dtype, device, cfg.model)
+        self.plan = net.plan
+        max_seq = min(cfg.max_seq_len or net.plan.max_positions, net.plan.max_positions)
+        if cfg.kv_cache_pages is not None:
+            n_pages = cfg.kv_cache_pages
+        elif cfg.kv_cache_tokens is not None:
+            n_pages = -(-cfg.kv_cache_tokens // cfg.page_size)
+        else:
+            n_pages = cfg.max_batch_size * -(-max_seq // cfg.page_size)
+        self.runner = make_runner(net, cfg.page_size, n_pages, cfg.max_batch_size,
+                                  max_tokens_per_step=cfg.max_num_batched_tokens)
+        self.scheduler = GenerationScheduler(self.runner, Sampler(device, cfg.seed), cfg.max_batch_size,
+                                             cfg.max_num_batched_tokens, net.plan.eos_token_ids, max_seq)
+
+    def _scheduler_loop(self) -> None:
+        try:
+            self._build()
+        except BaseException as exc:  # surfaced to the caller of start()
+            self._startup_error = exc
+            self._started.set()
+            return
+        self._started.set()
+        pending: Dict[int, _Pending] = {}
+        scheduler = self.scheduler
+        try:
+            while True:
+                block = not scheduler.has_pending_work()
+                while True:
+                    try:
+                        item = self._inbox.get(block=block, timeout=0.05 if block else None)
+                    except queue.Empty:
+                        break
+                    block = False
+                    if item is None:
+                        self._stop = True
+                        continue
+                    try:
+                        scheduler.enqueue_request(item.request)
+                        pending[item.request.request_id] = item
+                    except Exception as exc:
+                        self._deliver_error(item, exc)
+                if self._stop and not scheduler.has_pending_work():
+                    break
+                if scheduler.has_pending_work():
+                    scheduler.advance()
+                    for result in scheduler.pop_completed():
+                        self._deliver(pending.pop(result.request_id), result)
+        except BaseException as exc:
+            self._fatal = exc
+            for item in pending.values():
+                self._deliver_error(item, exc)
+            while True:
+                try:
+                    item = self._inbox.get_nowait()
+                except queue.Empty:
+                    break
+                if item is not None:
+                    self._deliver_error(item, exc)
+
+    def _deliver(self, item: _Pending, result: SchedulerResult) -> None:
+        if result.finish_reason == "error":
+            self._deliver_error(item, RuntimeError(result.error or "request failed"))
+            return
+        m = result.metrics
+        out = EngineResult(result.request_id, result.tokens, result.finish_reason,
+                           EngineMetrics(m.prompt_tokens, m.decode_tokens, m.prefill_time_ms, m.decode_time_ms, m.ttft_ms),
+                           {"tokens": result.tokens})
+        if item.stream is not None:
+            item.stream.put(None)
+        item.future.set_result(out)
+
+    def _deliver_error(self, item: _Pending, exc: BaseException) -> None:
+        if item.stream is not None:
+            item.stream.put(exc)
+        if not item.future.done():
+            item.future.set_exception(exc)
+
+    def shutdown_sync(self) -> None:
+        if self._thread is None:
+            return
+        self._inbox.put(None)
+        self._thread.join()
+        self._thread = None
+
+    async def shutdown(self) -> None:
+        await asyncio.get_running_loop().run_in_executor(None, self.shutdown_sync)
+
+    # ------------------------------------------------------------------ requests
+    def _make_request(self, prompt_ids, max_new_tokens, temperature, top_p, prefix_embeds, prefix_ids, stop_ids, seed,
+                      on_token) -> GenerationRequest:
+        if self._fatal is not None:
+            raise RuntimeError("the engine has stopped after an error") from self._fatal
+        if self._thread is None:
+            raise RuntimeError("the engine is not running")
+        temperature, top_p = _normalise(temperature, top_p)
+        if max_new_tokens is None or int(max_new_tokens) <= 0:
+            raise ValueError("max_new_tokens must be positive")
+        with self._id_lock:
+            request_id = self._next_id
+            self._next_id += 1
+        return GenerationRequest(request_id, list(prompt_ids), int(max_new_tokens), temperature, top_p, prefix_embeds,
+                                 tuple(prefix_ids), None if stop_ids is None else tuple(stop_ids), seed, on_token)
+
+    def submit_sync(self, prompt_ids: Sequence[int], *, max_new_tokens: int, temperature: Optional[float] = None,
+                    top_p: Optional[float] = None, prefix_embeds: Optional[torch.Tensor] = None,
+                    prefix_ids: Sequence[int] = (), stop_ids: Optional[Sequence[int]] = None,
+                    seed: Optional[int] = None, _stream: Optional["queue.Queue"] = None) -> Future:
+        """Queue a request; the returned future resolves to an ``EngineResult``."""
+        on_token = None
+        if _stream is not None:
+            def on_token(token, index, _q=_stream):
+                _q.put((token, index))
+        request = self._make_request(prompt_ids, max_new_tokens, temperature, top_p, prefix_embeds, prefix_ids,
+                                     stop_ids, seed, on_token)
+        future: Future = Future()
+        future.request_id = request.request_id
+        self._inbox.put(_Pending(request, future, _stream))
+        return future
+
+    def generate_sync(self, prompt_ids: Sequence[int], **options) -> EngineResult:
+        return self.submit_sync(prompt_ids, **options).result()
+
+    def generate_batch_sync(self, prompts: Sequence[Sequence[int]], **options) -> List[EngineResult]:
+        futures = [self.submit_sync(p, **options) for p in prompts]
+        return [f.result() for f in futures]
+
+    async def submit(self, prompt_ids: Sequence[int], *, max_new_tokens: int, temperature: Optional[float] = None,
+                     top_p: Optional[float] = None, prefix_embeds: Optional[torch.Tensor] = None,
+                     prefix_ids: Sequence[int] = (), stop_ids: Optional[Sequence[int]] = None,
+                     seed: Optional[int] = None) -> EngineResult:
+        future = self.submit_sync(prompt_ids, max_new_tokens=max_new_tokens, temperature=temperature, top_p=top_p,
+                                  prefix_embeds=prefix_embeds, prefix_ids=prefix_ids, stop_ids=stop_ids, seed=seed)
+        return await asyncio.wrap_future(future)
+
+    async def generate(self, prompt_ids: Sequence[int], *, settings: Optional[dict] = None, **options) -> EngineResult:
+        """``settings`` takes the reference's keys: ``temperature``, ``top_p``, ``max_tokens``."""
+        settings = dict(settings or {})
+        if "max_tokens" in settings:
+            options.setdefault("max_new_tokens", settings.pop("max_tokens"))
+        for key in ("temperature", "top_p"):
+            if key in settings:
+                options.setdefault(key, settings.pop(key))
+        if settings:
+            raise ValueError(f"unknown settings: {sorted(settings)}")
+        return await self.submit(prompt_ids, **options)
+
+    async def submit_streaming(self, prompt_ids: Sequence[int], **options) -> AsyncIterator[StreamUpdate]:
+        """Yields a ``StreamUpdate`` per token as it is committed."""
+        stream: "queue.Queue" = queue.Queue()
+        future = self.submit_sync(prompt_ids, _stream=stream, **options)
+        loop = asyncio.get_running_loop()
+        request_id = future.request_id
+        while True:
+            item = await loop.run_in_executor(None, stream.get)
+            if item is None:
+                break
+            if isinstance(item, BaseException):
+                raise item
+            token, index = item
+            yield StreamUpdate(request_id, token, index)
+        await asyncio.wrap_future(future)

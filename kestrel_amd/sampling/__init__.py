@@ -1,0 +1,3 @@
+from .sampler import GREEDY_EPS, Sampler, mix_key
+
+__all__ = ["GREEDY_EPS", "Sampler", "mix_key"]

@@ -1,0 +1,185 @@
+"""The scheduler's decisions, against a runner that only keeps books (no GPU)."""
+
+from types import SimpleNamespace
+
+import pytest
+import torch
+
+from kestrel_amd.cache import CacheManager
+from kestrel_amd.engine.scheduler import GenerationScheduler
+from kestrel_amd.engine.types import GenerationRequest
+from kestrel_amd.parts.specs import CacheSpec
+
+
+class FakeRunner:
+    """Implements what the scheduler uses of ``ModelRunner``; records every step."""
+
+    def __init__(self, n_pages=16, page_size=4, max_requests=4, max_positions=64, vocab=32):
+        self.cache = CacheManager([(CacheSpec(1, 8, None), None, None)], page_size, n_pages, max_requests)
+        self.model = SimpleNamespace(plan=SimpleNamespace(max_positions=max_positions, vocab_size=vocab))
+        self.held = {}
+        self.steps = []
+        self.vocab = vocab
+
+    def admit(self, reserve_length=0, portion=1):
+        slot = self.cache.admit(reserve_length, portion)
+        self.held[slot] = 0
+        return slot
+
+    def release(self, slot):
+        self.cache.release(slot)
+        del self.held[slot]
+
+    def step(self, entries):
+        record = []
+        wanted = 0
+        for e in entries:
+            start = self.held[e.slot] if e.start is None else e.start
+            assert start == self.held[e.slot], "portions must follow each other"
+            self.cache.ensure(e.slot, start + len(e.tokens))
+            self.held[e.slot] = start + len(e.tokens)
+            for lo, hi in e.bidirectional:
+                assert start <= lo and hi <= start + len(e.tokens), "a block was split"
+            record.append((e.slot, start, len(e.tokens), list(e.want)))
+            wanted += len(e.want)
+        self.steps.append(record)
+        self.cache.check()
+        return torch.zeros(wanted, self.vocab)
+
+
+class FakeSampler:
+    """Token = 10 + index of the token in its request; request seed 99 emits the stop id 0 at index 2."""
+
+    def sample(self, logits, temps, tops, seeds, indices):
+        assert logits.shape[0] == len(temps) == len(indices)
+        return torch.tensor([0 if (s == 99 and i == 2) else 10 + i for s, i in zip(seeds, indices)], dtype=torch.int32)
+
+
+def _scheduler(runner=None, max_batch_size=4, budget=16, **kw):
+    runner = runner or FakeRunner(**kw)
+    return GenerationScheduler(runner, FakeSampler(), max_batch_size, budget, eos_token_ids=(0,)), runner
+
+
+def _req(i, n_prompt, n_new, **kw):
+    return GenerationRequest(i, list(range(1, n_prompt + 1)), n_new, **kw)
+
+
+def test_prompt_is_cut_under_the_token_budget_and_then_decoded():
+    sched, runner = _scheduler(budget=16)
+    sched.enqueue_request(_req(0, 40, 3))
+    results = sched.run_until_done()
+    sizes = [[(n, want) for _s, _p, n, want in step] for step in runner.steps]
+    assert sizes[:3] == [[(16, [])], [(16, [])], [(8, [7])]]          # portions of 16, 16, 8; logits only at the end
+    assert sizes[3:] == [[(1, [0])], [(1, [0])]]                       # then one token a step
+    assert results[0].tokens == [10, 11, 12] and results[0].finish_reason == "length"
+    assert runner.cache.groups[0].pool.free_count == 16 and runner.cache.free_slots == 4
+
+
+def test_decodes_ride_beside_prompt_portions():
+    sched, runner = _scheduler(budget=8)
+    sched.enqueue_request(_req(0, 4, 6))
+    sched.advance()                                                     # request 0 prefilled, first token
+    sched.enqueue_request(_req(1, 20, 2))
+    sched.advance()
+    step = runner.steps[-1]
+    assert [(n, want) for _s, _p, n, want in step] == [(1, [0]), (7, [])]   # decode first, prompt gets the rest
+    sched.advance()
+    assert [n for _s, _p, n, _w in runner.steps[-1]] == [1, 7]
+    results = sched.run_until_done()
+    assert sorted(r.request_id for r in results) == [0, 1]
+
+
+def test_stop_token_and_length_finish():
+    sched, runner = _scheduler()
+    sched.enqueue_request(_req(0, 3, 10, seed=99))
+    sched.enqueue_request(_req(1, 3, 2))
+    results = {r.request_id: r for r in sched.run_until_done()}
+    assert results[0].tokens == [10, 11, 0] and results[0].finish_reason == "stop"
+    assert results[1].tokens == [10, 11] and results[1].finish_reason == "length"
+    # the context length ends a request too
+    sched, runner = _scheduler(max_positions=12)
+    sched.enqueue_request(_req(2, 8, 100))
+    (result,) = sched.run_until_done()
+    assert result.finish_reason == "length" and len(result.tokens) == 4     # 8 + 4 = 12 positions
+    assert result.metrics.prompt_tokens == 8 and result.metrics.decode_tokens == 4
+
+
+def test_at_most_max_batch_size_requests_are_live():
+    sched, runner = _scheduler(max_batch_size=2, budget=64, n_pages=64)
+    for i in range(5):
+        sched.enqueue_request(_req(i, 5, 3))
+    sched.advance()
+    assert len(runner.steps[-1]) == 2 and len(sched.waiting) == 3
+    results = sched.run_until_done()
+    assert len(results) == 5
+    assert max(len(step) for step in runner.steps) <= 2
+
+
+def test_a_request_waits_for_pages_and_a_smaller_one_may_pass():
+    # 8 pages of 4 = 32 tokens. Request 0 takes 6 pages (24); request 1 needs 5 and must wait;
+    # request 2 needs 2 and passes; request 1 runs once request 0 has given its pages back.
+    sched, runner = _scheduler(n_pages=8, budget=32)
+    sched.enqueue_request(_req(0, 20, 4))
+    sched.enqueue_request(_req(1, 16, 4))
+    sched.enqueue_request(_req(2, 4, 4))
+    sched.advance()
+    assert [s.request.request_id for s in sched.running] == [0, 2]
+    assert [s.request.request_id for s in sched.waiting] == [1]
+    results = sched.run_until_done()
+    assert [r.request_id for r in results] == [0, 2, 1]
+    assert all(r.finish_reason == "length" for r in results)
+    assert runner.cache.groups[0].pool.free_count == 8
+
+
+def test_a_request_that_can_never_fit_fails_alone():
+    sched, runner = _scheduler(n_pages=4, budget=32)      # 16 tokens in all
+    sched.enqueue_request(_req(0, 20, 10))
+    sched.enqueue_request(_req(1, 4, 2))
+    results = {r.request_id: r for r in sched.run_until_done()}
+    assert results[1].finish_reason == "length"
+    assert results[0].finish_reason == "error"
+    assert results[0].error == "Insufficient KV cache capacity for request 0 (needs 30 tokens)."
+
+
+def test_a_bidirectional_block_goes_in_one_portion():
+    sched, runner = _scheduler(budget=12, n_pages=32)
+    embeds = torch.zeros(7, 8)
+    sched.enqueue_request(_req(0, 9, 2))
+    sched.advance()
+    sched.enqueue_request(GenerationRequest(1, [5, 6, 7, 8, 9, 10], 2, prefix_embeds=embeds, prefix_ids=[0]))
+    sched.advance()
+    step = runner.steps[-1]
+    # 1 decode + 11 budget: block of 8 (BOS + 7 rows) and 3 text tokens
+    assert [(n, w) for _s, _p, n, w in step] == [(1, [0]), (11, [])]
+    sched.run_until_done()
+    # a block larger than what is left of the budget waits for a step with room; it is never split
+    sched, runner = _scheduler(budget=9, n_pages=32)
+    sched.enqueue_request(_req(0, 5, 2))
+    sched.enqueue_request(GenerationRequest(1, [5, 6], 1, prefix_embeds=embeds, prefix_ids=[0]))
+    sched.advance()
+    assert [n for _s, _p, n, _w in runner.steps[-1]] == [5]
+    sched.run_until_done()
+    assert any(n == 8 or n == 9 or n == 10 for step in runner.steps for _s, _p, n, _w in step)
+    with pytest.raises(ValueError, match="does not fit in one step"):
+        sched.enqueue_request(GenerationRequest(2, [1], 1, prefix_embeds=torch.zeros(20, 8)))
+
+
+def test_bad_requests_are_refused():
+    sched, _ = _scheduler()
+    for bad in (dict(max_new_tokens=0), dict(temperature=-1.0), dict(top_p=0.0), dict(top_p=1.5)):
+        kwargs = dict(max_new_tokens=2)
+        kwargs.update(bad)
+        with pytest.raises(ValueError):
+            sched.enqueue_request(GenerationRequest(0, [1, 2], **kwargs))
+    with pytest.raises(ValueError, match="at least one"):
+        sched.enqueue_request(GenerationRequest(0, [], 2))
+    with pytest.raises(ValueError, match="leaves no room"):
+        sched.enqueue_request(_req(0, 64, 2))
+
+
+def test_tokens_are_streamed_as_they_are_committed():
+    sched, _ = _scheduler()
+    seen = []
+    sched.enqueue_request(_req(0, 3, 3, on_token=lambda tok, i: seen.append((tok, i))))
+    sched.run_until_done()
+    assert seen == [(10, 0), (11, 1), (12, 2)]
