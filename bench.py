@@ -1,0 +1,230 @@
+"""Decode and prefill throughput of the engine on one MI355X.
+
+``python bench.py --gpus 1 --steps K --warmup W`` prints one JSON line. A step is one
+decode step of the default batch (8 requests, each holding ``context`` tokens: a block of
+prefix embeddings and text ids) through the engine's step function with greedy sampling
+on the GPU. The model has the layer sizes of the Moondream 2 text decoder with seeded
+random weights N(0, 0.02) in bf16; inputs are synthetic. Besides ``value`` (decoded tokens
+a second) the line carries a 2,048-token prefill, the decode step's HBM roofline and
+decode throughput at batch 1 and 64.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+# Layer sizes of the benchmark model (Moondream 2 text decoder) and its workload.
+MODEL = {"dim": 2048, "ff_dim": 8192, "n_layers": 24, "vocab_size": 51200, "max_context": 2048, "n_heads": 32,
+         "n_kv_heads": 32, "rope_theta": 10000.0, "prefix_attn": 730, "layer_norm_eps": 1e-5}
+CONTEXT = 1024          # tokens each request holds when decoding starts (730 prefix + 294 text)
+PREFILL_TOKENS = 2048
+PAGE_SIZE = 16
+SEED = 2
+PEAK_HBM = 8.0e12
+PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
+
+
+def build_model(layers: int, dtype, device):
+    """The benchmark model with random weights drawn on the GPU (nothing is read from disk)."""
+    import torch
+
+    from kestrel_amd.config import get_spec
+    from kestrel_amd.models import DecoderModel
+    from kestrel_amd.weights import InitRecipe, random_tensor
+
+    spec = get_spec("moondream2")
+    typed = spec.read_config({"text": dict(MODEL, n_layers=layers)})
+    net = DecoderModel(spec.build_plan(typed))
+    recipe = InitRecipe(std=0.02)
+    store = torch.bfloat16
+    tensors = {name: random_tensor(name, pspec, SEED, recipe, device=device).to(store if dtype == torch.bfloat16 else dtype)
+               for name, pspec in net.params().items()}
+    net.bind(tensors, dtype, device)
+    return net, typed
+
+
+def model_bytes(net, dtype_size: int) -> int:
+    """Bytes of weights a decode step reads once: every linear, norm and the head (the
+    embedding table is read only at the rows of the batch)."""
+    total = 0
+    emb = net.plan.names["embedding"]
+    for name, pspec in net.params().items():
+        if name == emb:
+            continue
+        count = 1
+        for s in pspec.shape:
+            count *= s
+        total += count * dtype_size
+    return total
+
+
+def prefill_flops(typed, tokens: int, prefix: int) -> float:
+    """Multiply-adds x 2 of one prompt of ``tokens`` positions whose first ``prefix`` are a
+    bidirectional block; the head runs on the last position only."""
+    d, ff, hd = typed.dim, typed.ff_dim, typed.head_dim
+    qkv = (typed.n_heads + 2 * typed.n_kv_heads) * hd
+    per_token_linear = 2 * (d * qkv + typed.n_heads * hd * d + 2 * d * ff)
+    pairs = prefix * prefix + sum(q + 1 for q in range(prefix, tokens))
+    attention = 4 * hd * typed.n_heads * pairs
+    return typed.n_layers * (tokens * per_token_linear + attention) + 2 * d * typed.vocab_size
+
+
+class DecodeBench:
+    """A batch of requests prefilled to ``context`` tokens, then decoded step by step."""
+
+    def __init__(self, net, typed, batch: int, context: int, steps_total: int):
+        import torch
+
+        from kestrel_amd.engine.loading import make_runner
+        from kestrel_amd.engine.step import StepEntry
+        from kestrel_amd.sampling import Sampler
+
+        self.torch, self.StepEntry = torch, StepEntry
+        self.net, self.typed, self.batch, self.context = net, typed, batch, context
+        pages_per_request = -(-(context + steps_total + 1) // PAGE_SIZE)
+        self.runner = make_runner(net, PAGE_SIZE, batch * pages_per_request, batch, max_tokens_per_step=4096)
+        self.sampler = Sampler(net.device)
+        gen = torch.Generator().manual_seed(SEED)
+        prefix = min(typed.prefix_attn, context - 1)
+        self.slots = []
+        last = []
+        for _ in range(batch):
+            slot = self.runner.admit()
+            embeds = torch.randn(prefix, typed.dim, generator=gen)
+            ids = torch.randint(0, typed.vocab_size, (context - prefix,), generator=gen).tolist()
+            entry = StepEntry(slot, [-1] * prefix + ids, want=[context - 1], embeds=embeds.to(net.device),
+                              bidirectional=[(0, prefix)] if prefix else [])
+            logits = self.runner.step([entry])
+            last.append(int(self.sampler.greedy(logits)[0]))
+            self.slots.append(slot)
+        self.last = last
+
+    def step(self):
+        entries = [self.StepEntry(slot, [tok], want=[0]) for slot, tok in zip(self.slots, self.last)]
+        logits = self.runner.step(entries)
+        self.last = self.sampler.greedy(logits).tolist()
+
+    def kv_bytes_now(self, dtype_size: int) -> int:
+        t = self.typed
+        per_token = 2 * t.n_kv_heads * t.head_dim * dtype_size * t.n_layers
+        return per_token * sum(self.runner.held[s] for s in self.slots)
+
+    def close(self):
+        for slot in self.slots:
+            self.runner.release(slot)
+        self.runner = None
+
+
+def time_decode(net, typed, batch, context, steps, warmup):
+    import torch
+
+    bench = DecodeBench(net, typed, batch, context, steps + warmup)
+    for _ in range(warmup):
+        bench.step()
+    torch.cuda.synchronize()
+    kv_start = bench.kv_bytes_now(2)
+    started = time.perf_counter()
+    for _ in range(steps):
+        bench.step()
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - started
+    kv_end = bench.kv_bytes_now(2)
+    bench.close()
+    torch.cuda.empty_cache()
+    return elapsed, 0.5 * (kv_start + kv_end)
+
+
+def time_prefill(net, typed, tokens, repeats=3):
+    import torch
+
+    from kestrel_amd.engine.loading import make_runner
+    from kestrel_amd.engine.step import StepEntry
+
+    runner = make_runner(net, PAGE_SIZE, -(-tokens // PAGE_SIZE) + 1, 1, max_tokens_per_step=tokens)
+    gen = torch.Generator().manual_seed(SEED + 1)
+    prefix = min(typed.prefix_attn, tokens - 1)
+    embeds = torch.randn(prefix, typed.dim, generator=gen).to(net.device)
+    ids = torch.randint(0, typed.vocab_size, (tokens - prefix,), generator=gen).tolist()
+    best = None
+    for i in range(repeats + 1):
+        slot = runner.admit()
+        entry = StepEntry(slot, [-1] * prefix + ids, want=[tokens - 1], embeds=embeds,
+                          bidirectional=[(0, prefix)] if prefix else [])
+        torch.cuda.synchronize()
+        started = time.perf_counter()
+        runner.step([entry])
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - started
+        runner.release(slot)
+        if i > 0:                      # the first run warms up
+            best = elapsed if best is None else min(best, elapsed)
+    return best
+
+
+def main() -> int:
+    parser = argparse.ArgumentParser()
+    parser.add_argument("--gpus", type=int, default=1)
+    parser.add_argument("--steps", type=int, default=128)
+    parser.add_argument("--warmup", type=int, default=8)
+    parser.add_argument("--batch", type=int, default=8)
+    parser.add_argument("--layers", type=int, default=MODEL["n_layers"], help="fewer layers than the model has (named in config)")
+    parser.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
+    parser.add_argument("--skip-points", action="store_true", help="only the default batch (no batch 1 / 64, no prefill)")
+    args = parser.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
+        return 2
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible")
+        return 1
+    device = torch.device("cuda:0")
+    torch.cuda.set_device(device)
+    dtype = torch.bfloat16 if args.dtype == "bf16" else torch.float32
+    size = 2 if dtype == torch.bfloat16 else 4
+    net, typed = build_model(args.layers, dtype, device)
+    weights = model_bytes(net, size)
+
+    elapsed, kv_bytes = time_decode(net, typed, args.batch, CONTEXT, args.steps, args.warmup)
+    ms_per_step = elapsed / args.steps * 1e3
+    value = args.batch * args.steps / elapsed
+    step_bytes = weights + kv_bytes * (size / 2) + args.batch * typed.dim * size
+    achieved = step_bytes / (elapsed / args.steps)
+    record = {
+        "metric": "decode tok/s (Moondream 2 text decoder sizes, batch 8, context 1024)", "value": round(value, 1),
+        "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": args.dtype, "data": "synthetic (seeded random token ids and prefix embeddings, random weights N(0,0.02))",
+        "config": {"model": "moondream2-text", "n_layers": args.layers, "n_layers_full": MODEL["n_layers"],
+                   "dim": typed.dim, "ff_dim": typed.ff_dim, "n_heads": typed.n_heads, "n_kv_heads": typed.n_kv_heads,
+                   "head_dim": typed.head_dim, "rotary_dim": typed.rotary_dim, "vocab_size": typed.vocab_size,
+                   "global_batch": args.batch, "seq_len": CONTEXT, "prefix_attn": typed.prefix_attn,
+                   "page_size": PAGE_SIZE, "parallelism": "single-gpu"},
+        "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": PEAK_HBM / 1e9, "unit": "GB/s",
+                     "frac": round(achieved / PEAK_HBM, 4)},
+    }
+    if not args.skip_points:
+        seconds = time_prefill(net, typed, PREFILL_TOKENS)
+        flops = prefill_flops(typed, PREFILL_TOKENS, min(typed.prefix_attn, PREFILL_TOKENS - 1))
+        record["prefill"] = {"value": round(PREFILL_TOKENS / seconds, 1), "tokens": PREFILL_TOKENS,
+                             "ms": round(seconds * 1e3, 3), "frac": round(flops / seconds / PEAK_FLOPS[args.dtype], 4)}
+        points = {}
+        for batch, steps in ((1, args.steps), (64, max(16, args.steps // 4))):
+            e, _ = time_decode(net, typed, batch, CONTEXT, steps, min(args.warmup, 4))
+            points[f"decode_b{batch}"] = round(batch * steps / e, 1)
+        record["points"] = points
+    print(json.dumps(record))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
