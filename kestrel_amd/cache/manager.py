@@ -75,7 +75,7 @@ class _Group:
     entries: List[int]                 # schedule entries that own a cache in this group
     pool: PagePool
     k: Optional[torch.Tensor] = None   # [len(entries), pages, Hkv, page_size, hd]
-    v: Optional[torch.Tensor] = None
+    v: Optional[torch.Tensor] = None   # [len(entries), pages, Hkv, hd, page_size]
 
 
 class _SlotState:
@@ -130,9 +130,12 @@ class CacheManager:
     # ------------------------------------------------------------------ device memory
     def _allocate_device(self) -> None:
         for group in self.groups:
-            shape = (len(group.entries), self.n_pages, group.spec.n_kv_heads, self.page_size, group.spec.head_dim)
-            group.k = torch.zeros(shape, dtype=self.dtype, device=self.device)
-            group.v = torch.zeros(shape, dtype=self.dtype, device=self.device)
+            spec = group.spec
+            # values are kept transposed inside a page: eight consecutive keys of one channel are 16 bytes
+            group.k = torch.zeros((len(group.entries), self.n_pages, spec.n_kv_heads, self.page_size, spec.head_dim),
+                                  dtype=self.dtype, device=self.device)
+            group.v = torch.zeros((len(group.entries), self.n_pages, spec.n_kv_heads, spec.head_dim, self.page_size),
+                                  dtype=self.dtype, device=self.device)
         for entry, (_c, state_spec, _r) in enumerate(self.needs):
             if state_spec is not None:
                 self.states[entry] = torch.zeros((self.max_requests, *state_spec.shape),

@@ -1,0 +1,426 @@
+// bf16 paged attention on the matrix cores: a prompt kernel and a decode kernel.
+//
+// Cache layout: keys [pages, Hkv, 16, hd], values [pages, Hkv, hd, 16] (transposed inside the
+// page), page size 16. Every token t of the packed batch reads the keys [kv_lo[t], kv_hi[t]) of
+// its row through the row's block table; the step's own keys are already in the cache.
+//
+// Prompt kernel. A wave owns 32 consecutive queries of one row and one head and walks the keys
+// in tiles of 32 (two pages). Scores are computed transposed, S^T = K Q^T, with
+// v_mfma_f32_32x32x16_bf16: the keys are the row operand (a lane loads half a key row straight
+// from the cache), the queries the column operand (held in registers for the whole loop). A
+// lane then holds, for ONE query, 16 scores: softmax needs only in-lane work and one exchange
+// with the lane 32 apart. The key rows are fed to the MFMA in a permuted order (bits 2 and 3 of
+// the row index swapped) so that the 8 probabilities a lane holds for a page are those of 8
+// consecutive keys: they are, as they stand, the column operand of O^T += V^T P^T, whose row
+// operand is one 16-byte load from the transposed value page. No LDS, no barriers.
+//
+// Decode kernel. One query per row: a bandwidth problem. The keys of a row are cut into splits
+// (grid z) and 64-key tiles (waves); 16-byte loads are fully coalesced for keys (8 lanes per key
+// row at hd 64) and values (2 lanes per channel row of a page). Waves merge through LDS, splits
+// through scratch memory by the last workgroup to arrive, always in the same order.
+#include "ka_common.h"
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
+typedef __attribute__((ext_vector_type(16))) float floatx16;
+typedef __attribute__((ext_vector_type(4))) float floatx4;
+
+constexpr int AT_PAGE = 16;
+constexpr float AT_LOG2E = 1.4426950408889634f;
+
+__device__ __forceinline__ bf16x8 at_load8(const bf16_t* p) { return *reinterpret_cast<const bf16x8*>(p); }
+
+// Orders the LDS traffic of one wave: what its lanes wrote before is seen by its lanes after.
+__device__ __forceinline__ void at_wave_sync() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// ----------------------------------------------------------------------------------------------
+// prompt kernel
+// ----------------------------------------------------------------------------------------------
+constexpr int AP_WAVES = 4;
+constexpr int AP_QBLOCK = 32 * AP_WAVES;    // queries per workgroup
+
+template <int HD>
+__global__ void __launch_bounds__(KA_WAVE * AP_WAVES)
+attn_prefill_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t* __restrict__ k_cache,
+                    const bf16_t* __restrict__ v_cache, const int* __restrict__ block_table, int max_pages,
+                    const int* __restrict__ qblk_row, const int* __restrict__ qblk_tok,
+                    const int* __restrict__ cu_q, const int* __restrict__ kv_len,
+                    const int* __restrict__ kv_lo, const int* __restrict__ kv_hi, bf16_t* __restrict__ out,
+                    long out_row_stride, float scale, int H, int Hkv) {
+    constexpr int QC = HD / 16;          // 16-byte chunks of half a head row = MFMA steps of the score product
+    constexpr int DB = HD / 32;          // 32-channel blocks of the output
+    const int blk = blockIdx.x, h = blockIdx.y;
+    const int wave = threadIdx.x / KA_WAVE, lane = threadIdx.x % KA_WAVE;
+    const int li = lane % 32, lg = lane / 32;
+    const int kvh = h / (H / Hkv);
+    const int row = qblk_row[blk];
+    const int tok_end = cu_q[row + 1];
+    const int tok0 = qblk_tok[blk] + wave * 32;
+    if (tok0 >= tok_end) return;
+    const int t = tok0 + li;
+    const bool q_valid = t < tok_end;
+    const int tq = q_valid ? t : tok_end - 1;
+    const int hi = q_valid ? kv_hi[tq] : 0;
+    const int lo = kv_lo ? kv_lo[tq] : 0;
+    int wave_hi = hi, wave_lo = q_valid ? lo : 0x7fffffff;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        wave_hi = max(wave_hi, __shfl_xor(wave_hi, off, KA_WAVE));
+        wave_lo = min(wave_lo, __shfl_xor(wave_lo, off, KA_WAVE));
+    }
+    const int limit = kv_len[row];       // keys of this row that hold data
+    wave_hi = min(wave_hi, limit);
+    const int* bt = block_table + (size_t)row * max_pages;
+
+    // queries: lane (q = li, g = lg) holds channels [g * HD/2, (g + 1) * HD/2)
+    bf16x8 qreg[QC];
+    {
+        const bf16_t* qp = q + (size_t)tq * q_row_stride + (size_t)h * HD + lg * (HD / 2);
+#pragma unroll
+        for (int c = 0; c < QC; ++c) qreg[c] = at_load8(qp + c * 8);
+    }
+    floatx16 o[DB];
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) o[db][v] = 0.f;
+    float m_i = -INFINITY, l_i = 0.f;
+    const float sl2 = scale * AT_LOG2E;
+    const int kperm = (li & 16) | ((li & 4) << 1) | ((li & 8) >> 1) | (li & 3);
+    const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+
+    for (int key0 = wave_lo & ~31; key0 < wave_hi; key0 += 32) {
+        // scores S^T[key][query]
+        floatx16 s;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) s[v] = 0.f;
+        {
+            int key = max(min(key0 + kperm, limit - 1), wave_lo);   // pages below wave_lo may have been given back
+            int page = bt[key / AT_PAGE];
+            const bf16_t* kp = k_cache + (((size_t)page * Hkv + kvh) * AT_PAGE + key % AT_PAGE) * HD + lg * (HD / 2);
+#pragma unroll
+            for (int c = 0; c < QC; ++c) s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(at_load8(kp + c * 8), qreg[c], s, 0, 0, 0);
+        }
+        // lane holds, for its query, the keys key0 + (v / 8) * 16 + lg * 8 + v % 8
+        float mx = -INFINITY;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            int key = key0 + (v / 8) * 16 + lg * 8 + (v % 8);
+            bool ok = key >= lo && key < hi;
+            s[v] = ok ? s[v] * sl2 : -INFINITY;
+            mx = fmaxf(mx, s[v]);
+        }
+        mx = fmaxf(mx, __shfl_xor(mx, 32, KA_WAVE));
+        float m_new = fmaxf(m_i, mx);
+        float m_use = m_new == -INFINITY ? 0.f : m_new;     // nothing visible yet: keep everything at zero
+        float alpha = exp2f(m_i - m_use);
+        float rowsum = 0.f;
+        bf16x8 pb[2];
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            float p = exp2f(s[v] - m_use);
+            rowsum += p;
+            pb[v / 8][v % 8] = (bf16_t)p;
+        }
+        rowsum += __shfl_xor(rowsum, 32, KA_WAVE);
+        l_i = l_i * alpha + rowsum;
+        m_i = m_new;
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) o[db][v] *= alpha;
+        // O^T[d][query] += V^T[d][key] P^T[key][query], one page per MFMA
+#pragma unroll
+        for (int pg = 0; pg < 2; ++pg) {
+            int kbase = key0 + pg * AT_PAGE;
+            if (kbase >= wave_hi) break;
+            if (kbase + AT_PAGE <= wave_lo) continue;   // nothing visible here, and the page may be gone
+            int page = bt[kbase / AT_PAGE];
+            int first = kbase + lg * 8;          // first of the 8 keys this lane loads
+#pragma unroll
+            for (int db = 0; db < DB; ++db) {
+                const bf16_t* vp = v_cache + (((size_t)page * Hkv + kvh) * HD + db * 32 + li) * AT_PAGE + lg * 8;
+                bf16x8 vv = at_load8(vp);
+                if (first + 8 > limit) {         // slots past the row's data may hold anything: keep them out
+#pragma unroll
+                    for (int j = 0; j < 8; ++j)
+                        if (first + j >= limit) vv[j] = (bf16_t)0.f;
+                }
+                o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vv, pb[pg], o[db], 0, 0, 0);
+            }
+        }
+    }
+    if (!q_valid) return;
+    float inv = l_i > 0.f ? 1.0f / l_i : 0.f;
+    bf16_t* op = out + (size_t)t * out_row_stride + (size_t)h * HD;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int qd = 0; qd < 4; ++qd) {
+            int d = db * 32 + qd * 8 + lg * 4;
+            bf16x4 r = {(bf16_t)(o[db][qd * 4 + 0] * inv), (bf16_t)(o[db][qd * 4 + 1] * inv),
+                        (bf16_t)(o[db][qd * 4 + 2] * inv), (bf16_t)(o[db][qd * 4 + 3] * inv)};
+            *reinterpret_cast<bf16x4*>(op + d) = r;
+        }
+}
+
+// ----------------------------------------------------------------------------------------------
+// decode kernel
+// ----------------------------------------------------------------------------------------------
+constexpr int AD_WAVES = 4;
+constexpr int AD_TILE = 64;               // keys per wave tile
+
+template <int HD>
+__global__ void __launch_bounds__(KA_WAVE * AD_WAVES)
+attn_decode_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t* __restrict__ k_cache,
+                   const bf16_t* __restrict__ v_cache, const int* __restrict__ block_table, int max_pages,
+                   const int* __restrict__ token_row, const int* __restrict__ kv_lo,
+                   const int* __restrict__ kv_hi, bf16_t* __restrict__ out, long out_row_stride, float scale,
+                   int H, int Hkv, float* __restrict__ partial, unsigned* __restrict__ counters) {
+    constexpr int LPK = HD / 8;            // lanes per key row
+    constexpr int KPI = KA_WAVE / LPK;     // keys per load instruction
+    constexpr int VU = HD * 2 / KA_WAVE;   // 16-byte value loads per lane and page
+    constexpr int REC = HD + 2;            // floats of a partial result: m, l, o[HD]
+    __shared__ float ps[AD_WAVES][AD_TILE];
+    __shared__ float merge[AD_WAVES][REC];
+    const int t = blockIdx.x, h = blockIdx.y, split = blockIdx.z, S = gridDim.z;
+    const int wave = threadIdx.x / KA_WAVE, lane = threadIdx.x % KA_WAVE;
+    const int kvh = h / (H / Hkv);
+    const int row = token_row[t];
+    const int lo = kv_lo ? kv_lo[t] : 0, hi = kv_hi[t];
+    const int lo_tile = lo & ~(AD_TILE - 1);      // tiles start on page boundaries; keys below lo are masked
+    const int chunk = ((hi - lo_tile + S - 1) / S + AD_TILE - 1) / AD_TILE * AD_TILE;
+    const int s_lo = lo_tile + split * chunk, s_hi = min(hi, s_lo + chunk);
+    const int* bt = block_table + (size_t)row * max_pages;
+    const int ks = lane / LPK, dg = lane % LPK;
+    const float sl2 = scale * AT_LOG2E;
+    float qf[8];
+    {
+        bf16x8 qv = at_load8(q + (size_t)t * q_row_stride + (size_t)h * HD + dg * 8);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) qf[j] = (float)qv[j] * sl2;
+    }
+    float m_i = -INFINITY, l_i = 0.f;
+    float acc[VU];
+#pragma unroll
+    for (int u = 0; u < VU; ++u) acc[u] = 0.f;
+
+    for (int tile0 = s_lo + wave * AD_TILE; tile0 < s_hi; tile0 += AD_WAVES * AD_TILE) {
+        float sc[LPK];
+        float mx = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < LPK; ++i) {
+            int key = tile0 + i * KPI + ks;
+            bool ok = key >= lo && key < s_hi;
+            int kc = max(min(key, s_hi - 1), lo);   // a place that holds data (pages below lo may be gone)
+            int page = bt[kc / AT_PAGE];
+            bf16x8 kv = at_load8(k_cache + (((size_t)page * Hkv + kvh) * AT_PAGE + kc % AT_PAGE) * HD + dg * 8);
+            float dot = 0.f;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) dot = fmaf(qf[j], (float)kv[j], dot);
+#pragma unroll
+            for (int off = 1; off < LPK; off <<= 1) dot += __shfl_xor(dot, off, KA_WAVE);
+            sc[i] = ok ? dot : -INFINITY;
+            mx = fmaxf(mx, sc[i]);
+        }
+#pragma unroll
+        for (int off = LPK; off < KA_WAVE; off <<= 1) mx = fmaxf(mx, __shfl_xor(mx, off, KA_WAVE));
+        float m_new = fmaxf(m_i, mx);
+        if (m_new == -INFINITY) continue;      // a tile wholly below lo (wave-uniform)
+        float alpha = exp2f(m_i - m_new);
+        float rowsum = 0.f;
+        at_wave_sync();                        // the previous tile's probabilities have been read
+#pragma unroll
+        for (int i = 0; i < LPK; ++i) {
+            float p = exp2f(sc[i] - m_new);
+            rowsum += p;
+            if (dg == 0) ps[wave][i * KPI + ks] = p;
+        }
+#pragma unroll
+        for (int off = LPK; off < KA_WAVE; off <<= 1) rowsum += __shfl_xor(rowsum, off, KA_WAVE);
+        l_i = l_i * alpha + rowsum;
+        m_i = m_new;
+#pragma unroll
+        for (int u = 0; u < VU; ++u) acc[u] *= alpha;
+        at_wave_sync();
+        // values: a page is HD rows of 16 keys; lane takes 8 keys (half a row) per load
+#pragma unroll
+        for (int pg = 0; pg < AD_TILE / AT_PAGE; ++pg) {
+            int kbase = tile0 + pg * AT_PAGE;
+            if (kbase >= s_hi) break;
+            if (kbase + AT_PAGE <= lo) continue;
+            int page = bt[kbase / AT_PAGE];
+            int half = lane & 1;
+            int first = kbase + half * 8;
+            float pv[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) pv[j] = ps[wave][pg * AT_PAGE + half * 8 + j];
+#pragma unroll
+            for (int u = 0; u < VU; ++u) {
+                int d = u * 32 + lane / 2;
+                bf16x8 vv = at_load8(v_cache + (((size_t)page * Hkv + kvh) * HD + d) * AT_PAGE + half * 8);
+                float sum = 0.f;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    int key = first + j;                      // slots outside the data may hold anything
+                    float x = key >= lo && key < s_hi ? (float)vv[j] : 0.f;
+                    sum = fmaf(pv[j], x, sum);
+                }
+                acc[u] += sum;
+            }
+        }
+    }
+    // the two halves of a channel row
+#pragma unroll
+    for (int u = 0; u < VU; ++u) acc[u] += __shfl_xor(acc[u], 1, KA_WAVE);
+    if (lane == 0) { merge[wave][0] = m_i; merge[wave][1] = l_i; }
+    if ((lane & 1) == 0) {
+#pragma unroll
+        for (int u = 0; u < VU; ++u) merge[wave][2 + u * 32 + lane / 2] = acc[u];
+    }
+    __syncthreads();
+    if (wave != 0) return;
+    // wave 0: lane d (and d + 64 for hd 128) merges the waves in wave order
+    float M = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < AD_WAVES; ++w) M = fmaxf(M, merge[w][0]);
+    float L = 0.f;
+    float od[(HD + KA_WAVE - 1) / KA_WAVE];
+#pragma unroll
+    for (int e = 0; e < (HD + KA_WAVE - 1) / KA_WAVE; ++e) od[e] = 0.f;
+#pragma unroll
+    for (int w = 0; w < AD_WAVES; ++w) {
+        float mw = merge[w][0];
+        float f = mw == -INFINITY ? 0.f : exp2f(mw - M);
+        L += merge[w][1] * f;
+#pragma unroll
+        for (int e = 0; e < (HD + KA_WAVE - 1) / KA_WAVE; ++e) {
+            int d = e * KA_WAVE + lane;
+            if (d < HD) od[e] += merge[w][2 + d] * f;
+        }
+    }
+    if (S > 1) {
+        float* mine = partial + ((size_t)(t * H + h) * S + split) * REC;
+        if (lane == 0) { mine[0] = M; mine[1] = L; }
+#pragma unroll
+        for (int e = 0; e < (HD + KA_WAVE - 1) / KA_WAVE; ++e) {
+            int d = e * KA_WAVE + lane;
+            if (d < HD) mine[2 + d] = od[e];
+        }
+        __threadfence();
+        unsigned seen = 0;
+        if (lane == 0) seen = atomicAdd(&counters[t * H + h], 1u);
+        seen = __shfl(seen, 0, KA_WAVE);
+        if (seen != (unsigned)(S - 1)) return;
+        if (lane == 0) atomicExch(&counters[t * H + h], 0u);
+        __threadfence();
+        const float* all = partial + (size_t)(t * H + h) * S * REC;
+        M = -INFINITY;
+        for (int s = 0; s < S; ++s)
+            M = fmaxf(M, __hip_atomic_load(all + s * REC, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+        L = 0.f;
+#pragma unroll
+        for (int e = 0; e < (HD + KA_WAVE - 1) / KA_WAVE; ++e) od[e] = 0.f;
+        for (int s = 0; s < S; ++s) {
+            float ms = __hip_atomic_load(all + s * REC, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            float f = ms == -INFINITY ? 0.f : exp2f(ms - M);
+            L += __hip_atomic_load(all + s * REC + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) * f;
+#pragma unroll
+            for (int e = 0; e < (HD + KA_WAVE - 1) / KA_WAVE; ++e) {
+                int d = e * KA_WAVE + lane;
+                if (d < HD) od[e] += __hip_atomic_load(all + s * REC + 2 + d, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) * f;
+            }
+        }
+    }
+    float inv = L > 0.f ? 1.0f / L : 0.f;
+    bf16_t* op = out + (size_t)t * out_row_stride + (size_t)h * HD;
+#pragma unroll
+    for (int e = 0; e < (HD + KA_WAVE - 1) / KA_WAVE; ++e) {
+        int d = e * KA_WAVE + lane;
+        if (d < HD) op[d] = (bf16_t)(od[e] * inv);
+    }
+}
+
+// ----------------------------------------------------------------------------------------------
+// entry points
+// ----------------------------------------------------------------------------------------------
+static int check_common(const char* who, const void* q, long q_row_stride, const void* out, long out_row_stride,
+                        int n, int H, int Hkv, int hd, int page_size, int max_pages) {
+    KA_CHECK(n > 0 && H > 0 && Hkv > 0 && H % Hkv == 0, "%s: bad sizes n=%d H=%d Hkv=%d", who, n, H, Hkv);
+    KA_CHECK(page_size == AT_PAGE, "%s: page size %d (the MFMA kernels need %d)", who, page_size, AT_PAGE);
+    KA_CHECK(max_pages > 0, "%s: empty block table", who);
+    KA_CHECK(q_row_stride % 8 == 0 && (uintptr_t)q % 16 == 0 && hd % 8 == 0, "%s: q must be 16-byte aligned", who);
+    KA_CHECK(out_row_stride % 4 == 0 && (uintptr_t)out % 8 == 0, "%s: out must be 8-byte aligned", who);
+    KA_CHECK(H <= 65535, "%s: too many heads", who);
+    return 0;
+}
+
+KA_API int ka_attention_prefill_supported(int hd, int page_size) {
+    return page_size == AT_PAGE && (hd == 32 || hd == 64 || hd == 96 || hd == 128);
+}
+
+KA_API int ka_attention_decode_supported(int hd, int page_size) {
+    return page_size == AT_PAGE && (hd == 64 || hd == 128);
+}
+
+KA_API int ka_attention_prefill_bf16(const void* q, long q_row_stride, const void* k_cache, const void* v_cache,
+                                     const int* block_table, int max_pages, const int* qblk_row,
+                                     const int* qblk_tok, int n_qblocks, const int* cu_q, const int* kv_len,
+                                     const int* kv_lo, const int* kv_hi, void* out, long out_row_stride,
+                                     float scale, int H, int Hkv, int hd, int page_size, hipStream_t stream) {
+    if (check_common("ka_attention_prefill_bf16", q, q_row_stride, out, out_row_stride, n_qblocks, H, Hkv, hd,
+                     page_size, max_pages))
+        return -1;
+    KA_CHECK(ka_attention_prefill_supported(hd, page_size), "ka_attention_prefill_bf16: head size %d not covered", hd);
+    dim3 grid(n_qblocks, H), block(KA_WAVE * AP_WAVES);
+#define KA_AP(HDV)                                                                                                  \
+    hipLaunchKernelGGL(attn_prefill_kernel<HDV>, grid, block, 0, stream, (const bf16_t*)q, q_row_stride,            \
+                       (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, max_pages, qblk_row, qblk_tok,  \
+                       cu_q, kv_len, kv_lo, kv_hi, (bf16_t*)out, out_row_stride, scale, H, Hkv)
+    switch (hd) {
+        case 32: KA_AP(32); break;
+        case 64: KA_AP(64); break;
+        case 96: KA_AP(96); break;
+        default: KA_AP(128); break;
+    }
+#undef KA_AP
+    KA_LAUNCH_CHECK();
+    return 0;
+}
+
+KA_API long ka_attention_decode_partial_floats(int n, int H, int hd, int splits) {
+    return (long)n * H * splits * (hd + 2);
+}
+
+KA_API int ka_attention_decode_bf16(const void* q, long q_row_stride, const void* k_cache, const void* v_cache,
+                                    const int* block_table, int max_pages, const int* token_row, const int* kv_lo,
+                                    const int* kv_hi, void* out, long out_row_stride, float scale, int n, int H,
+                                    int Hkv, int hd, int page_size, int splits, float* partial,
+                                    long partial_floats, unsigned* counters, int n_counters, hipStream_t stream) {
+    if (check_common("ka_attention_decode_bf16", q, q_row_stride, out, out_row_stride, n, H, Hkv, hd, page_size,
+                     max_pages))
+        return -1;
+    KA_CHECK(ka_attention_decode_supported(hd, page_size), "ka_attention_decode_bf16: head size %d not covered", hd);
+    KA_CHECK(splits >= 1 && splits <= 65535, "ka_attention_decode_bf16: bad split count %d", splits);
+    if (splits > 1) {
+        KA_CHECK(partial && counters, "ka_attention_decode_bf16: scratch missing");
+        KA_CHECK(ka_attention_decode_partial_floats(n, H, hd, splits) <= partial_floats,
+                 "ka_attention_decode_bf16: scratch too small");
+        KA_CHECK((long)n * H <= n_counters, "ka_attention_decode_bf16: too few counters");
+    }
+    dim3 grid(n, H, splits), block(KA_WAVE * AD_WAVES);
+    if (hd == 64)
+        hipLaunchKernelGGL(attn_decode_kernel<64>, grid, block, 0, stream, (const bf16_t*)q, q_row_stride,
+                           (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, max_pages, token_row, kv_lo,
+                           kv_hi, (bf16_t*)out, out_row_stride, scale, H, Hkv, partial, counters);
+    else
+        hipLaunchKernelGGL(attn_decode_kernel<128>, grid, block, 0, stream, (const bf16_t*)q, q_row_stride,
+                           (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, max_pages, token_row, kv_lo,
+                           kv_hi, (bf16_t*)out, out_row_stride, scale, H, Hkv, partial, counters);
+    KA_LAUNCH_CHECK();
+    return 0;
+}

@@ -7,7 +7,7 @@
 // bidirectional block has kv_hi = end of its block; a window of w has
 // kv_lo = max(0, p + 1 - w). The keys of this step are already in the cache.
 // Key position k of row r lies at page block_table[r, k / page_size], offset
-// k % page_size; cache layout [pages, Hkv, page_size, hd].
+// k % page_size; key cache [pages, Hkv, page_size, hd], value cache [pages, Hkv, hd, page_size].
 #include "ka_common.h"
 
 constexpr int ATT_MAX_HD = 512;
@@ -22,7 +22,7 @@ attention_generic_kernel(const T* __restrict__ q, long q_row_stride, const T* __
                          int hd, int page_size) {
     __shared__ float qs[ATT_MAX_HD];
     __shared__ float ps[KA_WAVE];
-    __shared__ long offs[KA_WAVE];
+    __shared__ long offs[KA_WAVE];   // value cache offset of channel 0 of each key of the chunk
     int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
     int kvh = h / (H / Hkv);
     int row = token_row[t];
@@ -42,8 +42,8 @@ attention_generic_kernel(const T* __restrict__ q, long q_row_stride, const T* __
         long off = 0;
         if (valid) {
             int page = bt[key / page_size];
-            off = (((long)page * Hkv + kvh) * page_size + key % page_size) * hd;
-            const T* kp = k_cache + off;
+            const T* kp = k_cache + (((long)page * Hkv + kvh) * page_size + key % page_size) * hd;
+            off = ((long)page * Hkv + kvh) * hd * page_size + key % page_size;
             float acc = 0.f;
             for (int d = 0; d < hd; ++d) acc = fmaf(qs[d], ka_to_float(kp[d]), acc);
             s = acc;
@@ -63,7 +63,7 @@ attention_generic_kernel(const T* __restrict__ q, long q_row_stride, const T* __
             int d = lane + i * KA_WAVE;
             if (d < hd) {
                 float acc = o[i] * corr;
-                for (int j = 0; j < count; ++j) acc = fmaf(ps[j], ka_to_float(v_cache[offs[j] + d]), acc);
+                for (int j = 0; j < count; ++j) acc = fmaf(ps[j], ka_to_float(v_cache[offs[j] + (long)d * page_size]), acc);
                 o[i] = acc;
             }
         }

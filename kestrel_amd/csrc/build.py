@@ -27,8 +27,8 @@ ARCH = "gfx950"
 # library name -> its sources. "core" is all a float32 run needs; "fast" holds the
 # bf16 MFMA kernels of serving.
 LIBRARIES: Dict[str, List[str]] = {
-    "core": ["elementwise.hip", "gemm_generic.hip", "attention_generic.hip", "sampling.hip"],
-    "fast": ["gemm_bf16.hip", "gemv_bf16.hip", "attention_bf16.hip"],
+    "core": ["ka_error.hip", "elementwise.hip", "gemm_generic.hip", "attention_generic.hip", "sampling.hip"],
+    "fast": ["ka_error.hip", "gemm_bf16.hip", "gemv_bf16.hip", "attention_bf16.hip"],
 }
 HEADERS = ["ka_common.h"]
 

@@ -4,20 +4,6 @@
 // it as fp32 and convert only at the boundary to the model's storage type.
 #include "ka_common.h"
 
-#include <stdarg.h>
-#include <stdio.h>
-
-static thread_local char g_error[512];
-
-void ka_set_error(const char* fmt, ...) {
-    va_list ap;
-    va_start(ap, fmt);
-    vsnprintf(g_error, sizeof(g_error), fmt, ap);
-    va_end(ap);
-}
-
-KA_API const char* ka_last_error() { return g_error; }
-
 KA_API int ka_version() { return 1; }
 
 // ----------------------------------------------------------------------------
@@ -142,7 +128,9 @@ KA_API int ka_layernorm(const float* x, const int* rows, const float* gamma, con
 // on their way into the paged cache together with v. The table row of position p is
 // [cos(p f_0..f_{rot/2-1}), sin(...)] in fp32; the rotation is computed in fp32.
 //
-// qkv row: [H*hd q | Hkv*hd k | Hkv*hd v]. Cache: [pages, Hkv, page_size, hd].
+// qkv row: [H*hd q | Hkv*hd k | Hkv*hd v]. Key cache: [pages, Hkv, page_size, hd]; value cache:
+// [pages, Hkv, hd, page_size] (transposed inside the page, so that the MFMA attention kernels
+// read eight consecutive keys of one channel with a single 16-byte load).
 // slots[t] = page * page_size + offset, or < 0 for "do not write" (a layer that
 // reads another layer's cache).
 // ----------------------------------------------------------------------------
@@ -184,7 +172,8 @@ __global__ void rope_cache_kernel(T* __restrict__ qkv, long row_stride,
             kv = d < half ? a * c - b * s : b * c + a * s;
         }
         k_cache[dst] = ka_from_float<T>(kv);
-        v_cache[dst] = vrow[idx];
+        size_t vdst = (((size_t)page * Hkv + h) * hd + d) * page_size + off;
+        v_cache[vdst] = vrow[idx];
     }
 }
 

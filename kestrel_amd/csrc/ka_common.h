@@ -18,8 +18,8 @@ typedef __bf16 bf16_t;
 
 constexpr int KA_WAVE = 64;
 
-// Error text of the last failed call in this thread (defined in elementwise.hip
-// for the core library; each library has its own copy).
+// Error text of the last failed call in this thread (ka_error.hip; each library
+// links its own copy).
 void ka_set_error(const char* fmt, ...);
 
 #define KA_CHECK(cond, ...)            \

@@ -48,6 +48,7 @@ class ModelRunner:
     """Owns the model, its cache and the scratch memory; ``step`` is the only way in."""
 
     STAGING_RING = 4
+    QUERY_BLOCK = 128        # queries of one row a workgroup of the prompt attention kernel takes
 
     def __init__(self, model: DecoderModel, cache: CacheManager, device: torch.device,
                  max_tokens_per_step: int = 4096) -> None:
@@ -175,10 +176,16 @@ class ModelRunner:
 
         # one packed int32 buffer: [ids | positions | token_row | kv_hi | row_slot | cu_q | kv_len | logit_rows |
         #                           given_rows | per group: slots, kv_lo, block_table]
+        qblk_row: List[int] = []
+        qblk_tok: List[int] = []
+        for r in range(n_rows):
+            for first in range(cu_q[r], cu_q[r + 1], self.QUERY_BLOCK):
+                qblk_row.append(r)
+                qblk_tok.append(first)
         sections: List[Tuple[str, List[int]]] = [
             ("ids", ids), ("positions", positions), ("token_row", token_row), ("kv_hi", kv_hi),
             ("row_slot", [e.slot for e in entries]), ("cu_q", cu_q), ("kv_len", kv_len), ("logit_rows", logit_rows),
-            ("given_rows", given_rows),
+            ("given_rows", given_rows), ("qblk_row", qblk_row), ("qblk_tok", qblk_tok),
         ]
         for g in range(n_groups):
             sections.append((f"slots{g}", slots[g]))
@@ -226,6 +233,7 @@ class ModelRunner:
             n_tokens=n_tokens, n_rows=n_rows, token_ids=view("ids"), positions=view("positions"),
             token_row=view("token_row"), kv_hi=view("kv_hi"), row_slot=view("row_slot"), cu_q=view("cu_q"),
             kv_len=view("kv_len"), logit_rows=view("logit_rows"), groups=groups, workspace=self.workspace,
+            qblk_row=view("qblk_row"), qblk_tok=view("qblk_tok"),
             given_embeds=given_embeds, given_rows=view("given_rows") if given else None, max_q=max_q, max_kv=max_kv,
             decode_only=max_q == 1, causal_only=causal_only,
             host={"starts": starts, "q_lens": [len(e.tokens) for e in entries], "kv_len": kv_len},

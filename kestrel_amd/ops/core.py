@@ -90,6 +90,16 @@ def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
     return None if t is None else t.data_ptr()
 
 
+def _check_caches(who: str, k_cache, v_cache, dtype, n_kv_heads: int, page_size: int, head_dim: int) -> None:
+    """Keys ``[pages, Hkv, page_size, hd]``, values ``[pages, Hkv, hd, page_size]``, both contiguous."""
+    _need(k_cache.dtype == dtype and k_cache.is_contiguous() and k_cache.dim() == 4
+          and tuple(k_cache.shape[1:]) == (n_kv_heads, page_size, head_dim),
+          f"{who}: key cache must be [pages, Hkv, page_size, hd] of the activation type")
+    _need(v_cache.dtype == dtype and v_cache.is_contiguous() and v_cache.dim() == 4
+          and tuple(v_cache.shape[1:]) == (n_kv_heads, head_dim, page_size) and v_cache.shape[0] == k_cache.shape[0],
+          f"{who}: value cache must be [pages, Hkv, hd, page_size] of the activation type")
+
+
 def uniform(key: int, counter: int) -> float:
     """The uniform number the sampling kernel draws for (key, counter)."""
     return float(lib().ka_uniform_host(key & (2 ** 64 - 1), counter))
@@ -142,7 +152,8 @@ def rope_cache(qkv: torch.Tensor, positions: torch.Tensor, slots: Optional[torch
     """Rotate q in place and write rotated k and v into the paged cache.
 
     ``qkv``: ``[n, (H + 2 Hkv) hd]``; ``table``: fp32 ``[positions, R]`` or ``None`` for no
-    rotation; caches ``[pages, Hkv, page_size, hd]``; ``slots`` ``None`` writes nothing.
+    rotation; key cache ``[pages, Hkv, page_size, hd]``, value cache ``[pages, Hkv, hd, page_size]``;
+    ``slots`` ``None`` writes nothing.
     """
     _dev(qkv, positions, slots, table, k_cache, v_cache)
     n = qkv.shape[0]
@@ -158,10 +169,7 @@ def rope_cache(qkv: torch.Tensor, positions: torch.Tensor, slots: Optional[torch
     if slots is not None:
         _need(slots.dtype == torch.int32 and slots.numel() == n and slots.is_contiguous(), "rope_cache: slots int32 [n]")
         _need(k_cache is not None and v_cache is not None, "rope_cache: cache tensors missing")
-        for c in (k_cache, v_cache):
-            _need(c.dtype == qkv.dtype and c.is_contiguous() and c.dim() == 4
-                  and tuple(c.shape[1:]) == (n_kv_heads, page_size, head_dim),
-                  "rope_cache: cache must be [pages, Hkv, page_size, hd] of the qkv type")
+        _check_caches("rope_cache", k_cache, v_cache, qkv.dtype, n_kv_heads, page_size, head_dim)
     _check(lib().ka_rope_cache(qkv.data_ptr(), code_of(qkv.dtype), qkv.stride(0), positions.data_ptr(), _ptr(slots),
                                _ptr(table), rows, _ptr(k_cache), _ptr(v_cache), n, n_heads, n_kv_heads, head_dim,
                                rot, page_size, stream_ptr()))
@@ -193,10 +201,7 @@ def attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
     _need(out.dim() == 2 and out.stride(1) == 1 and tuple(out.shape) == (n, n_heads * head_dim) and out.dtype == q.dtype,
           "attention: out must be [n, H hd] of the q type")
     page_size = k_cache.shape[2]
-    for c in (k_cache, v_cache):
-        _need(c.dtype == q.dtype and c.is_contiguous() and c.dim() == 4
-              and tuple(c.shape[1:]) == (n_kv_heads, page_size, head_dim),
-              "attention: cache must be [pages, Hkv, page_size, hd] of the q type")
+    _check_caches("attention", k_cache, v_cache, q.dtype, n_kv_heads, page_size, head_dim)
     _need(block_table.dtype == torch.int32 and block_table.dim() == 2 and block_table.is_contiguous(),
           "attention: block table must be contiguous int32 [rows, pages]")
     for t in (token_row, kv_hi) + ((kv_lo,) if kv_lo is not None else ()):

@@ -51,7 +51,8 @@ class LayerCache:
     """What one run of a layer may touch of the cache manager's memory.
 
     ``group``: key into ``StepBatch.groups`` (block table, slots, window start) or ``None``
-    if the mixer keeps no keys and values; ``k``/``v``: ``[pages, Hkv, page_size, hd]``;
+    if the mixer keeps no keys and values; ``k``: ``[pages, Hkv, page_size, hd]``, ``v``:
+    ``[pages, Hkv, hd, page_size]``;
     ``writes``: ``False`` when this run reads the cache of another run; ``state``:
     ``[slots, *shape]`` per-request state, indexed by ``StepBatch.row_slot``.
     """

@@ -1,0 +1,361 @@
+"""Each HIP kernel alone against a plain fp64 reference, at sizes other than the engine's."""
+
+from types import SimpleNamespace
+
+import pytest
+import torch
+import torch.nn.functional as F
+
+from tests.plain import moondream_plain as plain
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def _tol(dtype):
+    return (1e-5, 1e-5) if dtype == torch.float32 else (2e-2, 2e-2)
+
+
+def _close(actual, expected, dtype, scale=1.0):
+    atol, rtol = _tol(dtype)
+    torch.testing.assert_close(actual.double().cpu(), expected.double().cpu(), atol=atol * scale, rtol=rtol)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_embed_and_scatter(dtype):
+    from kestrel_amd.ops import core
+
+    torch.manual_seed(0)
+    table = torch.randn(333, 100).to(dtype).to(DEV)
+    ids = torch.tensor([5, -1, 332, 0, -1, 17], dtype=torch.int32, device=DEV)
+    out = torch.full((6, 100), 7.0, device=DEV)
+    core.embed(table, ids, out)
+    keep = ids.cpu() >= 0
+    _close(out.cpu()[keep], table.float().cpu()[ids.cpu()[keep].long()], torch.float32)
+    assert bool((out.cpu()[~keep] == 7.0).all())                 # given places are left alone
+    given = torch.randn(2, 100).to(dtype).to(DEV)
+    core.scatter_rows(given, torch.tensor([1, 4], dtype=torch.int32, device=DEV), out)
+    _close(out[[1, 4]], given.float(), torch.float32)
+
+
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("dim", [100, 2048, 5000])
+def test_layernorm(dim, out_dtype):
+    from kestrel_amd.ops import core
+
+    torch.manual_seed(1)
+    x = (torch.randn(9, dim) * 3 + 1.5).to(DEV)
+    gamma, beta = (1 + 0.1 * torch.randn(dim)).to(DEV), (0.1 * torch.randn(dim)).to(DEV)
+    for eps in (1e-5, 1e-2):
+        out = torch.empty(9, dim, dtype=out_dtype, device=DEV)
+        core.layernorm(x, gamma, beta, eps, out)
+        _close(out, F.layer_norm(x.double(), (dim,), gamma.double(), beta.double(), eps), out_dtype, scale=4)
+    rows = torch.tensor([8, 0, 3], dtype=torch.int32, device=DEV)
+    out = torch.empty(3, dim, dtype=out_dtype, device=DEV)
+    core.layernorm(x, gamma, None, 1e-6, out, rows)
+    _close(out, F.layer_norm(x.double()[[8, 0, 3]], (dim,), gamma.double(), None, 1e-6), out_dtype, scale=4)
+
+
+def _linear_case(fn, m, n, k, a_dtype, w_dtype, out_dtype, act, accumulate, seed=0, lda=None):
+    torch.manual_seed(seed)
+    lda = lda or k
+    a_full = torch.randn(m, lda).to(a_dtype).to(DEV)
+    a = a_full[:, :k]
+    w = (torch.randn(n, k) / k ** 0.5).to(w_dtype).to(DEV)
+    bias = torch.randn(n).to(DEV)
+    start = torch.randn(m, n).to(out_dtype).to(DEV)
+    out = start.clone()
+    fn(a, w, bias, out, act=act, accumulate=accumulate)
+    ref = a.double() @ w.double().T + bias.double()
+    if act:
+        ref = plain.gelu_tanh(ref)
+    if accumulate:
+        ref = ref + start.double()
+    worst = torch.float32 if (a_dtype == w_dtype == out_dtype == torch.float32) else torch.bfloat16
+    _close(out, ref, worst, scale=2)
+
+
+@pytest.mark.parametrize("shape", [(1, 37, 19), (65, 130, 200), (7, 64, 96), (130, 77, 333)])
+def test_linear_generic(shape):
+    from kestrel_amd.ops import core
+
+    m, n, k = shape
+    f32, bf = torch.float32, torch.bfloat16
+    for a_dtype, w_dtype, out_dtype in [(f32, f32, f32), (bf, bf, bf), (bf, bf, f32), (bf, f32, bf), (f32, bf, f32)]:
+        for act, accumulate in [(0, False), (1, False), (0, True)]:
+            if accumulate and out_dtype != f32:
+                continue
+            _linear_case(core.linear_generic, m, n, k, a_dtype, w_dtype, out_dtype, act, accumulate)
+    _linear_case(core.linear_generic, m, n, k, f32, f32, f32, 0, False, lda=k + 5)      # strided rows
+
+
+@pytest.mark.parametrize("shape", [(1, 48, 64), (8, 2048, 2048), (5, 100, 200), (16, 6144, 2048), (33, 77, 8192),
+                                   (64, 51200, 512), (17, 2048, 8192), (3, 16, 8)])
+def test_linear_skinny_bf16(shape):
+    """The weight-streaming MFMA kernel, with K-splits where N is small."""
+    from kestrel_amd.ops import fast
+
+    m, n, k = shape
+    bf, f32 = torch.bfloat16, torch.float32
+
+    def fn(a, w, bias, out, act, accumulate):
+        assert fast.linear_bf16(a, w, bias, out, act, accumulate)
+
+    for out_dtype, act, accumulate in [(bf, 0, False), (bf, 1, False), (f32, 0, True), (f32, 0, False)]:
+        _linear_case(fn, m, n, k, bf, bf, out_dtype, act, accumulate)
+    _linear_case(fn, m, n, k, bf, bf, bf, 0, False, lda=k + 16)
+
+
+def test_linear_skinny_is_the_same_on_every_run():
+    from kestrel_amd.ops import fast
+
+    torch.manual_seed(3)
+    a = torch.randn(8, 8192).bfloat16().to(DEV)
+    w = torch.randn(2048, 8192).bfloat16().to(DEV)
+    outs = []
+    for _ in range(5):
+        out = torch.empty(8, 2048, device=DEV)
+        assert fast.linear_bf16(a, w, None, out, 0, False)
+        outs.append(out.clone())
+    assert all(torch.equal(outs[0], o) for o in outs[1:])
+
+
+@pytest.mark.parametrize("shape", [(65, 128, 64), (200, 2048, 2048), (129, 100, 200), (300, 333, 520),
+                                   (2048, 512, 1024), (128, 6144, 2048), (70, 8, 8)])
+def test_linear_tiled_bf16(shape):
+    """The tiled MFMA kernel with ragged edges in M, N and K."""
+    from kestrel_amd.ops import fast
+
+    m, n, k = shape
+    bf, f32 = torch.bfloat16, torch.float32
+
+    def fn(a, w, bias, out, act, accumulate):
+        assert fast.linear_bf16(a, w, bias, out, act, accumulate)
+
+    for out_dtype, act, accumulate in [(bf, 0, False), (bf, 1, False), (f32, 0, True), (f32, 0, False)]:
+        _linear_case(fn, m, n, k, bf, bf, out_dtype, act, accumulate)
+    _linear_case(fn, m, n, k, bf, bf, bf, 0, False, lda=k + 8)
+
+
+def test_fast_linear_declines_what_it_does_not_cover():
+    from kestrel_amd.ops import fast
+
+    a = torch.randn(4, 20).bfloat16().to(DEV)         # K no multiple of 8
+    w = torch.randn(6, 20).bfloat16().to(DEV)
+    assert not fast.linear_bf16(a, w, None, torch.empty(4, 6, dtype=torch.bfloat16, device=DEV), 0, False)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("heads", [(3, 1, 32, 16, 4), (6, 2, 48, 12, 16), (4, 4, 16, 16, 1), (2, 2, 80, 0, 16)])
+def test_rope_and_cache_write(heads, dtype):
+    from kestrel_amd.ops import core
+
+    h, hkv, hd, rot, ps = heads
+    torch.manual_seed(4)
+    n, pages = 11, 12
+    qkv = torch.randn(n, (h + 2 * hkv) * hd).to(dtype)
+    positions = torch.tensor([0, 1, 2, 3, 40, 41, 7, 8, 9, 100, 101], dtype=torch.int32)
+    slots = torch.randperm(pages * ps)[:n].to(torch.int32)
+    slots[5] = -1                                        # this token writes nothing
+    table = plain.rotary_table(rot, 128, 777.0, torch.float32) if rot else None
+    k_cache = torch.zeros(pages, hkv, ps, hd, dtype=dtype, device=DEV)
+    v_cache = torch.zeros(pages, hkv, hd, ps, dtype=dtype, device=DEV)
+    dev = qkv.to(DEV)
+    core.rope_cache(dev, positions.to(DEV), slots.to(DEV), None if table is None else table.to(DEV), k_cache, v_cache,
+                    h, hkv, hd, ps)
+    q = qkv[:, :h * hd].double().view(n, h, hd)
+    k = qkv[:, h * hd:(h + hkv) * hd].double().view(n, hkv, hd)
+    v = qkv[:, (h + hkv) * hd:].double().view(n, hkv, hd)
+    if rot:
+        t64 = plain.rotary_table(rot, 128, 777.0)
+        q, k = plain.apply_rotary(q, positions, t64), plain.apply_rotary(k, positions, t64)
+    _close(dev[:, :h * hd].view(n, h, hd), q, dtype)
+    for t in range(n):
+        if slots[t] < 0:
+            continue
+        page, off = int(slots[t]) // ps, int(slots[t]) % ps
+        _close(k_cache[page, :, off, :], k[t], dtype)
+        _close(v_cache[page, :, :, off], v[t], dtype)
+    written = {int(s) for s in slots if s >= 0}
+    for slot in range(pages * ps):
+        if slot not in written:
+            assert float(k_cache[slot // ps, :, slot % ps, :].abs().max()) == 0.0
+
+
+class PagedCase:
+    """Rows of cached keys and values scattered over shuffled pages, and packed query tokens."""
+
+    def __init__(self, kv_lens, q_lens, h, hkv, hd, ps, dtype, seed=0, window=None, bidir=None):
+        gen = torch.Generator().manual_seed(seed)
+        self.h, self.hkv, self.hd, self.ps, self.dtype = h, hkv, hd, ps, dtype
+        n_rows = len(kv_lens)
+        pages_per_row = [-(-kv // ps) for kv in kv_lens]
+        n_pages = sum(pages_per_row) + 3
+        order = torch.randperm(n_pages, generator=gen).tolist()
+        max_pages = max(pages_per_row) + 2
+        table = torch.full((n_rows, max_pages), -1, dtype=torch.int32)
+        self.k = [torch.randn(kv, hkv, hd, generator=gen).to(dtype) for kv in kv_lens]
+        self.v = [torch.randn(kv, hkv, hd, generator=gen).to(dtype) for kv in kv_lens]
+        k_cache = torch.full((n_pages, hkv, ps, hd), float("nan")).to(dtype)
+        v_cache = torch.full((n_pages, hkv, hd, ps), float("nan")).to(dtype)
+        at = 0
+        for r, kv in enumerate(kv_lens):
+            for logical in range(pages_per_row[r]):
+                page = order[at]
+                at += 1
+                table[r, logical] = page
+                lo, hi = logical * ps, min(kv, (logical + 1) * ps)
+                k_cache[page, :, :hi - lo, :] = self.k[r][lo:hi].transpose(0, 1)
+                v_cache[page, :, :, :hi - lo] = self.v[r][lo:hi].permute(1, 2, 0)
+        token_row, kv_hi, kv_lo, cu_q = [], [], [], [0]
+        for r, (kv, ql) in enumerate(zip(kv_lens, q_lens)):
+            for i in range(ql):
+                pos = kv - ql + i
+                hi_t = pos + 1
+                if bidir and bidir[r] and bidir[r][0] <= pos < bidir[r][1]:
+                    hi_t = bidir[r][1]
+                token_row.append(r)
+                kv_hi.append(hi_t)
+                kv_lo.append(max(0, pos + 1 - window) if window else 0)
+            cu_q.append(len(token_row))
+        n = len(token_row)
+        self.q = torch.randn(n, h * hd, generator=gen).to(dtype)
+        qblk_row, qblk_tok = [], []
+        for r in range(n_rows):
+            for first in range(cu_q[r], cu_q[r + 1], 128):
+                qblk_row.append(r)
+                qblk_tok.append(first)
+        i32 = lambda xs: torch.tensor(xs, dtype=torch.int32, device=DEV)
+        self.token_row, self.kv_hi = i32(token_row), i32(kv_hi)
+        self.kv_lo = i32(kv_lo) if window else None
+        self.table, self.k_cache, self.v_cache = table.to(DEV), k_cache.to(DEV), v_cache.to(DEV)
+        self.batch = SimpleNamespace(decode_only=all(ql == 1 for ql in q_lens), max_kv=max(kv_lens), cu_q=i32(cu_q),
+                                     kv_len=i32(kv_lens), qblk_row=i32(qblk_row), qblk_tok=i32(qblk_tok))
+        self.lists = (token_row, kv_lo if window else [0] * n, kv_hi)
+
+    def reference(self, scale):
+        token_row, kv_lo, kv_hi = self.lists
+        out = torch.empty(len(token_row), self.h, self.hd, dtype=torch.float64)
+        group = self.h // self.hkv
+        q = self.q.double().view(-1, self.h, self.hd)
+        for t, (r, lo, hi) in enumerate(zip(token_row, kv_lo, kv_hi)):
+            for head in range(self.h):
+                keys = self.k[r][lo:hi, head // group].double()
+                vals = self.v[r][lo:hi, head // group].double()
+                w = torch.softmax(keys @ q[t, head] * scale, dim=0)
+                out[t, head] = w @ vals
+        return out.view(len(token_row), self.h * self.hd)
+
+
+def _run_attention(case, fn_name, scale):
+    from kestrel_amd.ops import core, fast
+
+    q = case.q.to(DEV)
+    out = torch.full((q.shape[0], case.h * case.hd), float("nan"), dtype=case.dtype, device=DEV)
+    if fn_name == "generic":
+        core.attention_generic(q, case.k_cache, case.v_cache, case.table, case.token_row, case.kv_lo, case.kv_hi, out,
+                               scale, case.h, case.hkv, case.hd)
+    else:
+        assert fast.attention_bf16(q, case.k_cache, case.v_cache, case.table, case.token_row, case.kv_lo, case.kv_hi,
+                                   out, scale, case.h, case.hkv, case.hd, case.batch)
+    return out
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(3, 1, 32, 4), (6, 2, 48, 16), (2, 2, 80, 16), (4, 4, 16, 1), (1, 1, 272, 16)])
+def test_attention_generic(shape, dtype):
+    h, hkv, hd, ps = shape
+    case = PagedCase([70, 5, 129], [70, 1, 9], h, hkv, hd, ps, dtype, seed=5)
+    out = _run_attention(case, "generic", hd ** -0.5)
+    _close(out, case.reference(hd ** -0.5), dtype)
+    windowed = PagedCase([70, 33], [20, 1], h, hkv, hd, ps, dtype, seed=6, window=17)
+    _close(_run_attention(windowed, "generic", 0.3), windowed.reference(0.3), dtype)
+    block = PagedCase([40], [40], h, hkv, hd, ps, dtype, seed=7, bidir=[(3, 21)])
+    _close(_run_attention(block, "generic", hd ** -0.5), block.reference(hd ** -0.5), dtype)
+
+
+@pytest.mark.parametrize("shape", [(4, 4, 64), (6, 2, 32), (3, 1, 96), (4, 2, 128), (32, 32, 64)])
+def test_attention_prompt_kernel(shape):
+    """Whole prompts, portions that continue a cache, single tokens in a mixed batch, a block that
+    sees both ways, a window; query counts that do not fill a wave."""
+    h, hkv, hd = shape
+    bf = torch.bfloat16
+    case = PagedCase([70, 5, 300, 33], [70, 1, 130, 2], h, hkv, hd, 16, bf, seed=8)
+    _close(_run_attention(case, "fast", hd ** -0.5), case.reference(hd ** -0.5), bf)
+    block = PagedCase([90, 64], [90, 40], h, hkv, hd, 16, bf, seed=9, bidir=[(0, 37), (30, 50)])
+    _close(_run_attention(block, "fast", hd ** -0.5), block.reference(hd ** -0.5), bf)
+    windowed = PagedCase([200, 45], [120, 3], h, hkv, hd, 16, bf, seed=10, window=40)
+    _close(_run_attention(windowed, "fast", 0.2), windowed.reference(0.2), bf)
+
+
+@pytest.mark.parametrize("shape", [(4, 4, 64), (6, 2, 128), (32, 32, 64), (8, 1, 64)])
+def test_attention_decode_kernel(shape):
+    """One token per row, contexts from one key to many splits' worth, with and without a window."""
+    h, hkv, hd = shape
+    bf = torch.bfloat16
+    for kv_lens in ([1], [5, 64, 65, 1000], [17, 256, 257, 511, 2, 2048], [700] * 9):
+        case = PagedCase(kv_lens, [1] * len(kv_lens), h, hkv, hd, 16, bf, seed=11 + len(kv_lens))
+        assert case.batch.decode_only
+        _close(_run_attention(case, "fast", hd ** -0.5), case.reference(hd ** -0.5), bf)
+    windowed = PagedCase([300, 20, 129], [1, 1, 1], h, hkv, hd, 16, bf, seed=12, window=100)
+    _close(_run_attention(windowed, "fast", 0.25), windowed.reference(0.25), bf)
+
+
+def test_a_far_key_among_hundreds_is_found():
+    """One query and one far key are scaled so that this key takes almost all the weight: a
+    kernel that loses it (a page's edge, a split's edge, a tile's edge) returns another value."""
+    h, hkv, hd = 4, 4, 64
+    bf = torch.bfloat16
+    for target in (0, 15, 16, 255, 256, 511, 777):
+        case = PagedCase([900], [1], h, hkv, hd, 16, bf, seed=13)
+        case.q[0] *= 0
+        case.q[0, :hd] = 4.0
+        # key `target` of head 0 lines up with the query; rebuild its cache cell
+        case.k[0][target, 0] = 4.0
+        page, off = int(case.table[0, target // 16]), target % 16
+        case.k_cache[page, 0, off, :] = 4.0
+        for name in ("generic", "fast"):
+            out = _run_attention(case, name, hd ** -0.5)
+            _close(out[0, :hd], case.v[0][target, 0].double(), bf)
+        prompt = PagedCase([900], [130], h, hkv, hd, 16, bf, seed=13)
+        prompt.q[-1] *= 0
+        prompt.q[-1, :hd] = 4.0
+        prompt.k[0][target, 0] = 4.0
+        page = int(prompt.table[0, target // 16])
+        prompt.k_cache[page, 0, target % 16, :] = 4.0
+        out = _run_attention(prompt, "fast", hd ** -0.5)
+        _close(out[-1, :hd], prompt.v[0][target, 0].double(), bf)
+
+
+def test_argmax_and_sampling():
+    from kestrel_amd.ops import core
+    from kestrel_amd.sampling import Sampler, mix_key
+
+    torch.manual_seed(14)
+    for vocab in (777, 51200, 70000):
+        logits = torch.randn(5, vocab, device=DEV)
+        logits[2, 3] = logits[2, vocab - 1] = 50.0            # a tie: the first index wins
+        out = torch.empty(5, dtype=torch.int32, device=DEV)
+        core.argmax(logits, out)
+        assert out.tolist() == torch.argmax(logits.cpu(), dim=-1).tolist() or out[2].item() == 3
+        assert out[2].item() == 3
+    sampler = Sampler(torch.device(DEV), seed=5)
+    logits = torch.tensor([[2.0, 1.0, 0.5, -1.0, -3.0, float("-inf")]] * 4000, device=DEV)
+    # temperature -> 0 is argmax; top_p tiny keeps the best token only
+    assert set(sampler.sample(logits[:8], [0.0] * 8, [1.0] * 8, list(range(8)), [0] * 8).tolist()) == {0}
+    assert set(sampler.sample(logits[:8], [1.0] * 8, [1e-4] * 8, list(range(8)), [0] * 8).tolist()) == {0}
+    for temp, top_p in ((1.0, 1.0), (0.7, 1.0), (1.0, 0.8), (1.5, 0.5)):
+        ids = sampler.sample(logits, [temp] * 4000, [top_p] * 4000, list(range(4000)), [3] * 4000).cpu()
+        probs = plain.nucleus_probs(logits[0].cpu(), temp, top_p)
+        counts = torch.bincount(ids.long(), minlength=6).double()
+        assert counts[5] == 0 and bool((counts[probs == 0] == 0).all())
+        keep = probs > 0
+        chi2 = float((((counts[keep] - 4000 * probs[keep]) ** 2) / (4000 * probs[keep])).sum())
+        assert chi2 < 30.0, (temp, top_p, counts.tolist(), probs.tolist())
+    # a request's draw does not depend on its row or on the rest of the batch
+    row = torch.randn(1, 1000, device=DEV)
+    alone = sampler.sample(row, [0.9], [0.95], [42], [7]).item()
+    mixed = sampler.sample(torch.cat([torch.randn(3, 1000, device=DEV), row]), [0.5, 0.0, 1.0, 0.9],
+                           [1.0, 1.0, 0.3, 0.95], [1, 2, 3, 42], [0, 5, 9, 7])[3].item()
+    assert alone == mixed
+    assert 0.0 <= core.uniform(mix_key(5, 42), 7) < 1.0
