@@ -90,7 +90,8 @@ class DecodeBench:
         self.torch, self.StepEntry = torch, StepEntry
         self.net, self.typed, self.batch, self.context = net, typed, batch, context
         pages_per_request = -(-(context + steps_total + 1) // PAGE_SIZE)
-        self.runner = make_runner(net, PAGE_SIZE, batch * pages_per_request, batch, max_tokens_per_step=4096)
+        self.runner = make_runner(net, PAGE_SIZE, batch * pages_per_request, batch, max_tokens_per_step=4096,
+                                  enable_graphs=True)
         self.sampler = Sampler(net.device)
         gen = torch.Generator().manual_seed(SEED)
         prefix = min(typed.prefix_attn, context - 1)

@@ -171,11 +171,10 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_
 // ----------------------------------------------------------------------------------------------
 // decode kernel
 // ----------------------------------------------------------------------------------------------
-constexpr int AD_WAVES = 4;
 constexpr int AD_TILE = 64;               // keys per wave tile
 
-template <int HD>
-__global__ void __launch_bounds__(KA_WAVE * AD_WAVES)
+template <int HD, int WAVES>
+__global__ void __launch_bounds__(KA_WAVE * WAVES)
 attn_decode_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t* __restrict__ k_cache,
                    const bf16_t* __restrict__ v_cache, const int* __restrict__ block_table, int max_pages,
                    const int* __restrict__ token_row, const int* __restrict__ kv_lo,
@@ -185,8 +184,8 @@ attn_decode_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t
     constexpr int KPI = KA_WAVE / LPK;     // keys per load instruction
     constexpr int VU = HD * 2 / KA_WAVE;   // 16-byte value loads per lane and page
     constexpr int REC = HD + 2;            // floats of a partial result: m, l, o[HD]
-    __shared__ float ps[AD_WAVES][AD_TILE];
-    __shared__ float merge[AD_WAVES][REC];
+    __shared__ float ps[WAVES][AD_TILE];
+    __shared__ float merge[WAVES][REC];
     const int t = blockIdx.x, h = blockIdx.y, split = blockIdx.z, S = gridDim.z;
     const int wave = threadIdx.x / KA_WAVE, lane = threadIdx.x % KA_WAVE;
     const int kvh = h / (H / Hkv);
@@ -209,7 +208,7 @@ attn_decode_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t
 #pragma unroll
     for (int u = 0; u < VU; ++u) acc[u] = 0.f;
 
-    for (int tile0 = s_lo + wave * AD_TILE; tile0 < s_hi; tile0 += AD_WAVES * AD_TILE) {
+    for (int tile0 = s_lo + wave * AD_TILE; tile0 < s_hi; tile0 += WAVES * AD_TILE) {
         float sc[LPK];
         float mx = -INFINITY;
 #pragma unroll
@@ -287,13 +286,13 @@ attn_decode_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t
     // wave 0: lane d (and d + 64 for hd 128) merges the waves in wave order
     float M = -INFINITY;
 #pragma unroll
-    for (int w = 0; w < AD_WAVES; ++w) M = fmaxf(M, merge[w][0]);
+    for (int w = 0; w < WAVES; ++w) M = fmaxf(M, merge[w][0]);
     float L = 0.f;
     float od[(HD + KA_WAVE - 1) / KA_WAVE];
 #pragma unroll
     for (int e = 0; e < (HD + KA_WAVE - 1) / KA_WAVE; ++e) od[e] = 0.f;
 #pragma unroll
-    for (int w = 0; w < AD_WAVES; ++w) {
+    for (int w = 0; w < WAVES; ++w) {
         float mw = merge[w][0];
         float f = mw == -INFINITY ? 0.f : exp2f(mw - M);
         L += merge[w][1] * f;
@@ -399,7 +398,7 @@ KA_API long ka_attention_decode_partial_floats(int n, int H, int hd, int splits)
 KA_API int ka_attention_decode_bf16(const void* q, long q_row_stride, const void* k_cache, const void* v_cache,
                                     const int* block_table, int max_pages, const int* token_row, const int* kv_lo,
                                     const int* kv_hi, void* out, long out_row_stride, float scale, int n, int H,
-                                    int Hkv, int hd, int page_size, int splits, float* partial,
+                                    int Hkv, int hd, int page_size, int splits, int waves, float* partial,
                                     long partial_floats, unsigned* counters, int n_counters, hipStream_t stream) {
     if (check_common("ka_attention_decode_bf16", q, q_row_stride, out, out_row_stride, n, H, Hkv, hd, page_size,
                      max_pages))
@@ -412,15 +411,18 @@ KA_API int ka_attention_decode_bf16(const void* q, long q_row_stride, const void
                  "ka_attention_decode_bf16: scratch too small");
         KA_CHECK((long)n * H <= n_counters, "ka_attention_decode_bf16: too few counters");
     }
-    dim3 grid(n, H, splits), block(KA_WAVE * AD_WAVES);
-    if (hd == 64)
-        hipLaunchKernelGGL(attn_decode_kernel<64>, grid, block, 0, stream, (const bf16_t*)q, q_row_stride,
-                           (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, max_pages, token_row, kv_lo,
-                           kv_hi, (bf16_t*)out, out_row_stride, scale, H, Hkv, partial, counters);
-    else
-        hipLaunchKernelGGL(attn_decode_kernel<128>, grid, block, 0, stream, (const bf16_t*)q, q_row_stride,
-                           (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, max_pages, token_row, kv_lo,
-                           kv_hi, (bf16_t*)out, out_row_stride, scale, H, Hkv, partial, counters);
+    KA_CHECK(waves == 4 || waves == 8 || waves == 16, "ka_attention_decode_bf16: waves must be 4, 8 or 16");
+    dim3 grid(n, H, splits), block(KA_WAVE * waves);
+#define KA_AD(HDV, WV)                                                                                              \
+    hipLaunchKernelGGL((attn_decode_kernel<HDV, WV>), grid, block, 0, stream, (const bf16_t*)q, q_row_stride,      \
+                       (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, max_pages, token_row, kv_lo,   \
+                       kv_hi, (bf16_t*)out, out_row_stride, scale, H, Hkv, partial, counters)
+    if (hd == 64) {
+        if (waves == 4) KA_AD(64, 4); else if (waves == 8) KA_AD(64, 8); else KA_AD(64, 16);
+    } else {
+        if (waves == 4) KA_AD(128, 4); else if (waves == 8) KA_AD(128, 8); else KA_AD(128, 16);
+    }
+#undef KA_AD
     KA_LAUNCH_CHECK();
     return 0;
 }

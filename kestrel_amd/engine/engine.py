@@ -127,7 +127,7 @@ class InferenceEngine:
         else:
             n_pages = cfg.max_batch_size * -(-max_seq // cfg.page_size)
         self.runner = make_runner(net, cfg.page_size, n_pages, cfg.max_batch_size,
-                                  max_tokens_per_step=cfg.max_num_batched_tokens)
+                                  max_tokens_per_step=cfg.max_num_batched_tokens, enable_graphs=cfg.enable_graphs)
         self.scheduler = GenerationScheduler(self.runner, Sampler(device, cfg.seed), cfg.max_batch_size,
                                              cfg.max_num_batched_tokens, net.plan.eos_token_ids, max_seq)
 

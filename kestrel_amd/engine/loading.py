@@ -33,6 +33,6 @@ def load_model(model_dir, dtype: torch.dtype, device: torch.device, model: Optio
 
 
 def make_runner(net: DecoderModel, page_size: int, n_pages: int, max_requests: int,
-                max_tokens_per_step: int = 4096) -> ModelRunner:
+                max_tokens_per_step: int = 4096, enable_graphs: bool = False) -> ModelRunner:
     cache = CacheManager(net.cache_needs(), page_size, n_pages, max_requests, dtype=net.dtype, device=net.device)
-    return ModelRunner(net, cache, net.device, max_tokens_per_step)
+    return ModelRunner(net, cache, net.device, max_tokens_per_step, enable_graphs=enable_graphs)

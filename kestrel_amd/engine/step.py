@@ -7,11 +7,15 @@ logits at the places asked for. The reference runs either padded whole prompts
 (``kestrel/models/moondream/runtime.py:1999-2157``) or one token per row
 (``runtime.py:2479-2586``); its metadata (slot mapping ``kv_cache.py:524-551``, per-row
 block table and key counts ``runtime.py:2283-2290``) is what is built here per token.
+
+Steps that hold one token per request are replayed as HIP graphs, one graph per batch
+size bucket (1, 2, 4, ... as in ``kestrel/runtime/decode_graph.py:20-25``): the metadata
+lives at fixed addresses, rows that pad the bucket see no keys and write nothing.
 """
 
 from __future__ import annotations
 
-from dataclasses import dataclass, field
+from dataclasses import dataclass
 from typing import Dict, List, Optional, Sequence, Tuple
 
 import torch
@@ -44,6 +48,27 @@ def _align(n: int) -> int:
     return (n + 3) & ~3
 
 
+def graph_buckets(max_batch: int) -> List[int]:
+    """Batch sizes graphs are captured for: powers of two up to ``max_batch``, and ``max_batch``
+    (``kestrel/runtime/decode_graph.py:20-25``; e.g. 33 -> 1, 2, 4, 8, 16, 32, 33)."""
+    sizes, size = [], 1
+    while size < max_batch:
+        sizes.append(size)
+        size *= 2
+    sizes.append(max_batch)
+    return sizes
+
+
+class _GraphState:
+    """A captured decode step of one bucket size: its metadata, scratch and graph."""
+
+    def __init__(self, device: torch.device) -> None:
+        self.workspace = Workspace(device)
+        self.meta: Optional[torch.Tensor] = None
+        self.graph: Optional[torch.cuda.CUDAGraph] = None
+        self.logits: Optional[torch.Tensor] = None
+
+
 class ModelRunner:
     """Owns the model, its cache and the scratch memory; ``step`` is the only way in."""
 
@@ -51,7 +76,8 @@ class ModelRunner:
     QUERY_BLOCK = 128        # queries of one row a workgroup of the prompt attention kernel takes
 
     def __init__(self, model: DecoderModel, cache: CacheManager, device: torch.device,
-                 max_tokens_per_step: int = 4096) -> None:
+                 max_tokens_per_step: int = 4096, enable_graphs: bool = False,
+                 max_graph_batch: Optional[int] = None) -> None:
         self.model, self.cache, self.device = model, cache, device
         self.max_tokens_per_step = max_tokens_per_step
         self.workspace = Workspace(device)
@@ -61,6 +87,11 @@ class ModelRunner:
         self._staging_events: List[Optional[torch.cuda.Event]] = [None] * self.STAGING_RING
         self._staging_next = 0
         self._meta_device: Optional[torch.Tensor] = None
+        self.enable_graphs = enable_graphs
+        self._buckets = graph_buckets(min(max_graph_batch or cache.max_requests, cache.max_requests))
+        self._graphs: Dict[int, _GraphState] = {}
+        self._pages_cap = -(-model.plan.max_positions // cache.page_size)
+        self.graph_replays = 0
 
     # ------------------------------------------------------------------ requests
     def admit(self, reserve_length: int = 0, portion: int = 1) -> int:
@@ -85,10 +116,8 @@ class ModelRunner:
             self._staging[index] = buf
         return buf, index
 
-    def build_batch(self, entries: Sequence[StepEntry]) -> StepBatch:
-        """Checks the entries, backs their positions with pages and lays the metadata out."""
-        cache, plan = self.cache, self.model.plan
-        ps = cache.page_size
+    def _check_entries(self, entries: Sequence[StepEntry]) -> List[int]:
+        plan = self.model.plan
         if not entries:
             raise ValueError("a step needs at least one entry")
         seen = set()
@@ -111,10 +140,23 @@ class ModelRunner:
             n_tokens += len(e.tokens)
         if n_tokens > self.max_tokens_per_step:
             raise ValueError(f"{n_tokens} tokens in one step exceed the limit of {self.max_tokens_per_step}")
+        return starts
+
+    def build_batch(self, entries: Sequence[StepEntry], pad_rows: int = 0, fixed_pages: int = 0,
+                    meta: Optional[torch.Tensor] = None, workspace: Optional[Workspace] = None) -> StepBatch:
+        """Checks the entries, backs their positions with pages and lays the metadata out.
+
+        ``pad_rows`` > number of entries adds rows of one token that see no keys and write
+        nothing; ``fixed_pages`` fixes the width of the block tables; ``meta`` is the device
+        buffer the metadata is copied into. With all three the layout depends on ``pad_rows``
+        alone, which is what a captured graph needs.
+        """
+        cache, plan = self.cache, self.model.plan
+        ps = cache.page_size
+        starts = self._check_entries(entries)
         for e, start in zip(entries, starts):
             cache.ensure(e.slot, start + len(e.tokens))
 
-        n_rows = len(entries)
         n_groups = len(cache.groups)
         ids: List[int] = []
         positions: List[int] = []
@@ -123,11 +165,12 @@ class ModelRunner:
         logit_rows: List[int] = []
         given_rows: List[int] = []
         given: List[torch.Tensor] = []
+        row_slot: List[int] = []
         cu_q = [0]
         kv_len: List[int] = []
         slots: List[List[int]] = [[] for _ in range(n_groups)]
         kv_lo: List[Optional[List[int]]] = [[] if g.spec.window is not None else None for g in cache.groups]
-        max_pages = 1
+        max_pages = max(1, fixed_pages)
         max_q = max_kv = 1
         causal_only = True
         for r, (e, start) in enumerate(zip(entries, starts)):
@@ -166,25 +209,43 @@ class ModelRunner:
                 logit_rows.append(base + int(w))
             cu_q.append(base + q)
             kv_len.append(start + q)
+            row_slot.append(e.slot)
             max_q, max_kv = max(max_q, q), max(max_kv, start + q)
             for g in range(n_groups):
                 table = cache.block_table(g, e.slot)
+                if fixed_pages and len(table) > fixed_pages:
+                    raise ValueError(f"slot {e.slot}: {len(table)} pages exceed the fixed table width {fixed_pages}")
                 max_pages = max(max_pages, len(table))
                 slots[g].extend(table[p // ps] * ps + p % ps for p in range(start, start + q))
                 if kv_lo[g] is not None:
                     kv_lo[g].extend(cache.window_start(g, p) for p in range(start, start + q))
+        n_real = len(entries)
+        for r in range(n_real, pad_rows):          # rows that only fill the bucket
+            ids.append(0)
+            positions.append(0)
+            token_row.append(r)
+            kv_hi.append(0)
+            logit_rows.append(len(ids) - 1)
+            cu_q.append(len(ids))
+            kv_len.append(0)
+            row_slot.append(-1)                    # no request: a mixer with state must pass these rows over
+            for g in range(n_groups):
+                slots[g].append(-1)
+                if kv_lo[g] is not None:
+                    kv_lo[g].append(0)
+        n_rows = max(n_real, pad_rows)
+        n_tokens = len(ids)
 
-        # one packed int32 buffer: [ids | positions | token_row | kv_hi | row_slot | cu_q | kv_len | logit_rows |
-        #                           given_rows | per group: slots, kv_lo, block_table]
         qblk_row: List[int] = []
         qblk_tok: List[int] = []
         for r in range(n_rows):
             for first in range(cu_q[r], cu_q[r + 1], self.QUERY_BLOCK):
                 qblk_row.append(r)
                 qblk_tok.append(first)
+        # one packed int32 buffer, every section starting on a 16-byte boundary
         sections: List[Tuple[str, List[int]]] = [
             ("ids", ids), ("positions", positions), ("token_row", token_row), ("kv_hi", kv_hi),
-            ("row_slot", [e.slot for e in entries]), ("cu_q", cu_q), ("kv_len", kv_len), ("logit_rows", logit_rows),
+            ("row_slot", row_slot), ("cu_q", cu_q), ("kv_len", kv_len), ("logit_rows", logit_rows),
             ("given_rows", given_rows), ("qblk_row", qblk_row), ("qblk_tok", qblk_tok),
         ]
         for g in range(n_groups):
@@ -196,6 +257,7 @@ class ModelRunner:
                 table = cache.block_table(g, e.slot)
                 flat.extend(table)
                 flat.extend([-1] * (max_pages - len(table)))
+            flat.extend([0] * (max_pages * (n_rows - n_real)))
             sections.append((f"table{g}", flat))
         offsets: Dict[str, Tuple[int, int]] = {}
         total = 0
@@ -208,9 +270,12 @@ class ModelRunner:
             off, count = offsets[name]
             if count:
                 host[off:off + count] = values
-        if self._meta_device is None or self._meta_device.numel() < total:
-            self._meta_device = torch.empty(max(total, 4096), dtype=torch.int32, device=self.device)
-        meta = self._meta_device
+        if meta is None:
+            if self._meta_device is None or self._meta_device.numel() < total:
+                self._meta_device = torch.empty(max(total, 4096), dtype=torch.int32, device=self.device)
+            meta = self._meta_device
+        elif meta.numel() < total:
+            raise ValueError("the metadata buffer of the graph is too small")
         meta[:total].copy_(staging[:total], non_blocking=True)
         event = self._staging_events[ring] or torch.cuda.Event()
         event.record()
@@ -232,12 +297,52 @@ class ModelRunner:
         return StepBatch(
             n_tokens=n_tokens, n_rows=n_rows, token_ids=view("ids"), positions=view("positions"),
             token_row=view("token_row"), kv_hi=view("kv_hi"), row_slot=view("row_slot"), cu_q=view("cu_q"),
-            kv_len=view("kv_len"), logit_rows=view("logit_rows"), groups=groups, workspace=self.workspace,
-            qblk_row=view("qblk_row"), qblk_tok=view("qblk_tok"),
+            kv_len=view("kv_len"), logit_rows=view("logit_rows"), groups=groups,
+            workspace=workspace or self.workspace, qblk_row=view("qblk_row"), qblk_tok=view("qblk_tok"),
             given_embeds=given_embeds, given_rows=view("given_rows") if given else None, max_q=max_q, max_kv=max_kv,
             decode_only=max_q == 1, causal_only=causal_only,
-            host={"starts": starts, "q_lens": [len(e.tokens) for e in entries], "kv_len": kv_len},
+            host={"starts": starts, "q_lens": [len(e.tokens) for e in entries], "kv_len": kv_len, "meta_ints": total},
         )
+
+    # ------------------------------------------------------------------ graphs
+    def _graph_bucket(self, entries: Sequence[StepEntry]) -> Optional[int]:
+        """The bucket a step can be replayed in, or ``None``: every entry one token with its
+        logits wanted, no given embedding, at most the largest bucket."""
+        if not self.enable_graphs or len(entries) > self._buckets[-1]:
+            return None
+        for e in entries:
+            if len(e.tokens) != 1 or int(e.tokens[0]) < 0 or list(e.want) != [0] or e.embeds is not None:
+                return None
+        return next(b for b in self._buckets if b >= len(entries))
+
+    def _step_graph(self, entries: Sequence[StepEntry], bucket: int) -> torch.Tensor:
+        state = self._graphs.get(bucket)
+        if state is None:
+            state = self._graphs[bucket] = _GraphState(self.device)
+        if state.meta is None:
+            probe = self.build_batch(entries, pad_rows=bucket, fixed_pages=self._pages_cap)
+            state.meta = torch.empty(probe.host["meta_ints"], dtype=torch.int32, device=self.device)
+        batch = self.build_batch(entries, pad_rows=bucket, fixed_pages=self._pages_cap, meta=state.meta,
+                                 workspace=state.workspace)
+        # the decode attention kernel cuts a row's keys by the longest context of the batch: a
+        # graph must cut the same way on every replay, so it is captured for the longest possible
+        batch.max_kv = self.model.plan.max_positions
+        if state.graph is None:
+            current = torch.cuda.current_stream()
+            side = torch.cuda.Stream()
+            side.wait_stream(current)
+            with torch.cuda.stream(side):          # first run outside capture: every buffer comes into being
+                self.model.forward(batch, self.layer_caches)
+            current.wait_stream(side)
+            torch.cuda.synchronize()
+            state.workspace.freeze()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                state.logits = self.model.forward(batch, self.layer_caches)
+            state.graph = graph
+        state.graph.replay()
+        self.graph_replays += 1
+        return state.logits[:len(entries)]
 
     # ------------------------------------------------------------------ the step
     @torch.inference_mode()
@@ -245,9 +350,15 @@ class ModelRunner:
         """Run the entries as one batch. Returns fp32 logits ``[wanted, vocab]`` in the order of
         the entries and of their ``want``; the tensor is scratch memory and is overwritten by
         the next step."""
-        batch = self.build_batch(entries)
-        logits = self.model.forward(batch, self.layer_caches)
-        for e, start in zip(entries, batch.host["starts"]):
+        bucket = self._graph_bucket(entries)
+        if bucket is not None:
+            logits = self._step_graph(entries, bucket)
+            starts = [self.held[e.slot] for e in entries]
+        else:
+            batch = self.build_batch(entries)
+            logits = self.model.forward(batch, self.layer_caches)
+            starts = batch.host["starts"]
+        for e, start in zip(entries, starts):
             self.held[e.slot] = start + len(e.tokens)
             self.cache.trim(e.slot, self.held[e.slot])
         return logits

@@ -18,8 +18,7 @@ _c_void_p, _c_int, _c_long, _c_float = ctypes.c_void_p, ctypes.c_int, ctypes.c_l
 
 _SIGNATURES = {
     "ka_linear_skinny_bf16": [_c_void_p, _c_long, _c_void_p, _c_long, _c_void_p, _c_void_p, _c_int, _c_long, _c_int,
-                              _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_long, _c_void_p, _c_int, _c_int,
-                              _c_void_p],
+                              _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
     "ka_linear_tiled_bf16": [_c_void_p, _c_long, _c_void_p, _c_long, _c_void_p, _c_void_p, _c_int, _c_long, _c_int,
                              _c_int, _c_int, _c_int, _c_int, _c_void_p],
     "ka_attention_prefill_bf16": [_c_void_p, _c_long, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p,
@@ -27,13 +26,13 @@ _SIGNATURES = {
                                   _c_int, _c_int, _c_int, _c_int, _c_void_p],
     "ka_attention_decode_bf16": [_c_void_p, _c_long, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p,
                                  _c_void_p, _c_void_p, _c_long, _c_float, _c_int, _c_int, _c_int, _c_int, _c_int,
-                                 _c_int, _c_void_p, _c_long, _c_void_p, _c_int, _c_void_p],
+                                 _c_int, _c_int, _c_void_p, _c_long, _c_void_p, _c_int, _c_void_p],
 }
 
 # Rows up to which the weight-streaming kernel is used instead of the tiled one.
 SKINNY_MAX_ROWS = 64
-# Workgroups the weight-streaming kernel aims for (256 CUs, a few workgroups each).
-SKINNY_TARGET_WORKGROUPS = 1024
+# Waves the weight-streaming kernel aims to have on the chip (256 CUs, 16 to 32 waves each).
+SKINNY_TARGET_WAVES = 6144
 SCRATCH_FLOATS = 8 << 20
 SCRATCH_COUNTERS = 1 << 16
 
@@ -92,11 +91,9 @@ def linear_bf16(a, weight, bias, out, act, accumulate) -> bool:
         raise KernelError("linear: accumulate needs an fp32 output")
     handle = lib()
     if m <= SKINNY_MAX_ROWS:
-        partial, counters = scratch(a.device)
         _check(handle.ka_linear_skinny_bf16(a.data_ptr(), a.stride(0), weight.data_ptr(), weight.stride(0), _ptr(bias),
                                             out.data_ptr(), _OUT_CODE[out.dtype], out.stride(0), m, n, k, act,
-                                            int(accumulate), partial.data_ptr(), partial.numel(), counters.data_ptr(),
-                                            counters.numel(), SKINNY_TARGET_WORKGROUPS, stream_ptr()))
+                                            int(accumulate), SKINNY_TARGET_WAVES, stream_ptr()))
     else:
         _check(handle.ka_linear_tiled_bf16(a.data_ptr(), a.stride(0), weight.data_ptr(), weight.stride(0), _ptr(bias),
                                            out.data_ptr(), _OUT_CODE[out.dtype], out.stride(0), m, n, k, act,
@@ -104,10 +101,17 @@ def linear_bf16(a, weight, bias, out, act, accumulate) -> bool:
     return True
 
 
-def decode_splits(n_tokens: int, n_heads: int, max_kv: int) -> int:
-    """Cuts of a row's keys so that about 512 workgroups run, each with at least 256 keys."""
-    wanted = -(-512 // max(1, n_tokens * n_heads))
-    return max(1, min(wanted, -(-max_kv // 256)))
+DECODE_KEYS_PER_WORKGROUP = 4096
+
+
+def decode_shape(max_kv: int):
+    """``(splits, waves)`` of the decode attention kernel: a workgroup of up to 16 waves takes a
+    64-key tile per wave and round; rows longer than 4096 keys are cut into splits that meet
+    through scratch memory."""
+    splits = max(1, -(-max_kv // DECODE_KEYS_PER_WORKGROUP))
+    tiles = -(-max_kv // (64 * splits))
+    waves = 4 if tiles <= 4 else 8 if tiles <= 8 else 16
+    return splits, waves
 
 
 def attention_bf16(q, k_cache, v_cache, block_table, token_row, kv_lo, kv_hi, out, scale, n_heads, n_kv_heads,
@@ -120,13 +124,13 @@ def attention_bf16(q, k_cache, v_cache, block_table, token_row, kv_lo, kv_hi, ou
         return False
     handle = lib()
     if batch.decode_only and handle.ka_attention_decode_supported(head_dim, page_size):
-        splits = decode_splits(n, n_heads, batch.max_kv)
+        splits, waves = decode_shape(batch.max_kv)
         partial, counters = scratch(q.device)
         if n * n_heads * splits * (head_dim + 2) <= partial.numel() and n * n_heads <= counters.numel():
             _check(handle.ka_attention_decode_bf16(
                 q.data_ptr(), q.stride(0), k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(),
                 block_table.shape[1], token_row.data_ptr(), _ptr(kv_lo), kv_hi.data_ptr(), out.data_ptr(),
-                out.stride(0), float(scale), n, n_heads, n_kv_heads, head_dim, page_size, splits, partial.data_ptr(),
+                out.stride(0), float(scale), n, n_heads, n_kv_heads, head_dim, page_size, splits, waves, partial.data_ptr(),
                 partial.numel(), counters.data_ptr(), counters.numel(), stream_ptr()))
             return True
     if handle.ka_attention_prefill_supported(head_dim, page_size) and batch.qblk_row is not None:
