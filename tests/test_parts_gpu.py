@@ -1,0 +1,316 @@
+"""Each part alone against the plain implementation, and parts of other kinds, defined here,
+registered, built and stepped without a change to the framework's files."""
+
+from dataclasses import dataclass
+from types import SimpleNamespace
+from typing import Optional
+
+import pytest
+import torch
+
+from tests import helpers
+from tests.plain import moondream_plain as plain
+
+pytestmark = pytest.mark.gpu
+DEV = torch.device("cuda:0")
+DTYPES = [torch.float32, torch.bfloat16]
+IDS = ["fp32", "bf16"]
+
+
+def _tensors(part, dtype, seed, std=0.2):
+    gen = torch.Generator().manual_seed(seed)
+    out = {}
+    for name, spec in part.params().items():
+        noise = torch.randn(spec.shape, generator=gen)
+        value = 1 + 0.1 * noise if spec.init == "gain" else std * noise
+        out[name] = value.to(torch.bfloat16).to(dtype if spec.role == "matrix" else torch.float32)
+    return out
+
+
+def _workspace_batch(n_tokens, **extra):
+    from kestrel_amd.engine.batch import Workspace
+
+    return SimpleNamespace(workspace=Workspace(DEV), n_tokens=n_tokens, **extra)
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+def test_layernorm_part(dtype):
+    from kestrel_amd.parts import NormSpec, build_part
+
+    part = build_part("norm", NormSpec("layernorm", 200, 3e-4, bias=True))
+    weights = _tensors(part, dtype, 0)
+    part.bind(weights, dtype, DEV)
+    x = torch.randn(7, 200) * 2 + 0.5
+    out = torch.empty(7, 200, dtype=dtype, device=DEV)
+    part.forward(x.to(DEV), out)
+    ref = plain.layer_norm(x.double(), weights["weight"].double(), weights["bias"].double(), 3e-4)
+    helpers.assert_close(out, ref, dtype, "layernorm part")
+
+
+def test_rotary_table_part():
+    from kestrel_amd.parts import PositionSpec, build_part
+
+    part = build_part("position", PositionSpec("rotary_neox", 12, 1234.5, 77))
+    table = part.table(DEV)
+    assert table.dtype == torch.float32 and tuple(table.shape) == (77, 12)
+    torch.testing.assert_close(table.cpu().double(), plain.rotary_table(12, 77, 1234.5), atol=2e-5, rtol=0)
+    assert build_part("position", PositionSpec("none")).table(DEV) is None
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+def test_feed_forward_part(dtype):
+    from kestrel_amd.parts import DenseFeedForwardSpec, build_part
+
+    part = build_part("feed_forward", DenseFeedForwardSpec("dense", 72, 200, "gelu_tanh", bias=True))
+    w = _tensors(part, dtype, 1)
+    part.bind(w, dtype, DEV)
+    h = (torch.randn(9, 72)).to(torch.bfloat16)
+    residual = torch.randn(9, 72)
+    out = residual.clone().to(DEV)
+    part.forward(h.to(dtype).to(DEV), _workspace_batch(9), out)
+    wd = {"p.mlp." + k: v.double() for k, v in w.items()}
+    ref = residual.double() + plain.mlp(h.double(), wd, "p.")
+    helpers.assert_close(out, ref, dtype, "feed-forward part")
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+@pytest.mark.parametrize("shape", [(4, 4, 16, 8), (6, 2, 48, 12), (3, 1, 64, 32)])
+def test_attention_part(shape, dtype):
+    """The mixer alone on a cache of its own: a prompt in two portions, then a decoded token."""
+    from kestrel_amd.cache import CacheManager
+    from kestrel_amd.engine.step import ModelRunner, StepEntry
+    from kestrel_amd.parts import AttentionSpec, PositionSpec, build_part
+
+    h, hkv, hd, rot = shape
+    dim = 40
+    spec = AttentionSpec("attention", dim, h, hkv, hd, PositionSpec("rotary_neox", rot, 500.0, 64), bias=True)
+    part = build_part("mixer", spec)
+    w = _tensors(part, dtype, 2, std=0.08)         # outputs of order 0.3: the tolerances are absolute
+    part.bind(w, dtype, DEV)
+    cache = CacheManager([(part.cache_spec(), None, None)], 16, 8, 2, dtype=dtype, device=DEV)
+    fake_model = SimpleNamespace(plan=SimpleNamespace(max_positions=64, vocab_size=10, dim=dim))
+    runner = ModelRunner(fake_model, cache, DEV)
+    slot = runner.admit()
+    total = 23
+    hs = torch.randn(total, dim).to(torch.bfloat16)
+    outs = []
+    for lo, hi in ((0, 17), (17, 22), (22, 23)):
+        batch = runner.build_batch([StepEntry(slot, [1] * (hi - lo))])
+        residual = torch.zeros(hi - lo, dim, device=DEV)
+        part.forward(hs[lo:hi].to(dtype).to(DEV), batch, runner.layer_caches[0], residual)
+        runner.held[slot] = hi
+        outs.append(residual.cpu())
+    cfg = {"n_heads": h, "n_kv_heads": hkv, "head_dim": hd}
+    wd = {"p.attn." + k: v.double() for k, v in w.items()}
+    positions = torch.arange(total)
+    ref = plain.attention(hs.double(), wd, "p.", cfg, positions, plain.visibility(positions, None),
+                          plain.rotary_table(rot, 64, 500.0))
+    helpers.assert_close(torch.cat(outs), ref, dtype, f"attention part {shape}")
+
+
+# ------------------------------------------------------------------------------------------------
+# parts of other kinds, defined in this test file
+# ------------------------------------------------------------------------------------------------
+
+@dataclass(frozen=True)
+class DecaySpec:
+    kind: str
+    dim: int
+    decay: float
+
+
+def _register_toys():
+    from kestrel_amd.parts import (FeedForward, Mixer, ParamSpec, PositionEncoding, StateSpec, register_feed_forward,
+                                   register_mixer, register_position)
+
+    class DecayMixer(Mixer):
+        """A mixer with state of its own and no keys or values: ``s <- decay * s + h W``, output ``s``.
+        The state lives in the cache manager's per-request slots."""
+
+        def params(self):
+            return {"w.weight": ParamSpec((self.spec.dim, self.spec.dim))}
+
+        def state_spec(self):
+            return StateSpec((self.spec.dim,), "float32")
+
+        def bind(self, tensors, dtype, device):
+            self.w = tensors["w.weight"].to(device).float()
+
+        def forward(self, h, batch, cache, residual):
+            # plain torch on the GPU: this toy shows the interfaces, not a kernel
+            rows = batch.token_row.long()
+            slots = batch.row_slot.long()
+            u = h.float() @ self.w.T
+            for t in range(h.shape[0]):
+                slot = slots[rows[t]]
+                if slot < 0:
+                    continue
+                cache.state[slot] = self.spec.decay * cache.state[slot] + u[t]
+                residual[t] += cache.state[slot]
+
+    class RoutedFeedForward(FeedForward):
+        """A feed-forward with routing: the router picks one of two experts per token."""
+
+        def params(self):
+            d = self.spec.dim
+            return {"router.weight": ParamSpec((2, d)), "e0.weight": ParamSpec((d, d)), "e1.weight": ParamSpec((d, d))}
+
+        def bind(self, tensors, dtype, device):
+            self.t = {k: v.to(device).float() for k, v in tensors.items()}
+
+        def forward(self, h, batch, residual):
+            x = h.float()
+            choice = (x @ self.t["router.weight"].T).argmax(dim=-1)
+            both = torch.stack([x @ self.t["e0.weight"].T, x @ self.t["e1.weight"].T])
+            residual += both[choice, torch.arange(x.shape[0], device=x.device)]
+
+    class LearnedPosition(PositionEncoding):
+        """Another position encoding: nothing to rotate, so no table."""
+
+    register_mixer("toy_decay", DecayMixer)
+    register_feed_forward("toy_routed", RoutedFeedForward)
+    register_position("toy_learned", LearnedPosition)
+
+
+def _toy_reference(ids, w, decay, eps):
+    """The toy model computed plainly: layer 0 (decay mixer, routed ff, sequential norms), then
+    layer 1 = attention + dense, then layer 0 again (its weights, a state of its own)."""
+    dim = w["emb"].shape[1]
+    x = w["emb"].double()[torch.tensor(ids)]
+    positions = torch.arange(len(ids))
+    allowed = plain.visibility(positions, None)
+
+    def toy_layer(x, state):
+        out = []
+        for t in range(x.shape[0]):
+            xt = x[t]
+            h = plain.layer_norm(xt, w["l0.n1.weight"].double(), w["l0.n1.bias"].double(), eps)
+            state = decay * state + w["l0.mix.w.weight"].double() @ h
+            xt = xt + state
+            h2 = plain.layer_norm(xt, w["l0.n2.weight"].double(), w["l0.n2.bias"].double(), eps)
+            e = int((w["l0.ff.router.weight"].double() @ h2).argmax())
+            xt = xt + w[f"l0.ff.e{e}.weight"].double() @ h2
+            out.append(xt)
+        return torch.stack(out)
+
+    x = toy_layer(x, torch.zeros(dim, dtype=torch.float64))
+    cfg = {"n_heads": 2, "n_kv_heads": 1, "head_dim": 16}
+    wd = {k.replace("l1.", "p."): v.double() for k, v in w.items() if k.startswith("l1.")}
+    xn = plain.layer_norm(x, wd["p.ln.weight"], wd["p.ln.bias"], eps)
+    x = x + plain.attention(xn, wd, "p.", cfg, positions, allowed, plain.rotary_table(8, 64, 100.0)) \
+        + plain.mlp(xn, wd, "p.")
+    x = toy_layer(x, torch.zeros(dim, dtype=torch.float64))
+    normed = plain.layer_norm(x, w["fn.weight"].double(), w["fn.bias"].double(), eps)
+    return normed @ w["emb"].double().T          # tied head, no bias
+
+
+def test_toy_parts_build_and_step():
+    """A mixer with state, a routed feed-forward and another position encoding are registered
+    from here; a plan names a layer twice in its schedule; the generic decoder, the cache
+    manager and the step function run it in portions and match a plain computation."""
+    from kestrel_amd.cache import CacheManager
+    from kestrel_amd.engine.step import ModelRunner, StepEntry
+    from kestrel_amd.models import DecoderModel
+    from kestrel_amd.parts import (AttentionSpec, DenseFeedForwardSpec, LayerSpec, ModelPlan, NormSpec, PositionSpec,
+                                   ScheduleEntry)
+
+    _register_toys()
+    dim, vocab, eps, decay = 32, 50, 1e-5, 0.5
+    norm = NormSpec("layernorm", dim, eps)
+    toy = LayerSpec("sequential", norm, DecaySpec("toy_decay", dim, decay), DecaySpec("toy_routed", dim, 0.0),
+                    norm2=norm, names={"norm.weight": "l0.n1.weight", "norm.bias": "l0.n1.bias",
+                                       "norm2.weight": "l0.n2.weight", "norm2.bias": "l0.n2.bias",
+                                       "mixer.w.weight": "l0.mix.w.weight",
+                                       "feed_forward.router.weight": "l0.ff.router.weight",
+                                       "feed_forward.e0.weight": "l0.ff.e0.weight",
+                                       "feed_forward.e1.weight": "l0.ff.e1.weight"})
+    attn = LayerSpec("parallel", norm,
+                     AttentionSpec("attention", dim, 2, 1, 16, PositionSpec("rotary_neox", 8, 100.0, 64)),
+                     DenseFeedForwardSpec("dense", dim, 48),
+                     names={"norm.weight": "l1.ln.weight", "norm.bias": "l1.ln.bias",
+                            "mixer.qkv.weight": "l1.attn.qkv.weight", "mixer.qkv.bias": "l1.attn.qkv.bias",
+                            "mixer.proj.weight": "l1.attn.proj.weight", "mixer.proj.bias": "l1.attn.proj.bias",
+                            "feed_forward.fc1.weight": "l1.mlp.fc1.weight", "feed_forward.fc1.bias": "l1.mlp.fc1.bias",
+                            "feed_forward.fc2.weight": "l1.mlp.fc2.weight", "feed_forward.fc2.bias": "l1.mlp.fc2.bias"})
+    plan = ModelPlan("toy", vocab, dim, 64, (toy, attn), (ScheduleEntry(0), ScheduleEntry(1), ScheduleEntry(0)),
+                     norm, head_bias=False, tied_head=True,
+                     names={"embedding": "emb", "final_norm.weight": "fn.weight", "final_norm.bias": "fn.bias"})
+    model = DecoderModel(plan)
+    gen = torch.Generator().manual_seed(3)
+    weights = {}
+    for name, spec in model.params().items():
+        noise = torch.randn(spec.shape, generator=gen)
+        weights[name] = (1 + 0.1 * noise) if spec.init == "gain" else 0.3 * noise
+    model.bind(weights, torch.float32, DEV)
+    needs = model.cache_needs()
+    assert [n[0] is None for n in needs] == [True, False, True] and [n[1] is None for n in needs] == [False, True, False]
+    cache = CacheManager(needs, 16, 8, 3, dtype=torch.float32, device=DEV)
+    assert cache.states[0] is not None and cache.states[2] is not None and cache.states[0] is not cache.states[2]
+    runner = ModelRunner(model, cache, DEV)
+    ids_a = helpers.random_ids(30, 21, vocab)
+    ids_b = helpers.random_ids(31, 9, vocab)
+    a, b = runner.admit(), runner.admit()
+    got_a, got_b = [], []
+    out = runner.step([StepEntry(a, ids_a[:12], want=list(range(12)))]).clone()
+    got_a.append(out)
+    out = runner.step([StepEntry(a, ids_a[12:20], want=list(range(8))), StepEntry(b, ids_b[:8], want=list(range(8)))]).clone()
+    got_a.append(out[:8])
+    got_b.append(out[8:])
+    out = runner.step([StepEntry(b, ids_b[8:], want=[0]), StepEntry(a, ids_a[20:], want=[0])]).clone()
+    got_b.append(out[:1])
+    got_a.append(out[1:])
+    helpers.assert_close(torch.cat(got_a), _toy_reference(ids_a, weights, decay, eps), torch.float32, "toy a")
+    helpers.assert_close(torch.cat(got_b), _toy_reference(ids_b, weights, decay, eps), torch.float32, "toy b")
+    # a slot that is used again starts from a zero state
+    runner.release(a)
+    c = runner.admit()
+    assert c == a
+    out = runner.step([StepEntry(c, ids_b, want=list(range(9)))]).clone()
+    helpers.assert_close(out, _toy_reference(ids_b, weights, decay, eps), torch.float32, "toy c")
+
+
+def test_a_layer_may_read_another_layers_cache():
+    """Schedule entry 1 keeps no keys and values and reads those of entry 0."""
+    from kestrel_amd.config import get_spec
+    from kestrel_amd.engine.loading import make_runner
+    from kestrel_amd.engine.step import StepEntry
+    from kestrel_amd.models import DecoderModel
+    from kestrel_amd.parts import ScheduleEntry
+    from dataclasses import replace
+
+    spec = get_spec("moondream2")
+    plan = spec.build_plan(spec.read_config(helpers.TINY_A))
+    plan = replace(plan, schedule=(ScheduleEntry(0), ScheduleEntry(1, reads_cache_of=0)))
+    model = DecoderModel(plan)
+    weights = {k: v.float() for k, v in helpers.stored_weights(helpers.model_dir("A")).items()}
+    model.bind(weights, torch.float32, DEV)
+    runner = make_runner(model, 16, 8, 2)
+    assert len(runner.cache.groups[0].entries) == 1            # one cache for both runs
+    ids = helpers.random_ids(40, 20, 512)
+    slot = runner.admit()
+    whole = runner.step([StepEntry(slot, ids, want=list(range(20)))]).clone()
+    runner.release(slot)
+    slot = runner.admit()
+    parts = [runner.step([StepEntry(slot, ids[:13], want=list(range(13)))]).clone()]
+    parts += [runner.step([StepEntry(slot, [t], want=[0])]).clone() for t in ids[13:]]
+    helpers.assert_close(torch.cat(parts), whole, torch.float32, "shared cache: portions against whole")
+    # and it equals the plain model whose second layer attends to the first layer's keys and values
+    cfg = helpers.flat_config("A")
+    w = {k: v.double() for k, v in weights.items()}
+    x = w["text.wte"][torch.tensor(ids)]
+    positions = torch.arange(20)
+    allowed = plain.visibility(positions, None)
+    table = plain.rotary_table(plain.rotary_dim_of(cfg), 20, cfg["rope_theta"])
+    hd, nh = plain.head_dim_of(cfg), cfg["n_heads"]
+    kv0 = None
+    for i in range(2):
+        p = f"text.blocks.{i}."
+        xn = plain.layer_norm(x, w[p + "ln.weight"], w[p + "ln.bias"], plain.eps_of(cfg))
+        qkv = plain.linear(xn, w[p + "attn.qkv.weight"], w[p + "attn.qkv.bias"])
+        q, k, v = qkv.split([nh * hd, nh * hd, nh * hd], dim=-1)
+        q = plain.apply_rotary(q.reshape(20, nh, hd), positions, table)
+        if i == 0:
+            kv0 = (plain.apply_rotary(k.reshape(20, nh, hd), positions, table), v.reshape(20, nh, hd))
+        o = plain.attention_core(q, kv0[0], kv0[1], allowed, hd ** -0.5).reshape(20, nh * hd)
+        x = x + plain.linear(o, w[p + "attn.proj.weight"], w[p + "attn.proj.bias"]) + plain.mlp(xn, w, p)
+    helpers.assert_close(whole, plain.head(x, w, cfg), torch.float32, "shared cache against plain")
