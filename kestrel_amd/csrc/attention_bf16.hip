@@ -173,13 +173,47 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_
 // ----------------------------------------------------------------------------------------------
 constexpr int AD_TILE = 64;               // keys per wave tile
 
+// What the decode kernel needs to take over the rotary encoding and the cache write of the
+// step's own token (slots null: that work was done before, and the token's key is in the cache).
+struct DecodeFuse {
+    const bf16_t* k_new;      // key and value rows of the tokens: [n, stride], heads side by side
+    const bf16_t* v_new;
+    long stride;
+    const float* table;       // fp32 [positions, rot]: cos then sin
+    int rot;
+    const int* slots;         // page * 16 + offset the token's key and value go to, < 0: nowhere
+    bf16_t* k_cache;
+    bf16_t* v_cache;
+};
+
+// Eight channels dg * 8 .. + 8 of one head row, rotated for the table row `cs` (non-interleaved
+// halves of the first `rot` channels), rounded to bf16 as the cache and the q buffer hold them.
+__device__ __forceinline__ void at_rotate8(const bf16_t* head, int dg, const float* cs, int rot, float out[8]) {
+    const int d0 = dg * 8, half = rot / 2;
+    bf16x8 own = at_load8(head + d0);
+    if (d0 >= rot) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) out[j] = (float)own[j];
+        return;
+    }
+    const bool first = d0 < half;
+    bf16x8 other = at_load8(head + (first ? d0 + half : d0 - half));
+    const int i0 = first ? d0 : d0 - half;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        float c = cs[i0 + j], sn = cs[half + i0 + j];
+        float v = first ? (float)own[j] * c - (float)other[j] * sn : (float)own[j] * c + (float)other[j] * sn;
+        out[j] = (float)(bf16_t)v;
+    }
+}
+
 template <int HD, int WAVES>
 __global__ void __launch_bounds__(KA_WAVE * WAVES)
 attn_decode_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t* __restrict__ k_cache,
                    const bf16_t* __restrict__ v_cache, const int* __restrict__ block_table, int max_pages,
                    const int* __restrict__ token_row, const int* __restrict__ kv_lo,
                    const int* __restrict__ kv_hi, bf16_t* __restrict__ out, long out_row_stride, float scale,
-                   int H, int Hkv, float* __restrict__ partial, unsigned* __restrict__ counters) {
+                   int H, int Hkv, float* __restrict__ partial, unsigned* __restrict__ counters, DecodeFuse fz) {
     constexpr int LPK = HD / 8;            // lanes per key row
     constexpr int KPI = KA_WAVE / LPK;     // keys per load instruction
     constexpr int VU = HD * 2 / KA_WAVE;   // 16-byte value loads per lane and page
@@ -190,7 +224,10 @@ attn_decode_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t
     const int wave = threadIdx.x / KA_WAVE, lane = threadIdx.x % KA_WAVE;
     const int kvh = h / (H / Hkv);
     const int row = token_row[t];
-    const int lo = kv_lo ? kv_lo[t] : 0, hi = kv_hi[t];
+    const int lo = kv_lo ? kv_lo[t] : 0;
+    const bool fused = fz.slots != nullptr && kv_hi[t] > 0;
+    const int pos = kv_hi[t] - 1;                 // fused: the token's own position, whose key is not cached yet
+    const int hi = fused ? pos : kv_hi[t];        // cached keys this token reads: [lo, hi)
     const int lo_tile = lo & ~(AD_TILE - 1);      // tiles start on page boundaries; keys below lo are masked
     const int chunk = ((hi - lo_tile + S - 1) / S + AD_TILE - 1) / AD_TILE * AD_TILE;
     const int s_lo = lo_tile + split * chunk, s_hi = min(hi, s_lo + chunk);
@@ -198,7 +235,11 @@ attn_decode_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t
     const int ks = lane / LPK, dg = lane % LPK;
     const float sl2 = scale * AT_LOG2E;
     float qf[8];
-    {
+    if (fused) {
+        at_rotate8(q + (size_t)t * q_row_stride + (size_t)h * HD, dg, fz.table + (size_t)pos * fz.rot, fz.rot, qf);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) qf[j] *= sl2;
+    } else {
         bf16x8 qv = at_load8(q + (size_t)t * q_row_stride + (size_t)h * HD + dg * 8);
 #pragma unroll
         for (int j = 0; j < 8; ++j) qf[j] = (float)qv[j] * sl2;
@@ -271,6 +312,45 @@ attn_decode_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t
                 }
                 acc[u] += sum;
             }
+        }
+    }
+    if (fused && wave == 0 && split == 0) {
+        // the token's own key and value: rotate the key, let one head of the group store both, and
+        // take them into this wave's sums straight from registers
+        float kn[8];
+        at_rotate8(fz.k_new + (size_t)t * fz.stride + (size_t)kvh * HD, dg, fz.table + (size_t)pos * fz.rot, fz.rot, kn);
+        const bf16_t* vrow = fz.v_new + (size_t)t * fz.stride + (size_t)kvh * HD;
+        const int slot = fz.slots[t];
+        if (slot >= 0 && h % (H / Hkv) == 0) {
+            const size_t page = slot / AT_PAGE, off = slot % AT_PAGE;
+            if (ks == 0) {
+                bf16x8 kb;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) kb[j] = (bf16_t)kn[j];
+                *reinterpret_cast<bf16x8*>(fz.k_cache + ((page * Hkv + kvh) * AT_PAGE + off) * HD + dg * 8) = kb;
+            }
+            if ((lane & 1) == 0) {
+#pragma unroll
+                for (int u = 0; u < VU; ++u) {
+                    int d = u * 32 + lane / 2;
+                    fz.v_cache[((page * Hkv + kvh) * HD + d) * AT_PAGE + off] = vrow[d];
+                }
+            }
+        }
+        float dot = 0.f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) dot = fmaf(qf[j], kn[j], dot);
+#pragma unroll
+        for (int off = 1; off < LPK; off <<= 1) dot += __shfl_xor(dot, off, KA_WAVE);
+        float m_new = fmaxf(m_i, dot);
+        float alpha = exp2f(m_i - m_new);
+        float pn = exp2f(dot - m_new);
+        l_i = l_i * alpha + pn;
+        m_i = m_new;
+#pragma unroll
+        for (int u = 0; u < VU; ++u) {
+            float vn = (lane & 1) == 0 ? (float)vrow[u * 32 + lane / 2] : 0.f;
+            acc[u] = acc[u] * alpha + pn * vn;
         }
     }
     // the two halves of a channel row
@@ -399,7 +479,9 @@ KA_API int ka_attention_decode_bf16(const void* q, long q_row_stride, const void
                                     const int* block_table, int max_pages, const int* token_row, const int* kv_lo,
                                     const int* kv_hi, void* out, long out_row_stride, float scale, int n, int H,
                                     int Hkv, int hd, int page_size, int splits, int waves, float* partial,
-                                    long partial_floats, unsigned* counters, int n_counters, hipStream_t stream) {
+                                    long partial_floats, unsigned* counters, int n_counters, const void* k_new,
+                                    const void* v_new, long new_stride, const float* table, int rot,
+                                    const int* slots, void* k_cache_w, void* v_cache_w, hipStream_t stream) {
     if (check_common("ka_attention_decode_bf16", q, q_row_stride, out, out_row_stride, n, H, Hkv, hd, page_size,
                      max_pages))
         return -1;
@@ -412,11 +494,19 @@ KA_API int ka_attention_decode_bf16(const void* q, long q_row_stride, const void
         KA_CHECK((long)n * H <= n_counters, "ka_attention_decode_bf16: too few counters");
     }
     KA_CHECK(waves == 4 || waves == 8 || waves == 16, "ka_attention_decode_bf16: waves must be 4, 8 or 16");
+    DecodeFuse fz = {};
+    if (slots) {
+        // the kernel rotates q and the new key itself and stores the token's key and value
+        KA_CHECK(k_new && v_new && k_cache_w && v_cache_w, "ka_attention_decode_bf16: fused mode needs the new key and value rows");
+        KA_CHECK(rot > 0 && rot <= hd && rot % 16 == 0 && table, "ka_attention_decode_bf16: fused mode needs a rotary width that is a multiple of 16 (got %d)", rot);
+        KA_CHECK(new_stride % 8 == 0 && (uintptr_t)k_new % 16 == 0 && (uintptr_t)v_new % 16 == 0, "ka_attention_decode_bf16: new key rows must be 16-byte aligned");
+        fz = DecodeFuse{(const bf16_t*)k_new, (const bf16_t*)v_new, new_stride, table, rot, slots, (bf16_t*)k_cache_w, (bf16_t*)v_cache_w};
+    }
     dim3 grid(n, H, splits), block(KA_WAVE * waves);
 #define KA_AD(HDV, WV)                                                                                              \
     hipLaunchKernelGGL((attn_decode_kernel<HDV, WV>), grid, block, 0, stream, (const bf16_t*)q, q_row_stride,      \
                        (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, max_pages, token_row, kv_lo,   \
-                       kv_hi, (bf16_t*)out, out_row_stride, scale, H, Hkv, partial, counters)
+                       kv_hi, (bf16_t*)out, out_row_stride, scale, H, Hkv, partial, counters, fz)
     if (hd == 64) {
         if (waves == 4) KA_AD(64, 4); else if (waves == 8) KA_AD(64, 8); else KA_AD(64, 16);
     } else {

@@ -106,18 +106,70 @@ layernorm_kernel(const float* __restrict__ x, const int* __restrict__ rows,
     }
 }
 
+// Rows of up to 256 * 4 * ITEMS values: every thread keeps its share of the row in registers, so
+// the row is read once.
+template <typename TOut, int ITEMS>
+__global__ void __launch_bounds__(LN_THREADS)
+layernorm_regs_kernel(const float* __restrict__ x, const int* __restrict__ rows,
+                      const float* __restrict__ gamma, const float* __restrict__ beta, float eps,
+                      TOut* __restrict__ out, int dim) {
+    typedef __attribute__((ext_vector_type(4))) float floatx4;
+    __shared__ float smem[LN_THREADS / KA_WAVE];
+    int i = blockIdx.x;
+    const float* src = x + (size_t)(rows ? rows[i] : i) * dim;
+    TOut* dst = out + (size_t)i * dim;
+    floatx4 v[ITEMS];
+    float s = 0.f;
+#pragma unroll
+    for (int j = 0; j < ITEMS; ++j) {
+        int d = (j * LN_THREADS + threadIdx.x) * 4;
+        v[j] = d < dim ? *reinterpret_cast<const floatx4*>(src + d) : floatx4{0.f, 0.f, 0.f, 0.f};
+        s += (v[j][0] + v[j][1]) + (v[j][2] + v[j][3]);
+    }
+    float mean = block_sum_256(s, smem) / (float)dim;
+    float q = 0.f;
+#pragma unroll
+    for (int j = 0; j < ITEMS; ++j) {
+        int d = (j * LN_THREADS + threadIdx.x) * 4;
+        if (d < dim) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) q += (v[j][e] - mean) * (v[j][e] - mean);
+        }
+    }
+    float rstd = 1.0f / sqrtf(block_sum_256(q, smem) / (float)dim + eps);
+#pragma unroll
+    for (int j = 0; j < ITEMS; ++j) {
+        int d = (j * LN_THREADS + threadIdx.x) * 4;
+        if (d < dim) {
+            floatx4 g = *reinterpret_cast<const floatx4*>(gamma + d);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                float y = (v[j][e] - mean) * rstd * g[e];
+                if (beta) y += beta[d + e];
+                dst[d + e] = ka_from_float<TOut>(y);
+            }
+        }
+    }
+}
+
 KA_API int ka_layernorm(const float* x, const int* rows, const float* gamma, const float* beta,
                         float eps, void* out, int out_dtype, int n, int dim, hipStream_t stream) {
     KA_CHECK(n >= 0 && dim > 0, "ka_layernorm: bad sizes n=%d dim=%d", n, dim);
     KA_CHECK(eps >= 0.f, "ka_layernorm: negative eps");
     if (n == 0) return 0;
     dim3 grid(n), block(LN_THREADS);
-    if (out_dtype == KA_F32)
+    KA_CHECK(out_dtype == KA_F32 || out_dtype == KA_BF16, "ka_layernorm: unsupported out dtype %d", out_dtype);
+    const bool aligned = dim % 4 == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)gamma % 16 == 0;
+    if (aligned && dim <= LN_THREADS * 4 * 4) {
+        if (out_dtype == KA_F32)
+            hipLaunchKernelGGL((layernorm_regs_kernel<float, 4>), grid, block, 0, stream, x, rows, gamma, beta, eps, (float*)out, dim);
+        else
+            hipLaunchKernelGGL((layernorm_regs_kernel<bf16_t, 4>), grid, block, 0, stream, x, rows, gamma, beta, eps, (bf16_t*)out, dim);
+    } else if (out_dtype == KA_F32) {
         hipLaunchKernelGGL(layernorm_kernel<float>, grid, block, 0, stream, x, rows, gamma, beta, eps, (float*)out, dim);
-    else if (out_dtype == KA_BF16)
+    } else {
         hipLaunchKernelGGL(layernorm_kernel<bf16_t>, grid, block, 0, stream, x, rows, gamma, beta, eps, (bf16_t*)out, dim);
-    else
-        KA_CHECK(false, "ka_layernorm: unsupported out dtype %d", out_dtype);
+    }
     KA_LAUNCH_CHECK();
     return 0;
 }

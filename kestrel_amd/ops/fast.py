@@ -19,6 +19,13 @@ _c_void_p, _c_int, _c_long, _c_float = ctypes.c_void_p, ctypes.c_int, ctypes.c_l
 _SIGNATURES = {
     "ka_linear_skinny_bf16": [_c_void_p, _c_long, _c_void_p, _c_long, _c_void_p, _c_void_p, _c_int, _c_long, _c_int,
                               _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
+    "ka_linear_skinny_fused": [
+        _c_void_p, _c_long, _c_int,                                   # A1, lda1, K1
+        _c_void_p, _c_long, _c_int, _c_void_p, _c_long, _c_void_p,    # A2, lda2, K2, W2, ldw2, bias2
+        _c_void_p, _c_void_p, _c_void_p, _c_float,                    # ln_x, gamma, beta, eps
+        _c_void_p, _c_long, _c_void_p, _c_void_p, _c_int, _c_long, _c_int, _c_int, _c_int,   # target a
+        _c_void_p, _c_long, _c_void_p, _c_void_p, _c_int, _c_long, _c_int, _c_int,           # target b
+        _c_int, _c_int, _c_void_p],                                   # M, target_waves, stream
     "ka_linear_tiled_bf16": [_c_void_p, _c_long, _c_void_p, _c_long, _c_void_p, _c_void_p, _c_int, _c_long, _c_int,
                              _c_int, _c_int, _c_int, _c_int, _c_void_p],
     "ka_attention_prefill_bf16": [_c_void_p, _c_long, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p,
@@ -26,18 +33,29 @@ _SIGNATURES = {
                                   _c_int, _c_int, _c_int, _c_int, _c_void_p],
     "ka_attention_decode_bf16": [_c_void_p, _c_long, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p,
                                  _c_void_p, _c_void_p, _c_long, _c_float, _c_int, _c_int, _c_int, _c_int, _c_int,
-                                 _c_int, _c_int, _c_void_p, _c_long, _c_void_p, _c_int, _c_void_p],
+                                 _c_int, _c_int, _c_void_p, _c_long, _c_void_p, _c_int,
+                                 _c_void_p, _c_void_p, _c_long, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p,
+                                 _c_void_p],
 }
 
 # Rows up to which the weight-streaming kernel is used instead of the tiled one.
 SKINNY_MAX_ROWS = 64
+# Rows (and their width) up to which the weight-streaming kernel can normalise its input itself.
+SKINNY_LN_MAX_ROWS = 16
+SKINNY_LN_MAX_WIDTH = 2048
+# Whether blocks let the weight-streaming kernel normalise its input itself. Every workgroup then
+# repeats the LayerNorm of all rows; measured on MI355X this costs more than the launch it saves.
+FUSE_LAYERNORM_PROLOGUE = False
 # Waves the weight-streaming kernel aims to have on the chip (256 CUs, 16 to 32 waves each).
 SKINNY_TARGET_WAVES = 6144
 SCRATCH_FLOATS = 8 << 20
 SCRATCH_COUNTERS = 1 << 16
+# Keys of one row a workgroup of the decode attention kernel takes before the row is split.
+DECODE_KEYS_PER_WORKGROUP = 4096
 
 _lib = None
 _scratch: Dict[torch.device, tuple] = {}
+_OUT_CODE = {torch.float32: KA_F32, torch.bfloat16: KA_BF16}
 
 
 def lib():
@@ -62,8 +80,8 @@ def _check(status: int) -> None:
 
 
 def scratch(device: torch.device):
-    """Partial sums and arrival counters the split kernels add up through (one pair per device;
-    the kernels leave the counters at zero). Calls on one device must not overlap."""
+    """Partial results and arrival counters that splits of a long row meet through (one pair per
+    device; the kernels leave the counters at zero). Calls on one device must not overlap."""
     key = torch.device(device)
     if key not in _scratch:
         _scratch[key] = (torch.zeros(SCRATCH_FLOATS, dtype=torch.float32, device=device),
@@ -71,7 +89,17 @@ def scratch(device: torch.device):
     return _scratch[key]
 
 
-_OUT_CODE = {torch.float32: KA_F32, torch.bfloat16: KA_BF16}
+def _operand_ok(t: torch.Tensor, k: int) -> bool:
+    return (t.dtype == torch.bfloat16 and t.dim() == 2 and t.shape[1] == k and t.stride(1) == 1 and t.stride(0) % 8 == 0
+            and t.data_ptr() % 16 == 0)
+
+
+def _bias_ok(bias: Optional[torch.Tensor], n: int) -> bool:
+    return bias is None or (bias.dtype == torch.float32 and bias.numel() == n and bias.is_contiguous())
+
+
+def _out_ok(out: torch.Tensor, m: int, n: int) -> bool:
+    return (out.dtype in _OUT_CODE and tuple(out.shape) == (m, n) and out.stride(1) == 1 and out.data_ptr() % 16 == 0)
 
 
 def linear_bf16(a, weight, bias, out, act, accumulate) -> bool:
@@ -79,13 +107,12 @@ def linear_bf16(a, weight, bias, out, act, accumulate) -> bool:
     n = weight.shape[0]
     if m == 0:
         return True
-    if (k % 8 or a.stride(0) % 8 or weight.stride(0) % 8 or a.data_ptr() % 16 or weight.data_ptr() % 16
-            or out.dtype not in _OUT_CODE or out.data_ptr() % 16 or a.stride(1) != 1 or weight.stride(1) != 1
-            or out.stride(1) != 1):
+    if k % 8 or not _operand_ok(a, k) or not _operand_ok(weight, k) or out.dtype not in _OUT_CODE \
+            or out.data_ptr() % 16 or out.stride(1) != 1:
         return False
-    if tuple(weight.shape) != (n, k) or tuple(out.shape) != (m, n):
+    if tuple(out.shape) != (m, n):
         raise KernelError(f"linear: shapes a {tuple(a.shape)}, weight {tuple(weight.shape)}, out {tuple(out.shape)}")
-    if bias is not None and (bias.dtype != torch.float32 or bias.numel() != n or not bias.is_contiguous()):
+    if not _bias_ok(bias, n):
         raise KernelError("linear: bias must be fp32 [N]")
     if accumulate and out.dtype != torch.float32:
         raise KernelError("linear: accumulate needs an fp32 output")
@@ -101,7 +128,67 @@ def linear_bf16(a, weight, bias, out, act, accumulate) -> bool:
     return True
 
 
-DECODE_KEYS_PER_WORKGROUP = 4096
+def linear_pair_accumulate(a1, w1, b1, a2, w2, b2, out) -> bool:
+    """``out += a1 @ w1.T + b1 + a2 @ w2.T + b2`` in one launch (few rows, fp32 ``out``)."""
+    m, k1 = a1.shape
+    k2 = a2.shape[1]
+    n = w1.shape[0]
+    if not (0 < m <= SKINNY_MAX_ROWS) or k1 % 8 or k2 % 8 or a2.shape[0] != m or w2.shape[0] != n:
+        return False
+    if not (_operand_ok(a1, k1) and _operand_ok(w1, k1) and _operand_ok(a2, k2) and _operand_ok(w2, k2)):
+        return False
+    if out.dtype != torch.float32 or not _out_ok(out, m, n) or not _bias_ok(b1, n) or not _bias_ok(b2, n):
+        return False
+    _check(lib().ka_linear_skinny_fused(
+        a1.data_ptr(), a1.stride(0), k1, a2.data_ptr(), a2.stride(0), k2, w2.data_ptr(), w2.stride(0), _ptr(b2),
+        None, None, None, 0.0,
+        w1.data_ptr(), w1.stride(0), _ptr(b1), out.data_ptr(), KA_F32, out.stride(0), n, 0, 1,
+        None, 0, None, None, 0, 0, 0, 0, m, SKINNY_TARGET_WAVES, stream_ptr()))
+    return True
+
+
+def linear_two_outputs(a, wa, ba, out_a, act_a, wb, bb, out_b, act_b) -> bool:
+    """``out_a = act_a(a @ wa.T + ba)`` and ``out_b = act_b(a @ wb.T + bb)`` in one launch (few rows)."""
+    m, k = a.shape
+    na, nb = wa.shape[0], wb.shape[0]
+    if not (0 < m <= SKINNY_MAX_ROWS) or k % 8:
+        return False
+    if not (_operand_ok(a, k) and _operand_ok(wa, k) and _operand_ok(wb, k) and _out_ok(out_a, m, na)
+            and _out_ok(out_b, m, nb) and _bias_ok(ba, na) and _bias_ok(bb, nb)):
+        return False
+    _check(lib().ka_linear_skinny_fused(
+        a.data_ptr(), a.stride(0), k, None, 0, 0, None, 0, None,
+        None, None, None, 0.0,
+        wa.data_ptr(), wa.stride(0), _ptr(ba), out_a.data_ptr(), _OUT_CODE[out_a.dtype], out_a.stride(0), na, act_a, 0,
+        wb.data_ptr(), wb.stride(0), _ptr(bb), out_b.data_ptr(), _OUT_CODE[out_b.dtype], out_b.stride(0), nb, act_b,
+        m, SKINNY_TARGET_WAVES, stream_ptr()))
+    return True
+
+
+def layernorm_linear_pair(x, gamma, beta, eps, wa, ba, out_a, act_a, wb, bb, out_b, act_b) -> bool:
+    """``h = LayerNorm(x)``; ``out_a = act_a(h @ wa.T + ba)``; ``out_b = act_b(h @ wb.T + bb)`` in one
+    launch: the kernel normalises the fp32 rows itself (at most 16 of them)."""
+    m, k = x.shape
+    if not (0 < m <= SKINNY_LN_MAX_ROWS) or k % 8 or k > SKINNY_LN_MAX_WIDTH or x.dtype != torch.float32 \
+            or not x.is_contiguous():
+        return False
+    if x.data_ptr() % 16 or gamma.dtype != torch.float32 or gamma.numel() != k or gamma.data_ptr() % 16:
+        return False
+    if beta is not None and (beta.dtype != torch.float32 or beta.numel() != k):
+        return False
+    na, nb = wa.shape[0], wb.shape[0]
+    if not (_operand_ok(wa, k) and _operand_ok(wb, k) and _out_ok(out_a, m, na) and _out_ok(out_b, m, nb)
+            and _bias_ok(ba, na) and _bias_ok(bb, nb)):
+        return False
+    if m * (k + 8) * 2 > 96 * 1024:
+        return False
+    _check(lib().ka_linear_skinny_fused(
+        None, 0, k, None, 0, 0, None, 0, None,
+        x.data_ptr(), gamma.data_ptr(), _ptr(beta), float(eps),
+        wa.data_ptr(), wa.stride(0), _ptr(ba), out_a.data_ptr(), _OUT_CODE[out_a.dtype], out_a.stride(0), na, act_a, 0,
+        wb.data_ptr(), wb.stride(0), _ptr(bb), out_b.data_ptr(), _OUT_CODE[out_b.dtype], out_b.stride(0), nb, act_b,
+        m, SKINNY_TARGET_WAVES, stream_ptr()))
+    return True
 
 
 def decode_shape(max_kv: int):
@@ -114,25 +201,56 @@ def decode_shape(max_kv: int):
     return splits, waves
 
 
+def _attention_operands_ok(q, out) -> bool:
+    return not (q.data_ptr() % 16 or q.stride(0) % 8 or out.data_ptr() % 16 or out.stride(0) % 4)
+
+
+def attention_decode_bf16(q, k_cache, v_cache, block_table, token_row, kv_lo, kv_hi, out, scale, n_heads,
+                          n_kv_heads, head_dim, batch, fuse=None) -> bool:
+    """One token per row. ``fuse = (k_new, v_new, table, slots)``: the kernel also rotates q and the
+    token's key and stores key and value in the cache (the rotary kernel is then not run)."""
+    n = q.shape[0]
+    page_size = k_cache.shape[2]
+    if n == 0:
+        return True
+    handle = lib()
+    if batch is None or not batch.decode_only or not _attention_operands_ok(q, out) \
+            or not handle.ka_attention_decode_supported(head_dim, page_size):
+        return False
+    splits, waves = decode_shape(batch.max_kv)
+    partial, counters = scratch(q.device)
+    if n * n_heads * splits * (head_dim + 2) > partial.numel() or n * n_heads > counters.numel():
+        return False
+    k_new = v_new = table = slots = None
+    new_stride = rot = 0
+    if fuse is not None:
+        k_new, v_new, table, slots = fuse
+        rot = int(table.shape[1])
+        new_stride = k_new.stride(0)
+        if rot % 16 or rot > head_dim or splits != 1 or k_new.data_ptr() % 16 or v_new.data_ptr() % 16 \
+                or new_stride % 8 or v_new.stride(0) != new_stride:
+            return False
+    _check(handle.ka_attention_decode_bf16(
+        q.data_ptr(), q.stride(0), k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(),
+        block_table.shape[1], token_row.data_ptr(), _ptr(kv_lo), kv_hi.data_ptr(), out.data_ptr(), out.stride(0),
+        float(scale), n, n_heads, n_kv_heads, head_dim, page_size, splits, waves, partial.data_ptr(), partial.numel(),
+        counters.data_ptr(), counters.numel(), _ptr(k_new), _ptr(v_new), new_stride, _ptr(table), rot, _ptr(slots),
+        k_cache.data_ptr(), v_cache.data_ptr(), stream_ptr()))
+    return True
+
+
 def attention_bf16(q, k_cache, v_cache, block_table, token_row, kv_lo, kv_hi, out, scale, n_heads, n_kv_heads,
                    head_dim, batch) -> bool:
     n = q.shape[0]
     page_size = k_cache.shape[2]
     if n == 0:
         return True
-    if batch is None or q.data_ptr() % 16 or q.stride(0) % 8 or out.data_ptr() % 16 or out.stride(0) % 4:
+    if batch is None or not _attention_operands_ok(q, out):
         return False
+    if attention_decode_bf16(q, k_cache, v_cache, block_table, token_row, kv_lo, kv_hi, out, scale, n_heads,
+                             n_kv_heads, head_dim, batch):
+        return True
     handle = lib()
-    if batch.decode_only and handle.ka_attention_decode_supported(head_dim, page_size):
-        splits, waves = decode_shape(batch.max_kv)
-        partial, counters = scratch(q.device)
-        if n * n_heads * splits * (head_dim + 2) <= partial.numel() and n * n_heads <= counters.numel():
-            _check(handle.ka_attention_decode_bf16(
-                q.data_ptr(), q.stride(0), k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(),
-                block_table.shape[1], token_row.data_ptr(), _ptr(kv_lo), kv_hi.data_ptr(), out.data_ptr(),
-                out.stride(0), float(scale), n, n_heads, n_kv_heads, head_dim, page_size, splits, waves, partial.data_ptr(),
-                partial.numel(), counters.data_ptr(), counters.numel(), stream_ptr()))
-            return True
     if handle.ka_attention_prefill_supported(head_dim, page_size) and batch.qblk_row is not None:
         _check(handle.ka_attention_prefill_bf16(
             q.data_ptr(), q.stride(0), k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(),

@@ -58,18 +58,39 @@ class PagedAttention(Mixer):
             self.proj_bias = tensors["proj.bias"].to(device=device, dtype=torch.float32).contiguous()
         self._table = self.position.table(device)
 
-    def forward(self, h, batch, cache: LayerCache, residual) -> None:
+    # The three stages are also offered one by one, so that a block may fuse the first with its
+    # norm and the last with its feed-forward (see ``Mixer.input_projection``).
+    def input_projection(self):
+        return self.qkv_weight, self.qkv_bias, self.qkv_dim
+
+    def output_projection(self):
+        return self.proj_weight, self.proj_bias
+
+    def attend(self, qkv, batch, cache: LayerCache):
+        """Position encoding, cache write and attention on the projected input ``[n, q|k|v]``."""
         spec = self.spec
-        n = h.shape[0]
-        ws = batch.workspace
-        qkv = ws.get("attn.qkv", (n, self.qkv_dim), self.dtype)
-        linear(h, self.qkv_weight, self.qkv_bias, qkv)
+        n = qkv.shape[0]
         group = batch.groups[cache.group]
+        out = batch.workspace.get("attn.out", (n, self.q_dim), self.dtype)
+        if qkv.dtype == torch.bfloat16 and batch.decode_only and cache.writes and self._table is not None:
+            # one token per row: the decode kernel rotates q and k and stores k and v itself
+            from ..ops import fast
+            k_new = qkv[:, self.q_dim:self.q_dim + self.kv_dim]
+            v_new = qkv[:, self.q_dim + self.kv_dim:]
+            if fast.attention_decode_bf16(qkv, cache.k, cache.v, group.block_table, batch.token_row, group.kv_lo,
+                                          batch.kv_hi, out, self.scale, spec.n_heads, spec.n_kv_heads, spec.head_dim,
+                                          batch, fuse=(k_new, v_new, self._table, group.slots)):
+                return out
         core.rope_cache(qkv, batch.positions, group.slots if cache.writes else None, self._table, cache.k, cache.v,
                         spec.n_heads, spec.n_kv_heads, spec.head_dim, group.page_size)
-        out = ws.get("attn.out", (n, self.q_dim), self.dtype)
         paged_attention(qkv, cache.k, cache.v, group.block_table, batch.token_row, group.kv_lo, batch.kv_hi, out,
                         self.scale, spec.n_heads, spec.n_kv_heads, spec.head_dim, batch)
+        return out
+
+    def forward(self, h, batch, cache: LayerCache, residual) -> None:
+        qkv = batch.workspace.get("attn.qkv", (h.shape[0], self.qkv_dim), self.dtype)
+        linear(h, self.qkv_weight, self.qkv_bias, qkv)
+        out = self.attend(qkv, batch, cache)
         linear(out, self.proj_weight, self.proj_bias, residual, accumulate=True)
 
 

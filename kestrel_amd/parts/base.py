@@ -77,11 +77,36 @@ class Mixer(Part):
         """Add the mixer's output for the normalised input ``h`` into fp32 ``residual``."""
         raise NotImplementedError
 
+    # Optional: a mixer that is "linear, core, linear" may offer its stages one by one. A block can
+    # then run the first linear together with its norm and the feed-forward's first linear, and
+    # the last linear together with the feed-forward's last (one kernel launch each when few rows
+    # are decoded). A mixer without these is always run through ``forward``.
+    def input_projection(self):
+        """``(weight [out, in], bias or None, out)`` of the first linear, or ``None``."""
+        return None
+
+    def attend(self, projected: torch.Tensor, batch, cache: LayerCache) -> torch.Tensor:
+        """The core on the projected input; returns the input of the output projection."""
+        raise NotImplementedError
+
+    def output_projection(self):
+        """``(weight, bias or None)`` of the last linear, whose result is added to the residual."""
+        return None
+
 
 class FeedForward(Part):
     def forward(self, h: torch.Tensor, batch, residual: torch.Tensor) -> None:
         """Add the feed-forward output for ``h`` into fp32 ``residual``."""
         raise NotImplementedError
+
+    # Optional, as for mixers: a feed-forward that is "linear + activation, linear".
+    def input_projection(self):
+        """``(weight, bias or None, out, activation code)`` of the first linear, or ``None``."""
+        return None
+
+    def output_projection(self):
+        """``(weight, bias or None)`` of the last linear, whose result is added to the residual."""
+        return None
 
 
 _REGISTRIES: Dict[str, Dict[str, Callable]] = {"mixer": {}, "feed_forward": {}, "norm": {}, "position": {}}

@@ -10,11 +10,48 @@ from .base import LayerCache, Part, build_part
 from .specs import LayerSpec, ParamSpec
 
 
+def _parallel_few_rows(block: "Block", x, batch, cache) -> bool:
+    """The parallel block for a few bf16 rows in three launches: norm + both first linears, the
+    mixer's core, both last linears + residual. Needs a mixer and a feed-forward that offer their
+    stages (``input_projection`` / ``output_projection``); returns ``False`` otherwise."""
+    from ..ops import fast
+    from ..ops.linear import linear
+
+    n = x.shape[0]
+    if block.dtype != torch.bfloat16 or n > fast.SKINNY_MAX_ROWS:
+        return False
+    m_in, f_in = block.mixer.input_projection(), block.feed_forward.input_projection()
+    m_out, f_out = block.mixer.output_projection(), block.feed_forward.output_projection()
+    if m_in is None or f_in is None or m_out is None or f_out is None:
+        return False
+    ws = batch.workspace
+    projected = ws.get("block.mixer_in", (n, m_in[2]), block.dtype)
+    hidden = ws.get("block.ff_hidden", (n, f_in[2]), block.dtype)
+    norm = block.norm
+    fused = False
+    if fast.FUSE_LAYERNORM_PROLOGUE and getattr(norm.spec, "kind", None) == "layernorm":
+        fused = fast.layernorm_linear_pair(x, norm.weight, norm.bias, norm.spec.eps, m_in[0], m_in[1], projected, 0,
+                                           f_in[0], f_in[1], hidden, f_in[3])
+    if not fused:
+        h = ws.get("block.h", tuple(x.shape), block.dtype)
+        norm.forward(x, h)
+        if not fast.linear_two_outputs(h, m_in[0], m_in[1], projected, 0, f_in[0], f_in[1], hidden, f_in[3]):
+            linear(h, m_in[0], m_in[1], projected)
+            linear(h, f_in[0], f_in[1], hidden, act=f_in[3])
+    mixed = block.mixer.attend(projected, batch, cache)
+    if not fast.linear_pair_accumulate(mixed, m_out[0], m_out[1], hidden, f_out[0], f_out[1], x):
+        linear(mixed, m_out[0], m_out[1], x, accumulate=True)
+        linear(hidden, f_out[0], f_out[1], x, accumulate=True)
+    return True
+
+
 def _parallel(block: "Block", x, batch, cache) -> None:
     """``x + mixer(norm(x)) + ff(norm(x))``: both branches read the same normalised input.
 
     Reference: ``kestrel/models/moondream/text.py:222-275``.
     """
+    if _parallel_few_rows(block, x, batch, cache):
+        return
     h = batch.workspace.get("block.h", tuple(x.shape), block.dtype)
     block.norm.forward(x, h)
     block.mixer.forward(h, batch, cache, x)

@@ -40,6 +40,12 @@ class DenseFeedForward(FeedForward):
             self.fc1_bias = tensors["fc1.bias"].to(device=device, dtype=torch.float32).contiguous()
             self.fc2_bias = tensors["fc2.bias"].to(device=device, dtype=torch.float32).contiguous()
 
+    def input_projection(self):
+        return self.fc1_weight, self.fc1_bias, self.spec.hidden_dim, self.act
+
+    def output_projection(self):
+        return self.fc2_weight, self.fc2_bias
+
     def forward(self, h, batch, residual) -> None:
         hidden = batch.workspace.get("ff.hidden", (h.shape[0], self.spec.hidden_dim), self.dtype)
         linear(h, self.fc1_weight, self.fc1_bias, hidden, act=self.act)

@@ -359,3 +359,98 @@ def test_argmax_and_sampling():
                            [1.0, 1.0, 0.3, 0.95], [1, 2, 3, 42], [0, 5, 9, 7])[3].item()
     assert alone == mixed
     assert 0.0 <= core.uniform(mix_key(5, 42), 7) < 1.0
+
+
+@pytest.mark.parametrize("shape", [(8, 2048, 2048, 8192), (1, 40, 64, 200), (16, 2048, 2048, 8192), (33, 96, 120, 320),
+                                   (64, 256, 8, 72)])
+def test_two_segment_skinny_linear(shape):
+    """out += a1 w1^T + b1 + a2 w2^T + b2 in one launch."""
+    from kestrel_amd.ops import fast
+
+    m, n, k1, k2 = shape
+    torch.manual_seed(20)
+    a1, a2 = torch.randn(m, k1).bfloat16().to(DEV), torch.randn(m, k2).bfloat16().to(DEV)
+    w1 = (torch.randn(n, k1) / k1 ** 0.5).bfloat16().to(DEV)
+    w2 = (torch.randn(n, k2) / k2 ** 0.5).bfloat16().to(DEV)
+    b1, b2 = torch.randn(n).to(DEV), torch.randn(n).to(DEV)
+    start = torch.randn(m, n).to(DEV)
+    out = start.clone()
+    assert fast.linear_pair_accumulate(a1, w1, b1, a2, w2, b2, out)
+    ref = start.double() + a1.double() @ w1.double().T + b1.double() + a2.double() @ w2.double().T + b2.double()
+    _close(out, ref, torch.float32, scale=200)          # bf16 operands, fp32 sums
+    out2 = start.clone()
+    assert fast.linear_pair_accumulate(a1, w1, None, a2, w2, None, out2)
+    _close(out2, ref - b1.double() - b2.double(), torch.float32, scale=200)
+
+
+@pytest.mark.parametrize("shape", [(8, 2048, 6144, 8192), (1, 64, 40, 24), (16, 320, 100, 200), (5, 2048, 48, 8)])
+def test_layernorm_prologue_skinny_linear(shape):
+    """LayerNorm, then two linears from the normalised rows, in one launch."""
+    from kestrel_amd.ops import fast
+
+    m, k, na, nb = shape
+    torch.manual_seed(21)
+    x = (torch.randn(m, k) * 2 + 0.3).to(DEV)
+    gamma, beta = (1 + 0.1 * torch.randn(k)).to(DEV), (0.1 * torch.randn(k)).to(DEV)
+    wa = (torch.randn(na, k) / k ** 0.5).bfloat16().to(DEV)
+    wb = (torch.randn(nb, k) / k ** 0.5).bfloat16().to(DEV)
+    ba, bb = torch.randn(na).to(DEV), torch.randn(nb).to(DEV)
+    out_a = torch.empty(m, na, dtype=torch.bfloat16, device=DEV)
+    out_b = torch.empty(m, nb, dtype=torch.bfloat16, device=DEV)
+    assert fast.layernorm_linear_pair(x, gamma, beta, 1e-5, wa, ba, out_a, 0, wb, bb, out_b, 1)
+    h = F.layer_norm(x.double(), (k,), gamma.double(), beta.double(), 1e-5).to(torch.bfloat16).double()
+    _close(out_a, h @ wa.double().T + ba.double(), torch.bfloat16, scale=2)
+    _close(out_b, plain.gelu_tanh(h @ wb.double().T + bb.double()), torch.bfloat16, scale=2)
+    assert not fast.layernorm_linear_pair(torch.randn(17, k, device=DEV), gamma, beta, 1e-5, wa, ba,
+                                          torch.empty(17, na, dtype=torch.bfloat16, device=DEV), 0, wb, bb,
+                                          torch.empty(17, nb, dtype=torch.bfloat16, device=DEV), 1)
+
+
+@pytest.mark.parametrize("shape", [(4, 4, 64, 32), (6, 2, 128, 64), (8, 1, 64, 16)])
+def test_decode_attention_that_rotates_and_stores(shape):
+    """The decode kernel with rotary encoding and cache write fused in, against the rotary kernel
+    followed by the plain decode kernel: same outputs, same cache."""
+    from kestrel_amd.ops import core, fast
+
+    h, hkv, hd, rot = shape
+    bf = torch.bfloat16
+    kv_lens = [1, 16, 17, 300, 1024]
+    case = PagedCase(kv_lens, [1] * len(kv_lens), h, hkv, hd, 16, bf, seed=22)
+    n = len(kv_lens)
+    torch.manual_seed(23)
+    qkv = torch.randn(n, (h + 2 * hkv) * hd).to(bf).to(DEV)
+    positions = torch.tensor([kv - 1 for kv in kv_lens], dtype=torch.int32, device=DEV)
+    slots = torch.tensor([int(case.table[r, (kv - 1) // 16]) * 16 + (kv - 1) % 16 for r, kv in enumerate(kv_lens)],
+                         dtype=torch.int32, device=DEV)
+    table = plain.rotary_table(rot, 2048, 10000.0, torch.float32).to(DEV)
+    # reference path
+    qkv_ref, k_ref, v_ref = qkv.clone(), case.k_cache.clone(), case.v_cache.clone()
+    core.rope_cache(qkv_ref, positions, slots, table, k_ref, v_ref, h, hkv, hd, 16)
+    out_ref = torch.empty(n, h * hd, dtype=bf, device=DEV)
+    assert fast.attention_decode_bf16(qkv_ref, k_ref, v_ref, case.table, case.token_row, None, case.kv_hi, out_ref,
+                                      hd ** -0.5, h, hkv, hd, case.batch)
+    # fused path
+    k_f, v_f = case.k_cache.clone(), case.v_cache.clone()
+    out_f = torch.empty(n, h * hd, dtype=bf, device=DEV)
+    q_dim, kv_dim = h * hd, hkv * hd
+    assert fast.attention_decode_bf16(qkv, k_f, v_f, case.table, case.token_row, None, case.kv_hi, out_f, hd ** -0.5,
+                                      h, hkv, hd, case.batch,
+                                      fuse=(qkv[:, q_dim:q_dim + kv_dim], qkv[:, q_dim + kv_dim:], table, slots))
+    _close(out_f, out_ref, bf)
+    for r, kv in enumerate(kv_lens):
+        page, off = int(slots[r]) // 16, int(slots[r]) % 16
+        assert torch.equal(k_f[page, :, off, :], k_ref[page, :, off, :])
+        assert torch.equal(v_f[page, :, :, off], v_ref[page, :, :, off])
+
+
+def test_decode_attention_splits_long_rows(monkeypatch):
+    """Rows longer than a workgroup's share are cut into splits that meet through scratch memory."""
+    from kestrel_amd.ops import fast
+
+    monkeypatch.setattr(fast, "DECODE_KEYS_PER_WORKGROUP", 256)
+    h, hkv, hd = 4, 2, 64
+    bf = torch.bfloat16
+    case = PagedCase([1000, 3, 257, 700], [1, 1, 1, 1], h, hkv, hd, 16, bf, seed=24)
+    assert fast.decode_shape(case.batch.max_kv)[0] == 4
+    for _ in range(2):                                   # twice: the counters must be left at zero
+        _close(_run_attention(case, "fast", hd ** -0.5), case.reference(hd ** -0.5), bf)
