@@ -16,21 +16,25 @@ typedef __attribute__((ext_vector_type(16))) float floatx16;
 typedef __attribute__((ext_vector_type(4))) float floatx4;
 
 constexpr int GB_N = 128;          // weight rows per tile
-constexpr int GB_M = 128;          // activation rows per tile
 constexpr int GB_K = 64;           // k per step
 constexpr int GB_LD = GB_K + 8;    // padded LDS row (144 bytes)
 constexpr int GB_THREADS = 256;
-constexpr int GB_SMEM = 2 * (GB_N + GB_M) * GB_LD * 2;   // bytes of LDS: two buffers of both operand tiles
+// Activation rows per tile: 64 * MT. MT = 2 is the square tile; MT = 1 doubles the number of
+// workgroups where N x M alone would leave CUs idle (the N = dim products of a 2048-token prompt).
+constexpr int gb_m(int mt) { return 64 * mt; }
+constexpr int gb_smem(int mt) { return 2 * (GB_N + gb_m(mt)) * GB_LD * 2; }   // two buffers of both tiles
 
 __device__ __forceinline__ bf16x8 gb_load8(const bf16_t* p) { return *reinterpret_cast<const bf16x8*>(p); }
 
+template <int MT>
 __global__ void __launch_bounds__(GB_THREADS)
 gemm_bf16_kernel(const bf16_t* __restrict__ A, long lda, const bf16_t* __restrict__ W, long ldw,
                  const float* __restrict__ bias, void* __restrict__ out, int out_dtype, long ldo, int M,
                  int N, int K, int act, int accumulate, int tiles_n, int tiles_m) {
-    extern __shared__ __attribute__((aligned(16))) unsigned char gb_smem[];
-    bf16_t (*Ws)[GB_N][GB_LD] = reinterpret_cast<bf16_t (*)[GB_N][GB_LD]>(gb_smem);
-    bf16_t (*Xs)[GB_M][GB_LD] = reinterpret_cast<bf16_t (*)[GB_M][GB_LD]>(gb_smem + 2 * GB_N * GB_LD * sizeof(bf16_t));
+    extern __shared__ __attribute__((aligned(16))) unsigned char gb_lds[];
+    bf16_t (*Ws)[GB_N][GB_LD] = reinterpret_cast<bf16_t (*)[GB_N][GB_LD]>(gb_lds);
+    constexpr int GB_M = gb_m(MT);
+    bf16_t (*Xs)[GB_M][GB_LD] = reinterpret_cast<bf16_t (*)[GB_M][GB_LD]>(gb_lds + 2 * GB_N * GB_LD * sizeof(bf16_t));
     // Tiles are numbered so that the workgroups one XCD gets (every 8th) walk down a column of
     // tiles that share the same weight rows, which then stay in that XCD's L2.
     int pid = blockIdx.x;
@@ -39,30 +43,35 @@ gemm_bf16_kernel(const bf16_t* __restrict__ A, long lda, const bf16_t* __restric
     int logical = (pid % 8) * per_xcd + pid / 8;
     if (logical >= total) return;
     int tn = logical / tiles_m, tm = logical % tiles_m;
-    const int n0 = tn * GB_N, m0 = tm * GB_M;
+    const int n0 = tn * GB_N, m0 = tm * gb_m(MT);
     const int tid = threadIdx.x, wave = tid / KA_WAVE, lane = tid % KA_WAVE;
     const int wn = wave / 2, wm = wave % 2;
     const int li = lane % 32, lg = lane / 32;
 
-    floatx16 acc[2][2];
+    floatx16 acc[2][MT];
 #pragma unroll
     for (int a = 0; a < 2; ++a)
 #pragma unroll
-        for (int b = 0; b < 2; ++b)
+        for (int b = 0; b < MT; ++b)
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[a][b][v] = 0.f;
 
     const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
-    bf16x8 wreg[4], xreg[4];
+    bf16x8 wreg[4], xreg[2 * MT];
     // chunk c = tid + i * 256: row c / 8, k-chunk c % 8
     auto fetch = [&](int k0) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             int c = tid + i * GB_THREADS;
-            int row = c >> 3, kc = (c & 7) * 8;
-            int k = k0 + kc;
-            int n = n0 + row, m = m0 + row;
+            int row = c >> 3, k = k0 + (c & 7) * 8;
+            int n = n0 + row;
             wreg[i] = (n < N && k < K) ? gb_load8(W + (size_t)n * ldw + k) : zero;
+        }
+#pragma unroll
+        for (int i = 0; i < 2 * MT; ++i) {
+            int c = tid + i * GB_THREADS;
+            int row = c >> 3, k = k0 + (c & 7) * 8;
+            int m = m0 + row;
             xreg[i] = (m < M && k < K) ? gb_load8(A + (size_t)m * lda + k) : zero;
         }
     };
@@ -70,9 +79,12 @@ gemm_bf16_kernel(const bf16_t* __restrict__ A, long lda, const bf16_t* __restric
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             int c = tid + i * GB_THREADS;
-            int row = c >> 3, kc = (c & 7) * 8;
-            *reinterpret_cast<bf16x8*>(&Ws[buf][row][kc]) = wreg[i];
-            *reinterpret_cast<bf16x8*>(&Xs[buf][row][kc]) = xreg[i];
+            *reinterpret_cast<bf16x8*>(&Ws[buf][c >> 3][(c & 7) * 8]) = wreg[i];
+        }
+#pragma unroll
+        for (int i = 0; i < 2 * MT; ++i) {
+            int c = tid + i * GB_THREADS;
+            *reinterpret_cast<bf16x8*>(&Xs[buf][c >> 3][(c & 7) * 8]) = xreg[i];
         }
     };
 
@@ -85,27 +97,28 @@ gemm_bf16_kernel(const bf16_t* __restrict__ A, long lda, const bf16_t* __restric
         if (s + 1 < steps) fetch((s + 1) * GB_K);
 #pragma unroll
         for (int ks = 0; ks < GB_K / 16; ++ks) {
-            bf16x8 wa[2], xb[2];
+            bf16x8 wa[2], xb[MT];
 #pragma unroll
-            for (int t = 0; t < 2; ++t) {
+            for (int t = 0; t < 2; ++t)
                 wa[t] = *reinterpret_cast<const bf16x8*>(&Ws[buf][wn * 64 + t * 32 + li][ks * 16 + lg * 8]);
-                xb[t] = *reinterpret_cast<const bf16x8*>(&Xs[buf][wm * 64 + t * 32 + li][ks * 16 + lg * 8]);
-            }
+#pragma unroll
+            for (int t = 0; t < MT; ++t)
+                xb[t] = *reinterpret_cast<const bf16x8*>(&Xs[buf][wm * 32 * MT + t * 32 + li][ks * 16 + lg * 8]);
 #pragma unroll
             for (int a = 0; a < 2; ++a)
 #pragma unroll
-                for (int b = 0; b < 2; ++b)
+                for (int b = 0; b < MT; ++b)
                     acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wa[a], xb[b], acc[a][b], 0, 0, 0);
         }
         if (s + 1 < steps) stash(buf ^ 1);
         __syncthreads();
     }
 
-    // epilogue: acc[a][b][v] is out[m][n] with n = n0 + wn*64 + a*32 + (v/4)*8 + lg*4 + v%4, m = m0 + wm*64 + b*32 + li
+    // epilogue: acc[a][b][v] is out[m][n] with n = n0 + wn*64 + a*32 + (v/4)*8 + lg*4 + v%4, m = m0 + wm*32*MT + b*32 + li
     const bool vec_ok = (N % 4 == 0) && (ldo % 4 == 0);
 #pragma unroll
-    for (int b = 0; b < 2; ++b) {
-        int m = m0 + wm * 64 + b * 32 + li;
+    for (int b = 0; b < MT; ++b) {
+        int m = m0 + wm * 32 * MT + b * 32 + li;
         if (m >= M) continue;
 #pragma unroll
         for (int a = 0; a < 2; ++a) {
@@ -157,19 +170,30 @@ KA_API int ka_linear_tiled_bf16(const void* A, long lda, const void* W, long ldw
     KA_CHECK(!(accumulate && out_dtype != KA_F32), "ka_linear_tiled_bf16: accumulate needs an fp32 output");
     uintptr_t obase = (uintptr_t)out;
     KA_CHECK(obase % 16 == 0, "ka_linear_tiled_bf16: output must be 16-byte aligned");
-    int tiles_n = ka_cdiv(N, GB_N), tiles_m = ka_cdiv(M, GB_M);
+    int tiles_n = ka_cdiv(N, GB_N);
+    // the square tile unless it would leave fewer than two workgroups per CU
+    int mt = (long)tiles_n * ka_cdiv(M, gb_m(2)) < 512 ? 1 : 2;
+    int tiles_m = ka_cdiv(M, gb_m(mt));
     long total = (long)tiles_n * tiles_m;
     long launched = ((total + 7) / 8) * 8;
     KA_CHECK(launched < (1L << 31), "ka_linear_tiled_bf16: too many tiles");
     static bool configured = false;
     if (!configured) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_bf16_kernel),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, GB_SMEM);
-        KA_CHECK(e == hipSuccess, "ka_linear_tiled_bf16: cannot reserve %d bytes of LDS: %s", GB_SMEM, hipGetErrorString(e));
+        hipError_t e1 = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_bf16_kernel<1>),
+                                            hipFuncAttributeMaxDynamicSharedMemorySize, gb_smem(1));
+        hipError_t e2 = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_bf16_kernel<2>),
+                                            hipFuncAttributeMaxDynamicSharedMemorySize, gb_smem(2));
+        KA_CHECK(e1 == hipSuccess && e2 == hipSuccess, "ka_linear_tiled_bf16: cannot reserve %d bytes of LDS", gb_smem(2));
         configured = true;
     }
-    hipLaunchKernelGGL(gemm_bf16_kernel, dim3((unsigned)launched), dim3(GB_THREADS), GB_SMEM, stream, (const bf16_t*)A, lda,
-                       (const bf16_t*)W, ldw, bias, out, out_dtype, ldo, M, N, K, act, accumulate, tiles_n, tiles_m);
+    if (mt == 1)
+        hipLaunchKernelGGL(gemm_bf16_kernel<1>, dim3((unsigned)launched), dim3(GB_THREADS), gb_smem(1), stream,
+                           (const bf16_t*)A, lda, (const bf16_t*)W, ldw, bias, out, out_dtype, ldo, M, N, K, act,
+                           accumulate, tiles_n, tiles_m);
+    else
+        hipLaunchKernelGGL(gemm_bf16_kernel<2>, dim3((unsigned)launched), dim3(GB_THREADS), gb_smem(2), stream,
+                           (const bf16_t*)A, lda, (const bf16_t*)W, ldw, bias, out, out_dtype, ldo, M, N, K, act,
+                           accumulate, tiles_n, tiles_m);
     KA_LAUNCH_CHECK();
     return 0;
 }

@@ -183,8 +183,9 @@ skinny_kernel(SkinnyArgs p) {
                     if (k >= K) break;
 #pragma unroll
                     for (int mb = 0; mb < MB; ++mb) {
-                        bf16x8 xa = k + g * 8 < K ? sk_load8(ap[mb] + k) : zero;
-                        bf16x8 xb = k + 32 + g * 8 < K ? sk_load8(ap[mb] + k + 32) : zero;
+                        const bool row = mb * 16 + r < M;      // rows past M are not fetched at all
+                        bf16x8 xa = row && k + g * 8 < K ? sk_load8(ap[mb] + k) : zero;
+                        bf16x8 xb = row && k + 32 + g * 8 < K ? sk_load8(ap[mb] + k + 32) : zero;
                         lo[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[u], xa, lo[mb], 0, 0, 0);
                         hi[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[u], xb, hi[mb], 0, 0, 0);
                     }
