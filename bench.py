@@ -179,6 +179,7 @@ def main() -> int:
     parser.add_argument("--layers", type=int, default=MODEL["n_layers"], help="fewer layers than the model has (named in config)")
     parser.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     parser.add_argument("--skip-points", action="store_true", help="only the default batch (no batch 1 / 64, no prefill)")
+    parser.add_argument("--only-prefill", action="store_true", help="only the 2,048-token prefill (for profiling)")
     args = parser.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -195,6 +196,10 @@ def main() -> int:
     net, typed = build_model(args.layers, dtype, device)
     weights = model_bytes(net, size)
 
+    if args.only_prefill:
+        seconds = time_prefill(net, typed, PREFILL_TOKENS)
+        print(json.dumps({"prefill_ms": round(seconds * 1e3, 3), "tokens": PREFILL_TOKENS, "dtype": args.dtype}))
+        return 0
     elapsed, kv_bytes = time_decode(net, typed, args.batch, CONTEXT, args.steps, args.warmup)
     ms_per_step = elapsed / args.steps * 1e3
     value = args.batch * args.steps / elapsed
