@@ -4,15 +4,17 @@
 // page), page size 16. Every token t of the packed batch reads the keys [kv_lo[t], kv_hi[t]) of
 // its row through the row's block table; the step's own keys are already in the cache.
 //
-// Prompt kernel. A wave owns 32 consecutive queries of one row and one head and walks the keys
-// in tiles of 32 (two pages). Scores are computed transposed, S^T = K Q^T, with
+// Prompt kernel. A workgroup owns 32 consecutive queries of one row and one head; its four waves
+// take every fourth tile of 32 keys (two pages) each and merge at the end, which gives the
+// chip eight waves per SIMD to hide the latency of the cache reads behind; the next tile's keys
+// and the current tile's values are in flight while the current scores are computed. Scores are computed transposed, S^T = K Q^T, with
 // v_mfma_f32_32x32x16_bf16: the keys are the row operand (a lane loads half a key row straight
 // from the cache), the queries the column operand (held in registers for the whole loop). A
 // lane then holds, for ONE query, 16 scores: softmax needs only in-lane work and one exchange
 // with the lane 32 apart. The key rows are fed to the MFMA in a permuted order (bits 2 and 3 of
 // the row index swapped) so that the 8 probabilities a lane holds for a page are those of 8
 // consecutive keys: they are, as they stand, the column operand of O^T += V^T P^T, whose row
-// operand is one 16-byte load from the transposed value page. No LDS, no barriers.
+// operand is one 16-byte load from the transposed value page. LDS is used for the merge only.
 //
 // Decode kernel. One query per row: a bandwidth problem. The keys of a row are cut into splits
 // (grid z) and 64-key tiles (waves); 16-byte loads are fully coalesced for keys (8 lanes per key
@@ -26,6 +28,7 @@ typedef __attribute__((ext_vector_type(16))) float floatx16;
 typedef __attribute__((ext_vector_type(4))) float floatx4;
 
 constexpr int AT_PAGE = 16;
+constexpr int AT_LDS_PAGES = 2048;        // block table entries of one row kept in LDS (32k keys)
 constexpr float AT_LOG2E = 1.4426950408889634f;
 
 __device__ __forceinline__ bf16x8 at_load8(const bf16_t* p) { return *reinterpret_cast<const bf16x8*>(p); }
@@ -40,8 +43,8 @@ __device__ __forceinline__ void at_wave_sync() {
 // ----------------------------------------------------------------------------------------------
 // prompt kernel
 // ----------------------------------------------------------------------------------------------
-constexpr int AP_WAVES = 4;
-constexpr int AP_QBLOCK = 32 * AP_WAVES;    // queries per workgroup
+constexpr int AP_WAVES = 4;                 // waves of a workgroup: all on the same 32 queries, keys interleaved
+constexpr int AP_QBLOCK = 32;               // queries per workgroup
 
 template <int HD>
 __global__ void __launch_bounds__(KA_WAVE * AP_WAVES)
@@ -53,15 +56,16 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_
                     long out_row_stride, float scale, int H, int Hkv) {
     constexpr int QC = HD / 16;          // 16-byte chunks of half a head row = MFMA steps of the score product
     constexpr int DB = HD / 32;          // 32-channel blocks of the output
+    constexpr int REC = DB * 16 + 2;     // floats a lane hands over at the merge: its outputs, m and l
+    __shared__ float mrg[AP_WAVES - 1][REC][KA_WAVE];
+    __shared__ int pages[AT_LDS_PAGES];
     const int blk = blockIdx.x, h = blockIdx.y;
     const int wave = threadIdx.x / KA_WAVE, lane = threadIdx.x % KA_WAVE;
     const int li = lane % 32, lg = lane / 32;
     const int kvh = h / (H / Hkv);
     const int row = qblk_row[blk];
     const int tok_end = cu_q[row + 1];
-    const int tok0 = qblk_tok[blk] + wave * 32;
-    if (tok0 >= tok_end) return;
-    const int t = tok0 + li;
+    const int t = qblk_tok[blk] + li;
     const bool q_valid = t < tok_end;
     const int tq = q_valid ? t : tok_end - 1;
     const int hi = q_valid ? kv_hi[tq] : 0;
@@ -74,7 +78,15 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_
     }
     const int limit = kv_len[row];       // keys of this row that hold data
     wave_hi = min(wave_hi, limit);
+    // The row's block table goes to LDS once: a look-up per tile in global memory would put a
+    // second trip to memory in front of every load of keys and values.
     const int* bt = block_table + (size_t)row * max_pages;
+    const int n_pages = (limit + AT_PAGE - 1) / AT_PAGE;
+    if (n_pages <= AT_LDS_PAGES) {
+        for (int i = threadIdx.x; i < n_pages; i += KA_WAVE * AP_WAVES) pages[i] = bt[i];
+        __syncthreads();
+        bt = pages;
+    }
 
     // queries: lane (q = li, g = lg) holds channels [g * HD/2, (g + 1) * HD/2)
     bf16x8 qreg[QC];
@@ -91,71 +103,146 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_
     float m_i = -INFINITY, l_i = 0.f;
     const float sl2 = scale * AT_LOG2E;
     const int kperm = (li & 16) | ((li & 4) << 1) | ((li & 8) >> 1) | (li & 3);
-    const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
 
-    for (int key0 = wave_lo & ~31; key0 < wave_hi; key0 += 32) {
-        // scores S^T[key][query]
+    // half a key row of tile `key0` for this lane's (permuted) key
+    auto load_keys = [&](int key0, bf16x8* dst) {
+        int key = max(min(key0 + kperm, limit - 1), wave_lo);   // pages below wave_lo may have been given back
+        int page = bt[key / AT_PAGE];
+        const bf16_t* kp = k_cache + (((size_t)page * Hkv + kvh) * AT_PAGE + key % AT_PAGE) * HD + lg * (HD / 2);
+#pragma unroll
+        for (int c = 0; c < QC; ++c) dst[c] = at_load8(kp + c * 8);
+    };
+
+    // the two value pages of tile `key0`: lane (d = li, g) loads 8 consecutive keys of channel d.
+    // `tail`: the tile reaches past the row's data, whose slots may hold anything: keep them out.
+    auto load_values = [&](int key0, bool tail, bf16x8 (*dst)[DB]) {
+#pragma unroll
+        for (int pg = 0; pg < 2; ++pg) {
+            int kbase = key0 + pg * AT_PAGE;
+            bool live = kbase < wave_hi && kbase + AT_PAGE > wave_lo;
+            int page = live ? bt[kbase / AT_PAGE] : 0;
+            const bf16_t* vp = v_cache + (((size_t)page * Hkv + kvh) * HD + li) * AT_PAGE + lg * 8;
+#pragma unroll
+            for (int db = 0; db < DB; ++db) {
+                bf16x8 vv = {0, 0, 0, 0, 0, 0, 0, 0};
+                if (live) vv = at_load8(vp + db * 32 * AT_PAGE);
+                dst[pg][db] = vv;
+            }
+            if (tail) {
+                int first = kbase + lg * 8;      // first of the 8 keys this lane loads
+#pragma unroll
+                for (int db = 0; db < DB; ++db)
+#pragma unroll
+                    for (int j = 0; j < 8; ++j)
+                        if (first + j >= limit) dst[pg][db][j] = (bf16_t)0.f;
+            }
+        }
+    };
+
+    // lowest end and highest start of the visible ranges of the wave's queries: a tile inside
+    // [max_lo, min_hi) is seen whole by every query and needs no mask
+    int min_hi = q_valid ? hi : 0, max_lo = q_valid ? lo : 0x7fffffff;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+        min_hi = min(min_hi, __shfl_xor(min_hi, off, KA_WAVE));
+        max_lo = max(max_lo, __shfl_xor(max_lo, off, KA_WAVE));
+    }
+
+    // one tile of 32 keys whose key rows are in `kr`
+    auto process = [&](int key0, const bf16x8* kr) {
+        bf16x8 vr[2][DB];
+        load_values(key0, key0 + 32 > limit, vr);          // in flight during the scores and the softmax
         floatx16 s;
 #pragma unroll
         for (int v = 0; v < 16; ++v) s[v] = 0.f;
-        {
-            int key = max(min(key0 + kperm, limit - 1), wave_lo);   // pages below wave_lo may have been given back
-            int page = bt[key / AT_PAGE];
-            const bf16_t* kp = k_cache + (((size_t)page * Hkv + kvh) * AT_PAGE + key % AT_PAGE) * HD + lg * (HD / 2);
 #pragma unroll
-            for (int c = 0; c < QC; ++c) s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(at_load8(kp + c * 8), qreg[c], s, 0, 0, 0);
-        }
+        for (int c = 0; c < QC; ++c) s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kr[c], qreg[c], s, 0, 0, 0);
         // lane holds, for its query, the keys key0 + (v / 8) * 16 + lg * 8 + v % 8
-        float mx = -INFINITY;
+        if (!(key0 >= max_lo && key0 + 32 <= min_hi)) {
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-            int key = key0 + (v / 8) * 16 + lg * 8 + (v % 8);
-            bool ok = key >= lo && key < hi;
-            s[v] = ok ? s[v] * sl2 : -INFINITY;
-            mx = fmaxf(mx, s[v]);
+            for (int v = 0; v < 16; ++v) {
+                int key = key0 + (v / 8) * 16 + lg * 8 + (v % 8);
+                if (!(key >= lo && key < hi)) s[v] = -INFINITY;
+            }
         }
-        mx = fmaxf(mx, __shfl_xor(mx, 32, KA_WAVE));
+        float mx = s[0];
+#pragma unroll
+        for (int v = 1; v < 16; ++v) mx = fmaxf(mx, s[v]);
+        mx = fmaxf(mx, __shfl_xor(mx, 32, KA_WAVE)) * sl2;   // the scale is positive: max and scale commute
         float m_new = fmaxf(m_i, mx);
         float m_use = m_new == -INFINITY ? 0.f : m_new;     // nothing visible yet: keep everything at zero
-        float alpha = exp2f(m_i - m_use);
+        float alpha = __builtin_amdgcn_exp2f(m_i - m_use);
         float rowsum = 0.f;
         bf16x8 pb[2];
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
-            float p = exp2f(s[v] - m_use);
+            float p = __builtin_amdgcn_exp2f(fmaf(s[v], sl2, -m_use));
             rowsum += p;
             pb[v / 8][v % 8] = (bf16_t)p;
         }
         rowsum += __shfl_xor(rowsum, 32, KA_WAVE);
         l_i = l_i * alpha + rowsum;
         m_i = m_new;
+        if (__any(alpha != 1.0f)) {
+#pragma unroll
+            for (int db = 0; db < DB; ++db)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) o[db][v] *= alpha;
+        }
+        // O^T[d][query] += V^T[d][key] P^T[key][query], one page per MFMA
+#pragma unroll
+        for (int pg = 0; pg < 2; ++pg)
+#pragma unroll
+            for (int db = 0; db < DB; ++db)
+                o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vr[pg][db], pb[pg], o[db], 0, 0, 0);
+    };
+
+    // two tiles per round, their key rows in two sets of registers: the next tile's keys are
+    // always in flight while a tile is processed
+    constexpr int STRIDE = 32 * AP_WAVES;
+    bf16x8 ka[QC], kb[QC];
+    int key0 = (wave_lo & ~31) + wave * 32;
+    if (key0 < wave_hi) load_keys(key0, ka);
+    while (key0 < wave_hi) {
+        if (key0 + STRIDE < wave_hi) load_keys(key0 + STRIDE, kb);
+        process(key0, ka);
+        key0 += STRIDE;
+        if (key0 >= wave_hi) break;
+        if (key0 + STRIDE < wave_hi) load_keys(key0 + STRIDE, ka);
+        process(key0, kb);
+        key0 += STRIDE;
+    }
+    // the waves took different keys of the same queries: merge in wave order
+    if (wave > 0) {
 #pragma unroll
         for (int db = 0; db < DB; ++db)
 #pragma unroll
-            for (int v = 0; v < 16; ++v) o[db][v] *= alpha;
-        // O^T[d][query] += V^T[d][key] P^T[key][query], one page per MFMA
-#pragma unroll
-        for (int pg = 0; pg < 2; ++pg) {
-            int kbase = key0 + pg * AT_PAGE;
-            if (kbase >= wave_hi) break;
-            if (kbase + AT_PAGE <= wave_lo) continue;   // nothing visible here, and the page may be gone
-            int page = bt[kbase / AT_PAGE];
-            int first = kbase + lg * 8;          // first of the 8 keys this lane loads
-#pragma unroll
-            for (int db = 0; db < DB; ++db) {
-                const bf16_t* vp = v_cache + (((size_t)page * Hkv + kvh) * HD + db * 32 + li) * AT_PAGE + lg * 8;
-                bf16x8 vv = at_load8(vp);
-                if (first + 8 > limit) {         // slots past the row's data may hold anything: keep them out
-#pragma unroll
-                    for (int j = 0; j < 8; ++j)
-                        if (first + j >= limit) vv[j] = (bf16_t)0.f;
-                }
-                o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vv, pb[pg], o[db], 0, 0, 0);
-            }
-        }
+            for (int v = 0; v < 16; ++v) mrg[wave - 1][db * 16 + v][lane] = o[db][v];
+        mrg[wave - 1][DB * 16][lane] = m_i;
+        mrg[wave - 1][DB * 16 + 1][lane] = l_i;
     }
-    if (!q_valid) return;
-    float inv = l_i > 0.f ? 1.0f / l_i : 0.f;
+    __syncthreads();
+    if (wave > 0 || !q_valid) return;
+    float M = m_i;
+#pragma unroll
+    for (int w = 0; w < AP_WAVES - 1; ++w) M = fmaxf(M, mrg[w][DB * 16][lane]);
+    float f0 = m_i == -INFINITY ? 0.f : exp2f(m_i - M);
+    float L = l_i * f0;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) o[db][v] *= f0;
+#pragma unroll
+    for (int w = 0; w < AP_WAVES - 1; ++w) {
+        float mw = mrg[w][DB * 16][lane];
+        float f = mw == -INFINITY ? 0.f : exp2f(mw - M);
+        L += mrg[w][DB * 16 + 1][lane] * f;
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) o[db][v] += mrg[w][db * 16 + v][lane] * f;
+    }
+    float inv = L > 0.f ? 1.0f / L : 0.f;
     bf16_t* op = out + (size_t)t * out_row_stride + (size_t)h * HD;
 #pragma unroll
     for (int db = 0; db < DB; ++db)
@@ -220,6 +307,7 @@ attn_decode_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t
     constexpr int REC = HD + 2;            // floats of a partial result: m, l, o[HD]
     __shared__ float ps[WAVES][AD_TILE];
     __shared__ float merge[WAVES][REC];
+    __shared__ int pages[AT_LDS_PAGES];
     const int t = blockIdx.x, h = blockIdx.y, split = blockIdx.z, S = gridDim.z;
     const int wave = threadIdx.x / KA_WAVE, lane = threadIdx.x % KA_WAVE;
     const int kvh = h / (H / Hkv);
@@ -232,6 +320,14 @@ attn_decode_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t
     const int chunk = ((hi - lo_tile + S - 1) / S + AD_TILE - 1) / AD_TILE * AD_TILE;
     const int s_lo = lo_tile + split * chunk, s_hi = min(hi, s_lo + chunk);
     const int* bt = block_table + (size_t)row * max_pages;
+    {   // the row's block table goes to LDS once (see the prompt kernel)
+        const int n_pages = (max(hi, 0) + AT_PAGE - 1) / AT_PAGE;
+        if (n_pages <= AT_LDS_PAGES) {
+            for (int i = threadIdx.x; i < n_pages; i += KA_WAVE * WAVES) pages[i] = bt[i];
+            __syncthreads();
+            bt = pages;
+        }
+    }
     const int ks = lane / LPK, dg = lane % LPK;
     const float sl2 = scale * AT_LOG2E;
     float qf[8];

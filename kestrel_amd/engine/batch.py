@@ -72,7 +72,7 @@ class StepBatch:
     logit_rows: torch.Tensor            # int32 [wanted]
     groups: Dict[int, GroupBatch]
     workspace: Workspace
-    qblk_row: Optional[torch.Tensor] = None       # int32 [blocks]: row of each block of 128 queries
+    qblk_row: Optional[torch.Tensor] = None       # int32 [blocks]: row of each block of 32 queries
     qblk_tok: Optional[torch.Tensor] = None       # int32 [blocks]: its first token
     given_embeds: Optional[torch.Tensor] = None   # [m, dim]
     given_rows: Optional[torch.Tensor] = None     # int32 [m] token indices they go to

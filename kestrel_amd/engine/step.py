@@ -73,7 +73,7 @@ class ModelRunner:
     """Owns the model, its cache and the scratch memory; ``step`` is the only way in."""
 
     STAGING_RING = 4
-    QUERY_BLOCK = 128        # queries of one row a workgroup of the prompt attention kernel takes
+    QUERY_BLOCK = 32         # queries of one row a workgroup of the prompt attention kernel takes
 
     def __init__(self, model: DecoderModel, cache: CacheManager, device: torch.device,
                  max_tokens_per_step: int = 4096, enable_graphs: bool = False,

@@ -19,13 +19,21 @@ TINY_B = {"text": {"dim": 96, "ff_dim": 320, "n_layers": 3, "vocab_size": 1000, 
 TINY_C = {"text": {"dim": 120, "ff_dim": 200, "n_layers": 2, "vocab_size": 777, "max_context": 320, "n_heads": 6,
                    "n_kv_heads": 2, "head_dim": 48, "rotary_dim": 12, "rope_theta": 1234.5, "prefix_attn": 5,
                    "layer_norm_eps": 3e-5}}
+# Head sizes the MFMA kernels take (64 with one shared kv head, 128 with as many kv heads as heads),
+# widths that are no multiple of 64: what serving runs, at toy size.
+TINY_D = {"text": {"dim": 128, "ff_dim": 136, "n_layers": 2, "vocab_size": 300, "max_context": 256, "n_heads": 2,
+                   "n_kv_heads": 1, "rope_theta": 10000.0, "prefix_attn": 9, "layer_norm_eps": 1e-5}}
+TINY_E = {"text": {"dim": 256, "ff_dim": 264, "n_layers": 2, "vocab_size": 411, "max_context": 192, "n_heads": 2,
+                   "n_kv_heads": 2, "rope_theta": 2500.0, "rotary_dim": 32, "prefix_attn": 6, "layer_norm_eps": 2e-6}}
 RECIPES = {
     "A": InitRecipe(std=0.02),
     "B": InitRecipe(std=0.03, gain_std=0.02, shift_std=0.02),
     "C": InitRecipe(std=0.05, bias_std=0.1, gain_std=0.1, shift_std=0.05),
+    "D": InitRecipe(std=0.04, gain_std=0.05, shift_std=0.05),
+    "E": InitRecipe(std=0.03, bias_std=0.05, gain_std=0.05, shift_std=0.02),
 }
-CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C}
-SEEDS = {"A": 0, "B": 1, "C": 2}
+CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D, "E": TINY_E}
+SEEDS = {"A": 0, "B": 1, "C": 2, "D": 3, "E": 4}
 
 
 @functools.lru_cache(maxsize=None)

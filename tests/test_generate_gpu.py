@@ -34,7 +34,7 @@ def _assert_greedy(result_tokens, expected, margins, slack, what):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B"])
+@pytest.mark.parametrize("name", ["A", "B", "D"])
 def test_greedy_generation_matches_the_plain_implementation(name, dtype):
     """Requests of different lengths submitted together: prompts are cut into portions of 48
     tokens beside the decoding of the others; with and without HIP graphs."""

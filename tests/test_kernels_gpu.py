@@ -222,7 +222,7 @@ class PagedCase:
         self.q = torch.randn(n, h * hd, generator=gen).to(dtype)
         qblk_row, qblk_tok = [], []
         for r in range(n_rows):
-            for first in range(cu_q[r], cu_q[r + 1], 128):
+            for first in range(cu_q[r], cu_q[r + 1], 32):
                 qblk_row.append(r)
                 qblk_tok.append(first)
         i32 = lambda xs: torch.tensor(xs, dtype=torch.int32, device=DEV)
