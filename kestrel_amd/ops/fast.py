@@ -27,7 +27,7 @@ _SIGNATURES = {
         _c_void_p, _c_long, _c_void_p, _c_void_p, _c_int, _c_long, _c_int, _c_int,           # target b
         _c_int, _c_int, _c_void_p],                                   # M, target_waves, stream
     "ka_linear_tiled_bf16": [_c_void_p, _c_long, _c_void_p, _c_long, _c_void_p, _c_void_p, _c_int, _c_long, _c_int,
-                             _c_int, _c_int, _c_int, _c_int, _c_void_p],
+                             _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
     "ka_attention_prefill_bf16": [_c_void_p, _c_long, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p,
                                   _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_long, _c_float,
                                   _c_int, _c_int, _c_int, _c_int, _c_void_p],
@@ -46,6 +46,8 @@ SKINNY_LN_MAX_WIDTH = 2048
 # Whether blocks let the weight-streaming kernel normalise its input itself. Every workgroup then
 # repeats the LayerNorm of all rows; measured on MI355X this costs more than the launch it saves.
 FUSE_LAYERNORM_PROLOGUE = False
+# Tile of the tiled kernel: 0 lets it choose by size; 421, 221, 211 force one (for measurements).
+TILED_CONFIG = 0
 # Waves the weight-streaming kernel aims to have on the chip (256 CUs, 16 to 32 waves each).
 SKINNY_TARGET_WAVES = 6144
 SCRATCH_FLOATS = 8 << 20
@@ -124,7 +126,7 @@ def linear_bf16(a, weight, bias, out, act, accumulate) -> bool:
     else:
         _check(handle.ka_linear_tiled_bf16(a.data_ptr(), a.stride(0), weight.data_ptr(), weight.stride(0), _ptr(bias),
                                            out.data_ptr(), _OUT_CODE[out.dtype], out.stride(0), m, n, k, act,
-                                           int(accumulate), stream_ptr()))
+                                           int(accumulate), TILED_CONFIG, stream_ptr()))
     return True
 
 
