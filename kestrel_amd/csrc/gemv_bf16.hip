@@ -30,10 +30,14 @@ constexpr int SK_KBLOCK = 64;      // k per wave and step
 constexpr int SK_LN_ROWS = 16;     // most rows the LayerNorm prologue takes
 constexpr int SK_PREFETCH = 4;     // weight blocks a wave loads before the LayerNorm prologue
 constexpr int SK_XV = 8;           // float4 per lane of a row kept in registers (rows up to 2048 wide)
-constexpr int SK_UNROLL = 4;       // k-blocks whose weight loads go out together
 constexpr int SK_PAD = 8;          // bf16 of padding per LDS row (keeps 16-byte reads off each other's banks)
 
 __device__ __forceinline__ bf16x8 sk_load8(const bf16_t* p) { return *reinterpret_cast<const bf16x8*>(p); }
+// Weights are read once and never again: a load that does not displace the activations,
+// which every workgroup of a CU reads, from the caches.
+__device__ __forceinline__ bf16x8 sk_load8_stream(const bf16_t* p) {
+    return __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(p));
+}
 
 struct SkinnyTarget {       // one weight matrix and where its product goes
     const bf16_t* W;
@@ -85,6 +89,28 @@ skinny_kernel(SkinnyArgs p) {
         hi[mb] = floatx4{0.f, 0.f, 0.f, 0.f};
     }
     const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+    // What the 32 finishing lanes add at the end (bias, and the output's old value when the
+    // product is accumulated) is fetched now: its latency hides behind the weight stream.
+    floatx4 addend[MB];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) addend[mb] = floatx4{0.f, 0.f, 0.f, 0.f};
+    if (wave == 0 && lane < 32) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            int n = n0 + g * 4 + i;
+            if (n >= N) continue;
+            float b = tg.bias ? tg.bias[n] : 0.f;
+            if (!second && p.bias2) b += p.bias2[n];
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb) {
+                int m = mb * 16 + r;
+                float old = 0.f;
+                if (tg.accumulate && m < M) old = reinterpret_cast<const float*>(tg.out)[(size_t)m * tg.ldo + n];
+                addend[mb][i] = b;
+                if (tg.accumulate) lo[mb][i] = old;     // wave 0's own sum starts from the old value
+            }
+        }
+    }
 
     if constexpr (LN) {
         // Weight loads of this wave's first blocks go out first: they do not depend on the rows,
@@ -95,12 +121,20 @@ skinny_kernel(SkinnyArgs p) {
 #pragma unroll
         for (int j = 0; j < SK_PREFETCH; ++j) {
             int k = (wave + j * WAVES) * SK_KBLOCK;
-            wpre[j] = k + koff < K ? sk_load8(wp + k) : zero;
+            wpre[j] = k + koff < K ? sk_load8_stream(wp + k) : zero;
         }
-        // normalise rows w, w + WAVES, ... of x into LDS: [M][K + pad] bf16
+        // the rows go to LDS as [M][K + pad] bf16: copied as they are, or normalised on the way
+        // (rows w, w + WAVES, ... by wave w)
         bf16_t* xs = reinterpret_cast<bf16_t*>(sk_dyn);
         const int ld = K + SK_PAD;
-        for (int m = wave; m < M; m += WAVES) {
+        if (p.ln_x == nullptr) {
+            const int cpr = K / 8;
+            for (int c = threadIdx.x; c < M * cpr; c += WAVES * KA_WAVE) {
+                int m = c / cpr, kc = (c % cpr) * 8;
+                *reinterpret_cast<bf16x8*>(xs + m * ld + kc) = sk_load8(p.A[0] + (size_t)m * p.lda[0] + kc);
+            }
+        }
+        for (int m = wave; m < M && p.ln_x != nullptr; m += WAVES) {
             const float* src = p.ln_x + (size_t)m * K;
             {
                 // the row stays in registers (K <= SK_XV * 256, checked by the host): one trip to memory
@@ -168,26 +202,33 @@ skinny_kernel(SkinnyArgs p) {
             const bf16_t* ap[MB];
 #pragma unroll
             for (int mb = 0; mb < MB; ++mb) ap[mb] = p.A[seg] + (size_t)min(mb * 16 + r, M - 1) * p.lda[seg] + g * 8;
-            // K is a multiple of 8: a lane's 8 values are all inside or all outside. Four blocks
-            // at a time, all their weight loads first: more bytes in flight per wave.
-            for (int k0 = wave * SK_KBLOCK; k0 < K; k0 += SK_UNROLL * WAVES * SK_KBLOCK) {
-                bf16x8 w[SK_UNROLL];
+            // K is a multiple of 8: a lane's 8 values are all inside or all outside. UN blocks at a
+            // time, and ALL their loads (weights and activations) before the first MFMA: an
+            // activation load issued between MFMAs puts a trip to L2 on the critical path per block.
+            constexpr int UN = MB == 1 ? 4 : MB == 2 ? 2 : 1;
+            for (int k0 = wave * SK_KBLOCK; k0 < K; k0 += UN * WAVES * SK_KBLOCK) {
+                bf16x8 w[UN], xa[UN][MB], xb[UN][MB];
 #pragma unroll
-                for (int u = 0; u < SK_UNROLL; ++u) {
+                for (int u = 0; u < UN; ++u) {
                     int k = k0 + u * WAVES * SK_KBLOCK;
-                    w[u] = k + koff < K ? sk_load8(wp + k) : zero;
+                    w[u] = k + koff < K ? sk_load8_stream(wp + k) : zero;
                 }
 #pragma unroll
-                for (int u = 0; u < SK_UNROLL; ++u) {
+                for (int u = 0; u < UN; ++u) {
                     int k = k0 + u * WAVES * SK_KBLOCK;
-                    if (k >= K) break;
 #pragma unroll
                     for (int mb = 0; mb < MB; ++mb) {
                         const bool row = mb * 16 + r < M;      // rows past M are not fetched at all
-                        bf16x8 xa = row && k + g * 8 < K ? sk_load8(ap[mb] + k) : zero;
-                        bf16x8 xb = row && k + 32 + g * 8 < K ? sk_load8(ap[mb] + k + 32) : zero;
-                        lo[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[u], xa, lo[mb], 0, 0, 0);
-                        hi[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[u], xb, hi[mb], 0, 0, 0);
+                        xa[u][mb] = row && k + g * 8 < K ? sk_load8(ap[mb] + k) : zero;
+                        xb[u][mb] = row && k + 32 + g * 8 < K ? sk_load8(ap[mb] + k + 32) : zero;
+                    }
+                }
+#pragma unroll
+                for (int u = 0; u < UN; ++u) {
+#pragma unroll
+                    for (int mb = 0; mb < MB; ++mb) {
+                        lo[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[u], xa[u][mb], lo[mb], 0, 0, 0);
+                        hi[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[u], xb[u][mb], hi[mb], 0, 0, 0);
                     }
                 }
             }
@@ -211,13 +252,11 @@ skinny_kernel(SkinnyArgs p) {
         for (int i = 0; i < 4; ++i) {
             int n = n0 + g * 4 + i;
             if (n >= N) continue;
-            float v = s[i] + (tg.bias ? tg.bias[n] : 0.f);
-            if (!second && p.bias2) v += p.bias2[n];
+            float v = s[i] + addend[mb][i];
             if (tg.act == 1) v = ka_gelu_tanh(v);
             size_t o = (size_t)m * tg.ldo + n;
             if (tg.out_dtype == KA_F32) {
-                float* op = reinterpret_cast<float*>(tg.out);
-                op[o] = tg.accumulate ? op[o] + v : v;
+                reinterpret_cast<float*>(tg.out)[o] = v;       // an accumulated product already holds the old value
             } else {
                 reinterpret_cast<bf16_t*>(tg.out)[o] = (bf16_t)v;
             }
@@ -307,9 +346,12 @@ KA_API int ka_linear_skinny_fused(const void* A1, long lda1, int K1, const void*
     if (waves > kblocks) waves = kblocks;
     if (MB > 2 && waves > 8) waves = 8;       // LDS of the final sum grows with MB
     int rc;
-    if (ln) {
-        waves = 8;                            // one or two rows per wave keep the prologue short
-        size_t dyn = (size_t)M * (K1 + SK_PAD) * sizeof(bf16_t);
+    // Staging plain rows in LDS (the copy path of the kernel) is measured slower than fetching
+    // them block by block, so only the LayerNorm prologue goes through LDS.
+    size_t dyn = (size_t)M * (K1 + SK_PAD) * sizeof(bf16_t);
+    const bool staged = ln;
+    if (staged) {
+        if (ln || waves < 4) waves = ln ? 8 : 4;     // one or two rows per wave keep a LayerNorm prologue short
         KA_CHECK(dyn <= 96 * 1024, "%s: %d rows of %d do not fit in LDS", who, M, K1);
         rc = launch_mb<1, true>(waves, strips, dyn, stream, args);
     } else {
