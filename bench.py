@@ -84,15 +84,18 @@ class DecodeBench:
         import torch
 
         from kestrel_amd.engine.loading import make_runner
-        from kestrel_amd.engine.step import StepEntry
+        from kestrel_amd.engine.step import PENDING_TOKEN, StepEntry
         from kestrel_amd.sampling import Sampler
 
-        self.torch, self.StepEntry = torch, StepEntry
+        self.torch, self.StepEntry, self.PENDING = torch, StepEntry, PENDING_TOKEN
         self.net, self.typed, self.batch, self.context = net, typed, batch, context
         pages_per_request = -(-(context + steps_total + 1) // PAGE_SIZE)
         self.runner = make_runner(net, PAGE_SIZE, batch * pages_per_request, batch, max_tokens_per_step=4096,
                                   enable_graphs=True)
-        self.sampler = Sampler(net.device)
+        self.sampler = Sampler(net.device, pending=self.runner.pending)
+        self.host = [torch.empty(batch, dtype=torch.int32, pin_memory=True) for _ in range(2)]
+        self.unread = None                      # (event, pinned tokens) of the step launched last
+        self.n_steps = 0
         gen = torch.Generator().manual_seed(SEED)
         prefix = min(typed.prefix_attn, context - 1)
         self.slots = []
@@ -104,14 +107,27 @@ class DecodeBench:
             entry = StepEntry(slot, [-1] * prefix + ids, want=[context - 1], embeds=embeds.to(net.device),
                               bidirectional=[(0, prefix)] if prefix else [])
             logits = self.runner.step([entry])
-            last.append(int(self.sampler.greedy(logits)[0]))
+            last.append(int(self.sampler.greedy(logits, slots=[slot])[0]))
             self.slots.append(slot)
         self.last = last
 
     def step(self):
-        entries = [self.StepEntry(slot, [tok], want=[0]) for slot, tok in zip(self.slots, self.last)]
+        """One decode step as the scheduler runs it with two steps in flight: the next step is
+        launched with the tokens that sampling left on the device, then the tokens of the step
+        before are read on the host."""
+        torch = self.torch
+        entries = [self.StepEntry(slot, [self.PENDING], want=[0]) for slot in self.slots]
         logits = self.runner.step(entries)
-        self.last = self.sampler.greedy(logits).tolist()
+        ids = self.sampler.greedy(logits, slots=self.slots)
+        host = self.host[self.n_steps % 2]
+        host.copy_(ids, non_blocking=True)
+        event = torch.cuda.Event()
+        event.record()
+        if self.unread is not None:
+            self.unread[0].synchronize()
+            self.last = self.unread[1].tolist()
+        self.unread = (event, host)
+        self.n_steps += 1
 
     def kv_bytes_now(self, dtype_size: int) -> int:
         t = self.typed

@@ -26,6 +26,8 @@ def _add_runtime_options(parser: argparse.ArgumentParser) -> None:
     parser.add_argument("--max-num-batched-tokens", type=int, default=2048)
     parser.add_argument("--seed", type=int, default=0)
     parser.add_argument("--disable-graphs", action="store_true", help="do not replay decode steps as HIP graphs")
+    parser.add_argument("--pipeline-depth", type=int, default=2, choices=(1, 2),
+                        help="2: launch a step before the previous step's tokens have reached the host")
 
 
 def _parse_ids(text: str) -> List[int]:
@@ -48,7 +50,7 @@ def _generate(args) -> int:
     cfg = RuntimeConfig(model_path=args.model_path, model=args.model, device=args.device, dtype=args.dtype,
                         max_batch_size=args.max_batch_size, page_size=args.page_size,
                         kv_cache_pages=args.kv_cache_pages, max_num_batched_tokens=args.max_num_batched_tokens,
-                        seed=args.seed, enable_graphs=not args.disable_graphs)
+                        seed=args.seed, enable_graphs=not args.disable_graphs, pipeline_depth=args.pipeline_depth)
     engine = InferenceEngine.create_sync(cfg)
     try:
         if args.random_prompts:

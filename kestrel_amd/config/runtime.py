@@ -38,6 +38,8 @@ class RuntimeConfig:
     ``kv_cache_tokens`` or, failing that, for ``max_batch_size`` full contexts.
     ``max_num_batched_tokens``: token budget of one step (prompt portions are cut to it).
     ``enable_graphs``: replay decode-only steps as captured HIP graphs.
+    ``pipeline_depth``: 2 launches a step before the tokens of the one before have reached
+    the host (``kestrel/scheduler/pipeline.py:49-65``); 1 reads every step first.
     ``seed``: base of the sampling generator.
     """
 
@@ -50,6 +52,7 @@ class RuntimeConfig:
     kv_cache_tokens: Optional[int] = None
     max_num_batched_tokens: int = 2048
     enable_graphs: bool = True
+    pipeline_depth: int = 2
     model: Optional[str] = None
     seed: int = 0
     max_seq_len: Optional[int] = None
@@ -66,6 +69,8 @@ class RuntimeConfig:
             raise ValueError("kv_cache_tokens must be a positive integer")
         if self.max_num_batched_tokens <= 0:
             raise ValueError("max_num_batched_tokens must be a positive integer")
+        if self.pipeline_depth not in (1, 2):
+            raise ValueError("pipeline_depth must be 1 or 2")
         if self.max_seq_len is not None and self.max_seq_len <= 0:
             raise ValueError("max_seq_len must be a positive integer")
         device = torch.device(self.device)

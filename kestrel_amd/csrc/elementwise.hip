@@ -7,29 +7,40 @@
 KA_API int ka_version() { return 1; }
 
 // ----------------------------------------------------------------------------
-// Embedding: out[t, :] = table[ids[t], :] as fp32; rows with ids[t] < 0 are left
-// as they are (their embedding was given by the caller).
+// Embedding: out[t, :] = table[ids[t], :] as fp32. A row with ids[t] == -1 is left as it
+// is (its embedding was given by the caller). ids[t] <= -2 names the entry -2 - ids[t] of
+// `pending`, a device table of token ids that an earlier step's sampling filled: the id of
+// a decoded token can so reach the next step without passing through the host.
 // ----------------------------------------------------------------------------
 template <typename T>
 __global__ void embed_kernel(const T* __restrict__ table, const int* __restrict__ ids,
+                             const int* __restrict__ pending, int n_pending, int vocab,
                              float* __restrict__ out, int dim) {
     int t = blockIdx.x;
     int id = ids[t];
-    if (id < 0) return;
+    if (id == -1) return;
+    if (id < 0) {
+        int at = -2 - id;
+        if (!pending || at >= n_pending) return;
+        id = pending[at];
+        if ((unsigned)id >= (unsigned)vocab) id = 0;   // never an address outside the table
+    }
     const T* src = table + (size_t)id * dim;
     float* dst = out + (size_t)t * dim;
     for (int d = threadIdx.x; d < dim; d += blockDim.x) dst[d] = ka_to_float(src[d]);
 }
 
-KA_API int ka_embed(const void* table, int table_dtype, const int* ids, float* out, int n,
-                    int dim, hipStream_t stream) {
-    KA_CHECK(n >= 0 && dim > 0, "ka_embed: bad sizes n=%d dim=%d", n, dim);
+KA_API int ka_embed(const void* table, int table_dtype, const int* ids, const int* pending, int n_pending,
+                    int vocab, float* out, int n, int dim, hipStream_t stream) {
+    KA_CHECK(n >= 0 && dim > 0 && vocab > 0 && n_pending >= 0, "ka_embed: bad sizes n=%d dim=%d vocab=%d", n, dim, vocab);
     if (n == 0) return 0;
     dim3 grid(n), block(256);
     if (table_dtype == KA_F32)
-        hipLaunchKernelGGL(embed_kernel<float>, grid, block, 0, stream, (const float*)table, ids, out, dim);
+        hipLaunchKernelGGL(embed_kernel<float>, grid, block, 0, stream, (const float*)table, ids, pending, n_pending,
+                           vocab, out, dim);
     else if (table_dtype == KA_BF16)
-        hipLaunchKernelGGL(embed_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)table, ids, out, dim);
+        hipLaunchKernelGGL(embed_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)table, ids, pending,
+                           n_pending, vocab, out, dim);
     else
         KA_CHECK(false, "ka_embed: unsupported table dtype %d", table_dtype);
     KA_LAUNCH_CHECK();

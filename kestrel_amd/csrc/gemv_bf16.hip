@@ -343,6 +343,7 @@ KA_API int ka_linear_skinny_fused(const void* A1, long lda1, int K1, const void*
     int MB = ka_cdiv(M, 16);
     int waves = ka_cdiv(target_waves, strips);
     int kblocks = ka_cdiv(K1 + (A2 ? K2 : 0), SK_KBLOCK);
+    if (waves < 4) waves = 4;                 // fewer waves leave too few loads in flight per CU
     if (waves > kblocks) waves = kblocks;
     if (MB > 2 && waves > 8) waves = 8;       // LDS of the final sum grows with MB
     int rc;

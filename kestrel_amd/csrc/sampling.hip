@@ -44,13 +44,40 @@ __host__ __device__ inline float ka_uniform(unsigned long long key, unsigned lon
     return (float)(z >> 40) * (1.0f / 16777216.0f);
 }
 
+// The chosen token goes to out[r] and, if the caller keeps a device table of the requests'
+// latest tokens, to pending[pending_at[r]] (a negative place is passed over).
+struct PendingTable {
+    int* tokens;          // nullptr: none kept
+    const int* at;        // per row of logits: the place in `tokens`
+    int n;                // places in `tokens`
+};
+
+__device__ __forceinline__ void ka_store_token(int* out, const PendingTable& pending, int r, int token) {
+    out[r] = token;
+    if (pending.tokens) {
+        int at = pending.at[r];
+        if (at >= 0 && at < pending.n) pending.tokens[at] = token;
+    }
+}
+
 // Index of the maximum (lowest index on ties) of one row, by all threads.
 __device__ int block_argmax(const float* __restrict__ row, int V, float* smem_f, int* smem_i) {
     float best = -INFINITY;
     int best_i = 0x7fffffff;
-    for (int i = threadIdx.x; i < V; i += SM_THREADS) {
-        float v = row[i];
-        if (v > best || (v == best && i < best_i)) { best = v; best_i = i; }
+    // eight loads in flight per thread: a row is read in a few trips to memory, not in V / threads
+    constexpr int UN = 8;
+    for (int base = threadIdx.x; base < V; base += SM_THREADS * UN) {
+        float v[UN];
+#pragma unroll
+        for (int u = 0; u < UN; ++u) {
+            int i = base + u * SM_THREADS;
+            v[u] = i < V ? row[i] : -INFINITY;
+        }
+#pragma unroll
+        for (int u = 0; u < UN; ++u) {
+            int i = base + u * SM_THREADS;
+            if (i < V && (v[u] > best || (v[u] == best && i < best_i))) { best = v[u]; best_i = i; }
+        }
     }
 #pragma unroll
     for (int off = KA_WAVE / 2; off > 0; off >>= 1) {
@@ -71,18 +98,20 @@ __device__ int block_argmax(const float* __restrict__ row, int V, float* smem_f,
 }
 
 __global__ void __launch_bounds__(SM_THREADS)
-argmax_kernel(const float* __restrict__ logits, long ld, int* __restrict__ out, int V) {
+argmax_kernel(const float* __restrict__ logits, long ld, int* __restrict__ out, int V,
+              PendingTable pending) {
     __shared__ float sf[SM_WAVES];
     __shared__ int si[SM_WAVES];
     int r = blockIdx.x;
     int idx = block_argmax(logits + (size_t)r * ld, V, sf, si);
-    if (threadIdx.x == 0) out[r] = idx;
+    if (threadIdx.x == 0) ka_store_token(out, pending, r, idx);
 }
 
 __global__ void __launch_bounds__(SM_THREADS)
 sample_kernel(const float* __restrict__ logits, long ld, const float* __restrict__ temps,
               const float* __restrict__ top_ps, const unsigned long long* __restrict__ rng_key,
-              const int* __restrict__ rng_counter, int* __restrict__ out, int V) {
+              const int* __restrict__ rng_counter, int* __restrict__ out, int V,
+              PendingTable pending) {
     __shared__ float sf[SM_WAVES];
     __shared__ int si[SM_WAVES];
     __shared__ float wave_tot[SM_WAVES];
@@ -92,7 +121,7 @@ sample_kernel(const float* __restrict__ logits, long ld, const float* __restrict
     float T = temps[r];
     int greedy = block_argmax(row, V, sf, si);
     if (!(T > SM_GREEDY_EPS)) {
-        if (threadIdx.x == 0) out[r] = greedy;
+        if (threadIdx.x == 0) ka_store_token(out, pending, r, greedy);
         return;
     }
     float inv_t = 1.0f / T;
@@ -159,25 +188,29 @@ sample_kernel(const float* __restrict__ logits, long ld, const float* __restrict
         __syncthreads();
         if (found_idx >= 0) break;
     }
-    if (threadIdx.x == 0) out[r] = found_idx >= 0 ? found_idx : greedy;
+    if (threadIdx.x == 0) ka_store_token(out, pending, r, found_idx >= 0 ? found_idx : greedy);
 }
 
-KA_API int ka_argmax(const float* logits, long ld, int* out, int rows, int V, hipStream_t stream) {
+KA_API int ka_argmax(const float* logits, long ld, int* out, int rows, int V, int* pending,
+                     const int* pending_at, int n_pending, hipStream_t stream) {
+    KA_CHECK(!pending || (pending_at && n_pending > 0), "ka_argmax: a pending table needs its places");
     KA_CHECK(rows >= 0 && V > 0 && ld >= V, "ka_argmax: bad sizes rows=%d V=%d ld=%ld", rows, V, ld);
     if (rows == 0) return 0;
-    hipLaunchKernelGGL(argmax_kernel, dim3(rows), dim3(SM_THREADS), 0, stream, logits, ld, out, V);
+    hipLaunchKernelGGL(argmax_kernel, dim3(rows), dim3(SM_THREADS), 0, stream, logits, ld, out, V,
+                       PendingTable{pending, pending_at, n_pending});
     KA_LAUNCH_CHECK();
     return 0;
 }
 
 KA_API int ka_sample(const float* logits, long ld, const float* temps, const float* top_ps,
                      const unsigned long long* rng_key, const int* rng_counter, int* out, int rows,
-                     int V, hipStream_t stream) {
+                     int V, int* pending, const int* pending_at, int n_pending, hipStream_t stream) {
     KA_CHECK(rows >= 0 && V > 0 && ld >= V, "ka_sample: bad sizes rows=%d V=%d ld=%ld", rows, V, ld);
+    KA_CHECK(!pending || (pending_at && n_pending > 0), "ka_sample: a pending table needs its places");
     KA_CHECK(temps && rng_key && rng_counter, "ka_sample: temperatures and generator state are required");
     if (rows == 0) return 0;
     hipLaunchKernelGGL(sample_kernel, dim3(rows), dim3(SM_THREADS), 0, stream, logits, ld, temps, top_ps, rng_key,
-                       rng_counter, out, V);
+                       rng_counter, out, V, PendingTable{pending, pending_at, n_pending});
     KA_LAUNCH_CHECK();
     return 0;
 }

@@ -74,6 +74,7 @@ class StepBatch:
     workspace: Workspace
     qblk_row: Optional[torch.Tensor] = None       # int32 [blocks]: row of each block of 32 queries
     qblk_tok: Optional[torch.Tensor] = None       # int32 [blocks]: its first token
+    pending: Optional[torch.Tensor] = None        # int32 device table: an id <= -2 stands for pending[-2 - id]
     given_embeds: Optional[torch.Tensor] = None   # [m, dim]
     given_rows: Optional[torch.Tensor] = None     # int32 [m] token indices they go to
     # facts known on the host, for choosing kernels

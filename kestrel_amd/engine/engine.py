@@ -128,8 +128,9 @@ class InferenceEngine:
             n_pages = cfg.max_batch_size * -(-max_seq // cfg.page_size)
         self.runner = make_runner(net, cfg.page_size, n_pages, cfg.max_batch_size,
                                   max_tokens_per_step=cfg.max_num_batched_tokens, enable_graphs=cfg.enable_graphs)
-        self.scheduler = GenerationScheduler(self.runner, Sampler(device, cfg.seed), cfg.max_batch_size,
-                                             cfg.max_num_batched_tokens, net.plan.eos_token_ids, max_seq)
+        self.scheduler = GenerationScheduler(self.runner, Sampler(device, cfg.seed, pending=self.runner.pending),
+                                             cfg.max_batch_size, cfg.max_num_batched_tokens, net.plan.eos_token_ids,
+                                             max_seq, pipeline_depth=cfg.pipeline_depth)
 
     def _scheduler_loop(self) -> None:
         try:

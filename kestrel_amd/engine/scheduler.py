@@ -20,6 +20,16 @@ Reference: queues and phases ``scheduler.py:285-286``, ``types.py:24-31``; admis
 (``scheduler.py:2219-2240``); finishing ``scheduler.py:3058-3108``. The reference runs
 either prompts or decodes in a forward and never cuts a prompt; mixing both in one
 step and cutting prompts is this engine's own design.
+
+Pipelining (``pipeline_depth`` 2, ``scheduler.py:459-548``, ``pipeline.py:49-65``): a step is
+launched before the tokens of the step before it have reached the host. A request enters
+``running`` as soon as its first token is sampled on the device; its next step names that
+token as ``PENDING_TOKEN`` and the embedding kernel takes it from the device table that the
+sampling kernel filled. The host reads a step's tokens one step late, so its work between
+two steps overlaps the GPU's. A request that turns out to have stopped has then already
+been launched once more: that step's token is thrown away, and the slot and pages are given
+back when it has been read ("zombie" steps, ``scheduler.py:2482-2527``). Limits of length
+are known without the token, so no step is launched beyond them.
 """
 
 from __future__ import annotations
@@ -31,7 +41,7 @@ from typing import Deque, Dict, List, Optional, Tuple
 
 import torch
 
-from .step import StepEntry
+from .step import PENDING_TOKEN, StepEntry
 from .types import GenerationRequest, RequestMetrics, RequestPhase, SchedulerResult, Sequence_
 
 
@@ -52,10 +62,29 @@ class StepPlan:
         return sum(len(r.entry.tokens) for r in self.rows)
 
 
+@dataclass
+class LaunchedStep:
+    """A step whose forward and sampling are queued on the GPU and whose tokens are on
+    their way to ``ids`` (pinned host memory; ``event`` tells when they are there)."""
+
+    rows: List[PlannedRow]
+    ids: Optional[torch.Tensor]
+    event: Optional["torch.cuda.Event"]
+
+
 class GenerationScheduler:
+    HOST_RING = 4
+
     def __init__(self, runner, sampler, max_batch_size: int, max_num_batched_tokens: int,
-                 eos_token_ids: Tuple[int, ...] = (), max_positions: Optional[int] = None) -> None:
+                 eos_token_ids: Tuple[int, ...] = (), max_positions: Optional[int] = None,
+                 pipeline_depth: int = 1) -> None:
+        if pipeline_depth not in (1, 2):
+            raise ValueError("pipeline_depth must be 1 (every step read before the next) or 2")
         self.runner, self.sampler = runner, sampler
+        self.pipeline_depth = pipeline_depth
+        self._inflight: Deque[LaunchedStep] = deque()
+        self._host_ids: List[Optional[torch.Tensor]] = [None] * self.HOST_RING
+        self._host_next = 0
         self.max_batch_size = max_batch_size
         self.max_num_batched_tokens = max_num_batched_tokens
         self.eos_token_ids = tuple(eos_token_ids)
@@ -84,7 +113,7 @@ class GenerationScheduler:
         self.waiting.append(Sequence_(request))
 
     def has_pending_work(self) -> bool:
-        return bool(self.waiting or self.prefilling or self.running)
+        return bool(self.waiting or self.prefilling or self.running or self._inflight)
 
     def pop_completed(self) -> List[SchedulerResult]:
         out, self.completed = self.completed, []
@@ -130,7 +159,11 @@ class GenerationScheduler:
         budget = self.max_num_batched_tokens
         # 1. one token for every running request (stable cohort: the oldest first)
         for seq in self.running[: self.max_batch_size]:
-            entry = StepEntry(seq.slot, [seq.tokens[-1]], want=[0], start=seq.total_length - 1)
+            request = seq.request
+            if seq.launched >= request.max_new_tokens or request.prompt_length + seq.launched >= self.max_positions:
+                continue                  # its last token is on its way: it ends when that is read
+            token = seq.tokens[-1] if len(seq.tokens) == seq.launched else PENDING_TOKEN
+            entry = StepEntry(seq.slot, [token], want=[0], start=request.prompt_length + seq.launched - 1)
             plan.rows.append(PlannedRow(seq, entry, True, "decode"))
             budget -= 1
         # 2. prompts already being fed, in order of admission
@@ -168,39 +201,83 @@ class GenerationScheduler:
 
     # ------------------------------------------------------------------ running
     def advance(self) -> bool:
-        """Plan and run one step. Returns whether anything was done."""
+        """Launch the next step, then read the oldest one that may no longer wait. Returns
+        whether anything was done."""
         plan = self.plan_step()
-        if not plan.rows:
-            return self._fail_unfittable()
+        did = False
+        if plan.rows:
+            self._launch(plan)
+            did = True
+        keep = self.pipeline_depth - 1 if plan.rows else 0
+        while len(self._inflight) > keep:
+            self._commit_step(self._inflight.popleft())
+            did = True
+        return did or self._fail_unfittable()
+
+    def _launch(self, plan: StepPlan) -> None:
         self.steps += 1
         logits = self.runner.step([row.entry for row in plan.rows])
         sampled_rows = [row for row in plan.rows if row.samples]
+        ids = event = None
         if sampled_rows:
-            temps = [row.seq.request.temperature for row in sampled_rows]
-            tops = [row.seq.request.top_p for row in sampled_rows]
-            seeds = [row.seq.request.seed if row.seq.request.seed is not None else row.seq.request.request_id
-                     for row in sampled_rows]
-            indices = [len(row.seq.tokens) for row in sampled_rows]
-            ids = self.sampler.sample(logits, temps, tops, seeds, indices).tolist()
-        else:
-            ids = []
-        now = time.perf_counter()
-        at = 0
+            requests = [row.seq.request for row in sampled_rows]
+            temps = [r.temperature for r in requests]
+            tops = [r.top_p for r in requests]
+            seeds = [r.seed if r.seed is not None else r.request_id for r in requests]
+            indices = [row.seq.launched for row in sampled_rows]
+            if self.pipeline_depth > 1:
+                ids = self.sampler.sample(logits, temps, tops, seeds, indices, slots=[row.seq.slot for row in sampled_rows])
+            else:
+                ids = self.sampler.sample(logits, temps, tops, seeds, indices)
+            if ids.is_cuda:
+                ids, event = self._to_host(ids)
         for row in plan.rows:
             seq = row.seq
             if row.kind == "prefill":
                 seq.fed += len(row.entry.tokens)
             if not row.samples:
                 continue
-            token = int(ids[at])
-            at += 1
-            if row.kind == "prefill":
+            seq.launched += 1
+            seq.inflight += 1
+            if row.kind == "prefill":       # its first token exists on the device: it decodes from the next step on
                 self.prefilling.remove(seq)
                 self.running.append(seq)
                 seq.phase = RequestPhase.RUNNING
+        self._inflight.append(LaunchedStep(plan.rows, ids, event))
+
+    def _to_host(self, ids: torch.Tensor):
+        """Start the copy of a step's tokens into pinned memory; the event tells when it is done."""
+        index = self._host_next
+        self._host_next = (index + 1) % self.HOST_RING       # more buffers than steps in flight
+        buf = self._host_ids[index]
+        if buf is None or buf.numel() < ids.numel():
+            buf = self._host_ids[index] = torch.empty(max(ids.numel(), 256), dtype=torch.int32, pin_memory=True)
+        host = buf[:ids.numel()]
+        host.copy_(ids, non_blocking=True)
+        event = torch.cuda.Event()
+        event.record()
+        return host, event
+
+    def _commit_step(self, step: LaunchedStep) -> None:
+        if step.event is not None:
+            step.event.synchronize()
+        ids = step.ids.tolist() if step.ids is not None else []
+        now = time.perf_counter()
+        at = 0
+        for row in step.rows:
+            if not row.samples:
+                continue
+            seq = row.seq
+            token = int(ids[at])
+            at += 1
+            seq.inflight -= 1
+            if seq.finish_reason is not None:      # it stopped a step ago: this token is not part of it
+                if seq.inflight == 0:
+                    self._release(seq)
+                continue
+            if row.kind == "prefill":
                 seq.first_token_at = now
             self._commit(seq, token, now)
-        return True
 
     def _commit(self, seq: Sequence_, token: int, now: float) -> None:
         seq.tokens.append(token)
@@ -222,9 +299,8 @@ class GenerationScheduler:
             self.running.remove(seq)
         if seq in self.prefilling:
             self.prefilling.remove(seq)
-        if seq.slot is not None:
-            self.runner.release(seq.slot)
-            seq.slot = None
+        if seq.inflight == 0:
+            self._release(seq)             # else: when the step that is still in flight has been read
         started = seq.prefill_started_at if seq.prefill_started_at is not None else seq.submitted_at
         first = seq.first_token_at if seq.first_token_at is not None else now
         metrics = RequestMetrics(
@@ -233,10 +309,15 @@ class GenerationScheduler:
             decode_time_ms=(now - first) * 1e3)
         self.completed.append(SchedulerResult(seq.request.request_id, list(seq.tokens), reason, metrics, error))
 
+    def _release(self, seq: Sequence_) -> None:
+        if seq.slot is not None:
+            self.runner.release(seq.slot)
+            seq.slot = None
+
     def _fail_unfittable(self) -> bool:
         """Nothing could be planned. If nothing is live either, the first waiting request can
         never be served: fail it alone and go on."""
-        if self.running or self.prefilling or not self.waiting:
+        if self.running or self.prefilling or self._inflight or not self.waiting:
             return False
         seq = self.waiting.popleft()
         needed = self._target_length(seq.request)

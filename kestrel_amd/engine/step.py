@@ -25,12 +25,17 @@ from ..models.decoder import DecoderModel
 from .batch import GroupBatch, StepBatch, Workspace
 
 
+PENDING_TOKEN = -2     # "the token that sampling last left for this request on the device"
+
+
 @dataclass
 class StepEntry:
     """The next tokens of one request.
 
     ``tokens``: ids; ``-1`` marks a place whose embedding is given in ``embeds`` (rows in
-    order of the ``-1`` places). ``want``: indices into ``tokens`` whose logits are returned.
+    order of the ``-1`` places); ``PENDING_TOKEN`` stands for the id that the sampler last
+    stored for this request in ``ModelRunner.pending`` (it need not have reached the host,
+    ``kestrel/scheduler/scheduler.py:2289-2290``). ``want``: indices into ``tokens`` whose logits are returned.
     ``bidirectional``: position ranges ``[lo, hi)`` whose tokens see each other both ways
     (an image block); each must lie wholly inside this portion. ``start``: position of the
     first token; ``None`` means right after what the request already holds.
@@ -92,6 +97,8 @@ class ModelRunner:
         self._graphs: Dict[int, _GraphState] = {}
         self._pages_cap = -(-model.plan.max_positions // cache.page_size)
         self.graph_replays = 0
+        # the latest sampled token of every request slot, written by the sampling kernels
+        self.pending = torch.zeros(max(1, cache.max_requests), dtype=torch.int32, device=device)
 
     # ------------------------------------------------------------------ requests
     def admit(self, reserve_length: int = 0, portion: int = 1) -> int:
@@ -187,7 +194,9 @@ class ModelRunner:
             n_given = 0
             for i, tok in enumerate(e.tokens):
                 tok = int(tok)
-                if tok < 0:
+                if tok == PENDING_TOKEN:
+                    tok = PENDING_TOKEN - e.slot      # the embedding kernel reads pending[slot]
+                elif tok < 0:
                     given_rows.append(base + i)
                     n_given += 1
                     tok = -1
@@ -299,7 +308,7 @@ class ModelRunner:
             token_row=view("token_row"), kv_hi=view("kv_hi"), row_slot=view("row_slot"), cu_q=view("cu_q"),
             kv_len=view("kv_len"), logit_rows=view("logit_rows"), groups=groups,
             workspace=workspace or self.workspace, qblk_row=view("qblk_row"), qblk_tok=view("qblk_tok"),
-            given_embeds=given_embeds, given_rows=view("given_rows") if given else None, max_q=max_q, max_kv=max_kv,
+            pending=self.pending, given_embeds=given_embeds, given_rows=view("given_rows") if given else None, max_q=max_q, max_kv=max_kv,
             decode_only=max_q == 1, causal_only=causal_only,
             host={"starts": starts, "q_lens": [len(e.tokens) for e in entries], "kv_len": kv_len, "meta_ints": total},
         )
@@ -311,7 +320,8 @@ class ModelRunner:
         if not self.enable_graphs or len(entries) > self._buckets[-1]:
             return None
         for e in entries:
-            if len(e.tokens) != 1 or int(e.tokens[0]) < 0 or list(e.want) != [0] or e.embeds is not None:
+            token = int(e.tokens[0])
+            if len(e.tokens) != 1 or (token < 0 and token != PENDING_TOKEN) or list(e.want) != [0] or e.embeds is not None:
                 return None
         return next(b for b in self._buckets if b >= len(entries))
 

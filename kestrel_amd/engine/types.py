@@ -77,7 +77,9 @@ class Sequence_:
     phase: RequestPhase = RequestPhase.WAITING
     slot: Optional[int] = None
     fed: int = 0                                     # prompt places already run
-    tokens: List[int] = field(default_factory=list)  # generated so far
+    tokens: List[int] = field(default_factory=list)  # generated so far, as the host has read them
+    launched: int = 0                                # tokens sampled on the device (>= len(tokens))
+    inflight: int = 0                                # steps launched whose token the host has not read
     finish_reason: Optional[str] = None
     submitted_at: float = field(default_factory=time.perf_counter)
     first_token_at: Optional[float] = None

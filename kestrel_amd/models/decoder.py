@@ -80,7 +80,7 @@ class DecoderModel:
         plan = self.plan
         ws = batch.workspace
         x = ws.get("model.x", (batch.n_tokens, plan.dim), torch.float32)
-        core.embed(self.embedding, batch.token_ids, x)
+        core.embed(self.embedding, batch.token_ids, x, batch.pending)
         if batch.given_embeds is not None:
             core.scatter_rows(batch.given_embeds, batch.given_rows, x)
         for index, entry in enumerate(plan.schedule):

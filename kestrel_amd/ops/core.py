@@ -20,7 +20,7 @@ _DTYPE_CODE = {torch.float32: KA_F32, torch.bfloat16: KA_BF16}
 _c_void_p, _c_int, _c_long, _c_float = ctypes.c_void_p, ctypes.c_int, ctypes.c_long, ctypes.c_float
 
 _SIGNATURES = {
-    "ka_embed": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_void_p],
+    "ka_embed": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_void_p, _c_int, _c_int, _c_void_p],
     "ka_scatter_rows": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_void_p],
     "ka_layernorm": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_float, _c_void_p, _c_int, _c_int, _c_int,
                      _c_void_p],
@@ -31,9 +31,9 @@ _SIGNATURES = {
     "ka_attention_generic": [_c_void_p, _c_int, _c_long, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p,
                              _c_void_p, _c_void_p, _c_void_p, _c_long, _c_float, _c_int, _c_int, _c_int, _c_int,
                              _c_int, _c_void_p],
-    "ka_argmax": [_c_void_p, _c_long, _c_void_p, _c_int, _c_int, _c_void_p],
+    "ka_argmax": [_c_void_p, _c_long, _c_void_p, _c_int, _c_int, _c_void_p, _c_void_p, _c_int, _c_void_p],
     "ka_sample": [_c_void_p, _c_long, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int,
-                  _c_void_p],
+                  _c_void_p, _c_void_p, _c_int, _c_void_p],
 }
 
 _lib = None
@@ -105,14 +105,17 @@ def uniform(key: int, counter: int) -> float:
     return float(lib().ka_uniform_host(key & (2 ** 64 - 1), counter))
 
 
-def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor) -> None:
-    """``out[t] = table[ids[t]]`` in fp32; rows with a negative id are left untouched."""
-    _dev(table, ids, out)
+def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor, pending: Optional[torch.Tensor] = None) -> None:
+    """``out[t] = table[ids[t]]`` in fp32. A row with id -1 is left untouched; an id ``<= -2`` is
+    replaced by ``pending[-2 - id]`` (int32 token ids kept on the device by earlier sampling)."""
+    _dev(table, ids, out, pending)
+    _need(pending is None or (pending.dtype == torch.int32 and pending.is_contiguous()), "embed: pending must be int32")
     n, dim = out.shape
     _need(table.dim() == 2 and table.shape[1] == dim and table.is_contiguous(), "embed: table must be [vocab, dim]")
     _need(ids.dtype == torch.int32 and ids.numel() == n and ids.is_contiguous(), "embed: ids must be int32 [n]")
     _need(out.dtype == torch.float32 and out.is_contiguous(), "embed: out must be contiguous fp32")
-    _check(lib().ka_embed(table.data_ptr(), code_of(table.dtype), ids.data_ptr(), out.data_ptr(), n, dim,
+    _check(lib().ka_embed(table.data_ptr(), code_of(table.dtype), ids.data_ptr(), _ptr(pending),
+                          0 if pending is None else pending.numel(), table.shape[0], out.data_ptr(), n, dim,
                           stream_ptr()))
 
 
@@ -213,19 +216,33 @@ def attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
                                       stream_ptr()))
 
 
-def argmax(logits: torch.Tensor, out: torch.Tensor) -> None:
-    """Index of the largest logit of every fp32 row into int32 ``out``."""
-    _dev(logits, out)
+def _pending_args(who: str, rows: int, pending, pending_at):
+    if pending is None:
+        return None, None, 0
+    _need(pending.dtype == torch.int32 and pending.is_contiguous(), f"{who}: pending must be int32")
+    _need(pending_at is not None and pending_at.dtype == torch.int32 and pending_at.numel() == rows
+          and pending_at.is_contiguous(), f"{who}: pending_at int32 [rows]")
+    return pending.data_ptr(), pending_at.data_ptr(), pending.numel()
+
+
+def argmax(logits: torch.Tensor, out: torch.Tensor, pending: Optional[torch.Tensor] = None,
+           pending_at: Optional[torch.Tensor] = None) -> None:
+    """Index of the largest logit of every fp32 row into int32 ``out``, and into
+    ``pending[pending_at[row]]`` if a table of latest tokens is given (negative place: skipped)."""
+    _dev(logits, out, pending, pending_at)
     rows, vocab = logits.shape
     _need(logits.dtype == torch.float32 and logits.stride(1) == 1, "argmax: logits must be fp32 rows")
     _need(out.dtype == torch.int32 and out.numel() == rows and out.is_contiguous(), "argmax: out int32 [rows]")
-    _check(lib().ka_argmax(logits.data_ptr(), logits.stride(0), out.data_ptr(), rows, vocab, stream_ptr()))
+    _check(lib().ka_argmax(logits.data_ptr(), logits.stride(0), out.data_ptr(), rows, vocab,
+                           *_pending_args("argmax", rows, pending, pending_at), stream_ptr()))
 
 
 def sample(logits: torch.Tensor, temps: torch.Tensor, top_ps: Optional[torch.Tensor], rng_key: torch.Tensor,
-           rng_counter: torch.Tensor, out: torch.Tensor) -> None:
-    """Temperature and top-p sampling of every row (greedy where temperature <= 1e-6)."""
-    _dev(logits, temps, top_ps, rng_key, rng_counter, out)
+           rng_counter: torch.Tensor, out: torch.Tensor, pending: Optional[torch.Tensor] = None,
+           pending_at: Optional[torch.Tensor] = None) -> None:
+    """Temperature and top-p sampling of every row (greedy where temperature <= 1e-6); the
+    token also goes to ``pending[pending_at[row]]`` if given."""
+    _dev(logits, temps, top_ps, rng_key, rng_counter, out, pending, pending_at)
     rows, vocab = logits.shape
     _need(logits.dtype == torch.float32 and logits.stride(1) == 1, "sample: logits must be fp32 rows")
     _need(temps.dtype == torch.float32 and temps.numel() == rows, "sample: temps fp32 [rows]")
@@ -234,4 +251,5 @@ def sample(logits: torch.Tensor, temps: torch.Tensor, top_ps: Optional[torch.Ten
     _need(rng_counter.dtype == torch.int32 and rng_counter.numel() == rows, "sample: rng_counter int32 [rows]")
     _need(out.dtype == torch.int32 and out.numel() == rows and out.is_contiguous(), "sample: out int32 [rows]")
     _check(lib().ka_sample(logits.data_ptr(), logits.stride(0), temps.data_ptr(), _ptr(top_ps), rng_key.data_ptr(),
-                           rng_counter.data_ptr(), out.data_ptr(), rows, vocab, stream_ptr()))
+                           rng_counter.data_ptr(), out.data_ptr(), rows, vocab,
+                           *_pending_args("sample", rows, pending, pending_at), stream_ptr()))

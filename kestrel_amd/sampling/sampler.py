@@ -12,6 +12,7 @@ from __future__ import annotations
 
 from typing import List, Optional, Sequence
 
+import numpy as np
 import torch
 
 from ..ops import core
@@ -33,30 +34,86 @@ def _signed(value: int) -> int:
 
 
 class Sampler:
-    def __init__(self, device: torch.device, seed: int = 0) -> None:
-        self.device, self.seed = device, seed
+    """``pending`` (optional) is the step function's device table of the requests' latest tokens:
+    with ``slots`` given to a call, row ``r``'s token is also stored at ``pending[slots[r]]``, where
+    the next step's embedding can read it before the host has seen it."""
+
+    STAGING_RING = 4
+
+    def __init__(self, device: torch.device, seed: int = 0, pending: Optional[torch.Tensor] = None) -> None:
+        self.device, self.seed, self.pending = device, seed, pending
+        self._staging: List[Optional[torch.Tensor]] = [None] * self.STAGING_RING
+        self._events: List[Optional[torch.cuda.Event]] = [None] * self.STAGING_RING
+        self._device_args: List[Optional[torch.Tensor]] = [None] * self.STAGING_RING
+        self._next = 0
+
+    def _upload(self, columns: Sequence[np.ndarray]) -> List[torch.Tensor]:
+        """Per-row arguments (4- or 8-byte columns) to the device with one copy out of pinned memory."""
+        rows = len(columns[0])
+        words = [rows * (c.dtype.itemsize // 4) for c in columns]
+        padded = [(w + 3) & ~3 for w in words]                   # every column starts on 16 bytes
+        total = sum(padded)
+        index = self._next
+        self._next = (index + 1) % self.STAGING_RING
+        if self._events[index] is not None:
+            self._events[index].synchronize()
+        if self._staging[index] is None or self._staging[index].numel() < total:
+            self._staging[index] = torch.empty(max(total, 1024), dtype=torch.int32, pin_memory=True)
+            self._device_args[index] = torch.empty(max(total, 1024), dtype=torch.int32, device=self.device)
+        host, dev = self._staging[index], self._device_args[index]
+        raw = host.numpy()
+        views: List[torch.Tensor] = []
+        at = 0
+        for column, n, n_padded in zip(columns, words, padded):
+            raw[at:at + n] = column.view(np.int32)
+            kind = {np.dtype(np.float32): torch.float32, np.dtype(np.int64): torch.int64,
+                    np.dtype(np.int32): torch.int32}[column.dtype]
+            views.append(dev[at:at + n].view(kind))
+            at += n_padded
+        dev[:total].copy_(host[:total], non_blocking=True)
+        event = self._events[index] or torch.cuda.Event()
+        event.record()
+        self._events[index] = event
+        return views
 
     def sample(self, logits: torch.Tensor, temperatures: Sequence[float], top_ps: Sequence[float],
-               request_seeds: Sequence[int], token_indices: Sequence[int]) -> torch.Tensor:
+               request_seeds: Sequence[int], token_indices: Sequence[int],
+               slots: Optional[Sequence[int]] = None) -> torch.Tensor:
         """One token id per row of fp32 ``logits``; int32 on the device."""
         rows = logits.shape[0]
         if not (len(temperatures) == len(top_ps) == len(request_seeds) == len(token_indices) == rows):
             raise ValueError("sampling parameters must have one entry per row of logits")
+        if slots is not None and (self.pending is None or len(slots) != rows):
+            raise ValueError("slots need a pending table and one entry per row of logits")
         out = torch.empty(rows, dtype=torch.int32, device=self.device)
         if rows == 0:
             return out
-        if all(t <= GREEDY_EPS for t in temperatures):
-            core.argmax(logits, out)
-            return out
-        temps = torch.tensor(list(temperatures), dtype=torch.float32).to(self.device)
-        tops = torch.tensor(list(top_ps), dtype=torch.float32).to(self.device)
-        keys = torch.tensor([_signed(mix_key(self.seed, s)) for s in request_seeds], dtype=torch.int64).to(self.device)
-        counters = torch.tensor(list(token_indices), dtype=torch.int32).to(self.device)
-        core.sample(logits, temps, tops, keys, counters, out)
+        greedy = all(t <= GREEDY_EPS for t in temperatures)
+        columns: List[np.ndarray] = []
+        if slots is not None:
+            columns.append(np.asarray(slots, dtype=np.int32))
+        if not greedy:
+            columns.append(np.asarray(temperatures, dtype=np.float32))
+            columns.append(np.asarray(top_ps, dtype=np.float32))
+            columns.append(np.asarray([_signed(mix_key(self.seed, s)) for s in request_seeds], dtype=np.int64))
+            columns.append(np.asarray(token_indices, dtype=np.int32))
+        args = self._upload(columns) if columns else []
+        pending_at = args.pop(0) if slots is not None else None
+        pending = self.pending if slots is not None else None
+        if greedy:
+            core.argmax(logits, out, pending, pending_at)
+        else:
+            temps, tops, keys, counters = args
+            core.sample(logits, temps, tops, keys, counters, out, pending, pending_at)
         return out
 
-    def greedy(self, logits: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    def greedy(self, logits: torch.Tensor, out: Optional[torch.Tensor] = None,
+               slots: Optional[Sequence[int]] = None) -> torch.Tensor:
         if out is None:
             out = torch.empty(logits.shape[0], dtype=torch.int32, device=self.device)
-        core.argmax(logits, out)
+        if slots is None:
+            core.argmax(logits, out)
+        else:
+            (pending_at,) = self._upload([np.asarray(slots, dtype=np.int32)])
+            core.argmax(logits, out, self.pending, pending_at)
         return out

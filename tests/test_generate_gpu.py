@@ -37,15 +37,16 @@ def _assert_greedy(result_tokens, expected, margins, slack, what):
 @pytest.mark.parametrize("name", ["A", "B", "D"])
 def test_greedy_generation_matches_the_plain_implementation(name, dtype):
     """Requests of different lengths submitted together: prompts are cut into portions of 48
-    tokens beside the decoding of the others; with and without HIP graphs."""
+    tokens beside the decoding of the others; with and without HIP graphs, with every step read
+    before the next and with two steps in flight."""
     cfg = helpers.flat_config(name)
     weights = helpers.stored_weights(helpers.model_dir(name))
     prompts = [helpers.random_ids(900 + i, n, cfg["vocab_size"]) for i, n in enumerate([5, 17, 33, 70])]
     n_new = 16
     expected = [plain.greedy_generate(cfg, weights, p, n_new) for p in prompts]
     slack = 1e-4 if dtype == "float32" else 5e-2
-    for graphs in (False, True):
-        engine = _engine(name, dtype, enable_graphs=graphs)
+    for graphs, depth in ((False, 1), (True, 2), (False, 2)):
+        engine = _engine(name, dtype, enable_graphs=graphs, pipeline_depth=depth)
         try:
             results = engine.generate_batch_sync(prompts, max_new_tokens=n_new, temperature=0.0, stop_ids=())
             replays = engine.runner.graph_replays
@@ -54,7 +55,7 @@ def test_greedy_generation_matches_the_plain_implementation(name, dtype):
         assert (replays > 0) == graphs
         for result, (tokens, margins) in zip(results, expected):
             assert result.finish_reason == "length" and result.metrics.output_tokens == n_new
-            _assert_greedy(result.tokens, tokens, margins, slack, f"tiny {name} {dtype} graphs={graphs}")
+            _assert_greedy(result.tokens, tokens, margins, slack, f"tiny {name} {dtype} graphs={graphs} depth={depth}")
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])

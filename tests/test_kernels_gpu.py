@@ -38,6 +38,37 @@ def test_embed_and_scatter(dtype):
     _close(out[[1, 4]], given.float(), torch.float32)
 
 
+def test_tokens_kept_on_the_device_reach_the_embedding():
+    """Sampling stores a row's token at a place of the pending table; an id <= -2 makes the
+    embedding read that place. Rows whose place is negative are not stored."""
+    from kestrel_amd.ops import core
+
+    torch.manual_seed(3)
+    table = torch.randn(50, 24).to(DEV)
+    logits = torch.randn(4, 50).to(DEV)
+    pending = torch.full((6,), 49, dtype=torch.int32, device=DEV)
+    places = torch.tensor([4, -1, 0, 5], dtype=torch.int32, device=DEV)
+    out = torch.empty(4, dtype=torch.int32, device=DEV)
+    core.argmax(logits, out, pending, places)
+    best = logits.argmax(dim=1).cpu()
+    assert out.cpu().tolist() == best.tolist()
+    assert pending.cpu().tolist() == [int(best[2]), 49, 49, 49, int(best[0]), int(best[3])]
+    ids = torch.tensor([-2 - 4, 7, -1, -2 - 0, -2 - 1], dtype=torch.int32, device=DEV)
+    x = torch.full((5, 24), 3.0, device=DEV)
+    core.embed(table, ids, x, pending)
+    want = table.cpu()[[int(best[0]), 7, 0, int(best[2]), 49]]
+    want[2] = 3.0
+    assert torch.equal(x.cpu(), want)
+    # the sampling kernel stores the same way
+    temps = torch.tensor([0.0, 0.7, 0.0, 1.1], device=DEV)
+    keys = torch.tensor([1, 2, 3, 4], dtype=torch.int64, device=DEV)
+    counters = torch.zeros(4, dtype=torch.int32, device=DEV)
+    pending.fill_(49)
+    core.sample(logits, temps, None, keys, counters, out, pending, places)
+    got = out.cpu().tolist()
+    assert pending.cpu().tolist() == [got[2], 49, 49, 49, got[0], got[3]]
+
+
 @pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("dim", [100, 2048, 5000])
 def test_layernorm(dim, out_dtype):

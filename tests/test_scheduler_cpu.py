@@ -19,6 +19,7 @@ class FakeRunner:
         self.model = SimpleNamespace(plan=SimpleNamespace(max_positions=max_positions, vocab_size=vocab))
         self.held = {}
         self.steps = []
+        self.tokens = []
         self.vocab = vocab
 
     def admit(self, reserve_length=0, portion=1):
@@ -43,6 +44,7 @@ class FakeRunner:
             record.append((e.slot, start, len(e.tokens), list(e.want)))
             wanted += len(e.want)
         self.steps.append(record)
+        self.tokens.append([list(e.tokens) for e in entries])
         self.cache.check()
         return torch.zeros(wanted, self.vocab)
 
@@ -50,14 +52,16 @@ class FakeRunner:
 class FakeSampler:
     """Token = 10 + index of the token in its request; request seed 99 emits the stop id 0 at index 2."""
 
-    def sample(self, logits, temps, tops, seeds, indices):
+    def sample(self, logits, temps, tops, seeds, indices, slots=None):
         assert logits.shape[0] == len(temps) == len(indices)
+        assert slots is None or len(slots) == len(indices)
         return torch.tensor([0 if (s == 99 and i == 2) else 10 + i for s, i in zip(seeds, indices)], dtype=torch.int32)
 
 
-def _scheduler(runner=None, max_batch_size=4, budget=16, **kw):
+def _scheduler(runner=None, max_batch_size=4, budget=16, pipeline_depth=1, **kw):
     runner = runner or FakeRunner(**kw)
-    return GenerationScheduler(runner, FakeSampler(), max_batch_size, budget, eos_token_ids=(0,)), runner
+    return GenerationScheduler(runner, FakeSampler(), max_batch_size, budget, eos_token_ids=(0,),
+                               pipeline_depth=pipeline_depth), runner
 
 
 def _req(i, n_prompt, n_new, **kw):
@@ -183,3 +187,66 @@ def test_tokens_are_streamed_as_they_are_committed():
     sched.enqueue_request(_req(0, 3, 3, on_token=lambda tok, i: seen.append((tok, i))))
     sched.run_until_done()
     assert seen == [(10, 0), (11, 1), (12, 2)]
+
+
+# ---------------------------------------------------------------------- two steps in flight
+def _mixed_requests():
+    return [_req(0, 3, 10, seed=99), _req(1, 3, 2), _req(2, 21, 5), _req(3, 7, 1), _req(4, 5, 6, seed=99)]
+
+
+def test_pipelined_scheduling_gives_the_same_results():
+    outcomes = []
+    for depth in (1, 2):
+        sched, runner = _scheduler(pipeline_depth=depth, budget=16, max_batch_size=3, n_pages=24)
+        for request in _mixed_requests():
+            sched.enqueue_request(request)
+        results = {r.request_id: (r.tokens, r.finish_reason) for r in sched.run_until_done()}
+        assert runner.cache.groups[0].pool.free_count == 24 and runner.cache.free_slots == 4
+        assert not runner.held
+        outcomes.append(results)
+    assert outcomes[0] == outcomes[1]
+    assert outcomes[0][0] == ([10, 11, 0], "stop") and outcomes[0][3] == ([10], "length")
+
+
+def test_a_step_is_launched_before_the_last_one_is_read():
+    from kestrel_amd.engine.step import PENDING_TOKEN
+
+    sched, runner = _scheduler(pipeline_depth=2)
+    seen = []
+    sched.enqueue_request(_req(0, 3, 4, on_token=lambda tok, i: seen.append(i)))
+    sched.advance()                                    # the prompt is launched; nothing read yet
+    assert seen == [] and len(runner.steps) == 1
+    assert sched.running and sched.running[0].launched == 1 and sched.running[0].tokens == []
+    sched.advance()                                    # first decode launched with a token the host has not seen
+    assert runner.tokens[-1] == [[PENDING_TOKEN]] and seen == [0]
+    sched.run_until_done()
+    assert seen == [0, 1, 2, 3]
+    # the length limit is known without the token: prompt + 3 decode steps, none beyond
+    assert [n for step in runner.steps for _s, _p, n, _w in step] == [3, 1, 1, 1]
+    assert all(tokens == [[PENDING_TOKEN]] for tokens in runner.tokens[1:])
+
+
+def test_a_request_that_stopped_runs_one_step_too_many_and_is_freed_after_it():
+    sched, runner = _scheduler(pipeline_depth=2)
+    sched.enqueue_request(_req(0, 3, 10, seed=99))     # stops with its third token
+    done = []
+    while sched.has_pending_work():
+        sched.advance()
+        finished = sched.pop_completed()
+        if finished:
+            done.append((len(runner.steps), finished[0], dict(runner.held)))
+    (steps_then, result, held_then), = done
+    assert result.tokens == [10, 11, 0] and result.finish_reason == "stop"
+    # prompt, two decodes that count and one more that was already launched when the stop was read
+    assert len(runner.steps) == 4 and steps_then == 4
+    assert held_then, "the slot is still held while the extra step is in flight"
+    assert not runner.held and runner.cache.groups[0].pool.free_count == 16 and runner.cache.free_slots == 4
+
+
+def test_a_finished_request_makes_room_one_step_later_when_pipelined():
+    sched, runner = _scheduler(pipeline_depth=2, max_batch_size=1, n_pages=64, budget=64)
+    sched.enqueue_request(_req(0, 4, 2))
+    sched.enqueue_request(_req(1, 4, 2))
+    results = sched.run_until_done()
+    assert [r.request_id for r in results] == [0, 1] and all(r.tokens == [10, 11] for r in results)
+    assert max(len(step) for step in runner.steps) == 1
