@@ -2,41 +2,66 @@
 //
 // The weight matrix is streamed from HBM exactly once, and nothing is exchanged between
 // workgroups (no fences, no atomics: on a part with eight L2s they cost more than the whole
-// product). A workgroup owns a strip of 8 weight rows and all of K; its waves take interleaved
-// 64-wide k-blocks and add up through LDS in wave order, so the result is the same on every
-// run. 8 rows rather than the MFMA's 16 give N / 8 workgroups, enough to fill 256 CUs at
-// N = 2048. v_mfma_f32_16x16x32_bf16 wants 16 row-operand rows: rows 0..7 carry the strip's
-// k-block [k, k + 32), rows 8..15 the same weight rows' [k + 32, k + 64), so every lane's
-// 16-byte load is useful. Two MFMAs per block then multiply with the activations of the first
-// and of the second half; rows 0..7 of the first and rows 8..15 of the second are the wanted
-// sums, the other halves are never read.
+// product). The unit of work is a strip of 8 weight rows over all of K; the waves of a
+// workgroup take interleaved 64-wide k-blocks of it and add up through LDS in wave order, so the
+// result is the same on every run. 8 rows rather than the MFMA's 16 give N / 8 strips, enough
+// to fill 256 CUs at N = 2048. v_mfma_f32_16x16x32_bf16 wants 16 row-operand rows: rows 0..7
+// carry the strip's k-block [k, k + 32), rows 8..15 the same weight rows' [k + 32, k + 64), so
+// every lane's 16-byte load is useful. Two MFMAs per block then multiply with the activations
+// of the first and of the second half; rows 0..7 of the first and rows 8..15 of the second are
+// the wanted sums, the other halves are never read. With at most 8 rows of activations (HALF)
+// the activations play the same trick: MFMA columns 0..7 carry the rows' [k, k + 32), columns
+// 8..15 their [k + 32, k + 64); one MFMA and one activation load per block, and the wanted sums
+// are the two diagonal 8 x 8 quarters of the result.
 //
-// At these sizes a kernel costs more in launch and memory latency than in bytes, so one launch
-// does as much as the data flow allows:
-//  * two K-segments into one output (out += A1 W1^T + A2 W2^T + b1 + b2): the attention
-//    output projection and the second feed-forward linear of a parallel block in one pass;
-//  * two outputs from one input (strips of W_a, then strips of W_b): the fused q|k|v
-//    projection and the first feed-forward linear, which read the same normalised input;
-//  * a LayerNorm prologue (M <= 16): the workgroup normalises the fp32 rows itself (one wave
-//    per row, statistics in fp32, two passes) into LDS and feeds the MFMA from there.
+// Every load of the inner loops is unconditional: an address that would fall outside is moved
+// to the last valid place of the same row and the activation that multiplies it is zero. A
+// load under a branch makes the compiler wait for ALL loads in flight before the next MFMA,
+// and the loop then pays a trip to memory per round instead of streaming.
+//
+// Two kernels:
+//  * persistent (one K-segment, K up to 64 * 8 * 8): a workgroup loads its share of the
+//    activations into registers ONCE (normalising fp32 rows itself if asked to: the LayerNorm
+//    prologue) and then walks over strips blockIdx.x, + gridDim.x, ...: only weights are
+//    fetched inside the loop, one or two strips ahead of the arithmetic;
+//  * split (any K, two K-segments into one output: out += A1 W1^T + A2 W2^T + b1 + b2, the
+//    attention output projection and the second feed-forward linear of a parallel block in one
+//    pass): one strip per workgroup, up to 16 waves over K, rounds of blocks double-buffered.
+// Both take two targets (strips of W_a, then strips of W_b, from the same input): the fused
+// q|k|v projection and the first feed-forward linear.
 #include "ka_common.h"
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
 typedef __attribute__((ext_vector_type(4))) float floatx4;
 
-constexpr int SK_STRIP = 8;        // weight rows per workgroup
+constexpr int SK_STRIP = 8;        // weight rows per strip
 constexpr int SK_KBLOCK = 64;      // k per wave and step
 constexpr int SK_LN_ROWS = 16;     // most rows the LayerNorm prologue takes
-constexpr int SK_PREFETCH = 4;     // weight blocks a wave loads before the LayerNorm prologue
 constexpr int SK_XV = 8;           // float4 per lane of a row kept in registers (rows up to 2048 wide)
 constexpr int SK_PAD = 8;          // bf16 of padding per LDS row (keeps 16-byte reads off each other's banks)
+constexpr int SP_WAVES = 8;        // waves of a persistent workgroup
+constexpr int SP_MAX_PER = 8;      // most k-blocks per wave it keeps activations for
 
-__device__ __forceinline__ bf16x8 sk_load8(const bf16_t* p) { return *reinterpret_cast<const bf16x8*>(p); }
+// Every operand lives in global memory. Saying so at the load matters: a pointer that went
+// through sk_pinned() below is "generic" to the compiler, and generic (flat) loads count as LDS
+// traffic too, which forces a wait for everything in flight at each use.
+#define SK_GLOBAL __attribute__((address_space(1)))
+__device__ __forceinline__ bf16x8 sk_load8(const bf16_t* p) { return *(const SK_GLOBAL bf16x8*)p; }
 // Weights are read once and never again: a load that does not displace the activations,
 // which every workgroup of a CU reads, from the caches.
 __device__ __forceinline__ bf16x8 sk_load8_stream(const bf16_t* p) {
-    return __builtin_nontemporal_load(reinterpret_cast<const bf16x8*>(p));
+    return __builtin_nontemporal_load((const SK_GLOBAL bf16x8*)p);
+}
+
+// A kernel argument that is chosen between two at run time (target a or b, segment 1 or 2)
+// is pinned in scalar registers first: left alone, the compiler turns "choose one of two
+// loaded arguments" into "load from the chosen address", a trip to memory on which every
+// weight load of the round then depends.
+template <typename T>
+__device__ __forceinline__ T sk_pinned(T v) {
+    asm volatile("" : "+s"(v));
+    return v;
 }
 
 struct SkinnyTarget {       // one weight matrix and where its product goes
@@ -68,222 +93,505 @@ struct SkinnyArgs {
     int M;
 };
 
-template <int MB, int WAVES, bool LN>
-__global__ void __launch_bounds__(WAVES * KA_WAVE) __attribute__((amdgpu_waves_per_eu(4)))
-skinny_kernel(SkinnyArgs p) {
-    __shared__ floatx4 red[WAVES][MB][KA_WAVE];
+// bias[n .. n + 3] without a branch around the loads (values past N are never used).
+__device__ __forceinline__ floatx4 sk_bias4(const float* bias, int n, int N) {
+    floatx4 v = floatx4{0.f, 0.f, 0.f, 0.f};
+    if (bias == nullptr) return v;
+    if (N % 4 == 0 && (reinterpret_cast<uintptr_t>(bias) & 15) == 0) {     // n is a multiple of 4
+        v = *(const SK_GLOBAL floatx4*)(bias + min(n, N - 4));
+    } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] = *(const SK_GLOBAL float*)(bias + min(n + i, N - 1));
+    }
+    return v;
+}
+
+// The finishing lanes (g in {0, 1}, r; with HALF r < 8) own out[m = mb * 16 + r][n0 + g * 4 + i]:
+// they add the waves' partial sums in wave order, then bias / old value, activation, store.
+template <int MB, bool HALF, int NW>
+__device__ __forceinline__ void sk_finish(const floatx4 (*red)[MB][KA_WAVE], const floatx4 (&addend)[MB],
+                                          const SkinnyTarget& tg, int n0, int M, int lane) {
+    const int r = lane % 16, g = lane / 16;
+    // the other half of an output element: MFMA rows 8..15, and with HALF columns 8..15 as well
+    constexpr int OTHER = HALF ? 40 : 32;
+    const int n = n0 + g * 4;
+    const bool whole = n + 3 < tg.N && tg.ldo % 4 == 0 && (reinterpret_cast<uintptr_t>(tg.out) & 15) == 0;
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+        floatx4 s = addend[mb];
+#pragma unroll
+        for (int w = 0; w < NW; ++w) s += red[w][mb][lane] + red[w][mb][lane + OTHER];
+        const int m = mb * 16 + r;
+        if (m >= M) continue;
+        if (tg.act == 1) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) s[i] = ka_gelu_tanh(s[i]);
+        }
+        const size_t o = (size_t)m * tg.ldo + n;
+        if (whole) {
+            if (tg.out_dtype == KA_F32) {
+                *reinterpret_cast<floatx4*>(reinterpret_cast<float*>(tg.out) + o) = s;
+            } else {
+                bf16x4 y;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) y[i] = (bf16_t)s[i];
+                *reinterpret_cast<bf16x4*>(reinterpret_cast<bf16_t*>(tg.out) + o) = y;
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                if (n + i >= tg.N) continue;
+                if (tg.out_dtype == KA_F32) reinterpret_cast<float*>(tg.out)[o + i] = s[i];
+                else reinterpret_cast<bf16_t*>(tg.out)[o + i] = (bf16_t)s[i];
+            }
+        }
+    }
+}
+
+// LayerNorm of rows wave, wave + NW, ... of fp32 x [M, K] into LDS as bf16 [M][K + SK_PAD]
+// (statistics in fp32, two passes over a row kept in registers: K <= SK_XV * 256).
+template <int NW>
+__device__ __forceinline__ void sk_layernorm_rows(const SkinnyArgs& p, bf16_t* xs, int wave, int lane) {
+    const int K = p.K[0], M = p.M, ld = K + SK_PAD;
+    for (int m = wave; m < M; m += NW) {
+        const float* src = p.ln_x + (size_t)m * K;
+        floatx4 xv[SK_XV], gm[SK_XV], bt[SK_XV];
+        float s = 0.f;
+        // the row, and the scale and shift that meet it, in one trip to memory
+#pragma unroll
+        for (int j = 0; j < SK_XV; ++j) {
+            const int k = min((j * KA_WAVE + lane) * 4, K - 4);
+            xv[j] = *reinterpret_cast<const floatx4*>(src + k);
+            gm[j] = *reinterpret_cast<const floatx4*>(p.ln_gamma + k);
+            bt[j] = p.ln_beta ? *reinterpret_cast<const floatx4*>(p.ln_beta + k) : floatx4{0.f, 0.f, 0.f, 0.f};
+        }
+#pragma unroll
+        for (int j = 0; j < SK_XV; ++j) {
+            if ((j * KA_WAVE + lane) * 4 >= K) xv[j] = floatx4{0.f, 0.f, 0.f, 0.f};
+            s += (xv[j][0] + xv[j][1]) + (xv[j][2] + xv[j][3]);
+        }
+        float mean = ka_wave_sum(s) / (float)K;
+        float q = 0.f;
+#pragma unroll
+        for (int j = 0; j < SK_XV; ++j) {
+            if ((j * KA_WAVE + lane) * 4 < K) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) q += (xv[j][i] - mean) * (xv[j][i] - mean);
+            }
+        }
+        float rstd = 1.0f / sqrtf(ka_wave_sum(q) / (float)K + p.ln_eps);
+#pragma unroll
+        for (int j = 0; j < SK_XV; ++j) {
+            const int k = (j * KA_WAVE + lane) * 4;
+            if (k < K) {
+                bf16x4 y;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) y[i] = (bf16_t)((xv[j][i] - mean) * rstd * gm[j][i] + bt[j][i]);
+                *reinterpret_cast<bf16x4*>(xs + m * ld + k) = y;
+            }
+        }
+    }
+}
+
+// ----------------------------------------------------------------------------
+// The persistent kernel.
+// ----------------------------------------------------------------------------
+template <int PER, int MB, bool HALF, bool LN, int DEPTH>
+__global__ void __launch_bounds__(SP_WAVES * KA_WAVE)
+skinny_persistent_kernel(SkinnyArgs p, int total_strips) {
+    static_assert(!HALF || MB == 1, "the half-column form is for at most 8 rows");
+    static_assert(!LN || MB == 1, "the LayerNorm prologue takes at most 16 rows");
+    __shared__ floatx4 red[2][SP_WAVES][MB][KA_WAVE];
     extern __shared__ __attribute__((aligned(16))) unsigned char sk_dyn[];
     const int wave = threadIdx.x / KA_WAVE, lane = threadIdx.x % KA_WAVE;
+    const int r = lane % 16, g = lane / 16;
+    const int K = p.K[0], M = p.M;
+    const int koff = (r / 8) * 32 + g * 8;            // this lane's place inside a 64-wide k-block (weights)
+    const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+    const int grid = gridDim.x;
+    const int mine = (total_strips - (int)blockIdx.x + grid - 1) / grid;      // strips of this workgroup, >= 1
+
+    // where this lane reads its PER weight blocks of a row (an offset past K is moved inside:
+    // the activations that meet it are zero)
+    int wofs[PER];
+#pragma unroll
+    for (int u = 0; u < PER; ++u) wofs[u] = min((wave + u * SP_WAVES) * SK_KBLOCK + koff, K - 8);
+
+    bf16x8 w[DEPTH][PER];
+    floatx4 addend[DEPTH][MB];
+    const bf16_t* const Wa = sk_pinned(p.a.W);
+    const bf16_t* const Wb = sk_pinned(p.b.W);
+    const long ldwa = sk_pinned(p.a.ldw), ldwb = sk_pinned(p.b.ldw);
+    const int Na = sk_pinned(p.a.N), Nb = sk_pinned(p.b.N);
+    const float* const biasa = sk_pinned(p.a.bias);
+    const float* const biasb = sk_pinned(p.b.bias);
+    const int strips_a = sk_pinned(p.strips_a);
+
+    auto issue = [&](int slot, int i) {
+        const int strip = blockIdx.x + i * grid;
+        const bool second = strip >= strips_a;
+        const bf16_t* W = second ? Wb : Wa;
+        const long ldw = second ? ldwb : ldwa;
+        const int N = second ? Nb : Na;
+        const float* bias = second ? biasb : biasa;
+        const int n0 = (second ? strip - strips_a : strip) * SK_STRIP;
+        const bf16_t* wp = W + (size_t)min(n0 + r % 8, N - 1) * ldw;
+#pragma unroll
+        for (int u = 0; u < PER; ++u) w[slot][u] = sk_load8_stream(wp + wofs[u]);
+        // what the finishing lanes add at the end comes with the strip's weights (all waves ask
+        // for it: a load under a branch would break the stream)
+        floatx4 b4 = sk_bias4(bias, n0 + (g & 1) * 4, N);
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) addend[slot][mb] = b4;
+    };
+
+    // the first strips' weights are on their way while the activations come in
+    issue(0, 0);
+    if (DEPTH == 3 && mine > 1) issue(1, 1);
+
+    // activations of this wave's k-blocks wave, wave + 8, ...: fetched (or normalised) once
+    constexpr int XH = HALF ? 1 : 2;
+    bf16x8 x[PER][MB][XH];
+    if constexpr (LN) {
+        bf16_t* xs = reinterpret_cast<bf16_t*>(sk_dyn);
+        sk_layernorm_rows<SP_WAVES>(p, xs, wave, lane);
+        __syncthreads();
+        const int ld = K + SK_PAD;
+#pragma unroll
+        for (int u = 0; u < PER; ++u) {
+            const int k = (wave + u * SP_WAVES) * SK_KBLOCK;
+            if constexpr (HALF) {
+                const int m = r % 8;
+                x[u][0][0] = m < M && k + koff < K ? *reinterpret_cast<const bf16x8*>(xs + m * ld + k + koff) : zero;
+            } else {
+                const bf16_t* xp = xs + min(r, M - 1) * ld + k + g * 8;
+                x[u][0][0] = r < M && k + g * 8 < K ? *reinterpret_cast<const bf16x8*>(xp) : zero;
+                x[u][0][1] = r < M && k + 32 + g * 8 < K ? *reinterpret_cast<const bf16x8*>(xp + 32) : zero;
+            }
+        }
+    } else {
+#pragma unroll
+        for (int u = 0; u < PER; ++u) {
+            const int k = (wave + u * SP_WAVES) * SK_KBLOCK;
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb) {
+                if constexpr (HALF) {
+                    const int m = r % 8;
+                    bf16x8 v = sk_load8(p.A[0] + (size_t)min(m, M - 1) * p.lda[0] + min(k + koff, K - 8));
+                    x[u][mb][0] = m < M && k + koff < K ? v : zero;
+                } else {
+                    const int m = mb * 16 + r;
+                    const bf16_t* ap = p.A[0] + (size_t)min(m, M - 1) * p.lda[0];
+                    bf16x8 va = sk_load8(ap + min(k + g * 8, K - 8));
+                    bf16x8 vb = sk_load8(ap + min(k + 32 + g * 8, K - 8));
+                    x[u][mb][0] = m < M && k + g * 8 < K ? va : zero;
+                    x[u][mb][1] = m < M && k + 32 + g * 8 < K ? vb : zero;
+                }
+            }
+        }
+    }
+
+    const bool finishing_lane = lane < 32 && (!HALF || r < 8);
+
+    auto compute = [&](int slot, int i) {
+        floatx4 lo[MB], hi[MB];
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) {
+            lo[mb] = floatx4{0.f, 0.f, 0.f, 0.f};
+            hi[mb] = floatx4{0.f, 0.f, 0.f, 0.f};
+        }
+#pragma unroll
+        for (int u = 0; u < PER; ++u) {
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb) {
+                lo[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[slot][u], x[u][mb][0], lo[mb], 0, 0, 0);
+                if constexpr (!HALF) hi[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[slot][u], x[u][mb][1], hi[mb], 0, 0, 0);
+            }
+        }
+        const int buf = i & 1;
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) red[buf][wave][mb][lane] = HALF || g < 2 ? lo[mb] : hi[mb];
+        // One barrier per strip is enough: a buffer is written again two strips later, after the
+        // barrier of the strip between, which the finishing wave reaches only when it has read it.
+        __syncthreads();
+        if (wave != i % SP_WAVES || !finishing_lane) return;
+        const int strip = blockIdx.x + i * grid;
+        const bool second = strip >= strips_a;
+        const int n0 = (second ? strip - strips_a : strip) * SK_STRIP;
+        sk_finish<MB, HALF, SP_WAVES>(red[buf], addend[slot], second ? p.b : p.a, n0, M, lane);
+    };
+
+    // Strip i + DEPTH - 1 is asked for before strip i is multiplied. No load of the loop stands
+    // under a condition, and the last strips are written out case by case without any: the
+    // compiler can then wait for exactly the strip it needs and leave the others in flight.
+    int i = 0;
+    if constexpr (DEPTH == 2) {
+        for (; i + 2 < mine; i += 2) {
+            issue(1, i + 1);
+            compute(0, i);
+            issue(0, i + 2);
+            compute(1, i + 1);
+        }
+        if (mine - i == 2) {
+            issue(1, i + 1);
+            compute(0, i);
+            compute(1, i + 1);
+        } else {
+            compute(0, i);
+        }
+    } else {
+        static_assert(DEPTH == 3, "one or two strips ahead");
+        if (mine == 1) {
+            compute(0, 0);
+            return;
+        }
+        for (; i + 5 <= mine; i += 3) {
+            issue(2, i + 2);
+            compute(0, i);
+            issue(0, i + 3);
+            compute(1, i + 1);
+            issue(1, i + 4);
+            compute(2, i + 2);
+        }
+        const int left = mine - i;          // 2, 3 or 4
+        if (left == 2) {
+            compute(0, i);
+            compute(1, i + 1);
+        } else if (left == 3) {
+            issue(2, i + 2);
+            compute(0, i);
+            compute(1, i + 1);
+            compute(2, i + 2);
+        } else {
+            issue(2, i + 2);
+            compute(0, i);
+            issue(0, i + 3);
+            compute(1, i + 1);
+            compute(2, i + 2);
+            compute(0, i + 3);
+        }
+    }
+}
+
+// ----------------------------------------------------------------------------
+// The split kernel: one strip per workgroup, WAVES waves over the k-blocks of both segments.
+// ----------------------------------------------------------------------------
+template <int MB, int WAVES, bool HALF>
+__global__ void __launch_bounds__(WAVES * KA_WAVE)
+skinny_split_kernel(SkinnyArgs p) {
+    static_assert(!HALF || MB == 1, "the half-column form is for at most 8 rows");
+    __shared__ floatx4 red[WAVES][MB][KA_WAVE];
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / KA_WAVE), lane = threadIdx.x % KA_WAVE;
     const int r = lane % 16, g = lane / 16;
     const bool second = (int)blockIdx.x >= p.strips_a;
     const SkinnyTarget& tg = second ? p.b : p.a;
     const int n0 = (second ? blockIdx.x - p.strips_a : blockIdx.x) * SK_STRIP;
     const int M = p.M, N = tg.N;
-    const int koff = (r / 8) * 32 + g * 8;            // this lane's place inside a 64-wide k-block
+    const int koff = (r / 8) * 32 + g * 8;
     const size_t wrow = (size_t)min(n0 + r % 8, N - 1);
+    const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
 
+    // What the finishing lanes add at the end (biases, and the output's old value when the
+    // product is accumulated) is fetched first: its latency hides behind the weight stream.
+    floatx4 addend[MB];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) addend[mb] = floatx4{0.f, 0.f, 0.f, 0.f};
+    const bool finishing_lane = wave == 0 && lane < 32 && (!HALF || r < 8);
+    if (finishing_lane) {
+        floatx4 b4 = sk_bias4(tg.bias, n0 + g * 4, N);
+        if (!second && p.bias2) b4 += sk_bias4(p.bias2, n0 + g * 4, N);
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) {
+            addend[mb] = b4;
+            // the old values of a row are read like a bias (rows and columns past the end are
+            // moved inside and never used)
+            if (tg.accumulate)
+                addend[mb] += sk_bias4(reinterpret_cast<const float*>(tg.out) + (size_t)min(mb * 16 + r, M - 1) * tg.ldo,
+                                       n0 + g * 4, N);
+        }
+    }
+
+    const int nb1 = (p.K[0] + SK_KBLOCK - 1) / SK_KBLOCK;
+    const int nb = nb1 + (p.A[1] ? (p.K[1] + SK_KBLOCK - 1) / SK_KBLOCK : 0);
+    constexpr int UN = MB == 1 ? 4 : MB == 2 ? 2 : 1;      // blocks of a round
+    constexpr int XH = HALF ? 1 : 2;
+    const int rounds = (nb + WAVES * UN - 1) / (WAVES * UN);
+
+    bf16x8 w[2][UN], x[2][UN][MB][XH];
     floatx4 lo[MB], hi[MB];
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
         lo[mb] = floatx4{0.f, 0.f, 0.f, 0.f};
         hi[mb] = floatx4{0.f, 0.f, 0.f, 0.f};
     }
-    const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
-    // What the 32 finishing lanes add at the end (bias, and the output's old value when the
-    // product is accumulated) is fetched now: its latency hides behind the weight stream.
-    floatx4 addend[MB];
-#pragma unroll
-    for (int mb = 0; mb < MB; ++mb) addend[mb] = floatx4{0.f, 0.f, 0.f, 0.f};
-    if (wave == 0 && lane < 32) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            int n = n0 + g * 4 + i;
-            if (n >= N) continue;
-            float b = tg.bias ? tg.bias[n] : 0.f;
-            if (!second && p.bias2) b += p.bias2[n];
-#pragma unroll
-            for (int mb = 0; mb < MB; ++mb) {
-                int m = mb * 16 + r;
-                float old = 0.f;
-                if (tg.accumulate && m < M) old = reinterpret_cast<const float*>(tg.out)[(size_t)m * tg.ldo + n];
-                addend[mb][i] = b;
-                if (tg.accumulate) lo[mb][i] = old;     // wave 0's own sum starts from the old value
-            }
-        }
-    }
 
-    if constexpr (LN) {
-        // Weight loads of this wave's first blocks go out first: they do not depend on the rows,
-        // and their latency then hides behind the LayerNorm below.
-        const int K = p.K[0];
-        const bf16_t* wp = tg.W + wrow * tg.ldw + koff;
-        bf16x8 wpre[SK_PREFETCH];
-#pragma unroll
-        for (int j = 0; j < SK_PREFETCH; ++j) {
-            int k = (wave + j * WAVES) * SK_KBLOCK;
-            wpre[j] = k + koff < K ? sk_load8_stream(wp + k) : zero;
-        }
-        // the rows go to LDS as [M][K + pad] bf16: copied as they are, or normalised on the way
-        // (rows w, w + WAVES, ... by wave w)
-        bf16_t* xs = reinterpret_cast<bf16_t*>(sk_dyn);
-        const int ld = K + SK_PAD;
-        if (p.ln_x == nullptr) {
-            const int cpr = K / 8;
-            for (int c = threadIdx.x; c < M * cpr; c += WAVES * KA_WAVE) {
-                int m = c / cpr, kc = (c % cpr) * 8;
-                *reinterpret_cast<bf16x8*>(xs + m * ld + kc) = sk_load8(p.A[0] + (size_t)m * p.lda[0] + kc);
-            }
-        }
-        for (int m = wave; m < M && p.ln_x != nullptr; m += WAVES) {
-            const float* src = p.ln_x + (size_t)m * K;
-            {
-                // the row stays in registers (K <= SK_XV * 256, checked by the host): one trip to memory
-                floatx4 xv[SK_XV];
-                float s = 0.f;
-#pragma unroll
-                for (int j = 0; j < SK_XV; ++j) {
-                    int k = (j * KA_WAVE + lane) * 4;
-                    xv[j] = k < K ? *reinterpret_cast<const floatx4*>(src + k) : floatx4{0.f, 0.f, 0.f, 0.f};
-                    s += (xv[j][0] + xv[j][1]) + (xv[j][2] + xv[j][3]);
-                }
-                float mean = ka_wave_sum(s) / (float)K;
-                float q = 0.f;
-#pragma unroll
-                for (int j = 0; j < SK_XV; ++j) {
-                    int k = (j * KA_WAVE + lane) * 4;
-                    if (k < K) {
-#pragma unroll
-                        for (int i = 0; i < 4; ++i) q += (xv[j][i] - mean) * (xv[j][i] - mean);
-                    }
-                }
-                float rstd = 1.0f / sqrtf(ka_wave_sum(q) / (float)K + p.ln_eps);
-#pragma unroll
-                for (int j = 0; j < SK_XV; ++j) {
-                    int k = (j * KA_WAVE + lane) * 4;
-                    if (k < K) {
-                        floatx4 gm = *reinterpret_cast<const floatx4*>(p.ln_gamma + k);
-                        bf16x4 y;
-#pragma unroll
-                        for (int i = 0; i < 4; ++i) {
-                            float v = (xv[j][i] - mean) * rstd * gm[i];
-                            if (p.ln_beta) v += p.ln_beta[k + i];
-                            y[i] = (bf16_t)v;
-                        }
-                        *reinterpret_cast<bf16x4*>(xs + m * ld + k) = y;
-                    }
-                }
-            }
-        }
-        __syncthreads();
-        const bf16_t* xp = xs + min(r, M - 1) * ld + g * 8;
-#pragma unroll
-        for (int j = 0; j < SK_PREFETCH; ++j) {
-            int k = (wave + j * WAVES) * SK_KBLOCK;
-            if (k < K) {
-                bf16x8 xa = k + g * 8 < K ? *reinterpret_cast<const bf16x8*>(xp + k) : zero;
-                bf16x8 xb = k + 32 + g * 8 < K ? *reinterpret_cast<const bf16x8*>(xp + k + 32) : zero;
-                lo[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wpre[j], xa, lo[0], 0, 0, 0);
-                hi[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wpre[j], xb, hi[0], 0, 0, 0);
-            }
-        }
-        for (int k = (wave + SK_PREFETCH * WAVES) * SK_KBLOCK; k < K; k += WAVES * SK_KBLOCK) {
-            bf16x8 w = k + koff < K ? sk_load8(wp + k) : zero;
-            bf16x8 xa = k + g * 8 < K ? *reinterpret_cast<const bf16x8*>(xp + k) : zero;
-            bf16x8 xb = k + 32 + g * 8 < K ? *reinterpret_cast<const bf16x8*>(xp + k + 32) : zero;
-            lo[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w, xa, lo[0], 0, 0, 0);
-            hi[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w, xb, hi[0], 0, 0, 0);
-        }
-    } else {
-#pragma unroll
-        for (int seg = 0; seg < 2; ++seg) {
-            if (seg == 1 && p.A[1] == nullptr) break;
-            const int K = p.K[seg];
-            const bf16_t* wp = (seg == 0 ? tg.W + wrow * tg.ldw : p.W2 + wrow * p.ldw2) + koff;
-            const bf16_t* ap[MB];
-#pragma unroll
-            for (int mb = 0; mb < MB; ++mb) ap[mb] = p.A[seg] + (size_t)min(mb * 16 + r, M - 1) * p.lda[seg] + g * 8;
-            // K is a multiple of 8: a lane's 8 values are all inside or all outside. UN blocks at a
-            // time, and ALL their loads (weights and activations) before the first MFMA: an
-            // activation load issued between MFMAs puts a trip to L2 on the critical path per block.
-            constexpr int UN = MB == 1 ? 4 : MB == 2 ? 2 : 1;
-            for (int k0 = wave * SK_KBLOCK; k0 < K; k0 += UN * WAVES * SK_KBLOCK) {
-                bf16x8 w[UN], xa[UN][MB], xb[UN][MB];
-#pragma unroll
-                for (int u = 0; u < UN; ++u) {
-                    int k = k0 + u * WAVES * SK_KBLOCK;
-                    w[u] = k + koff < K ? sk_load8_stream(wp + k) : zero;
-                }
-#pragma unroll
-                for (int u = 0; u < UN; ++u) {
-                    int k = k0 + u * WAVES * SK_KBLOCK;
-#pragma unroll
-                    for (int mb = 0; mb < MB; ++mb) {
-                        const bool row = mb * 16 + r < M;      // rows past M are not fetched at all
-                        xa[u][mb] = row && k + g * 8 < K ? sk_load8(ap[mb] + k) : zero;
-                        xb[u][mb] = row && k + 32 + g * 8 < K ? sk_load8(ap[mb] + k + 32) : zero;
-                    }
-                }
-#pragma unroll
-                for (int u = 0; u < UN; ++u) {
-#pragma unroll
-                    for (int mb = 0; mb < MB; ++mb) {
-                        lo[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[u], xa[u][mb], lo[mb], 0, 0, 0);
-                        hi[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[u], xb[u][mb], hi[mb], 0, 0, 0);
-                    }
-                }
-            }
-        }
-    }
-    // A lane holds the MFMA rows g * 4 + i: lanes g < 2 keep rows 0..7 of `lo`, lanes g >= 2 rows
-    // 8..15 of `hi`; lanes g and g + 2 hold the two halves of the same output elements.
-#pragma unroll
-    for (int mb = 0; mb < MB; ++mb) red[wave][mb][lane] = g < 2 ? lo[mb] : hi[mb];
-    __syncthreads();
-    if (wave != 0 || lane >= 32) return;
-    // 32 lanes finish: lane (g in {0, 1}, r) owns out[m = mb * 16 + r][n = n0 + g * 4 + i]
+    // this lane's rows of the weights and of the activations, per segment (the second segment's
+    // are never followed when there is none)
+    const int K0 = sk_pinned(p.K[0]), K1 = sk_pinned(p.K[1]);
+    const bf16_t* const wrow0 = tg.W + wrow * tg.ldw;
+    const bf16_t* const wrow1 = p.W2 + wrow * p.ldw2;
+    const bf16_t* arow0[MB];
+    const bf16_t* arow1[MB];
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
-        floatx4 s = floatx4{0.f, 0.f, 0.f, 0.f};
+        const int m = min(HALF ? r % 8 : mb * 16 + r, M - 1);
+        arow0[mb] = p.A[0] + (size_t)m * p.lda[0];
+        arow1[mb] = p.A[1] + (size_t)m * p.lda[1];
+    }
+
+    auto issue = [&](int slot, int round) {
 #pragma unroll
-        for (int w = 0; w < WAVES; ++w) s += red[w][mb][lane] + red[w][mb][lane + 32];
-        int m = mb * 16 + r;
-        if (m >= M) continue;
+        for (int u = 0; u < UN; ++u) {
+            // a block past the end reads the last one again and multiplies it with zeros
+            const int b = wave + (round * UN + u) * WAVES;
+            const bool live = b < nb;
+            const int bc = min(b, nb - 1);
+            const bool seg = bc >= nb1;
+            const int Ks = seg ? K1 : K0;
+            const int k = (seg ? bc - nb1 : bc) * SK_KBLOCK;
+            const bf16_t* wp = seg ? wrow1 : wrow0;
+            w[slot][u] = sk_load8_stream(wp + min(k + koff, Ks - 8));
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            int n = n0 + g * 4 + i;
-            if (n >= N) continue;
-            float v = s[i] + addend[mb][i];
-            if (tg.act == 1) v = ka_gelu_tanh(v);
-            size_t o = (size_t)m * tg.ldo + n;
-            if (tg.out_dtype == KA_F32) {
-                reinterpret_cast<float*>(tg.out)[o] = v;       // an accumulated product already holds the old value
-            } else {
-                reinterpret_cast<bf16_t*>(tg.out)[o] = (bf16_t)v;
+            for (int mb = 0; mb < MB; ++mb) {
+                const bf16_t* ap = seg ? arow1[mb] : arow0[mb];
+                if constexpr (HALF) {
+                    const int m = r % 8;
+                    bf16x8 v = sk_load8(ap + min(k + koff, Ks - 8));
+                    x[slot][u][mb][0] = live && m < M && k + koff < Ks ? v : zero;
+                } else {
+                    const int m = mb * 16 + r;
+                    bf16x8 va = sk_load8(ap + min(k + g * 8, Ks - 8));
+                    bf16x8 vb = sk_load8(ap + min(k + 32 + g * 8, Ks - 8));
+                    x[slot][u][mb][0] = live && m < M && k + g * 8 < Ks ? va : zero;
+                    x[slot][u][mb][1] = live && m < M && k + 32 + g * 8 < Ks ? vb : zero;
+                }
             }
         }
+    };
+    auto compute = [&](int slot) {
+#pragma unroll
+        for (int u = 0; u < UN; ++u) {
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb) {
+                lo[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[slot][u], x[slot][u][mb][0], lo[mb], 0, 0, 0);
+                if constexpr (!HALF) hi[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[slot][u], x[slot][u][mb][1], hi[mb], 0, 0, 0);
+            }
+        }
+    };
+
+    // round i + 1 is asked for before round i is multiplied; the tail is written out so that no
+    // load of the loop stands under a condition
+    issue(0, 0);
+    int i = 0;
+    for (; i + 2 < rounds; i += 2) {
+        issue(1, i + 1);
+        compute(0);
+        issue(0, i + 2);
+        compute(1);
+    }
+    if (rounds - i == 2) {
+        issue(1, i + 1);
+        compute(0);
+        compute(1);
+    } else {
+        compute(0);
+    }
+
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) red[wave][mb][lane] = HALF || g < 2 ? lo[mb] : hi[mb];
+    __syncthreads();
+    if (!finishing_lane) return;
+    sk_finish<MB, HALF, WAVES>(red, addend, tg, n0, M, lane);
+}
+
+// ----------------------------------------------------------------------------
+// Host side
+// ----------------------------------------------------------------------------
+static int sk_compute_units() {
+    static int cus = 0;
+    if (cus == 0) {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) == hipSuccess &&
+            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
+            cus = n;
+        else
+            cus = 256;
+    }
+    return cus;
+}
+
+// The persistent kernel is used wherever it fits; switching it off is for measurements and for
+// tests of the split kernel on sizes that it otherwise never sees.
+static int sk_persistent_enabled = 1;
+KA_API void ka_skinny_set_persistent(int enabled) { sk_persistent_enabled = enabled; }
+
+template <int PER, int MB, bool HALF, bool LN>
+static int launch_persistent_one(int grid, size_t dyn, int strips, hipStream_t stream, const SkinnyArgs& args) {
+    // two strips ahead where one workgroup has a CU (and its registers) to itself
+    constexpr int DEPTH = LN ? 3 : 2;
+    if (dyn > 0) {
+        static size_t reserved = 0;
+        if (dyn > reserved) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(skinny_persistent_kernel<PER, MB, HALF, LN, DEPTH>),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)dyn);
+            KA_CHECK(e == hipSuccess, "skinny linear: cannot reserve %zu bytes of LDS", dyn);
+            reserved = dyn;
+        }
+    }
+    hipLaunchKernelGGL((skinny_persistent_kernel<PER, MB, HALF, LN, DEPTH>), dim3(grid), dim3(SP_WAVES * KA_WAVE), dyn,
+                       stream, args, strips);
+    return 0;
+}
+
+template <int MB, bool HALF, bool LN>
+static int launch_persistent_per(int per, int grid, size_t dyn, int strips, hipStream_t stream, const SkinnyArgs& args) {
+    if (per <= 1) return launch_persistent_one<1, MB, HALF, LN>(grid, dyn, strips, stream, args);
+    if (per <= 2) return launch_persistent_one<2, MB, HALF, LN>(grid, dyn, strips, stream, args);
+    if (per <= 4) return launch_persistent_one<4, MB, HALF, LN>(grid, dyn, strips, stream, args);
+    // (the LayerNorm prologue takes rows of at most 2048: four blocks per wave)
+    if constexpr (MB == 1 && !LN) return launch_persistent_one<8, MB, HALF, LN>(grid, dyn, strips, stream, args);
+    return 1;
+}
+
+// Whether the persistent kernel takes these sizes.
+static bool persistent_fits(int M, int kblocks) {
+    const int per = ka_cdiv(kblocks, SP_WAVES);
+    return per <= (M <= 16 ? SP_MAX_PER : 4);
+}
+
+static int launch_persistent(int strips, int M, int kblocks, bool ln, size_t dyn, hipStream_t stream,
+                             const SkinnyArgs& args) {
+    const int per = ka_cdiv(kblocks, SP_WAVES);
+    const int MB = ka_cdiv(M, 16);
+    // workgroups: as many as the chip holds at once (two of 8 waves per CU while registers
+    // allow), cut so that every one walks over the same number of strips
+    const bool two = MB <= 1 && per <= 4 && !ln;      // the LayerNorm prologue's registers leave room for one
+    const int slots = sk_compute_units() * (two ? 2 : 1);
+    const int rounds = ka_cdiv(strips, slots);
+    const int grid = ka_cdiv(strips, rounds);
+    if (ln) {
+        if (M <= 8) return launch_persistent_per<1, true, true>(per, grid, dyn, strips, stream, args);
+        return launch_persistent_per<1, false, true>(per, grid, dyn, strips, stream, args);
+    }
+    if (M <= 8) return launch_persistent_per<1, true, false>(per, grid, 0, strips, stream, args);
+    switch (MB) {
+        case 1: return launch_persistent_per<1, false, false>(per, grid, 0, strips, stream, args);
+        case 2: return launch_persistent_per<2, false, false>(per, grid, 0, strips, stream, args);
+        case 3: return launch_persistent_per<3, false, false>(per, grid, 0, strips, stream, args);
+        default: return launch_persistent_per<4, false, false>(per, grid, 0, strips, stream, args);
     }
 }
 
-template <int MB, bool LN>
-static int launch_mb(int waves, int strips, size_t dyn, hipStream_t stream, const SkinnyArgs& args) {
-#define KA_SK(WV)                                                                                       \
-    do {                                                                                                \
-        if (dyn > 0) {                                                                                  \
-            static size_t reserved = 0;                                                                 \
-            if (dyn > reserved) {                                                                       \
-                hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(skinny_kernel<MB, WV, LN>), \
-                                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)dyn);   \
-                KA_CHECK(e == hipSuccess, "skinny linear: cannot reserve %zu bytes of LDS", dyn);       \
-                reserved = dyn;                                                                         \
-            }                                                                                           \
-        }                                                                                               \
-        hipLaunchKernelGGL((skinny_kernel<MB, WV, LN>), dim3(strips), dim3(WV * KA_WAVE), dyn, stream, args); \
-    } while (0)
-    if (waves >= 16) KA_SK(16);
-    else if (waves >= 8) KA_SK(8);
-    else if (waves >= 4) KA_SK(4);
-    else KA_SK(2);
-#undef KA_SK
+template <int MB, bool HALF>
+static int launch_split(int waves, int strips, hipStream_t stream, const SkinnyArgs& args) {
+    if (waves >= 16) {
+        if constexpr (HALF) {      // 16 waves leave 128 registers a lane: enough only for the half-column form
+            hipLaunchKernelGGL((skinny_split_kernel<MB, 16, HALF>), dim3(strips), dim3(16 * KA_WAVE), 0, stream, args);
+            return 0;
+        }
+    }
+    if (waves >= 8) hipLaunchKernelGGL((skinny_split_kernel<MB, 8, HALF>), dim3(strips), dim3(8 * KA_WAVE), 0, stream, args);
+    else hipLaunchKernelGGL((skinny_split_kernel<MB, 4, HALF>), dim3(strips), dim3(4 * KA_WAVE), 0, stream, args);
     return 0;
 }
 
@@ -299,7 +607,7 @@ static int check_target(const char* who, const SkinnyTarget& t, int K) {
 
 // The general entry point. Segments: A1 [M, K1] with W (target a) and optionally A2 [M, K2] with
 // W2 (same rows as target a; not with a second target). ln_x non-null: A1 is replaced by
-// LayerNorm(ln_x) (M <= 16, K1 % 4 == 0). Target b (Wb non-null) shares the input.
+// LayerNorm(ln_x) (M <= 16, K1 <= 2048). Target b (Wb non-null) shares the input.
 KA_API int ka_linear_skinny_fused(const void* A1, long lda1, int K1, const void* A2, long lda2, int K2,
                                   const void* W2, long ldw2, const float* bias2, const float* ln_x,
                                   const float* ln_gamma, const float* ln_beta, float ln_eps, const void* Wa,
@@ -319,8 +627,9 @@ KA_API int ka_linear_skinny_fused(const void* A1, long lda1, int K1, const void*
     if (ln) {
         KA_CHECK(M <= SK_LN_ROWS, "%s: the LayerNorm prologue takes at most %d rows", who, SK_LN_ROWS);
         KA_CHECK(K1 <= SK_XV * KA_WAVE * 4, "%s: the LayerNorm prologue takes rows of at most %d", who, SK_XV * KA_WAVE * 4);
-        KA_CHECK(ln_gamma && ln_eps >= 0.f && (uintptr_t)ln_x % 16 == 0 && (uintptr_t)ln_gamma % 16 == 0, "%s: LayerNorm operands", who);
-        KA_CHECK(A2 == nullptr, "%s: no second segment with a LayerNorm prologue", who);
+        KA_CHECK(ln_gamma && ln_eps >= 0.f && (uintptr_t)ln_x % 16 == 0 && (uintptr_t)ln_gamma % 16 == 0 &&
+                     (uintptr_t)ln_beta % 16 == 0, "%s: LayerNorm operands must be 16-byte aligned", who);
+        KA_CHECK(A2 == nullptr && !accumulate_a, "%s: no second segment and no accumulation with a LayerNorm prologue", who);
         args.ln_x = ln_x; args.ln_gamma = ln_gamma; args.ln_beta = ln_beta; args.ln_eps = ln_eps;
     } else {
         KA_CHECK(A1 && lda1 % 8 == 0 && lda1 >= K1 && (uintptr_t)A1 % 16 == 0, "%s: input rows must be 16-byte aligned and >= K", who);
@@ -340,28 +649,32 @@ KA_API int ka_linear_skinny_fused(const void* A1, long lda1, int K1, const void*
         if (check_target(who, args.b, K1)) return -1;
         strips += ka_cdiv(Nb, SK_STRIP);
     }
-    int MB = ka_cdiv(M, 16);
-    int waves = ka_cdiv(target_waves, strips);
-    int kblocks = ka_cdiv(K1 + (A2 ? K2 : 0), SK_KBLOCK);
-    if (waves < 4) waves = 4;                 // fewer waves leave too few loads in flight per CU
-    if (waves > kblocks) waves = kblocks;
-    if (MB > 2 && waves > 8) waves = 8;       // LDS of the final sum grows with MB
-    int rc;
-    // Staging plain rows in LDS (the copy path of the kernel) is measured slower than fetching
-    // them block by block, so only the LayerNorm prologue goes through LDS.
-    size_t dyn = (size_t)M * (K1 + SK_PAD) * sizeof(bf16_t);
-    const bool staged = ln;
-    if (staged) {
-        if (ln || waves < 4) waves = ln ? 8 : 4;     // one or two rows per wave keep a LayerNorm prologue short
+    const int MB = ka_cdiv(M, 16);
+    const int kblocks = ka_cdiv(K1, SK_KBLOCK) + (A2 ? ka_cdiv(K2, SK_KBLOCK) : 0);
+    if (ln) {
+        const size_t dyn = (size_t)M * (K1 + SK_PAD) * sizeof(bf16_t);
         KA_CHECK(dyn <= 96 * 1024, "%s: %d rows of %d do not fit in LDS", who, M, K1);
-        rc = launch_mb<1, true>(waves, strips, dyn, stream, args);
-    } else {
-        switch (MB) {
-            case 1: rc = launch_mb<1, false>(waves, strips, 0, stream, args); break;
-            case 2: rc = launch_mb<2, false>(waves, strips, 0, stream, args); break;
-            case 3: rc = launch_mb<3, false>(waves, strips, 0, stream, args); break;
-            default: rc = launch_mb<4, false>(waves, strips, 0, stream, args); break;
-        }
+        KA_CHECK(persistent_fits(M, kblocks), "%s: K=%d is too wide for the LayerNorm prologue", who, K1);
+        if (launch_persistent(strips, M, kblocks, true, dyn, stream, args)) return -1;
+        KA_LAUNCH_CHECK();
+        return 0;
+    }
+    if (!A2 && !accumulate_a && sk_persistent_enabled && persistent_fits(M, kblocks)) {
+        if (launch_persistent(strips, M, kblocks, false, 0, stream, args)) return -1;
+        KA_LAUNCH_CHECK();
+        return 0;
+    }
+    // waves over K: enough workgroups x waves to fill the chip, no more than there are rounds for
+    int waves = ka_cdiv(target_waves, strips);
+    const int un = MB == 1 ? 4 : MB == 2 ? 2 : 1;
+    if (waves > ka_cdiv(kblocks, un)) waves = ka_cdiv(kblocks, un);
+    int rc;
+    if (M <= 8) rc = launch_split<1, true>(waves, strips, stream, args);
+    else switch (MB) {
+        case 1: rc = launch_split<1, false>(waves, strips, stream, args); break;
+        case 2: rc = launch_split<2, false>(waves, strips, stream, args); break;
+        case 3: rc = launch_split<3, false>(waves, strips, stream, args); break;
+        default: rc = launch_split<4, false>(waves, strips, stream, args); break;
     }
     if (rc) return rc;
     KA_LAUNCH_CHECK();

@@ -43,13 +43,15 @@ SKINNY_MAX_ROWS = 64
 # Rows (and their width) up to which the weight-streaming kernel can normalise its input itself.
 SKINNY_LN_MAX_ROWS = 16
 SKINNY_LN_MAX_WIDTH = 2048
-# Whether blocks let the weight-streaming kernel normalise its input itself. Every workgroup then
-# repeats the LayerNorm of all rows; measured on MI355X this costs more than the launch it saves.
-FUSE_LAYERNORM_PROLOGUE = False
+# Whether blocks let the weight-streaming kernel normalise its input itself. Every workgroup of
+# the persistent kernel then repeats the LayerNorm of all rows once; with a few hundred workgroups
+# that is cheaper than a launch of its own (measured on MI355X: 3 % of a decode step at batch 8).
+FUSE_LAYERNORM_PROLOGUE = True
 # Tile of the tiled kernel: 0 lets it choose by size; 421, 221, 211 force one (for measurements).
 TILED_CONFIG = 0
-# Waves the weight-streaming kernel aims to have on the chip (256 CUs, 16 to 32 waves each).
-SKINNY_TARGET_WAVES = 6144
+# Waves the split weight-streaming kernel aims to have on the chip: 8 per workgroup at 256 strips
+# (measured best for the output projection + second feed-forward linear of Moondream 2).
+SKINNY_TARGET_WAVES = 2048
 SCRATCH_FLOATS = 8 << 20
 SCRATCH_COUNTERS = 1 << 16
 # Keys of one row a workgroup of the decode attention kernel takes before the row is split.
@@ -69,11 +71,20 @@ def lib():
             fn.argtypes = argtypes
             fn.restype = _c_int
         handle.ka_last_error.restype = ctypes.c_char_p
+        handle.ka_skinny_set_persistent.argtypes = [_c_int]
+        handle.ka_skinny_set_persistent.restype = None
         for name in ("ka_attention_prefill_supported", "ka_attention_decode_supported"):
             getattr(handle, name).argtypes = [_c_int, _c_int]
             getattr(handle, name).restype = _c_int
         _lib = handle
     return _lib
+
+
+def set_skinny_persistent(enabled: bool) -> None:
+    """Whether one-segment skinny linears use the persistent kernel (activations in registers,
+    workgroups walking over strips) where it fits: on by default; off is for measurements and
+    for tests of the kernel that otherwise only takes what the persistent one does not."""
+    lib().ka_skinny_set_persistent(int(enabled))
 
 
 def _check(status: int) -> None:

@@ -120,10 +120,14 @@ def test_linear_generic(shape):
     _linear_case(core.linear_generic, m, n, k, f32, f32, f32, 0, False, lda=k + 5)      # strided rows
 
 
+@pytest.mark.parametrize("persistent", [True, False])
 @pytest.mark.parametrize("shape", [(1, 48, 64), (8, 2048, 2048), (5, 100, 200), (16, 6144, 2048), (33, 77, 8192),
-                                   (64, 51200, 512), (17, 2048, 8192), (3, 16, 8)])
-def test_linear_skinny_bf16(shape):
-    """The weight-streaming MFMA kernel, with K-splits where N is small."""
+                                   (64, 51200, 512), (17, 2048, 8192), (3, 16, 8), (9, 20000, 1032), (40, 4100, 2048),
+                                   (8, 1000, 4096), (12, 515, 3000), (64, 9000, 1024)])
+def test_linear_skinny_bf16(shape, persistent):
+    """The weight-streaming MFMA kernels: the persistent one (activations in registers, workgroups
+    walk over strips; a form of its own for at most 8 rows) and the one with K-splits that takes
+    the rest, which is tested on the same shapes with the persistent one switched off."""
     from kestrel_amd.ops import fast
 
     m, n, k = shape
@@ -132,9 +136,13 @@ def test_linear_skinny_bf16(shape):
     def fn(a, w, bias, out, act, accumulate):
         assert fast.linear_bf16(a, w, bias, out, act, accumulate)
 
-    for out_dtype, act, accumulate in [(bf, 0, False), (bf, 1, False), (f32, 0, True), (f32, 0, False)]:
-        _linear_case(fn, m, n, k, bf, bf, out_dtype, act, accumulate)
-    _linear_case(fn, m, n, k, bf, bf, bf, 0, False, lda=k + 16)
+    fast.set_skinny_persistent(persistent)
+    try:
+        for out_dtype, act, accumulate in [(bf, 0, False), (bf, 1, False), (f32, 0, True), (f32, 0, False)]:
+            _linear_case(fn, m, n, k, bf, bf, out_dtype, act, accumulate)
+        _linear_case(fn, m, n, k, bf, bf, bf, 0, False, lda=k + 16)
+    finally:
+        fast.set_skinny_persistent(True)
 
 
 def test_linear_skinny_is_the_same_on_every_run():
