@@ -273,29 +273,61 @@ struct DecodeFuse {
     bf16_t* v_cache;
 };
 
-// Eight channels dg * 8 .. + 8 of one head row, rotated for the table row `cs` (non-interleaved
-// halves of the first `rot` channels), rounded to bf16 as the cache and the q buffer hold them.
-__device__ __forceinline__ void at_rotate8(const bf16_t* head, int dg, const float* cs, int rot, float out[8]) {
+// What a lane needs to rotate eight channels dg * 8 .. + 8 of one head row: the channels, their
+// partners in the other half of the rotated part, and cos / sin of the position. Fetched in one
+// go (at_fetch_rotary) and used later (at_rotated), so that the trip to memory overlaps others.
+struct RotaryOperands {
+    bf16x8 own, other;
+};
+struct RotaryAngles {        // of one position: the same for q and for the key
+    floatx4 c[2], s[2];
+};
+
+// lanes past the rotated part fetch lane 0's operands (valid addresses, never used)
+__device__ __forceinline__ RotaryOperands at_fetch_rotary(const bf16_t* head, int dg, int rot) {
     const int d0 = dg * 8, half = rot / 2;
-    bf16x8 own = at_load8(head + d0);
+    RotaryOperands r;
+    r.own = at_load8(head + d0);
+    const bool rotated = d0 < rot, first = d0 < half;
+    r.other = at_load8(head + (rotated ? (first ? d0 + half : d0 - half) : 0));
+    return r;
+}
+
+__device__ __forceinline__ RotaryAngles at_fetch_angles(const float* cs, int dg, int rot) {
+    const int d0 = dg * 8, half = rot / 2;
+    const bool rotated = d0 < rot, first = d0 < half;
+    const int i0 = rotated ? (first ? d0 : d0 - half) : 0;
+    RotaryAngles a;
+    a.c[0] = *reinterpret_cast<const floatx4*>(cs + i0);
+    a.c[1] = *reinterpret_cast<const floatx4*>(cs + i0 + 4);
+    a.s[0] = *reinterpret_cast<const floatx4*>(cs + half + i0);
+    a.s[1] = *reinterpret_cast<const floatx4*>(cs + half + i0 + 4);
+    return a;
+}
+
+// The eight channels rotated (non-interleaved halves of the first `rot` channels), rounded to
+// bf16 as the cache and the q buffer hold them.
+__device__ __forceinline__ void at_rotated(const RotaryOperands& r, const RotaryAngles& a, int dg, int rot, float out[8]) {
+    const int d0 = dg * 8, half = rot / 2;
     if (d0 >= rot) {
 #pragma unroll
-        for (int j = 0; j < 8; ++j) out[j] = (float)own[j];
+        for (int j = 0; j < 8; ++j) out[j] = (float)r.own[j];
         return;
     }
     const bool first = d0 < half;
-    bf16x8 other = at_load8(head + (first ? d0 + half : d0 - half));
-    const int i0 = first ? d0 : d0 - half;
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-        float c = cs[i0 + j], sn = cs[half + i0 + j];
-        float v = first ? (float)own[j] * c - (float)other[j] * sn : (float)own[j] * c + (float)other[j] * sn;
+        float c = a.c[j / 4][j % 4], sn = a.s[j / 4][j % 4];
+        float v = first ? (float)r.own[j] * c - (float)r.other[j] * sn : (float)r.own[j] * c + (float)r.other[j] * sn;
         out[j] = (float)(bf16_t)v;
     }
 }
 
+// (four waves per SIMD are all that a workgroup of 16 waves allows, two with the registers that
+// head size 128 needs; saying so keeps the compiler from trading loads in flight for an
+// occupancy the kernel cannot have)
 template <int HD, int WAVES>
-__global__ void __launch_bounds__(KA_WAVE * WAVES)
+__global__ void __launch_bounds__(KA_WAVE * WAVES) __attribute__((amdgpu_waves_per_eu(HD <= 64 ? 4 : 2, HD <= 64 ? 4 : 2)))
 attn_decode_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t* __restrict__ k_cache,
                    const bf16_t* __restrict__ v_cache, const int* __restrict__ block_table, int max_pages,
                    const int* __restrict__ token_row, const int* __restrict__ kv_lo,
@@ -304,6 +336,7 @@ attn_decode_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t
     constexpr int LPK = HD / 8;            // lanes per key row
     constexpr int KPI = KA_WAVE / LPK;     // keys per load instruction
     constexpr int VU = HD * 2 / KA_WAVE;   // 16-byte value loads per lane and page
+    constexpr int TP = AD_TILE / AT_PAGE;  // pages of a tile
     constexpr int REC = HD + 2;            // floats of a partial result: m, l, o[HD]
     __shared__ float ps[WAVES][AD_TILE];
     __shared__ float merge[WAVES][REC];
@@ -319,6 +352,30 @@ attn_decode_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t
     const int lo_tile = lo & ~(AD_TILE - 1);      // tiles start on page boundaries; keys below lo are masked
     const int chunk = ((hi - lo_tile + S - 1) / S + AD_TILE - 1) / AD_TILE * AD_TILE;
     const int s_lo = lo_tile + split * chunk, s_hi = min(hi, s_lo + chunk);
+    const int ks = lane / LPK, dg = lane % LPK;
+    const float sl2 = scale * AT_LOG2E;
+    const bool takes_new = fused && wave == 0 && split == 0;     // this wave adds the token's own key and value
+
+    // The operands of q (and, for the wave that takes them, of the token's own key and value) are
+    // asked for first and used after the first tile's keys and values have been asked for.
+    const bf16_t* qhead = q + (size_t)t * q_row_stride + (size_t)h * HD;
+    RotaryOperands qr, kr;
+    RotaryAngles angles;
+    bf16x8 qplain;
+    bf16_t vnew[VU];
+    if (fused) {
+        qr = at_fetch_rotary(qhead, dg, fz.rot);
+        angles = at_fetch_angles(fz.table + (size_t)pos * fz.rot, dg, fz.rot);
+    } else {
+        qplain = at_load8(qhead + dg * 8);
+    }
+    if (takes_new) {
+        kr = at_fetch_rotary(fz.k_new + (size_t)t * fz.stride + (size_t)kvh * HD, dg, fz.rot);
+        const bf16_t* vrow = fz.v_new + (size_t)t * fz.stride + (size_t)kvh * HD;
+#pragma unroll
+        for (int u = 0; u < VU; ++u) vnew[u] = vrow[u * 32 + lane / 2];
+    }
+
     const int* bt = block_table + (size_t)row * max_pages;
     {   // the row's block table goes to LDS once (see the prompt kernel)
         const int n_pages = (max(hi, 0) + AT_PAGE - 1) / AT_PAGE;
@@ -328,36 +385,74 @@ attn_decode_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t
             bt = pages;
         }
     }
-    const int ks = lane / LPK, dg = lane % LPK;
-    const float sl2 = scale * AT_LOG2E;
+    // q, and the token's own key and value, have had the time of the block table's trip
     float qf[8];
-    if (fused) {
-        at_rotate8(q + (size_t)t * q_row_stride + (size_t)h * HD, dg, fz.table + (size_t)pos * fz.rot, fz.rot, qf);
+    if (fused) at_rotated(qr, angles, dg, fz.rot, qf);
+    else {
 #pragma unroll
-        for (int j = 0; j < 8; ++j) qf[j] *= sl2;
-    } else {
-        bf16x8 qv = at_load8(q + (size_t)t * q_row_stride + (size_t)h * HD + dg * 8);
-#pragma unroll
-        for (int j = 0; j < 8; ++j) qf[j] = (float)qv[j] * sl2;
+        for (int j = 0; j < 8; ++j) qf[j] = (float)qplain[j];
     }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) qf[j] *= sl2;
     float m_i = -INFINITY, l_i = 0.f;
     float acc[VU];
 #pragma unroll
     for (int u = 0; u < VU; ++u) acc[u] = 0.f;
+    if (takes_new) {
+        // the token's own key and value: rotate the key, let one head of the group store both, and
+        // start this wave's sums with them, straight from registers
+        float kn[8];
+        at_rotated(kr, angles, dg, fz.rot, kn);
+        const int slot = fz.slots[t];
+        if (slot >= 0 && h % (H / Hkv) == 0) {
+            const size_t page = slot / AT_PAGE, off = slot % AT_PAGE;
+            if (ks == 0) {
+                bf16x8 kb;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) kb[j] = (bf16_t)kn[j];
+                *reinterpret_cast<bf16x8*>(fz.k_cache + ((page * Hkv + kvh) * AT_PAGE + off) * HD + dg * 8) = kb;
+            }
+            if ((lane & 1) == 0) {
+#pragma unroll
+                for (int u = 0; u < VU; ++u) {
+                    int d = u * 32 + lane / 2;
+                    fz.v_cache[((page * Hkv + kvh) * HD + d) * AT_PAGE + off] = vnew[u];
+                }
+            }
+        }
+        float dot = 0.f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) dot = fmaf(qf[j], kn[j], dot);
+#pragma unroll
+        for (int off = 1; off < LPK; off <<= 1) dot += __shfl_xor(dot, off, KA_WAVE);
+        m_i = dot;                // the only key so far: its weight is 1
+        l_i = 1.f;
+#pragma unroll
+        for (int u = 0; u < VU; ++u) acc[u] = (lane & 1) == 0 ? (float)vnew[u] : 0.f;
+    }
 
     for (int tile0 = s_lo + wave * AD_TILE; tile0 < s_hi; tile0 += WAVES * AD_TILE) {
+        // All key loads of the tile go out before any arithmetic, and none stands under a
+        // condition: a place outside [lo, s_hi) is moved to one inside and masked afterwards. The
+        // compiler can then wait for exactly the register it needs instead of for everything.
+        bf16x8 kreg[LPK];
+#pragma unroll
+        for (int i = 0; i < LPK; ++i) {
+            int key = tile0 + i * KPI + ks;
+            int kc = max(min(key, s_hi - 1), lo);   // a place that holds data (pages below lo may be gone)
+            int page = bt[kc / AT_PAGE];
+            kreg[i] = at_load8(k_cache + (((size_t)page * Hkv + kvh) * AT_PAGE + kc % AT_PAGE) * HD + dg * 8);
+        }
+        __builtin_amdgcn_sched_barrier(0);     // all of them, before the first is used
         float sc[LPK];
         float mx = -INFINITY;
 #pragma unroll
         for (int i = 0; i < LPK; ++i) {
             int key = tile0 + i * KPI + ks;
             bool ok = key >= lo && key < s_hi;
-            int kc = max(min(key, s_hi - 1), lo);   // a place that holds data (pages below lo may be gone)
-            int page = bt[kc / AT_PAGE];
-            bf16x8 kv = at_load8(k_cache + (((size_t)page * Hkv + kvh) * AT_PAGE + kc % AT_PAGE) * HD + dg * 8);
             float dot = 0.f;
 #pragma unroll
-            for (int j = 0; j < 8; ++j) dot = fmaf(qf[j], (float)kv[j], dot);
+            for (int j = 0; j < 8; ++j) dot = fmaf(qf[j], (float)kreg[i][j], dot);
 #pragma unroll
             for (int off = 1; off < LPK; off <<= 1) dot += __shfl_xor(dot, off, KA_WAVE);
             sc[i] = ok ? dot : -INFINITY;
@@ -367,6 +462,20 @@ attn_decode_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t
         for (int off = LPK; off < KA_WAVE; off <<= 1) mx = fmaxf(mx, __shfl_xor(mx, off, KA_WAVE));
         float m_new = fmaxf(m_i, mx);
         if (m_new == -INFINITY) continue;      // a tile wholly below lo (wave-uniform)
+        // the values: asked for as soon as the keys' registers are free, all at once and, like
+        // the keys, without a condition; the softmax below runs while they are on their way
+        bf16x8 vreg[TP][VU];
+#pragma unroll
+        for (int pg = 0; pg < TP; ++pg) {
+            int kc = max(min(tile0 + pg * AT_PAGE, s_hi - 1), lo);
+            int page = bt[kc / AT_PAGE];
+#pragma unroll
+            for (int u = 0; u < VU; ++u) {
+                int d = u * 32 + lane / 2;
+                vreg[pg][u] = at_load8(v_cache + (((size_t)page * Hkv + kvh) * HD + d) * AT_PAGE + (lane & 1) * 8);
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
         float alpha = exp2f(m_i - m_new);
         float rowsum = 0.f;
         at_wave_sync();                        // the previous tile's probabilities have been read
@@ -383,70 +492,25 @@ attn_decode_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t
 #pragma unroll
         for (int u = 0; u < VU; ++u) acc[u] *= alpha;
         at_wave_sync();
-        // values: a page is HD rows of 16 keys; lane takes 8 keys (half a row) per load
+        // values: a page is HD rows of 16 keys; a lane holds 8 keys (half a row) per load
 #pragma unroll
-        for (int pg = 0; pg < AD_TILE / AT_PAGE; ++pg) {
-            int kbase = tile0 + pg * AT_PAGE;
-            if (kbase >= s_hi) break;
-            if (kbase + AT_PAGE <= lo) continue;
-            int page = bt[kbase / AT_PAGE];
-            int half = lane & 1;
-            int first = kbase + half * 8;
+        for (int pg = 0; pg < TP; ++pg) {
+            const int half = lane & 1;
+            const int first = tile0 + pg * AT_PAGE + half * 8;
             float pv[8];
 #pragma unroll
             for (int j = 0; j < 8; ++j) pv[j] = ps[wave][pg * AT_PAGE + half * 8 + j];
 #pragma unroll
             for (int u = 0; u < VU; ++u) {
-                int d = u * 32 + lane / 2;
-                bf16x8 vv = at_load8(v_cache + (((size_t)page * Hkv + kvh) * HD + d) * AT_PAGE + half * 8);
                 float sum = 0.f;
 #pragma unroll
                 for (int j = 0; j < 8; ++j) {
                     int key = first + j;                      // slots outside the data may hold anything
-                    float x = key >= lo && key < s_hi ? (float)vv[j] : 0.f;
+                    float x = key >= lo && key < s_hi ? (float)vreg[pg][u][j] : 0.f;
                     sum = fmaf(pv[j], x, sum);
                 }
                 acc[u] += sum;
             }
-        }
-    }
-    if (fused && wave == 0 && split == 0) {
-        // the token's own key and value: rotate the key, let one head of the group store both, and
-        // take them into this wave's sums straight from registers
-        float kn[8];
-        at_rotate8(fz.k_new + (size_t)t * fz.stride + (size_t)kvh * HD, dg, fz.table + (size_t)pos * fz.rot, fz.rot, kn);
-        const bf16_t* vrow = fz.v_new + (size_t)t * fz.stride + (size_t)kvh * HD;
-        const int slot = fz.slots[t];
-        if (slot >= 0 && h % (H / Hkv) == 0) {
-            const size_t page = slot / AT_PAGE, off = slot % AT_PAGE;
-            if (ks == 0) {
-                bf16x8 kb;
-#pragma unroll
-                for (int j = 0; j < 8; ++j) kb[j] = (bf16_t)kn[j];
-                *reinterpret_cast<bf16x8*>(fz.k_cache + ((page * Hkv + kvh) * AT_PAGE + off) * HD + dg * 8) = kb;
-            }
-            if ((lane & 1) == 0) {
-#pragma unroll
-                for (int u = 0; u < VU; ++u) {
-                    int d = u * 32 + lane / 2;
-                    fz.v_cache[((page * Hkv + kvh) * HD + d) * AT_PAGE + off] = vrow[d];
-                }
-            }
-        }
-        float dot = 0.f;
-#pragma unroll
-        for (int j = 0; j < 8; ++j) dot = fmaf(qf[j], kn[j], dot);
-#pragma unroll
-        for (int off = 1; off < LPK; off <<= 1) dot += __shfl_xor(dot, off, KA_WAVE);
-        float m_new = fmaxf(m_i, dot);
-        float alpha = exp2f(m_i - m_new);
-        float pn = exp2f(dot - m_new);
-        l_i = l_i * alpha + pn;
-        m_i = m_new;
-#pragma unroll
-        for (int u = 0; u < VU; ++u) {
-            float vn = (lane & 1) == 0 ? (float)vrow[u * 32 + lane / 2] : 0.f;
-            acc[u] = acc[u] * alpha + pn * vn;
         }
     }
     // the two halves of a channel row
@@ -598,6 +662,7 @@ KA_API int ka_attention_decode_bf16(const void* q, long q_row_stride, const void
         KA_CHECK(new_stride % 8 == 0 && (uintptr_t)k_new % 16 == 0 && (uintptr_t)v_new % 16 == 0, "ka_attention_decode_bf16: new key rows must be 16-byte aligned");
         fz = DecodeFuse{(const bf16_t*)k_new, (const bf16_t*)v_new, new_stride, table, rot, slots, (bf16_t*)k_cache_w, (bf16_t*)v_cache_w};
     }
+    if (hd == 128 && waves == 16) waves = 8;   // 16 waves leave 128 registers a lane: too few for a tile's loads
     dim3 grid(n, H, splits), block(KA_WAVE * waves);
 #define KA_AD(HDV, WV)                                                                                              \
     hipLaunchKernelGGL((attn_decode_kernel<HDV, WV>), grid, block, 0, stream, (const bf16_t*)q, q_row_stride,      \
@@ -606,7 +671,7 @@ KA_API int ka_attention_decode_bf16(const void* q, long q_row_stride, const void
     if (hd == 64) {
         if (waves == 4) KA_AD(64, 4); else if (waves == 8) KA_AD(64, 8); else KA_AD(64, 16);
     } else {
-        if (waves == 4) KA_AD(128, 4); else if (waves == 8) KA_AD(128, 8); else KA_AD(128, 16);
+        if (waves == 4) KA_AD(128, 4); else KA_AD(128, 8);
     }
 #undef KA_AD
     KA_LAUNCH_CHECK();

@@ -238,9 +238,16 @@ skinny_persistent_kernel(SkinnyArgs p, int total_strips) {
         const bf16_t* wp = W + (size_t)min(n0 + r % 8, N - 1) * ldw;
 #pragma unroll
         for (int u = 0; u < PER; ++u) w[slot][u] = sk_load8_stream(wp + wofs[u]);
-        // what the finishing lanes add at the end comes with the strip's weights (all waves ask
-        // for it: a load under a branch would break the stream)
-        floatx4 b4 = sk_bias4(bias, n0 + (g & 1) * 4, N);
+        // what the finishing lanes add at the end comes with the strip's weights. Every lane
+        // asks (a load under a branch would break the stream), but all except the finishing
+        // lanes of the strip's finishing wave ask for the bias's first line, which costs nothing
+        // (exactly one load whatever the bias is: the host sends biases that are not 16-byte
+        // aligned or whose N is no multiple of 4 to the split kernel, and "no bias" reads a
+        // line of the weights and throws it away)
+        const bool finisher = wave == i % SP_WAVES && lane < 32;
+        const float* bp = bias ? bias + (finisher ? min(n0 + (g & 1) * 4, N - 4) : 0) : reinterpret_cast<const float*>(Wa);
+        floatx4 b4 = *(const SK_GLOBAL floatx4*)bp;
+        if (!bias) b4 = floatx4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb) addend[slot][mb] = b4;
     };
@@ -553,10 +560,14 @@ static int launch_persistent_per(int per, int grid, size_t dyn, int strips, hipS
     return 1;
 }
 
-// Whether the persistent kernel takes these sizes.
-static bool persistent_fits(int M, int kblocks) {
+// Whether the persistent kernel takes these sizes and operands (it reads four bias values of a
+// strip with one aligned load).
+static bool persistent_bias_ok(const SkinnyTarget& t) {
+    return t.W == nullptr || t.bias == nullptr || (t.N % 4 == 0 && (uintptr_t)t.bias % 16 == 0);
+}
+static bool persistent_fits(int M, int kblocks, const SkinnyArgs& args) {
     const int per = ka_cdiv(kblocks, SP_WAVES);
-    return per <= (M <= 16 ? SP_MAX_PER : 4);
+    return per <= (M <= 16 ? SP_MAX_PER : 4) && persistent_bias_ok(args.a) && persistent_bias_ok(args.b);
 }
 
 static int launch_persistent(int strips, int M, int kblocks, bool ln, size_t dyn, hipStream_t stream,
@@ -654,12 +665,12 @@ KA_API int ka_linear_skinny_fused(const void* A1, long lda1, int K1, const void*
     if (ln) {
         const size_t dyn = (size_t)M * (K1 + SK_PAD) * sizeof(bf16_t);
         KA_CHECK(dyn <= 96 * 1024, "%s: %d rows of %d do not fit in LDS", who, M, K1);
-        KA_CHECK(persistent_fits(M, kblocks), "%s: K=%d is too wide for the LayerNorm prologue", who, K1);
+        KA_CHECK(persistent_fits(M, kblocks, args), "%s: K=%d or the biases do not suit the LayerNorm prologue", who, K1);
         if (launch_persistent(strips, M, kblocks, true, dyn, stream, args)) return -1;
         KA_LAUNCH_CHECK();
         return 0;
     }
-    if (!A2 && !accumulate_a && sk_persistent_enabled && persistent_fits(M, kblocks)) {
+    if (!A2 && !accumulate_a && sk_persistent_enabled && persistent_fits(M, kblocks, args)) {
         if (launch_persistent(strips, M, kblocks, false, 0, stream, args)) return -1;
         KA_LAUNCH_CHECK();
         return 0;

@@ -178,30 +178,42 @@ def linear_two_outputs(a, wa, ba, out_a, act_a, wb, bb, out_b, act_b) -> bool:
     return True
 
 
-def layernorm_linear_pair(x, gamma, beta, eps, wa, ba, out_a, act_a, wb, bb, out_b, act_b) -> bool:
-    """``h = LayerNorm(x)``; ``out_a = act_a(h @ wa.T + ba)``; ``out_b = act_b(h @ wb.T + bb)`` in one
-    launch: the kernel normalises the fp32 rows itself (at most 16 of them)."""
+def layernorm_linear(x, gamma, beta, eps, wa, ba, out_a, act_a, wb=None, bb=None, out_b=None, act_b=0) -> bool:
+    """``h = LayerNorm(x)``; ``out_a = act_a(h @ wa.T + ba)`` and, if a second target is given,
+    ``out_b = act_b(h @ wb.T + bb)`` in one launch: the kernel normalises the fp32 rows itself
+    (at most 16 of them, at most 2048 wide)."""
     m, k = x.shape
     if not (0 < m <= SKINNY_LN_MAX_ROWS) or k % 8 or k > SKINNY_LN_MAX_WIDTH or x.dtype != torch.float32 \
             or not x.is_contiguous():
         return False
     if x.data_ptr() % 16 or gamma.dtype != torch.float32 or gamma.numel() != k or gamma.data_ptr() % 16:
         return False
-    if beta is not None and (beta.dtype != torch.float32 or beta.numel() != k):
+    if beta is not None and (beta.dtype != torch.float32 or beta.numel() != k or beta.data_ptr() % 16):
         return False
-    na, nb = wa.shape[0], wb.shape[0]
-    if not (_operand_ok(wa, k) and _operand_ok(wb, k) and _out_ok(out_a, m, na) and _out_ok(out_b, m, nb)
-            and _bias_ok(ba, na) and _bias_ok(bb, nb)):
+    na = wa.shape[0]
+    if not (_operand_ok(wa, k) and _out_ok(out_a, m, na) and _bias_ok(ba, na)):
+        return False
+    two = wb is not None
+    nb = wb.shape[0] if two else 0
+    if two and not (_operand_ok(wb, k) and _out_ok(out_b, m, nb) and _bias_ok(bb, nb)):
         return False
     if m * (k + 8) * 2 > 96 * 1024:
         return False
+    for bias, n in ((ba, na), (bb, nb)):
+        if bias is not None and (n % 4 or bias.data_ptr() % 16):
+            return False
     _check(lib().ka_linear_skinny_fused(
         None, 0, k, None, 0, 0, None, 0, None,
         x.data_ptr(), gamma.data_ptr(), _ptr(beta), float(eps),
         wa.data_ptr(), wa.stride(0), _ptr(ba), out_a.data_ptr(), _OUT_CODE[out_a.dtype], out_a.stride(0), na, act_a, 0,
-        wb.data_ptr(), wb.stride(0), _ptr(bb), out_b.data_ptr(), _OUT_CODE[out_b.dtype], out_b.stride(0), nb, act_b,
+        _ptr(wb), wb.stride(0) if two else 0, _ptr(bb) if two else None, _ptr(out_b),
+        _OUT_CODE[out_b.dtype] if two else 0, out_b.stride(0) if two else 0, nb, act_b,
         m, SKINNY_TARGET_WAVES, stream_ptr()))
     return True
+
+
+def layernorm_linear_pair(x, gamma, beta, eps, wa, ba, out_a, act_a, wb, bb, out_b, act_b) -> bool:
+    return layernorm_linear(x, gamma, beta, eps, wa, ba, out_a, act_a, wb, bb, out_b, act_b)
 
 
 def decode_shape(max_kv: int):
