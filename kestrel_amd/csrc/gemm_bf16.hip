@@ -9,11 +9,13 @@
 // and stores them as one vector. Bias, GELU-tanh and the fp32 residual accumulate run in the
 // epilogue.
 //
-// The 2 x 2 wave tile (128 x 128 per workgroup) is used where it gives every CU two workgroups,
-// 2 x 1 otherwise; other shapes can be forced for measurements.
+// That kernel takes any K (in steps of 8); where K is a multiple of 64 the large-tile kernel
+// further down, which loads straight into LDS, is used instead.
 #include "ka_common.h"
 
 #include <stdlib.h>
+
+#include <type_traits>
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
@@ -162,6 +164,225 @@ gemm_bf16_kernel(const bf16_t* __restrict__ A, long lda, const bf16_t* __restric
     }
 }
 
+// ----------------------------------------------------------------------------
+// The large-tile kernel. Four (2 x 2) or eight (4 x 2) waves, each with WN x WM MFMA tiles of
+// 32 x 32. K-steps of BK go from global memory straight into LDS (global_load_lds_dwordx4: no
+// registers, no ds_write), NS stages, one barrier per step. Chunk c (16 bytes) of tile row r
+// lies at place c ^ swizzle(r) of its row, chosen by which chunk each lane of the load asks
+// for, so that the rows that one pass of a 16-byte LDS read touches fall on different banks
+// without padding. Rows past the end of a matrix are read from its last row (and never stored);
+// K must be a multiple of BK.
+// ----------------------------------------------------------------------------
+constexpr int gd_smem(int bn, int bm, int bk, int ns) { return ns * (bn + bm) * bk * 2; }
+
+// A loop whose index is a compile-time constant in every round (the accumulators are up to 256
+// registers: an index the compiler does not resolve would put them in memory).
+template <int I, int N, typename F>
+__device__ __forceinline__ void gd_static_for(F&& f) {
+    if constexpr (I < N) {
+        f(std::integral_constant<int, I>{});
+        gd_static_for<I + 1, N>(f);
+    }
+}
+
+#define GD_GLOBAL __attribute__((address_space(1)))
+#define GD_LDS __attribute__((address_space(3)))
+
+// s_waitcnt vmcnt(n) alone (gfx9 encoding: vmcnt in bits 3:0 and 15:14, the other counters at their maximum)
+template <int N>
+__device__ __forceinline__ void gd_wait_loads() {
+    __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | 0x0f70);
+}
+
+// The barrier alone, without the fence that __syncthreads() puts before it: that fence waits
+// for every load in flight, the younger stages' too. What must be ordered here is ordered by
+// hand: a wave has waited for its own loads of the stage (vmcnt) and for its LDS reads of the
+// stage before (their values were used) when it arrives.
+__device__ __forceinline__ void gd_barrier() {
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+}
+
+template <int WN, int WM, int GN, int GM, int BK, int NS>
+__global__ void __launch_bounds__(KA_WAVE * GN * GM)
+    __attribute__((amdgpu_waves_per_eu(GN * GM / 4, (WN * WM > 8 ? 1 : 2) * (GN * GM / 4))))
+gemm_dma_kernel(const bf16_t* __restrict__ A, long lda, const bf16_t* __restrict__ W, long ldw,
+                const float* __restrict__ bias, void* __restrict__ out, int out_dtype, long ldo, int M,
+                int N, int K, int act, int accumulate, int tiles_n, int tiles_m) {
+    static_assert(BK == 32 || BK == 64, "K-steps of 32 or 64");
+    static_assert(NS >= 2 && NS <= 4, "two to four stages");
+    static_assert(GN * GM == 4 || GN * GM == 8, "four or eight waves");
+    constexpr int WAVES = GN * GM;
+    constexpr int BN = 32 * WN * GN, BM = 32 * WM * GM;
+    constexpr int ROW = BK * 2;                          // bytes of a tile row
+    constexpr int CPR = BK / 8;                          // 16-byte chunks of a tile row
+    constexpr int RPL = KA_WAVE / CPR;                   // rows that one load of 1 KB brings
+    constexpr int STAGE = (BN + BM) * ROW;               // bytes of one stage: W rows, then X rows
+    constexpr int W_LOADS = BN / RPL / WAVES, X_LOADS = BM / RPL / WAVES;   // loads per wave and stage
+    static_assert(W_LOADS * RPL * WAVES == BN && X_LOADS * RPL * WAVES == BM, "the tile does not divide over the waves' loads");
+    constexpr int LPW = W_LOADS + X_LOADS;
+    extern __shared__ __attribute__((aligned(16))) unsigned char gb_lds[];
+    int pid = blockIdx.x;
+    int total = tiles_n * tiles_m;
+    int per_xcd = (total + 7) / 8;
+    int logical = (pid % 8) * per_xcd + pid / 8;
+    if (logical >= total) return;
+    int tn = logical / tiles_m, tm = logical % tiles_m;
+    const int n0 = tn * BN, m0 = tm * BM;
+    const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid / KA_WAVE), lane = tid % KA_WAVE;
+    const int wn = wave / GM, wm = wave % GM;
+    const int li = lane % 32, lg = lane / 32;
+
+    floatx16 acc[WN][WM];
+#pragma unroll
+    for (int a = 0; a < WN; ++a)
+#pragma unroll
+        for (int b = 0; b < WM; ++b)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[a][b][v] = 0.f;
+
+    // Chunk c of row r lies at place c ^ swizzle(r) of its row: with rows of 128 bytes the eight
+    // rows that one pass of a 16-byte LDS read touches then fall on different banks (r & 7); with
+    // rows of 64 bytes two rows share a bank line, so pairs of rows take turns ((r >> 1) & 3).
+    auto swizzle = [](int r) { return CPR == 8 ? (r & 7) : ((r >> 1) & 3); };
+    // What this lane asks for in a load of RPL rows: row lane / CPR of them, and the chunk that
+    // belongs at place lane % CPR of that row.
+    const int lrow = lane / CPR, lchunk = (lane % CPR) ^ swizzle(lrow);
+    const bf16_t* wsrc[W_LOADS];
+    const bf16_t* xsrc[X_LOADS];
+#pragma unroll
+    for (int i = 0; i < W_LOADS; ++i) {
+        int r = (wave * W_LOADS + i) * RPL + lrow;
+        wsrc[i] = W + (size_t)min(n0 + r, N - 1) * ldw + lchunk * 8;
+    }
+#pragma unroll
+    for (int i = 0; i < X_LOADS; ++i) {
+        int r = (wave * X_LOADS + i) * RPL + lrow;
+        xsrc[i] = A + (size_t)min(m0 + r, M - 1) * lda + lchunk * 8;
+    }
+    auto fetch = [&](int stage, int k0) {
+        unsigned char* base = gb_lds + stage * STAGE;
+#pragma unroll
+        for (int i = 0; i < W_LOADS; ++i)
+            __builtin_amdgcn_global_load_lds((const GD_GLOBAL void*)(wsrc[i] + k0),
+                                             (GD_LDS void*)(base + (wave * W_LOADS + i) * RPL * ROW), 16, 0, 0);
+#pragma unroll
+        for (int i = 0; i < X_LOADS; ++i)
+            __builtin_amdgcn_global_load_lds((const GD_GLOBAL void*)(xsrc[i] + k0),
+                                             (GD_LDS void*)(base + BN * ROW + (wave * X_LOADS + i) * RPL * ROW), 16, 0, 0);
+    };
+
+    // operand addresses inside a stage: tile row li of each of this wave's tiles; the k-chunk
+    // of k-step ks is ks * 2 + lg
+    int wrow_off[WN], xrow_off[WM];
+#pragma unroll
+    for (int a = 0; a < WN; ++a) wrow_off[a] = (wn * 32 * WN + a * 32 + li) * ROW;
+#pragma unroll
+    for (int b = 0; b < WM; ++b) xrow_off[b] = BN * ROW + (wm * 32 * WM + b * 32 + li) * ROW;
+    const int swz = swizzle(li);
+
+    // NS - 1 stages are on their way while one is multiplied. A wave waits for its own loads of
+    // the stage it needs (the younger ones may stay in flight), the barrier then tells it that
+    // everybody's have landed and that the stage read last has been left by all.
+    const int steps = K / BK;
+#pragma unroll
+    for (int st = 0; st < NS - 1; ++st)
+        if (st < steps) fetch(st, st * BK);
+    for (int s = 0; s < steps; ++s) {
+        const int younger = min(NS - 2, steps - 1 - s);          // stages asked for after stage s
+        if (NS >= 4 && younger >= 2) gd_wait_loads<2 * LPW>();
+        else if (NS >= 3 && younger >= 1) gd_wait_loads<LPW>();
+        else gd_wait_loads<0>();
+        gd_barrier();
+        if (s + NS - 1 < steps) fetch((s + NS - 1) % NS, (s + NS - 1) * BK);
+        const unsigned char* base = gb_lds + (s % NS) * STAGE;
+        bf16x8 wa[2][WN], xb[2][WM];
+        auto operands = [&](int slot, int ks) {
+            const int place = ((ks * 2 + lg) ^ swz) * 16;
+#pragma unroll
+            for (int a = 0; a < WN; ++a) wa[slot][a] = *reinterpret_cast<const bf16x8*>(base + wrow_off[a] + place);
+#pragma unroll
+            for (int b = 0; b < WM; ++b) xb[slot][b] = *reinterpret_cast<const bf16x8*>(base + xrow_off[b] + place);
+        };
+        operands(0, 0);
+#pragma unroll
+        for (int ks = 0; ks < BK / 16; ++ks) {
+            if (ks + 1 < BK / 16) operands((ks + 1) & 1, ks + 1);
+#pragma unroll
+            for (int a = 0; a < WN; ++a)
+#pragma unroll
+                for (int b = 0; b < WM; ++b)
+                    acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wa[ks & 1][a], xb[ks & 1][b], acc[a][b], 0, 0, 0);
+        }
+    }
+
+    // epilogue: acc[a][b][v] is out[m][n] with n = n0 + wn*32*WN + a*32 + (v/4)*8 + lg*4 + v%4,
+    // m = m0 + wm*32*WM + b*32 + li
+    const bool vec_ok = (N % 4 == 0) && (ldo % 4 == 0);
+    gd_static_for<0, WM>([&](auto bc) {
+        constexpr int b = decltype(bc)::value;
+        const int m = m0 + wm * 32 * WM + b * 32 + li;
+        gd_static_for<0, WN>([&](auto ac) {
+            constexpr int a = decltype(ac)::value;
+            gd_static_for<0, 4>([&](auto qc) {
+                constexpr int q = decltype(qc)::value;
+                const int n = n0 + wn * 32 * WN + a * 32 + q * 8 + lg * 4;
+                if (m >= M || n >= N) return;
+                float v[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    float x = acc[a][b][q * 4 + i];
+                    if (bias && n + i < N) x += bias[n + i];
+                    if (act == 1) x = ka_gelu_tanh(x);
+                    v[i] = x;
+                }
+                size_t o = (size_t)m * ldo + n;
+                if (out_dtype == KA_F32) {
+                    float* op = reinterpret_cast<float*>(out) + o;
+                    if (vec_ok) {
+                        floatx4 cur = accumulate ? *reinterpret_cast<floatx4*>(op) : floatx4{0.f, 0.f, 0.f, 0.f};
+                        floatx4 res = {cur[0] + v[0], cur[1] + v[1], cur[2] + v[2], cur[3] + v[3]};
+                        *reinterpret_cast<floatx4*>(op) = res;
+                    } else {
+                        for (int i = 0; i < 4 && n + i < N; ++i) op[i] = accumulate ? op[i] + v[i] : v[i];
+                    }
+                } else {
+                    bf16_t* op = reinterpret_cast<bf16_t*>(out) + o;
+                    if (vec_ok) {
+                        bf16x4 res = {(bf16_t)v[0], (bf16_t)v[1], (bf16_t)v[2], (bf16_t)v[3]};
+                        *reinterpret_cast<bf16x4*>(op) = res;
+                    } else {
+                        for (int i = 0; i < 4 && n + i < N; ++i) op[i] = (bf16_t)v[i];
+                    }
+                }
+            });
+        });
+    });
+}
+
+template <int WN, int WM, int GN, int GM, int BK, int NS>
+static int launch_dma(const bf16_t* A, long lda, const bf16_t* W, long ldw, const float* bias, void* out,
+                      int out_dtype, long ldo, int M, int N, int K, int act, int accumulate, hipStream_t stream) {
+    static bool configured = false;
+    constexpr int BN = 32 * WN * GN, BM = 32 * WM * GM;
+    constexpr int smem = gd_smem(BN, BM, BK, NS);
+    static_assert(smem <= 160 * 1024, "the stages do not fit in LDS");
+    if (!configured) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_dma_kernel<WN, WM, GN, GM, BK, NS>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+        KA_CHECK(e == hipSuccess, "ka_linear_tiled_bf16: cannot reserve %d bytes of LDS: %s", smem, hipGetErrorString(e));
+        configured = true;
+    }
+    int tiles_n = ka_cdiv(N, BN), tiles_m = ka_cdiv(M, BM);
+    long total = (long)tiles_n * tiles_m;
+    long launched = ((total + 7) / 8) * 8;
+    KA_CHECK(launched < (1L << 31), "ka_linear_tiled_bf16: too many tiles");
+    hipLaunchKernelGGL((gemm_dma_kernel<WN, WM, GN, GM, BK, NS>), dim3((unsigned)launched), dim3(KA_WAVE * GN * GM), smem,
+                       stream, A, lda, W, ldw, bias, out, out_dtype, ldo, M, N, K, act, accumulate, tiles_n, tiles_m);
+    return 0;
+}
+
 template <int NT, int MT, int BK>
 static int launch_config(const bf16_t* A, long lda, const bf16_t* W, long ldw, const float* bias, void* out,
                          int out_dtype, long ldo, int M, int N, int K, int act, int accumulate,
@@ -183,7 +404,7 @@ static int launch_config(const bf16_t* A, long lda, const bf16_t* W, long ldw, c
     return 0;
 }
 
-// `config`: 0 chooses by size; 421 / 221 / 211 force the 4x2 (BK 32), 2x2 (BK 64), 2x1 (BK 64) tile.
+// `config`: 0 chooses by size; other values force a tile (for measurements and tests).
 KA_API int ka_linear_tiled_bf16(const void* A, long lda, const void* W, long ldw, const float* bias,
                                 void* out, int out_dtype, long ldo, int M, int N, int K, int act,
                                 int accumulate, int config, hipStream_t stream) {
@@ -196,20 +417,35 @@ KA_API int ka_linear_tiled_bf16(const void* A, long lda, const void* W, long ldw
     KA_CHECK(!(accumulate && out_dtype != KA_F32), "ka_linear_tiled_bf16: accumulate needs an fp32 output");
     KA_CHECK((uintptr_t)out % 16 == 0, "ka_linear_tiled_bf16: output must be 16-byte aligned");
     if (config == 0) {
-        // the square tile unless it leaves fewer than two workgroups per CU (measured: the bigger
-        // 4 x 2 tile is slower at every size tried, the loop being bound by latency, not by LDS)
-        long t22 = (long)ka_cdiv(N, 128) * ka_cdiv(M, 128);
-        config = t22 >= 512 ? 221 : 211;
+        if (K % 64 == 0) {
+            // Tiles of 128 x 128 read 64 flops' worth of operands per byte from L2, which is what
+            // bounds them (measured: 11 TB/s of L2 traffic at 800 TFLOP/s); 256 x 256 halves that
+            // and wins where its tiles fill the CUs evenly, i.e. come in whole rounds of one per CU.
+            long t256 = (long)ka_cdiv(N, 256) * ka_cdiv(M, 256);
+            int cus = 256;
+            long rounds = (t256 + cus - 1) / cus;
+            config = t256 * 10 >= rounds * cus * 9 ? 22224 : 12222;
+        } else {
+            long t22 = (long)ka_cdiv(N, 128) * ka_cdiv(M, 128);
+            config = t22 >= 512 ? 221 : 211;
+        }
     }
     const bf16_t* a = (const bf16_t*)A;
     const bf16_t* w = (const bf16_t*)W;
     int rc;
     switch (config) {
-        case 421: rc = launch_config<4, 2, 32>(a, lda, w, ldw, bias, out, out_dtype, ldo, M, N, K, act, accumulate, stream); break;
         case 221: rc = launch_config<2, 2, 64>(a, lda, w, ldw, bias, out, out_dtype, ldo, M, N, K, act, accumulate, stream); break;
         case 211: rc = launch_config<2, 1, 64>(a, lda, w, ldw, bias, out, out_dtype, ldo, M, N, K, act, accumulate, stream); break;
-        case 222: rc = launch_config<2, 2, 32>(a, lda, w, ldw, bias, out, out_dtype, ldo, M, N, K, act, accumulate, stream); break;
-        case 441: rc = launch_config<4, 4, 32>(a, lda, w, ldw, bias, out, out_dtype, ldo, M, N, K, act, accumulate, stream); break;
+#define KA_DMA(CODE, WNV, WMV, GNV, GMV, BKV, NSV)                                                               \
+        case CODE:                                                                                                \
+            KA_CHECK(K % BKV == 0, "ka_linear_tiled_bf16: this tile needs K to be a multiple of %d", BKV);        \
+            rc = launch_dma<WNV, WMV, GNV, GMV, BKV, NSV>(a, lda, w, ldw, bias, out, out_dtype, ldo, M, N, K, act, accumulate, stream); \
+            break;
+        // 10000 (four waves, 2 x 2) or 20000 (eight waves, 4 x 2) + stages * 1000 + (K-step / 32) * 100 + wave tile
+        KA_DMA(12222, 2, 2, 2, 2, 64, 2)      // 128 x 128, two workgroups per CU
+        KA_DMA(22224, 2, 4, 4, 2, 64, 2)      // 256 x 256, one workgroup of eight waves per CU
+        KA_DMA(13122, 2, 2, 2, 2, 32, 3)      // (measured slower everywhere; kept as the test of three stages and K-steps of 32)
+#undef KA_DMA
         default: KA_CHECK(false, "ka_linear_tiled_bf16: unknown tile configuration %d", config);
     }
     if (rc) return rc;

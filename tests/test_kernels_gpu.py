@@ -176,6 +176,27 @@ def test_linear_tiled_bf16(shape):
     _linear_case(fn, m, n, k, bf, bf, bf, 0, False, lda=k + 8)
 
 
+@pytest.mark.parametrize("config", [12222, 22224, 13122])
+@pytest.mark.parametrize("shape", [(65, 128, 64), (300, 333, 512), (513, 700, 192), (2048, 512, 1024), (100, 2048, 2048), (70, 90, 32)])
+def test_linear_large_tile_bf16(shape, config, monkeypatch):
+    """The kernel that loads straight into LDS, at every wave tile, with ragged edges in M and N
+    (K in steps of 64)."""
+    from kestrel_amd.ops import fast
+
+    m, n, k = shape
+    bf, f32 = torch.bfloat16, torch.float32
+    if k % (32 * (config // 100 % 10)):
+        pytest.skip("K is no multiple of this tile's K-step")
+    monkeypatch.setattr(fast, "TILED_CONFIG", config)
+
+    def fn(a, w, bias, out, act, accumulate):
+        assert fast.linear_bf16(a, w, bias, out, act, accumulate)
+
+    for out_dtype, act, accumulate in [(bf, 0, False), (bf, 1, False), (f32, 0, True), (f32, 0, False)]:
+        _linear_case(fn, m, n, k, bf, bf, out_dtype, act, accumulate)
+    _linear_case(fn, m, n, k, bf, bf, bf, 0, False, lda=k + 8)
+
+
 def test_fast_linear_declines_what_it_does_not_cover():
     from kestrel_amd.ops import fast
 
