@@ -137,7 +137,7 @@ gemm_bf16_kernel(const bf16_t* __restrict__ A, long lda, const bf16_t* __restric
                 for (int i = 0; i < 4; ++i) {
                     float x = acc[a][b][q * 4 + i];
                     if (bias && n + i < N) x += bias[n + i];
-                    if (act == 1) x = ka_gelu_tanh(x);
+                    if (act == 1) x = ka_gelu_tanh_fast(x);
                     v[i] = x;
                 }
                 size_t o = (size_t)m * ldo + n;
@@ -320,6 +320,7 @@ gemm_dma_kernel(const bf16_t* __restrict__ A, long lda, const bf16_t* __restrict
     // epilogue: acc[a][b][v] is out[m][n] with n = n0 + wn*32*WN + a*32 + (v/4)*8 + lg*4 + v%4,
     // m = m0 + wm*32*WM + b*32 + li
     const bool vec_ok = (N % 4 == 0) && (ldo % 4 == 0);
+    const bool bias_vec = (N % 4 == 0) && (reinterpret_cast<uintptr_t>(bias) % 16 == 0);
     gd_static_for<0, WM>([&](auto bc) {
         constexpr int b = decltype(bc)::value;
         const int m = m0 + wm * 32 * WM + b * 32 + li;
@@ -329,12 +330,17 @@ gemm_dma_kernel(const bf16_t* __restrict__ A, long lda, const bf16_t* __restrict
                 constexpr int q = decltype(qc)::value;
                 const int n = n0 + wn * 32 * WN + a * 32 + q * 8 + lg * 4;
                 if (m >= M || n >= N) return;
+                floatx4 bv = {0.f, 0.f, 0.f, 0.f};
+                if (bias) {
+                    if (bias_vec) bv = *reinterpret_cast<const floatx4*>(bias + n);       // n + 3 < N: N % 4 == 0
+                    else
+                        for (int i = 0; i < 4 && n + i < N; ++i) bv[i] = bias[n + i];
+                }
                 float v[4];
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
-                    float x = acc[a][b][q * 4 + i];
-                    if (bias && n + i < N) x += bias[n + i];
-                    if (act == 1) x = ka_gelu_tanh(x);
+                    float x = acc[a][b][q * 4 + i] + bv[i];
+                    if (act == 1) x = ka_gelu_tanh_fast(x);
                     v[i] = x;
                 }
                 size_t o = (size_t)m * ldo + n;

@@ -125,7 +125,7 @@ __device__ __forceinline__ void sk_finish(const floatx4 (*red)[MB][KA_WAVE], con
         if (m >= M) continue;
         if (tg.act == 1) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) s[i] = ka_gelu_tanh(s[i]);
+            for (int i = 0; i < 4; ++i) s[i] = ka_gelu_tanh_fast(s[i]);
         }
         const size_t o = (size_t)m * tg.ldo + n;
         if (whole) {

@@ -69,4 +69,15 @@ __device__ __forceinline__ float ka_gelu_tanh(float x) {
     return 0.5f * x * (1.0f + tanhf(inner));
 }
 
+// The same with tanh(u) = 1 - 2 / (1 + e^(2u)) on the hardware's exponential: a few instructions
+// instead of the library routine's many. 1 + tanh is exact to about 1e-7, far below what a bf16
+// result keeps; the kernels that write bf16 activations use it.
+__device__ __forceinline__ float ka_gelu_tanh_fast(float x) {
+    const float k0 = 0.7978845608028654f;
+    const float k1 = 0.044715f;
+    float inner = k0 * (x + k1 * x * x * x);
+    float e = __expf(2.0f * inner);               // inf for large inner: 2 / inf = 0, tanh = 1
+    return x * (1.0f - __fdividef(1.0f, 1.0f + e));   // 0.5 x (1 + tanh) = x (1 - 1 / (1 + e))
+}
+
 static inline int ka_cdiv(long a, long b) { return (int)((a + b - 1) / b); }
