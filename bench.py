@@ -222,7 +222,8 @@ def main() -> int:
     step_bytes = weights + kv_bytes * (size / 2) + args.batch * typed.dim * size
     achieved = step_bytes / (elapsed / args.steps)
     record = {
-        "metric": "decode tok/s (Moondream 2 text decoder sizes, batch 8, context 1024)", "value": round(value, 1),
+        "metric": f"decode tok/s (Moondream 2 text decoder sizes, batch {args.batch}, context {CONTEXT})",
+        "value": round(value, 1),
         "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": args.dtype, "data": "synthetic (seeded random token ids and prefix embeddings, random weights N(0,0.02))",

@@ -108,9 +108,10 @@ __device__ __forceinline__ floatx4 sk_bias4(const float* bias, int n, int N) {
 
 // The finishing lanes (g in {0, 1}, r; with HALF r < 8) own out[m = mb * 16 + r][n0 + g * 4 + i]:
 // they add the waves' partial sums in wave order, then bias / old value, activation, store.
-template <int MB, bool HALF, int NW>
+// `mine(mb)` says whether the calling wave finishes block mb of 16 rows.
+template <int MB, bool HALF, int NW, typename Mine>
 __device__ __forceinline__ void sk_finish(const floatx4 (*red)[MB][KA_WAVE], const floatx4 (&addend)[MB],
-                                          const SkinnyTarget& tg, int n0, int M, int lane) {
+                                          const SkinnyTarget& tg, int n0, int M, int lane, Mine mine) {
     const int r = lane % 16, g = lane / 16;
     // the other half of an output element: MFMA rows 8..15, and with HALF columns 8..15 as well
     constexpr int OTHER = HALF ? 40 : 32;
@@ -118,6 +119,7 @@ __device__ __forceinline__ void sk_finish(const floatx4 (*red)[MB][KA_WAVE], con
     const bool whole = n + 3 < tg.N && tg.ldo % 4 == 0 && (reinterpret_cast<uintptr_t>(tg.out) & 15) == 0;
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
+        if (!mine(mb)) continue;
         floatx4 s = addend[mb];
 #pragma unroll
         for (int w = 0; w < NW; ++w) s += red[w][mb][lane] + red[w][mb][lane + OTHER];
@@ -240,11 +242,11 @@ skinny_persistent_kernel(SkinnyArgs p, int total_strips) {
         for (int u = 0; u < PER; ++u) w[slot][u] = sk_load8_stream(wp + wofs[u]);
         // what the finishing lanes add at the end comes with the strip's weights. Every lane
         // asks (a load under a branch would break the stream), but all except the finishing
-        // lanes of the strip's finishing wave ask for the bias's first line, which costs nothing
+        // lanes of the strip's finishing waves ask for the bias's first line, which costs nothing
         // (exactly one load whatever the bias is: the host sends biases that are not 16-byte
         // aligned or whose N is no multiple of 4 to the split kernel, and "no bias" reads a
         // line of the weights and throws it away)
-        const bool finisher = wave == i % SP_WAVES && lane < 32;
+        const bool finisher = (wave - i % SP_WAVES + SP_WAVES) % SP_WAVES < MB && lane < 32;
         const float* bp = bias ? bias + (finisher ? min(n0 + (g & 1) * 4, N - 4) : 0) : reinterpret_cast<const float*>(Wa);
         floatx4 b4 = *(const SK_GLOBAL floatx4*)bp;
         if (!bias) b4 = floatx4{0.f, 0.f, 0.f, 0.f};
@@ -321,11 +323,14 @@ skinny_persistent_kernel(SkinnyArgs p, int total_strips) {
         // One barrier per strip is enough: a buffer is written again two strips later, after the
         // barrier of the strip between, which the finishing wave reaches only when it has read it.
         __syncthreads();
-        if (wave != i % SP_WAVES || !finishing_lane) return;
+        // the strip's blocks of 16 rows are finished by waves i, i + 1, ... (mod 8), one each
+        const int turn = (wave - i % SP_WAVES + SP_WAVES) % SP_WAVES;
+        if (turn >= MB || !finishing_lane) return;
         const int strip = blockIdx.x + i * grid;
         const bool second = strip >= strips_a;
         const int n0 = (second ? strip - strips_a : strip) * SK_STRIP;
-        sk_finish<MB, HALF, SP_WAVES>(red[buf], addend[slot], second ? p.b : p.a, n0, M, lane);
+        sk_finish<MB, HALF, SP_WAVES>(red[buf], addend[slot], second ? p.b : p.a, n0, M, lane,
+                                      [turn](int mb) { return mb == turn; });
     };
 
     // Strip i + DEPTH - 1 is asked for before strip i is multiplied. No load of the loop stands
@@ -508,7 +513,7 @@ skinny_split_kernel(SkinnyArgs p) {
     for (int mb = 0; mb < MB; ++mb) red[wave][mb][lane] = HALF || g < 2 ? lo[mb] : hi[mb];
     __syncthreads();
     if (!finishing_lane) return;
-    sk_finish<MB, HALF, WAVES>(red, addend, tg, n0, M, lane);
+    sk_finish<MB, HALF, WAVES>(red, addend, tg, n0, M, lane, [](int) { return true; });
 }
 
 // ----------------------------------------------------------------------------
