@@ -426,11 +426,17 @@ KA_API int ka_linear_tiled_bf16(const void* A, long lda, const void* W, long ldw
         if (K % 64 == 0) {
             // Tiles of 128 x 128 read 64 flops' worth of operands per byte from L2, which is what
             // bounds them (measured: 11 TB/s of L2 traffic at 800 TFLOP/s); 256 x 256 halves that
-            // and wins where its tiles fill the CUs evenly, i.e. come in whole rounds of one per CU.
+            // and wins where its tiles fill most of the CUs in every round (measured inside the
+            // model at 2048 rows: N = 6144 and 8192). Where 128 x 128 tiles leave a CU with one
+            // workgroup only, eight waves and three stages hide the trip to HBM that two
+            // workgroups would otherwise hide for each other (N = 2048: 35 us of 120 at K = 8192).
+            const int cus = 256;
             long t256 = (long)ka_cdiv(N, 256) * ka_cdiv(M, 256);
-            int cus = 256;
+            long t128 = (long)ka_cdiv(N, 128) * ka_cdiv(M, 128);
             long rounds = (t256 + cus - 1) / cus;
-            config = t256 * 10 >= rounds * cus * 9 ? 22224 : 12222;
+            if (t256 * 10 >= rounds * cus * 7) config = 22224;
+            else if (t128 <= cus) config = 23212;
+            else config = 12222;
         } else {
             long t22 = (long)ka_cdiv(N, 128) * ka_cdiv(M, 128);
             config = t22 >= 512 ? 221 : 211;
@@ -449,8 +455,9 @@ KA_API int ka_linear_tiled_bf16(const void* A, long lda, const void* W, long ldw
             break;
         // 10000 (four waves, 2 x 2) or 20000 (eight waves, 4 x 2) + stages * 1000 + (K-step / 32) * 100 + wave tile
         KA_DMA(12222, 2, 2, 2, 2, 64, 2)      // 128 x 128, two workgroups per CU
+        KA_DMA(23212, 1, 2, 4, 2, 64, 3)      // 128 x 128 by eight waves, three stages: for one workgroup per CU
         KA_DMA(22224, 2, 4, 4, 2, 64, 2)      // 256 x 256, one workgroup of eight waves per CU
-        KA_DMA(13122, 2, 2, 2, 2, 32, 3)      // (measured slower everywhere; kept as the test of three stages and K-steps of 32)
+        KA_DMA(13122, 2, 2, 2, 2, 32, 3)      // (slower everywhere; kept as the test of K-steps of 32)
 #undef KA_DMA
         default: KA_CHECK(false, "ka_linear_tiled_bf16: unknown tile configuration %d", config);
     }
