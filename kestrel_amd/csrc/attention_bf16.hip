@@ -46,8 +46,11 @@ __device__ __forceinline__ void at_wave_sync() {
 constexpr int AP_WAVES = 4;                 // waves of a workgroup: all on the same 32 queries, keys interleaved
 constexpr int AP_QBLOCK = 32;               // queries per workgroup
 
+// (At least two waves per SIMD, except at head size 128, which needs more registers: with 256 registers a lane the compiler lets the MFMAs write
+// ordinary registers. Left to itself it puts their results in accumulator registers and then
+// spends a third of the loop's instructions moving them to where the softmax can read them.)
 template <int HD>
-__global__ void __launch_bounds__(KA_WAVE * AP_WAVES)
+__global__ void __launch_bounds__(KA_WAVE * AP_WAVES) __attribute__((amdgpu_waves_per_eu(HD <= 96 ? 2 : 1)))
 attn_prefill_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t* __restrict__ k_cache,
                     const bf16_t* __restrict__ v_cache, const int* __restrict__ block_table, int max_pages,
                     const int* __restrict__ qblk_row, const int* __restrict__ qblk_tok,
