@@ -387,6 +387,28 @@ def test_a_far_key_among_hundreds_is_found():
         _close(out[-1, :hd], prompt.v[0][target, 0].double(), bf)
 
 
+def test_a_windows_edge_is_kept():
+    """The key just outside a window lines up with the query far better than any other, the
+    first key inside it second best: a kernel that lets the edge slip by one returns the wrong
+    value. Edges on a page's first and last slot, on a tile's edge and in between."""
+    h, hkv, hd = 4, 4, 64
+    bf = torch.bfloat16
+    for window in (100, 101, 115, 132, 388, 389):
+        for q_len in (1, 130):
+            case = PagedCase([900], [q_len], h, hkv, hd, 16, bf, seed=21, window=window)
+            first = 900 - window                       # first key the last query sees
+            case.q[-1] *= 0
+            case.q[-1, :hd] = 4.0
+            for key, strength in ((first - 1, 6.0), (first, 3.0)):
+                case.k[0][key, 0] = strength
+                page = int(case.table[0, key // 16])
+                case.k_cache[page, 0, key % 16, :] = strength
+            for name in ("generic", "fast"):
+                out = _run_attention(case, name, hd ** -0.5)
+                _close(out[-1, :hd], case.v[0][first, 0].double(), bf)
+            _close(_run_attention(case, "fast", hd ** -0.5), case.reference(hd ** -0.5), bf)
+
+
 def test_argmax_and_sampling():
     from kestrel_amd.ops import core
     from kestrel_amd.sampling import Sampler, mix_key
