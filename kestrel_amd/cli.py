@@ -63,14 +63,17 @@ def _generate(args) -> int:
             return 2
         started = time.perf_counter()
         results = engine.generate_batch_sync(prompts, max_new_tokens=args.max_tokens, temperature=args.temperature,
-                                             top_p=args.top_p)
+                                             top_p=args.top_p, return_logprobs=args.logprobs,
+                                             suppressed_token_ids=_parse_ids(args.suppress_ids or ""))
         elapsed = time.perf_counter() - started
         for result in results:
-            print(json.dumps({"request_id": result.request_id, "tokens": result.tokens,
-                              "finish_reason": result.finish_reason, "input_tokens": result.metrics.input_tokens,
-                              "output_tokens": result.metrics.output_tokens,
-                              "ttft_ms": round(result.metrics.ttft_ms, 3),
-                              "decode_time_ms": round(result.metrics.decode_time_ms, 3)}))
+            record = {"request_id": result.request_id, "tokens": result.tokens,
+                      "finish_reason": result.finish_reason, "input_tokens": result.metrics.input_tokens,
+                      "output_tokens": result.metrics.output_tokens, "ttft_ms": round(result.metrics.ttft_ms, 3),
+                      "decode_time_ms": round(result.metrics.decode_time_ms, 3)}
+            if result.logprobs is not None:
+                record["logprobs"] = [round(lp, 6) for lp in result.logprobs]
+            print(json.dumps(record))
         total = sum(r.metrics.output_tokens for r in results)
         print(f"# {len(results)} requests, {total} tokens in {elapsed:.3f} s", file=sys.stderr)
     finally:
@@ -108,6 +111,8 @@ def main(argv=None) -> int:
     gen.add_argument("--prompt-file", help="JSON file with a list of prompts, each a list of token ids")
     gen.add_argument("--random-prompts", type=int, default=0, help="this many random prompts")
     gen.add_argument("--prompt-len", type=int, default=32, help="length of the random prompts")
+    gen.add_argument("--logprobs", action="store_true", help="also print the log-probability of every generated token")
+    gen.add_argument("--suppress-ids", help="token ids that must never be generated, e.g. '0,50256'")
     gen.add_argument("--max-tokens", type=int, default=16, help="tokens to generate per prompt")
     gen.add_argument("--temperature", type=float, default=0.0)
     gen.add_argument("--top-p", type=float, default=1.0)

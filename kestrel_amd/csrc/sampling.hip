@@ -215,5 +215,93 @@ KA_API int ka_sample(const float* logits, long ld, const float* temps, const flo
     return 0;
 }
 
+// ----------------------------------------------------------------------------
+// Masks before sampling (kestrel/scheduler/scheduler.py:2563-2604,2854-2927): tokens a request
+// suppresses get -inf; a request with an allow-list keeps only the tokens on it.
+// ----------------------------------------------------------------------------
+__global__ void suppress_kernel(float* __restrict__ logits, long ld, const int* __restrict__ rows,
+                                const int* __restrict__ tokens, int n, int V) {
+    int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    int token = tokens[i];
+    if (token >= 0 && token < V) logits[(size_t)rows[i] * ld + token] = -INFINITY;
+}
+
+// Row r keeps the tokens allowed[starts[r] .. starts[r + 1]) (sorted ascending); an empty list
+// means no restriction.
+__global__ void __launch_bounds__(256)
+allow_kernel(float* __restrict__ logits, long ld, const int* __restrict__ starts,
+             const int* __restrict__ allowed, int V) {
+    const int r = blockIdx.y;
+    const int lo0 = starts[r], hi0 = starts[r + 1];
+    if (hi0 <= lo0) return;
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < V; i += gridDim.x * blockDim.x) {
+        int lo = lo0, hi = hi0;            // first entry >= i
+        while (lo < hi) {
+            int mid = (lo + hi) >> 1;
+            if (allowed[mid] < i) lo = mid + 1; else hi = mid;
+        }
+        if (!(lo < hi0 && allowed[lo] == i)) logits[(size_t)r * ld + i] = -INFINITY;
+    }
+}
+
+KA_API int ka_suppress_tokens(float* logits, long ld, const int* rows, const int* tokens, int n, int V,
+                              hipStream_t stream) {
+    KA_CHECK(n >= 0 && V > 0 && ld >= V, "ka_suppress_tokens: bad sizes n=%d V=%d ld=%ld", n, V, ld);
+    if (n == 0) return 0;
+    hipLaunchKernelGGL(suppress_kernel, dim3((n + 255) / 256), dim3(256), 0, stream, logits, ld, rows, tokens, n, V);
+    KA_LAUNCH_CHECK();
+    return 0;
+}
+
+KA_API int ka_allow_tokens(float* logits, long ld, const int* starts, const int* allowed, int rows, int V,
+                           hipStream_t stream) {
+    KA_CHECK(rows >= 0 && V > 0 && ld >= V, "ka_allow_tokens: bad sizes rows=%d V=%d ld=%ld", rows, V, ld);
+    if (rows == 0) return 0;
+    int blocks = (V + 255) / 256;
+    if (blocks > 64) blocks = 64;
+    hipLaunchKernelGGL(allow_kernel, dim3(blocks, rows), dim3(256), 0, stream, logits, ld, starts, allowed, V);
+    KA_LAUNCH_CHECK();
+    return 0;
+}
+
+// ----------------------------------------------------------------------------
+// Log-probability of the chosen token (kestrel/scheduler/scheduler.py:3019-3042): with a
+// temperature above 1e-6, log softmax(logits / T)[token]; otherwise (greedy, or a row whose
+// normaliser is not finite) 0 if the token is the argmax and -inf if not.
+// ----------------------------------------------------------------------------
+__global__ void __launch_bounds__(SM_THREADS)
+logprob_kernel(const float* __restrict__ logits, long ld, const int* __restrict__ ids,
+               const float* __restrict__ temps, float* __restrict__ out, int V) {
+    __shared__ float sf[SM_WAVES];
+    __shared__ int si[SM_WAVES];
+    const int r = blockIdx.x;
+    const float* row = logits + (size_t)r * ld;
+    const int greedy = block_argmax(row, V, sf, si);
+    const float T = temps ? fmaxf(temps[r], 0.f) : 0.f;
+    const float eff = T > SM_GREEDY_EPS ? T : 1.0f;
+    const float mx = row[greedy] / eff;
+    float z = 0.f;
+    for (int i = threadIdx.x; i < V; i += SM_THREADS) z += expf(row[i] / eff - mx);
+    z = block_reduce_sum(z, sf);
+    if (threadIdx.x != 0) return;
+    const float normaliser = mx + logf(z);
+    const int id = ids[r];
+    const bool force_greedy = !(T > SM_GREEDY_EPS) || !isfinite(normaliser);
+    float lp;
+    if (force_greedy) lp = id == greedy ? 0.f : -INFINITY;
+    else lp = (id >= 0 && id < V ? row[id] / eff : -INFINITY) - normaliser;
+    out[r] = lp;
+}
+
+KA_API int ka_token_logprobs(const float* logits, long ld, const int* ids, const float* temps, float* out,
+                             int rows, int V, hipStream_t stream) {
+    KA_CHECK(rows >= 0 && V > 0 && ld >= V, "ka_token_logprobs: bad sizes rows=%d V=%d ld=%ld", rows, V, ld);
+    if (rows == 0) return 0;
+    hipLaunchKernelGGL(logprob_kernel, dim3(rows), dim3(SM_THREADS), 0, stream, logits, ld, ids, temps, out, V);
+    KA_LAUNCH_CHECK();
+    return 0;
+}
+
 // The uniform number the kernel draws, for tests and host-side replay.
 KA_API float ka_uniform_host(unsigned long long key, unsigned long long counter) { return ka_uniform(key, counter); }

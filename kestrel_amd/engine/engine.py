@@ -48,6 +48,7 @@ class EngineResult:
     finish_reason: str
     metrics: EngineMetrics
     output: Dict[str, object]
+    logprobs: Optional[List[float]] = None      # of the tokens, if the request asked for them
 
 
 @dataclass
@@ -184,7 +185,7 @@ class InferenceEngine:
         m = result.metrics
         out = EngineResult(result.request_id, result.tokens, result.finish_reason,
                            EngineMetrics(m.prompt_tokens, m.decode_tokens, m.prefill_time_ms, m.decode_time_ms, m.ttft_ms),
-                           {"tokens": result.tokens})
+                           {"tokens": result.tokens}, result.logprobs)
         if item.stream is not None:
             item.stream.put(None)
         item.future.set_result(out)
@@ -207,7 +208,8 @@ class InferenceEngine:
 
     # ------------------------------------------------------------------ requests
     def _make_request(self, prompt_ids, max_new_tokens, temperature, top_p, prefix_embeds, prefix_ids, stop_ids, seed,
-                      on_token) -> GenerationRequest:
+                      on_token, return_logprobs=False, suppress_next_token_ids=(), suppressed_token_ids=(),
+                      allowed_token_ids=None) -> GenerationRequest:
         if self._fatal is not None:
             raise RuntimeError("the engine has stopped after an error") from self._fatal
         if self._thread is None:
@@ -219,19 +221,29 @@ class InferenceEngine:
             request_id = self._next_id
             self._next_id += 1
         return GenerationRequest(request_id, list(prompt_ids), int(max_new_tokens), temperature, top_p, prefix_embeds,
-                                 tuple(prefix_ids), None if stop_ids is None else tuple(stop_ids), seed, on_token)
+                                 tuple(prefix_ids), None if stop_ids is None else tuple(stop_ids), seed, on_token,
+                                 return_logprobs=bool(return_logprobs),
+                                 suppress_next_token_ids=tuple(int(t) for t in suppress_next_token_ids or ()),
+                                 suppressed_token_ids=tuple(int(t) for t in suppressed_token_ids or ()),
+                                 allowed_token_ids=None if allowed_token_ids is None
+                                 else tuple(int(t) for t in allowed_token_ids))
 
     def submit_sync(self, prompt_ids: Sequence[int], *, max_new_tokens: int, temperature: Optional[float] = None,
                     top_p: Optional[float] = None, prefix_embeds: Optional[torch.Tensor] = None,
                     prefix_ids: Sequence[int] = (), stop_ids: Optional[Sequence[int]] = None,
-                    seed: Optional[int] = None, _stream: Optional["queue.Queue"] = None) -> Future:
-        """Queue a request; the returned future resolves to an ``EngineResult``."""
+                    seed: Optional[int] = None, _stream: Optional["queue.Queue"] = None, **sampling) -> Future:
+        """Queue a request; the returned future resolves to an ``EngineResult``. ``sampling`` takes
+        ``return_logprobs``, ``suppress_next_token_ids``, ``suppressed_token_ids`` and
+        ``allowed_token_ids`` (``kestrel/engine/core.py:556-597``)."""
+        unknown = set(sampling) - {"return_logprobs", "suppress_next_token_ids", "suppressed_token_ids", "allowed_token_ids"}
+        if unknown:
+            raise TypeError(f"unknown options: {sorted(unknown)}")
         on_token = None
         if _stream is not None:
             def on_token(token, index, _q=_stream):
                 _q.put((token, index))
         request = self._make_request(prompt_ids, max_new_tokens, temperature, top_p, prefix_embeds, prefix_ids,
-                                     stop_ids, seed, on_token)
+                                     stop_ids, seed, on_token, **sampling)
         future: Future = Future()
         future.request_id = request.request_id
         self._inbox.put(_Pending(request, future, _stream))
@@ -247,16 +259,22 @@ class InferenceEngine:
     async def submit(self, prompt_ids: Sequence[int], *, max_new_tokens: int, temperature: Optional[float] = None,
                      top_p: Optional[float] = None, prefix_embeds: Optional[torch.Tensor] = None,
                      prefix_ids: Sequence[int] = (), stop_ids: Optional[Sequence[int]] = None,
-                     seed: Optional[int] = None) -> EngineResult:
+                     seed: Optional[int] = None, **sampling) -> EngineResult:
         future = self.submit_sync(prompt_ids, max_new_tokens=max_new_tokens, temperature=temperature, top_p=top_p,
-                                  prefix_embeds=prefix_embeds, prefix_ids=prefix_ids, stop_ids=stop_ids, seed=seed)
+                                  prefix_embeds=prefix_embeds, prefix_ids=prefix_ids, stop_ids=stop_ids, seed=seed,
+                                  **sampling)
         return await asyncio.wrap_future(future)
 
     async def generate(self, prompt_ids: Sequence[int], *, settings: Optional[dict] = None, **options) -> EngineResult:
-        """``settings`` takes the reference's keys: ``temperature``, ``top_p``, ``max_tokens``."""
+        """``settings`` takes the reference's keys: ``temperature``, ``top_p``, ``max_tokens`` and the
+        private ``_logprobs`` and ``_suppress_next_token_ids`` (``kestrel/engine/core.py:556-597``)."""
         settings = dict(settings or {})
         if "max_tokens" in settings:
             options.setdefault("max_new_tokens", settings.pop("max_tokens"))
+        if "_logprobs" in settings:
+            options.setdefault("return_logprobs", bool(settings.pop("_logprobs")))
+        if "_suppress_next_token_ids" in settings:
+            options.setdefault("suppress_next_token_ids", settings.pop("_suppress_next_token_ids"))
         for key in ("temperature", "top_p"):
             if key in settings:
                 options.setdefault(key, settings.pop(key))

@@ -70,10 +70,11 @@ class LaunchedStep:
     rows: List[PlannedRow]
     ids: Optional[torch.Tensor]
     event: Optional["torch.cuda.Event"]
+    logprobs: Optional[torch.Tensor] = None
 
 
 class GenerationScheduler:
-    HOST_RING = 4
+    HOST_RING = 8
 
     def __init__(self, runner, sampler, max_batch_size: int, max_num_batched_tokens: int,
                  eos_token_ids: Tuple[int, ...] = (), max_positions: Optional[int] = None,
@@ -103,6 +104,8 @@ class GenerationScheduler:
             raise ValueError("temperature must be non-negative")
         if not 0 < request.top_p <= 1:
             raise ValueError("top_p must be in (0, 1]")
+        if request.allowed_token_ids is not None and len(request.allowed_token_ids) == 0:
+            raise ValueError("an allow-list needs at least one token")
         if request.prompt_length == 0:
             raise ValueError("a request needs at least one prompt token or embedding")
         if request.prompt_length >= self.max_positions:
@@ -218,19 +221,35 @@ class GenerationScheduler:
         self.steps += 1
         logits = self.runner.step([row.entry for row in plan.rows])
         sampled_rows = [row for row in plan.rows if row.samples]
-        ids = event = None
+        ids = event = logprobs = None
         if sampled_rows:
             requests = [row.seq.request for row in sampled_rows]
             temps = [r.temperature for r in requests]
             tops = [r.top_p for r in requests]
             seeds = [r.seed if r.seed is not None else r.request_id for r in requests]
             indices = [row.seq.launched for row in sampled_rows]
+            # masks: what a request never wants, and what it does not want as its first token
+            suppress = [(i, int(t)) for i, r in enumerate(requests) for t in r.suppressed_token_ids]
+            suppress += [(i, int(t)) for i, (row, r) in enumerate(zip(sampled_rows, requests))
+                         if row.seq.launched == 0 for t in r.suppress_next_token_ids]
+            allowed = [r.allowed_token_ids for r in requests]
+            extras = {}
+            if suppress:
+                extras["suppress"] = suppress
+            if any(a for a in allowed):
+                extras["allowed"] = allowed
+            if any(r.return_logprobs for r in requests):
+                extras["logprobs"] = True
             if self.pipeline_depth > 1:
-                ids = self.sampler.sample(logits, temps, tops, seeds, indices, slots=[row.seq.slot for row in sampled_rows])
+                extras["slots"] = [row.seq.slot for row in sampled_rows]
+            if extras.keys() - {"slots"}:
+                ids, logprobs = self.sampler.sample_step(logits, temps, tops, seeds, indices, **extras)
             else:
-                ids = self.sampler.sample(logits, temps, tops, seeds, indices)
+                ids = self.sampler.sample(logits, temps, tops, seeds, indices, **extras)
             if ids.is_cuda:
                 ids, event = self._to_host(ids)
+                if logprobs is not None:
+                    logprobs, event = self._to_host(logprobs)
         for row in plan.rows:
             seq = row.seq
             if row.kind == "prefill":
@@ -243,17 +262,18 @@ class GenerationScheduler:
                 self.prefilling.remove(seq)
                 self.running.append(seq)
                 seq.phase = RequestPhase.RUNNING
-        self._inflight.append(LaunchedStep(plan.rows, ids, event))
+        self._inflight.append(LaunchedStep(plan.rows, ids, event, logprobs))
 
-    def _to_host(self, ids: torch.Tensor):
-        """Start the copy of a step's tokens into pinned memory; the event tells when it is done."""
+    def _to_host(self, values: torch.Tensor):
+        """Start the copy of a step's tokens (or their log-probabilities) into pinned memory; the
+        event tells when it is done."""
         index = self._host_next
-        self._host_next = (index + 1) % self.HOST_RING       # more buffers than steps in flight
+        self._host_next = (index + 1) % self.HOST_RING       # more buffers than copies in flight
         buf = self._host_ids[index]
-        if buf is None or buf.numel() < ids.numel():
-            buf = self._host_ids[index] = torch.empty(max(ids.numel(), 256), dtype=torch.int32, pin_memory=True)
-        host = buf[:ids.numel()]
-        host.copy_(ids, non_blocking=True)
+        if buf is None or buf.numel() < values.numel():
+            buf = self._host_ids[index] = torch.empty(max(values.numel(), 256), dtype=torch.int32, pin_memory=True)
+        host = buf[:values.numel()].view(values.dtype)        # int32 or float32: four bytes either way
+        host.copy_(values, non_blocking=True)
         event = torch.cuda.Event()
         event.record()
         return host, event
@@ -262,6 +282,7 @@ class GenerationScheduler:
         if step.event is not None:
             step.event.synchronize()
         ids = step.ids.tolist() if step.ids is not None else []
+        logprobs = step.logprobs.tolist() if step.logprobs is not None else None
         now = time.perf_counter()
         at = 0
         for row in step.rows:
@@ -269,6 +290,7 @@ class GenerationScheduler:
                 continue
             seq = row.seq
             token = int(ids[at])
+            logprob = logprobs[at] if logprobs is not None else None
             at += 1
             seq.inflight -= 1
             if seq.finish_reason is not None:      # it stopped a step ago: this token is not part of it
@@ -277,6 +299,8 @@ class GenerationScheduler:
                 continue
             if row.kind == "prefill":
                 seq.first_token_at = now
+            if seq.request.return_logprobs and logprob is not None:
+                seq.logprobs.append(float(logprob))
             self._commit(seq, token, now)
 
     def _commit(self, seq: Sequence_, token: int, now: float) -> None:
@@ -307,7 +331,8 @@ class GenerationScheduler:
             prompt_tokens=seq.request.prompt_length, decode_tokens=len(seq.tokens),
             prefill_time_ms=(first - started) * 1e3, ttft_ms=(first - seq.submitted_at) * 1e3,
             decode_time_ms=(now - first) * 1e3)
-        self.completed.append(SchedulerResult(seq.request.request_id, list(seq.tokens), reason, metrics, error))
+        self.completed.append(SchedulerResult(seq.request.request_id, list(seq.tokens), reason, metrics, error,
+                                              list(seq.logprobs) if seq.request.return_logprobs else None))
 
     def _release(self, seq: Sequence_) -> None:
         if seq.slot is not None:

@@ -39,6 +39,11 @@ class GenerationRequest:
     stop_ids: Optional[Tuple[int, ...]] = None      # None: the model's end-of-sequence ids
     seed: Optional[int] = None                      # None: the request id
     on_token: Optional[Callable[[int, int], None]] = None   # (token, index) as they are committed
+    # masks before sampling and scores after it (``kestrel/scheduler/scheduler.py:2563-2604,3019-3042``)
+    return_logprobs: bool = False                   # the chosen tokens' log-probabilities come back too
+    suppress_next_token_ids: Sequence[int] = ()     # not to be the first generated token
+    suppressed_token_ids: Sequence[int] = ()        # never to be generated
+    allowed_token_ids: Optional[Sequence[int]] = None   # if given, the only tokens that may be generated
 
     @property
     def block_length(self) -> int:
@@ -67,6 +72,7 @@ class SchedulerResult:
     finish_reason: str              # "stop", "length" or "error"
     metrics: RequestMetrics
     error: Optional[str] = None
+    logprobs: Optional[List[float]] = None          # one per token, if the request asked for them
 
 
 @dataclass
@@ -78,6 +84,7 @@ class Sequence_:
     slot: Optional[int] = None
     fed: int = 0                                     # prompt places already run
     tokens: List[int] = field(default_factory=list)  # generated so far, as the host has read them
+    logprobs: List[float] = field(default_factory=list)
     launched: int = 0                                # tokens sampled on the device (>= len(tokens))
     inflight: int = 0                                # steps launched whose token the host has not read
     finish_reason: Optional[str] = None

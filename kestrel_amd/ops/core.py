@@ -32,6 +32,9 @@ _SIGNATURES = {
                              _c_void_p, _c_void_p, _c_void_p, _c_long, _c_float, _c_int, _c_int, _c_int, _c_int,
                              _c_int, _c_void_p],
     "ka_argmax": [_c_void_p, _c_long, _c_void_p, _c_int, _c_int, _c_void_p, _c_void_p, _c_int, _c_void_p],
+    "ka_suppress_tokens": [_c_void_p, _c_long, _c_void_p, _c_void_p, _c_int, _c_int, _c_void_p],
+    "ka_allow_tokens": [_c_void_p, _c_long, _c_void_p, _c_void_p, _c_int, _c_int, _c_void_p],
+    "ka_token_logprobs": [_c_void_p, _c_long, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_void_p],
     "ka_sample": [_c_void_p, _c_long, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int,
                   _c_void_p, _c_void_p, _c_int, _c_void_p],
 }
@@ -253,3 +256,42 @@ def sample(logits: torch.Tensor, temps: torch.Tensor, top_ps: Optional[torch.Ten
     _check(lib().ka_sample(logits.data_ptr(), logits.stride(0), temps.data_ptr(), _ptr(top_ps), rng_key.data_ptr(),
                            rng_counter.data_ptr(), out.data_ptr(), rows, vocab,
                            *_pending_args("sample", rows, pending, pending_at), stream_ptr()))
+
+
+def _logit_rows(who: str, logits: torch.Tensor):
+    _need(logits.dim() == 2 and logits.dtype == torch.float32 and logits.stride(1) == 1, f"{who}: logits must be fp32 rows")
+    return logits.shape
+
+
+def suppress_tokens(logits: torch.Tensor, rows: torch.Tensor, tokens: torch.Tensor) -> None:
+    """``logits[rows[i], tokens[i]] = -inf`` (ids outside the vocabulary are passed over)."""
+    _dev(logits, rows, tokens)
+    n_rows, vocab = _logit_rows("suppress_tokens", logits)
+    _need(rows.dtype == torch.int32 and tokens.dtype == torch.int32 and rows.numel() == tokens.numel()
+          and rows.is_contiguous() and tokens.is_contiguous(), "suppress_tokens: rows and tokens int32 of one length")
+    _check(lib().ka_suppress_tokens(logits.data_ptr(), logits.stride(0), rows.data_ptr(), tokens.data_ptr(),
+                                    rows.numel(), vocab, stream_ptr()))
+
+
+def allow_tokens(logits: torch.Tensor, starts: torch.Tensor, allowed: torch.Tensor) -> None:
+    """Row ``r`` keeps only the tokens ``allowed[starts[r]:starts[r + 1]]`` (sorted ascending);
+    a row with an empty list is left alone."""
+    _dev(logits, starts, allowed)
+    n_rows, vocab = _logit_rows("allow_tokens", logits)
+    _need(starts.dtype == torch.int32 and starts.numel() == n_rows + 1 and starts.is_contiguous(),
+          "allow_tokens: starts int32 [rows + 1]")
+    _need(allowed.dtype == torch.int32 and allowed.is_contiguous(), "allow_tokens: allowed int32")
+    _check(lib().ka_allow_tokens(logits.data_ptr(), logits.stride(0), starts.data_ptr(), allowed.data_ptr(), n_rows,
+                                 vocab, stream_ptr()))
+
+
+def token_logprobs(logits: torch.Tensor, ids: torch.Tensor, temps: Optional[torch.Tensor], out: torch.Tensor) -> None:
+    """Log-probability of ``ids[r]`` under ``softmax(logits[r] / T)``; greedy rows (``T <= 1e-6`` or
+    no temperatures) give 0 for the argmax and -inf otherwise."""
+    _dev(logits, ids, temps, out)
+    n_rows, vocab = _logit_rows("token_logprobs", logits)
+    _need(ids.dtype == torch.int32 and ids.numel() == n_rows and ids.is_contiguous(), "token_logprobs: ids int32 [rows]")
+    _need(temps is None or (temps.dtype == torch.float32 and temps.numel() == n_rows), "token_logprobs: temps fp32 [rows]")
+    _need(out.dtype == torch.float32 and out.numel() == n_rows and out.is_contiguous(), "token_logprobs: out fp32 [rows]")
+    _check(lib().ka_token_logprobs(logits.data_ptr(), logits.stride(0), ids.data_ptr(), _ptr(temps), out.data_ptr(),
+                                   n_rows, vocab, stream_ptr()))

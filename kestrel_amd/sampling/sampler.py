@@ -2,7 +2,9 @@
 
 Reference: ``kestrel/scheduler/scheduler.py:2929-2993``: all rows greedy -> argmax;
 otherwise per-row temperature and top-p, rows with temperature <= 1e-6 greedy
-(``scheduler.py:55``). The reference draws from one device generator seeded from
+(``scheduler.py:55``). Before that, tokens a request suppresses get -inf and a request with an
+allow-list keeps only the tokens on it (``scheduler.py:2563-2604,2854-2927``); after it, the
+log-probability of the chosen token can be had (``scheduler.py:3019-3042``). The reference draws from one device generator seeded from
 ``torch.seed()`` (``scheduler.py:404-405``) and is not reproducible; here every draw comes
 from a counter-based generator keyed by (engine seed, request seed, index of the token),
 so a request's tokens do not depend on what else is in the batch.
@@ -10,7 +12,7 @@ so a request's tokens do not depend on what else is in the batch.
 
 from __future__ import annotations
 
-from typing import List, Optional, Sequence
+from typing import List, Optional, Sequence, Tuple
 
 import numpy as np
 import torch
@@ -48,9 +50,9 @@ class Sampler:
         self._next = 0
 
     def _upload(self, columns: Sequence[np.ndarray]) -> List[torch.Tensor]:
-        """Per-row arguments (4- or 8-byte columns) to the device with one copy out of pinned memory."""
-        rows = len(columns[0])
-        words = [rows * (c.dtype.itemsize // 4) for c in columns]
+        """Small arguments (4- or 8-byte columns of any length) to the device with one copy out of
+        pinned memory."""
+        words = [len(c) * (c.dtype.itemsize // 4) for c in columns]
         padded = [(w + 3) & ~3 for w in words]                   # every column starts on 16 bytes
         total = sum(padded)
         index = self._next
@@ -80,32 +82,72 @@ class Sampler:
                request_seeds: Sequence[int], token_indices: Sequence[int],
                slots: Optional[Sequence[int]] = None) -> torch.Tensor:
         """One token id per row of fp32 ``logits``; int32 on the device."""
+        return self.sample_step(logits, temperatures, top_ps, request_seeds, token_indices, slots=slots)[0]
+
+    def sample_step(self, logits: torch.Tensor, temperatures: Sequence[float], top_ps: Sequence[float],
+                    request_seeds: Sequence[int], token_indices: Sequence[int],
+                    slots: Optional[Sequence[int]] = None,
+                    suppress: Sequence[Tuple[int, int]] = (),
+                    allowed: Optional[Sequence[Optional[Sequence[int]]]] = None,
+                    logprobs: bool = False) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+        """Masks, then one token id per row, then (if asked) the chosen tokens' log-probabilities.
+
+        ``suppress``: pairs (row, token) whose logit becomes -inf. ``allowed``: per row ``None`` or
+        the only tokens the row may choose. Both change ``logits`` in place. Returns int32 ids and
+        fp32 log-probabilities (or ``None``), both on the device.
+        """
         rows = logits.shape[0]
         if not (len(temperatures) == len(top_ps) == len(request_seeds) == len(token_indices) == rows):
             raise ValueError("sampling parameters must have one entry per row of logits")
         if slots is not None and (self.pending is None or len(slots) != rows):
             raise ValueError("slots need a pending table and one entry per row of logits")
+        if allowed is not None and len(allowed) != rows:
+            raise ValueError("allowed needs one entry per row of logits")
         out = torch.empty(rows, dtype=torch.int32, device=self.device)
         if rows == 0:
-            return out
+            return out, (torch.empty(0, dtype=torch.float32, device=self.device) if logprobs else None)
         greedy = all(t <= GREEDY_EPS for t in temperatures)
+        restrict = allowed is not None and any(a for a in allowed)
         columns: List[np.ndarray] = []
+        names: List[str] = []
+
+        def column(name: str, values, dtype) -> None:
+            names.append(name)
+            columns.append(np.asarray(values, dtype=dtype))
+
         if slots is not None:
-            columns.append(np.asarray(slots, dtype=np.int32))
+            column("slots", slots, np.int32)
+        if suppress:
+            column("suppress_rows", [r for r, _ in suppress], np.int32)
+            column("suppress_tokens", [t for _, t in suppress], np.int32)
+        if restrict:
+            starts, flat = [0], []
+            for a in allowed:
+                flat.extend(sorted(set(int(t) for t in a)) if a else [])
+                starts.append(len(flat))
+            column("allow_starts", starts, np.int32)
+            column("allow_tokens", flat, np.int32)
+        if not greedy or logprobs:
+            column("temps", temperatures, np.float32)
         if not greedy:
-            columns.append(np.asarray(temperatures, dtype=np.float32))
-            columns.append(np.asarray(top_ps, dtype=np.float32))
-            columns.append(np.asarray([_signed(mix_key(self.seed, s)) for s in request_seeds], dtype=np.int64))
-            columns.append(np.asarray(token_indices, dtype=np.int32))
-        args = self._upload(columns) if columns else []
-        pending_at = args.pop(0) if slots is not None else None
+            column("tops", top_ps, np.float32)
+            column("keys", [_signed(mix_key(self.seed, s)) for s in request_seeds], np.int64)
+            column("counters", token_indices, np.int32)
+        arg = dict(zip(names, self._upload(columns))) if columns else {}
+        if suppress:
+            core.suppress_tokens(logits, arg["suppress_rows"], arg["suppress_tokens"])
+        if restrict:
+            core.allow_tokens(logits, arg["allow_starts"], arg["allow_tokens"])
         pending = self.pending if slots is not None else None
         if greedy:
-            core.argmax(logits, out, pending, pending_at)
+            core.argmax(logits, out, pending, arg.get("slots"))
         else:
-            temps, tops, keys, counters = args
-            core.sample(logits, temps, tops, keys, counters, out, pending, pending_at)
-        return out
+            core.sample(logits, arg["temps"], arg["tops"], arg["keys"], arg["counters"], out, pending, arg.get("slots"))
+        chosen = None
+        if logprobs:
+            chosen = torch.empty(rows, dtype=torch.float32, device=self.device)
+            core.token_logprobs(logits, out, arg["temps"], chosen)
+        return out, chosen
 
     def greedy(self, logits: torch.Tensor, out: Optional[torch.Tensor] = None,
                slots: Optional[Sequence[int]] = None) -> torch.Tensor:

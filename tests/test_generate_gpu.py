@@ -95,6 +95,37 @@ def test_sampling_is_reproducible_and_independent_of_the_batch():
     assert all(0 <= t < cfg["vocab_size"] for r in mixed for t in r.tokens)
 
 
+@pytest.mark.parametrize("depth", [1, 2])
+def test_masks_and_logprobs_through_the_entry_point(depth):
+    """Greedy generation with the chosen tokens' log-probabilities, a token that may not come
+    first, tokens that may never come and an allow-list, against the plain implementation."""
+    name = "A"
+    cfg = helpers.flat_config(name)
+    weights = helpers.stored_weights(helpers.model_dir(name))
+    prompt = helpers.random_ids(975, 11, cfg["vocab_size"])
+    tokens, margins = plain.greedy_generate(cfg, weights, prompt, 6)
+    engine = _engine(name, "float32", pipeline_depth=depth)
+    try:
+        scored = engine.generate_sync(prompt, max_new_tokens=6, stop_ids=(), return_logprobs=True)
+        barred = engine.generate_sync(prompt, max_new_tokens=3, stop_ids=(), suppress_next_token_ids=[tokens[0]],
+                                      return_logprobs=True, temperature=0.7, top_p=1.0, seed=3)
+        never = engine.generate_sync(prompt, max_new_tokens=6, stop_ids=(), suppressed_token_ids=tokens[:2])
+        only = engine.generate_sync(prompt, max_new_tokens=6, stop_ids=(), allowed_token_ids=[3, 5, 8])
+    finally:
+        engine.shutdown_sync()
+    _assert_greedy(scored.tokens, tokens, margins, 1e-4, "with log-probabilities")
+    assert scored.logprobs == [0.0] * len(scored.tokens)            # greedy: the argmax has log-probability 0
+    assert barred.tokens[0] != tokens[0]
+    # its first token's score under softmax(logits / 0.7) with the barred token at -inf
+    logits = plain.forward(cfg, weights, prompt)[-1].clone()
+    logits[tokens[0]] = float("-inf")
+    expected = torch.log_softmax(logits.double() / 0.7, dim=-1)[barred.tokens[0]]
+    assert abs(barred.logprobs[0] - float(expected)) < 1e-3
+    assert len(barred.logprobs) == 3 and all(lp <= 0.0 for lp in barred.logprobs)
+    assert not set(never.tokens) & set(tokens[:2])
+    assert set(only.tokens) <= {3, 5, 8} and only.logprobs is None
+
+
 def test_stop_ids_max_tokens_and_errors():
     cfg = helpers.flat_config("A")
     weights = helpers.stored_weights(helpers.model_dir("A"))

@@ -443,6 +443,60 @@ def test_argmax_and_sampling():
     assert 0.0 <= core.uniform(mix_key(5, 42), 7) < 1.0
 
 
+def test_masks_before_sampling_and_logprobs_after():
+    """Vectors of the reference's own tests (``tests/scheduler/test_logprobs.py``): suppression
+    composes with an allow-list (``:923-939``); the log-probability of the chosen token follows the
+    sampling epsilon (``:899-920``: temperatures 0, 5e-7, 2e-6 give 0, -inf and the temperature-scaled
+    log-softmax); and both on a vocabulary that is no power of two against torch."""
+    from kestrel_amd.ops import core
+    from kestrel_amd.sampling import Sampler
+
+    sampler = Sampler(torch.device(DEV), seed=1)
+    logits = torch.tensor([[5.0, 4.0, 3.0]], device=DEV)
+    ids, _ = sampler.sample_step(logits, [0.0], [1.0], [0], [0], suppress=[(0, 0)], allowed=[[0, 1]])
+    assert ids.cpu().tolist() == [1]
+
+    logits = torch.tensor([[1.0, 0.0, -1.0], [1.0, 0.0, -1.0], [0.0, -1e-6, -2e-6]], device=DEV)
+    chosen = torch.tensor([0, 1, 1], dtype=torch.int32, device=DEV)
+    temps = torch.tensor([0.0, 5e-7, 2e-6], device=DEV)
+    out = torch.empty(3, device=DEV)
+    core.token_logprobs(logits, chosen, temps, out)
+    got = out.cpu()
+    expected = torch.log_softmax(logits[2].cpu().double() / 2e-6, dim=-1)[1]
+    assert got[0].item() == 0.0 and torch.isneginf(got[1]).item()
+    assert abs(got[2].item() - expected.item()) < 1e-5
+
+    torch.manual_seed(4)
+    big = (torch.randn(5, 1003) * 3).to(DEV)
+    work = big.clone()
+    rows = torch.tensor([0, 0, 3, 4], dtype=torch.int32, device=DEV)
+    tokens = torch.tensor([5, 1002, 0, 2000], dtype=torch.int32, device=DEV)     # the last lies outside: passed over
+    core.suppress_tokens(work, rows, tokens)
+    want = big.clone()
+    want[0, 5] = want[0, 1002] = want[3, 0] = float("-inf")
+    assert torch.equal(work, want)
+    starts = torch.tensor([0, 0, 3, 3, 3, 4], dtype=torch.int32, device=DEV)      # rows 1 and 4 are restricted
+    allowed = torch.tensor([7, 500, 1002, 64], dtype=torch.int32, device=DEV)
+    core.allow_tokens(work, starts, allowed)
+    keep = torch.full_like(want, float("-inf"))
+    keep[1, [7, 500, 1002]] = want[1, [7, 500, 1002]]
+    keep[4, 64] = want[4, 64]
+    want[1], want[4] = keep[1], keep[4]
+    assert torch.equal(work, want)
+    temps = torch.tensor([0.7, 1.0, 0.0, 1.3, 2.0], device=DEV)
+    chosen = torch.tensor([9, 500, int(want[2].argmax()), 11, 64], dtype=torch.int32, device=DEV)
+    out = torch.empty(5, device=DEV)
+    core.token_logprobs(work, chosen, temps, out)
+    ref = []
+    for r in range(5):
+        t = float(temps[r])
+        if t <= 1e-6:
+            ref.append(0.0)
+        else:
+            ref.append(float(torch.log_softmax(want[r].cpu().double() / t, dim=-1)[int(chosen[r])]))
+    assert torch.allclose(out.cpu().double(), torch.tensor(ref, dtype=torch.float64), atol=2e-5, rtol=1e-5)
+
+
 @pytest.mark.parametrize("shape", [(8, 2048, 2048, 8192), (1, 40, 64, 200), (16, 2048, 2048, 8192), (33, 96, 120, 320),
                                    (64, 256, 8, 72)])
 def test_two_segment_skinny_linear(shape):

@@ -52,6 +52,14 @@ class FakeRunner:
 class FakeSampler:
     """Token = 10 + index of the token in its request; request seed 99 emits the stop id 0 at index 2."""
 
+    def __init__(self):
+        self.calls = []
+
+    def sample_step(self, logits, temps, tops, seeds, indices, slots=None, suppress=(), allowed=None, logprobs=False):
+        self.calls.append(dict(suppress=list(suppress), allowed=allowed, logprobs=logprobs, indices=list(indices)))
+        ids = self.sample(logits, temps, tops, seeds, indices, slots)
+        return ids, (torch.tensor([-0.5 * (i + 1) for i in indices]) if logprobs else None)
+
     def sample(self, logits, temps, tops, seeds, indices, slots=None):
         assert logits.shape[0] == len(temps) == len(indices)
         assert slots is None or len(slots) == len(indices)
@@ -250,3 +258,23 @@ def test_a_finished_request_makes_room_one_step_later_when_pipelined():
     results = sched.run_until_done()
     assert [r.request_id for r in results] == [0, 1] and all(r.tokens == [10, 11] for r in results)
     assert max(len(step) for step in runner.steps) == 1
+
+
+# ---------------------------------------------------------------------- masks and scores
+@pytest.mark.parametrize("depth", [1, 2])
+def test_masks_and_logprobs_reach_the_sampler(depth):
+    sched, runner = _scheduler(pipeline_depth=depth)
+    sched.enqueue_request(_req(0, 3, 3, return_logprobs=True, suppress_next_token_ids=(7, 8), suppressed_token_ids=(5,)))
+    sched.enqueue_request(_req(1, 4, 2, allowed_token_ids=(10, 11, 12)))
+    sched.enqueue_request(_req(2, 2, 2))
+    results = {r.request_id: r for r in sched.run_until_done()}
+    calls = sched.sampler.calls
+    # first step: all three prompts end; request 0 is row 0 and suppresses 5 always and 7, 8 for its first token
+    assert sorted(calls[0]["suppress"]) == [(0, 5), (0, 7), (0, 8)]
+    assert calls[0]["allowed"] == [None, (10, 11, 12), None] and calls[0]["logprobs"] is True
+    # afterwards only the lasting suppression is left
+    assert all(sorted(c["suppress"]) == [(0, 5)] for c in calls[1:] if c["suppress"])
+    assert results[0].logprobs == [-0.5, -1.0, -1.5] and len(results[0].tokens) == 3
+    assert results[1].logprobs is None and results[2].logprobs is None
+    with pytest.raises(ValueError, match="allow-list"):
+        sched.enqueue_request(_req(3, 2, 2, allowed_token_ids=()))
