@@ -152,45 +152,51 @@ __device__ __forceinline__ void sk_finish(const floatx4 (*red)[MB][KA_WAVE], con
 
 // LayerNorm of rows wave, wave + NW, ... of fp32 x [M, K] into LDS as bf16 [M][K + SK_PAD]
 // (statistics in fp32, two passes over a row kept in registers: K <= SK_XV * 256).
-template <int NW>
-__device__ __forceinline__ void sk_layernorm_rows(const SkinnyArgs& p, bf16_t* xs, int wave, int lane) {
-    const int K = p.K[0], M = p.M, ld = K + SK_PAD;
-    for (int m = wave; m < M; m += NW) {
-        const float* src = p.ln_x + (size_t)m * K;
-        floatx4 xv[SK_XV], gm[SK_XV], bt[SK_XV];
-        float s = 0.f;
-        // the row, and the scale and shift that meet it, in one trip to memory
+// A row to be normalised, with the scale and shift that meet it: fetched in one trip to memory
+// (sk_fetch_row) and turned into bf16 in LDS later (sk_normalise_row), so that other loads can
+// be issued in between without standing in front of these in the wave's queue.
+struct RowOperands {
+    floatx4 x[SK_XV], gamma[SK_XV], beta[SK_XV];
+};
+
+__device__ __forceinline__ void sk_fetch_row(const SkinnyArgs& p, int m, int lane, RowOperands& row) {
+    const int K = p.K[0];
+    const float* src = p.ln_x + (size_t)m * K;
 #pragma unroll
-        for (int j = 0; j < SK_XV; ++j) {
-            const int k = min((j * KA_WAVE + lane) * 4, K - 4);
-            xv[j] = *reinterpret_cast<const floatx4*>(src + k);
-            gm[j] = *reinterpret_cast<const floatx4*>(p.ln_gamma + k);
-            bt[j] = p.ln_beta ? *reinterpret_cast<const floatx4*>(p.ln_beta + k) : floatx4{0.f, 0.f, 0.f, 0.f};
+    for (int j = 0; j < SK_XV; ++j) {
+        const int k = min((j * KA_WAVE + lane) * 4, K - 4);
+        row.x[j] = *reinterpret_cast<const floatx4*>(src + k);
+        row.gamma[j] = *reinterpret_cast<const floatx4*>(p.ln_gamma + k);
+        row.beta[j] = p.ln_beta ? *reinterpret_cast<const floatx4*>(p.ln_beta + k) : floatx4{0.f, 0.f, 0.f, 0.f};
+    }
+}
+
+__device__ __forceinline__ void sk_normalise_row(const SkinnyArgs& p, bf16_t* xs, int m, int lane, RowOperands& row) {
+    const int K = p.K[0], ld = K + SK_PAD;
+    float s = 0.f;
+#pragma unroll
+    for (int j = 0; j < SK_XV; ++j) {
+        if ((j * KA_WAVE + lane) * 4 >= K) row.x[j] = floatx4{0.f, 0.f, 0.f, 0.f};
+        s += (row.x[j][0] + row.x[j][1]) + (row.x[j][2] + row.x[j][3]);
+    }
+    float mean = ka_wave_sum(s) / (float)K;
+    float q = 0.f;
+#pragma unroll
+    for (int j = 0; j < SK_XV; ++j) {
+        if ((j * KA_WAVE + lane) * 4 < K) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) q += (row.x[j][i] - mean) * (row.x[j][i] - mean);
         }
+    }
+    float rstd = 1.0f / sqrtf(ka_wave_sum(q) / (float)K + p.ln_eps);
 #pragma unroll
-        for (int j = 0; j < SK_XV; ++j) {
-            if ((j * KA_WAVE + lane) * 4 >= K) xv[j] = floatx4{0.f, 0.f, 0.f, 0.f};
-            s += (xv[j][0] + xv[j][1]) + (xv[j][2] + xv[j][3]);
-        }
-        float mean = ka_wave_sum(s) / (float)K;
-        float q = 0.f;
+    for (int j = 0; j < SK_XV; ++j) {
+        const int k = (j * KA_WAVE + lane) * 4;
+        if (k < K) {
+            bf16x4 y;
 #pragma unroll
-        for (int j = 0; j < SK_XV; ++j) {
-            if ((j * KA_WAVE + lane) * 4 < K) {
-#pragma unroll
-                for (int i = 0; i < 4; ++i) q += (xv[j][i] - mean) * (xv[j][i] - mean);
-            }
-        }
-        float rstd = 1.0f / sqrtf(ka_wave_sum(q) / (float)K + p.ln_eps);
-#pragma unroll
-        for (int j = 0; j < SK_XV; ++j) {
-            const int k = (j * KA_WAVE + lane) * 4;
-            if (k < K) {
-                bf16x4 y;
-#pragma unroll
-                for (int i = 0; i < 4; ++i) y[i] = (bf16_t)((xv[j][i] - mean) * rstd * gm[j][i] + bt[j][i]);
-                *reinterpret_cast<bf16x4*>(xs + m * ld + k) = y;
-            }
+            for (int i = 0; i < 4; ++i) y[i] = (bf16_t)((row.x[j][i] - mean) * rstd * row.gamma[j][i] + row.beta[j][i]);
+            *reinterpret_cast<bf16x4*>(xs + m * ld + k) = y;
         }
     }
 }
@@ -254,7 +260,14 @@ skinny_persistent_kernel(SkinnyArgs p, int total_strips) {
         for (int mb = 0; mb < MB; ++mb) addend[slot][mb] = b4;
     };
 
-    // the first strips' weights are on their way while the activations come in
+    // The first strips' weights are on their way while the activations come in. A wave's loads
+    // come back in the order in which it asked, so the row that it is to normalise is asked for
+    // before the weights: the LayerNorm would otherwise wait for them.
+    RowOperands row;
+    if constexpr (LN) {
+        if (wave < M) sk_fetch_row(p, wave, lane, row);
+        __builtin_amdgcn_sched_barrier(0);
+    }
     issue(0, 0);
     if (DEPTH == 3 && mine > 1) issue(1, 1);
 
@@ -263,7 +276,12 @@ skinny_persistent_kernel(SkinnyArgs p, int total_strips) {
     bf16x8 x[PER][MB][XH];
     if constexpr (LN) {
         bf16_t* xs = reinterpret_cast<bf16_t*>(sk_dyn);
-        sk_layernorm_rows<SP_WAVES>(p, xs, wave, lane);
+        __builtin_amdgcn_sched_barrier(0);
+        if (wave < M) sk_normalise_row(p, xs, wave, lane, row);
+        for (int m = wave + SP_WAVES; m < M; m += SP_WAVES) {
+            sk_fetch_row(p, m, lane, row);
+            sk_normalise_row(p, xs, m, lane, row);
+        }
         __syncthreads();
         const int ld = K + SK_PAD;
 #pragma unroll

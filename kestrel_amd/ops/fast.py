@@ -81,10 +81,10 @@ def lib():
     return _lib
 
 
-def set_skinny_persistent(enabled: bool) -> None:
-    """Whether one-segment skinny linears use the persistent kernel (activations in registers,
-    workgroups walking over strips) where it fits: on by default; off is for measurements and
-    for tests of the kernel that otherwise only takes what the persistent one does not."""
+def set_skinny_persistent(enabled: int) -> None:
+    """Whether one-segment skinny linears may use the persistent kernel where it fits (1, the
+    default) or all go to the split kernel (0): for measurements, and for tests of the split kernel
+    on sizes that it otherwise never sees."""
     lib().ka_skinny_set_persistent(int(enabled))
 
 

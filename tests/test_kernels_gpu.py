@@ -120,7 +120,7 @@ def test_linear_generic(shape):
     _linear_case(core.linear_generic, m, n, k, f32, f32, f32, 0, False, lda=k + 5)      # strided rows
 
 
-@pytest.mark.parametrize("persistent", [True, False])
+@pytest.mark.parametrize("persistent", [1, 0])
 @pytest.mark.parametrize("shape", [(1, 48, 64), (8, 2048, 2048), (5, 100, 200), (16, 6144, 2048), (33, 77, 8192),
                                    (64, 51200, 512), (17, 2048, 8192), (3, 16, 8), (9, 20000, 1032), (40, 4100, 2048),
                                    (8, 1000, 4096), (12, 515, 3000), (64, 9000, 1024)])
@@ -142,7 +142,7 @@ def test_linear_skinny_bf16(shape, persistent):
             _linear_case(fn, m, n, k, bf, bf, out_dtype, act, accumulate)
         _linear_case(fn, m, n, k, bf, bf, bf, 0, False, lda=k + 16)
     finally:
-        fast.set_skinny_persistent(True)
+        fast.set_skinny_persistent(1)
 
 
 def test_linear_skinny_is_the_same_on_every_run():
@@ -519,7 +519,8 @@ def test_two_segment_skinny_linear(shape):
     _close(out2, ref - b1.double() - b2.double(), torch.float32, scale=200)
 
 
-@pytest.mark.parametrize("shape", [(8, 2048, 6144, 8192), (1, 64, 40, 24), (16, 320, 100, 200), (5, 2048, 48, 8)])
+@pytest.mark.parametrize("shape", [(8, 2048, 6144, 8192), (1, 64, 40, 24), (16, 320, 100, 200), (5, 2048, 48, 8),
+                                   (12, 1000, 24, 20000), (3, 2048, 8192, 16384)])
 def test_layernorm_prologue_skinny_linear(shape):
     """LayerNorm, then two linears from the normalised rows, in one launch."""
     from kestrel_amd.ops import fast
