@@ -45,6 +45,7 @@ __device__ __forceinline__ void at_wave_sync() {
 // ----------------------------------------------------------------------------------------------
 constexpr int AP_WAVES = 4;                 // waves of a workgroup: all on the same 32 queries, keys interleaved
 constexpr int AP_QBLOCK = 32;               // queries per workgroup
+constexpr int AP_MAX_TABLE = 24576;         // block table entries of one row that fit in LDS beside the merge (393k keys)
 
 // (At least two waves per SIMD, except at head size 128, which needs more registers: with 256 registers a lane the compiler lets the MFMAs write
 // ordinary registers. Left to itself it puts their results in accumulator registers and then
@@ -56,14 +57,18 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_
                     const int* __restrict__ qblk_row, const int* __restrict__ qblk_tok,
                     const int* __restrict__ cu_q, const int* __restrict__ kv_len,
                     const int* __restrict__ kv_lo, const int* __restrict__ kv_hi, bf16_t* __restrict__ out,
-                    long out_row_stride, float scale, int H, int Hkv) {
+                    long out_row_stride, float scale, int H, int Hkv, int table_entries) {
     constexpr int QC = HD / 16;          // 16-byte chunks of half a head row = MFMA steps of the score product
     constexpr int DB = HD / 32;          // 32-channel blocks of the output
     constexpr int REC = DB * 16 + 2;     // floats a lane hands over at the merge: its outputs, m and l
     __shared__ float mrg[AP_WAVES - 1][REC][KA_WAVE];
-    __shared__ int pages[AT_LDS_PAGES];
-    const int blk = blockIdx.x, h = blockIdx.y;
-    const int wave = threadIdx.x / KA_WAVE, lane = threadIdx.x % KA_WAVE;
+    extern __shared__ int pages[];       // the row's block table: `table_entries` of them
+    // Heads are the fast index of the grid: the workgroups that run side by side then have the
+    // same amount of work (the host lists the blocks of queries with the most keys first, so
+    // the launch ends with the short ones), and an XCD, which gets every eighth workgroup,
+    // keeps to the keys and values of a few heads.
+    const int h = blockIdx.x, blk = blockIdx.y;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / KA_WAVE), lane = threadIdx.x % KA_WAVE;
     const int li = lane % 32, lg = lane / 32;
     const int kvh = h / (H / Hkv);
     const int row = qblk_row[blk];
@@ -80,15 +85,18 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_
         wave_lo = min(wave_lo, __shfl_xor(wave_lo, off, KA_WAVE));
     }
     const int limit = kv_len[row];       // keys of this row that hold data
-    wave_hi = min(wave_hi, limit);
+    // (the same in every lane: told to the compiler, which then counts tiles and looks up whole
+    // pages in scalar registers)
+    wave_hi = __builtin_amdgcn_readfirstlane(min(wave_hi, limit));
+    wave_lo = __builtin_amdgcn_readfirstlane(wave_lo);
     // The row's block table goes to LDS once: a look-up per tile in global memory would put a
-    // second trip to memory in front of every load of keys and values.
-    const int* bt = block_table + (size_t)row * max_pages;
-    const int n_pages = (limit + AT_PAGE - 1) / AT_PAGE;
-    if (n_pages <= AT_LDS_PAGES) {
+    // second trip to memory in front of every load of keys and values. (The host sees to it that
+    // the table is long enough for every row of the launch.)
+    const int n_pages = min((limit + AT_PAGE - 1) / AT_PAGE, table_entries);
+    {
+        const int* bt = block_table + (size_t)row * max_pages;
         for (int i = threadIdx.x; i < n_pages; i += KA_WAVE * AP_WAVES) pages[i] = bt[i];
         __syncthreads();
-        bt = pages;
     }
 
     // queries: lane (q = li, g = lg) holds channels [g * HD/2, (g + 1) * HD/2)
@@ -107,54 +115,75 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_
     const float sl2 = scale * AT_LOG2E;
     const int kperm = (li & 16) | ((li & 4) << 1) | ((li & 8) >> 1) | (li & 3);
 
+    // Every load of the loop is issued whether its tile exists or not, from an address moved
+    // inside the row's live keys: a load under a branch would make the compiler wait for
+    // everything in flight, and the loop would pay a trip to the cache per tile.
+    const int last_live = n_pages * AT_PAGE < limit ? n_pages * AT_PAGE - 1 : limit - 1;   // (inside the table in LDS, whatever the host said)
+    const int first_live = min(wave_lo, last_live);                  // pages below wave_lo may have been given back
+    const size_t page_stride = (size_t)Hkv * AT_PAGE * HD;           // elements of a page, keys or values
+    const unsigned k_lane = (unsigned)(kvh * AT_PAGE * HD + lg * (HD / 2));
+    const unsigned v_lane = (unsigned)((kvh * HD + li) * AT_PAGE + lg * 8);
+
     // half a key row of tile `key0` for this lane's (permuted) key
     auto load_keys = [&](int key0, bf16x8* dst) {
-        int key = max(min(key0 + kperm, limit - 1), wave_lo);   // pages below wave_lo may have been given back
-        int page = bt[key / AT_PAGE];
-        const bf16_t* kp = k_cache + (((size_t)page * Hkv + kvh) * AT_PAGE + key % AT_PAGE) * HD + lg * (HD / 2);
+        unsigned key = (unsigned)min(max(key0 + kperm, first_live), last_live);
+        unsigned page = (unsigned)pages[key / AT_PAGE];
+        const bf16_t* kp = k_cache + ((size_t)page * page_stride + (k_lane + (key % AT_PAGE) * HD));
 #pragma unroll
         for (int c = 0; c < QC; ++c) dst[c] = at_load8(kp + c * 8);
     };
 
     // the two value pages of tile `key0`: lane (d = li, g) loads 8 consecutive keys of channel d.
-    // `tail`: the tile reaches past the row's data, whose slots may hold anything: keep them out.
-    auto load_values = [&](int key0, bool tail, bf16x8 (*dst)[DB]) {
+    // The page is the same for all lanes: its address is made in scalar registers.
+    auto load_values = [&](int key0, bf16x8 (*dst)[DB]) {
+#pragma unroll
+        for (int pg = 0; pg < 2; ++pg) {
+            unsigned kbase = (unsigned)min(max(key0 + pg * AT_PAGE, first_live), last_live);
+            unsigned page = (unsigned)__builtin_amdgcn_readfirstlane(pages[kbase / AT_PAGE]);
+            const bf16_t* vp = v_cache + (size_t)page * page_stride;
+#pragma unroll
+            for (int db = 0; db < DB; ++db) dst[pg][db] = at_load8(vp + (v_lane + db * 32 * AT_PAGE));
+        }
+    };
+    // what of them may be used: nothing of a page outside the wave's keys (another page was
+    // loaded in its place), and nothing past the row's data, whose slots may hold anything
+    auto mask_values = [&](int key0, bf16x8 (*dst)[DB]) {
+        const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
         for (int pg = 0; pg < 2; ++pg) {
             int kbase = key0 + pg * AT_PAGE;
             bool live = kbase < wave_hi && kbase + AT_PAGE > wave_lo;
-            int page = live ? bt[kbase / AT_PAGE] : 0;
-            const bf16_t* vp = v_cache + (((size_t)page * Hkv + kvh) * HD + li) * AT_PAGE + lg * 8;
+            int first = kbase + lg * 8;      // first of the 8 keys this lane loaded
 #pragma unroll
             for (int db = 0; db < DB; ++db) {
-                bf16x8 vv = {0, 0, 0, 0, 0, 0, 0, 0};
-                if (live) vv = at_load8(vp + db * 32 * AT_PAGE);
-                dst[pg][db] = vv;
-            }
-            if (tail) {
-                int first = kbase + lg * 8;      // first of the 8 keys this lane loads
-#pragma unroll
-                for (int db = 0; db < DB; ++db)
+                if (!live) dst[pg][db] = zero;
+                else if (kbase + AT_PAGE > limit) {
 #pragma unroll
                     for (int j = 0; j < 8; ++j)
                         if (first + j >= limit) dst[pg][db][j] = (bf16_t)0.f;
+                }
             }
         }
     };
 
     // lowest end and highest start of the visible ranges of the wave's queries: a tile inside
     // [max_lo, min_hi) is seen whole by every query and needs no mask
-    int min_hi = q_valid ? hi : 0, max_lo = q_valid ? lo : 0x7fffffff;
+    int min_hi = q_valid ? hi : 0x7fffffff, max_lo = q_valid ? lo : 0;
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) {
         min_hi = min(min_hi, __shfl_xor(min_hi, off, KA_WAVE));
         max_lo = max(max_lo, __shfl_xor(max_lo, off, KA_WAVE));
     }
+    min_hi = __builtin_amdgcn_readfirstlane(min_hi);
+    max_lo = __builtin_amdgcn_readfirstlane(max_lo);
 
-    // one tile of 32 keys whose key rows are in `kr`
-    auto process = [&](int key0, const bf16x8* kr) {
+    constexpr int STRIDE = 32 * AP_WAVES;
+    // one tile of 32 keys whose key rows are in `kr`; the next tile's go to `kr_next`
+    auto process = [&](int key0, const bf16x8* kr, bf16x8* kr_next) {
         bf16x8 vr[2][DB];
-        load_values(key0, key0 + 32 > limit, vr);          // in flight during the scores and the softmax
+        load_values(key0, vr);                             // in flight during the scores and the softmax
+        load_keys(key0 + STRIDE, kr_next);                 // in flight until the next tile
+        __builtin_amdgcn_sched_barrier(0);
         floatx16 s;
 #pragma unroll
         for (int v = 0; v < 16; ++v) s[v] = 0.f;
@@ -193,6 +222,7 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_
                 for (int v = 0; v < 16; ++v) o[db][v] *= alpha;
         }
         // O^T[d][query] += V^T[d][key] P^T[key][query], one page per MFMA
+        if (key0 + 32 > min(wave_hi, limit) || key0 < wave_lo) mask_values(key0, vr);
 #pragma unroll
         for (int pg = 0; pg < 2; ++pg)
 #pragma unroll
@@ -202,17 +232,14 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_
 
     // two tiles per round, their key rows in two sets of registers: the next tile's keys are
     // always in flight while a tile is processed
-    constexpr int STRIDE = 32 * AP_WAVES;
     bf16x8 ka[QC], kb[QC];
     int key0 = (wave_lo & ~31) + wave * 32;
-    if (key0 < wave_hi) load_keys(key0, ka);
+    load_keys(key0, ka);
     while (key0 < wave_hi) {
-        if (key0 + STRIDE < wave_hi) load_keys(key0 + STRIDE, kb);
-        process(key0, ka);
+        process(key0, ka, kb);
         key0 += STRIDE;
         if (key0 >= wave_hi) break;
-        if (key0 + STRIDE < wave_hi) load_keys(key0 + STRIDE, ka);
-        process(key0, kb);
+        process(key0, kb, ka);
         key0 += STRIDE;
     }
     // the waves took different keys of the same queries: merge in wave order
@@ -613,16 +640,34 @@ KA_API int ka_attention_prefill_bf16(const void* q, long q_row_stride, const voi
                                      const int* block_table, int max_pages, const int* qblk_row,
                                      const int* qblk_tok, int n_qblocks, const int* cu_q, const int* kv_len,
                                      const int* kv_lo, const int* kv_hi, void* out, long out_row_stride,
-                                     float scale, int H, int Hkv, int hd, int page_size, hipStream_t stream) {
+                                     float scale, int H, int Hkv, int hd, int page_size, int longest_row,
+                                     hipStream_t stream) {
     if (check_common("ka_attention_prefill_bf16", q, q_row_stride, out, out_row_stride, n_qblocks, H, Hkv, hd,
                      page_size, max_pages))
         return -1;
     KA_CHECK(ka_attention_prefill_supported(hd, page_size), "ka_attention_prefill_bf16: head size %d not covered", hd);
-    dim3 grid(n_qblocks, H), block(KA_WAVE * AP_WAVES);
+    // `longest_row`: no row of the launch holds more keys than this (0: not known, the whole
+    // width of the block table is kept in LDS)
+    int table_entries = max_pages;
+    if (longest_row > 0 && ka_cdiv(longest_row, AT_PAGE) < max_pages) table_entries = ka_cdiv(longest_row, AT_PAGE);
+    KA_CHECK(table_entries <= AP_MAX_TABLE, "ka_attention_prefill_bf16: a row of %d keys is longer than the %d this kernel takes",
+             table_entries * AT_PAGE, AP_MAX_TABLE * AT_PAGE);
+    const size_t table_bytes = (size_t)table_entries * sizeof(int);
+    KA_CHECK(n_qblocks <= 65535, "ka_attention_prefill_bf16: more than 65535 blocks of queries in one launch");
+    dim3 grid(H, n_qblocks), block(KA_WAVE * AP_WAVES);
 #define KA_AP(HDV)                                                                                                  \
-    hipLaunchKernelGGL(attn_prefill_kernel<HDV>, grid, block, 0, stream, (const bf16_t*)q, q_row_stride,            \
+    {                                                                                                               \
+        static bool configured = false;                                                                             \
+        if (!configured) {                                                                                          \
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(attn_prefill_kernel<HDV>),             \
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, AP_MAX_TABLE * sizeof(int)); \
+            KA_CHECK(e == hipSuccess, "ka_attention_prefill_bf16: cannot reserve LDS: %s", hipGetErrorString(e));   \
+            configured = true;                                                                                      \
+        }                                                                                                           \
+    }                                                                                                               \
+    hipLaunchKernelGGL(attn_prefill_kernel<HDV>, grid, block, table_bytes, stream, (const bf16_t*)q, q_row_stride,  \
                        (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, max_pages, qblk_row, qblk_tok,  \
-                       cu_q, kv_len, kv_lo, kv_hi, (bf16_t*)out, out_row_stride, scale, H, Hkv)
+                       cu_q, kv_len, kv_lo, kv_hi, (bf16_t*)out, out_row_stride, scale, H, Hkv, table_entries)
     switch (hd) {
         case 32: KA_AP(32); break;
         case 64: KA_AP(64); break;

@@ -242,24 +242,26 @@ gemm_dma_kernel(const bf16_t* __restrict__ A, long lda, const bf16_t* __restrict
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[a][b][v] = 0.f;
 
-    // Chunk c of row r lies at place c ^ swizzle(r) of its row: with rows of 128 bytes the eight
-    // rows that one pass of a 16-byte LDS read touches then fall on different banks (r & 7); with
-    // rows of 64 bytes two rows share a bank line, so pairs of rows take turns ((r >> 1) & 3).
-    auto swizzle = [](int r) { return CPR == 8 ? (r & 7) : ((r >> 1) & 3); };
+    // Chunk c of row r lies at place c ^ swizzle(r) of its row. One pass of a 16-byte LDS read
+    // serves 16 lanes, which here read the same chunk of 16 consecutive rows, and the 64 banks
+    // hold 256 bytes: two rows of 128 bytes, so rows of the same parity must differ in their
+    // place ((r >> 1) & 7), or four rows of 64 bytes ((r >> 2) & 3). (Measured with r & 7: half
+    // of the LDS cycles were bank conflicts, rows r and r + 8 meeting in one pass.)
+    auto swizzle = [](int r) { return CPR == 8 ? ((r >> 1) & 7) : ((r >> 2) & 3); };
     // What this lane asks for in a load of RPL rows: row lane / CPR of them, and the chunk that
     // belongs at place lane % CPR of that row.
-    const int lrow = lane / CPR, lchunk = (lane % CPR) ^ swizzle(lrow);
+    const int lrow = lane / CPR;
     const bf16_t* wsrc[W_LOADS];
     const bf16_t* xsrc[X_LOADS];
 #pragma unroll
     for (int i = 0; i < W_LOADS; ++i) {
         int r = (wave * W_LOADS + i) * RPL + lrow;
-        wsrc[i] = W + (size_t)min(n0 + r, N - 1) * ldw + lchunk * 8;
+        wsrc[i] = W + (size_t)min(n0 + r, N - 1) * ldw + ((lane % CPR) ^ swizzle(r)) * 8;
     }
 #pragma unroll
     for (int i = 0; i < X_LOADS; ++i) {
         int r = (wave * X_LOADS + i) * RPL + lrow;
-        xsrc[i] = A + (size_t)min(m0 + r, M - 1) * lda + lchunk * 8;
+        xsrc[i] = A + (size_t)min(m0 + r, M - 1) * lda + ((lane % CPR) ^ swizzle(r)) * 8;
     }
     auto fetch = [&](int stage, int k0) {
         unsigned char* base = gb_lds + stage * STAGE;

@@ -247,10 +247,12 @@ class ModelRunner:
 
         qblk_row: List[int] = []
         qblk_tok: List[int] = []
-        for r in range(n_rows):
-            for first in range(cu_q[r], cu_q[r + 1], self.QUERY_BLOCK):
-                qblk_row.append(r)
-                qblk_tok.append(first)
+        blocks = [(r, first) for r in range(n_rows) for first in range(cu_q[r], cu_q[r + 1], self.QUERY_BLOCK)]
+        # the blocks that see the most keys first: a launch then ends with short ones
+        blocks.sort(key=lambda b: -max(kv_hi[b[1]:min(b[1] + self.QUERY_BLOCK, cu_q[b[0] + 1])]))
+        for r, first in blocks:
+            qblk_row.append(r)
+            qblk_tok.append(first)
         # one packed int32 buffer, every section starting on a 16-byte boundary
         sections: List[Tuple[str, List[int]]] = [
             ("ids", ids), ("positions", positions), ("token_row", token_row), ("kv_hi", kv_hi),

@@ -30,7 +30,7 @@ _SIGNATURES = {
                              _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
     "ka_attention_prefill_bf16": [_c_void_p, _c_long, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p,
                                   _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_long, _c_float,
-                                  _c_int, _c_int, _c_int, _c_int, _c_void_p],
+                                  _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
     "ka_attention_decode_bf16": [_c_void_p, _c_long, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p,
                                  _c_void_p, _c_void_p, _c_long, _c_float, _c_int, _c_int, _c_int, _c_int, _c_int,
                                  _c_int, _c_int, _c_void_p, _c_long, _c_void_p, _c_int,
@@ -282,6 +282,7 @@ def attention_bf16(q, k_cache, v_cache, block_table, token_row, kv_lo, kv_hi, ou
             q.data_ptr(), q.stride(0), k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(),
             block_table.shape[1], batch.qblk_row.data_ptr(), batch.qblk_tok.data_ptr(), int(batch.qblk_row.numel()),
             batch.cu_q.data_ptr(), batch.kv_len.data_ptr(), _ptr(kv_lo), kv_hi.data_ptr(), out.data_ptr(),
-            out.stride(0), float(scale), n_heads, n_kv_heads, head_dim, page_size, stream_ptr()))
+            out.stride(0), float(scale), n_heads, n_kv_heads, head_dim, page_size,
+            int(batch.max_kv) if batch.max_kv > 1 else 0, stream_ptr()))
         return True
     return False
