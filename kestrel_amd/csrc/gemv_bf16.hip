@@ -535,6 +535,219 @@ skinny_split_kernel(SkinnyArgs p) {
 }
 
 // ----------------------------------------------------------------------------
+// The wide kernel, for 17 to 64 rows. With that many rows the activations are what the kernels
+// above read most of: every strip of 8 weight rows meets all of them, from L2. Here a workgroup
+// of eight waves takes eight neighbouring strips and a part of K, brings the activations of that
+// part into LDS once (in chunks of 256 k, two buffers in turn) and every
+// wave multiplies its own strip with them; the parts of K meet in fp32 partial sums that a
+// second kernel adds up, in the order of the parts, with bias, activation and the output's old
+// value. Nothing crosses between workgroups inside a launch.
+//
+// LDS layout of a chunk: row m is 512 bytes, its 16-byte unit u lies at place u ^ (m & 15): the
+// 16 lanes that one pass of an MFMA operand read serves (16 rows, the same unit) then fall on 16
+// different bank groups.
+// ----------------------------------------------------------------------------
+constexpr int WD_WAVES = 8;        // strips of a workgroup
+constexpr int WD_CB = 4;           // k-blocks of a chunk
+constexpr int WD_DEPTH = 2;        // chunks of weights in flight per wave
+constexpr int WD_ROW_BYTES = WD_CB * SK_KBLOCK * 2;
+
+struct WideArgs {
+    const bf16_t* A[2];     // [M, K[s]] per segment (A[1] null: one segment)
+    long lda[2];
+    const bf16_t* W[2];     // [N, K[s]]
+    long ldw[2];
+    int K[2];
+    int M, N, splits;
+    float* partial;         // [splits, M, N]
+};
+
+// (Two workgroups per CU, which is what hides the trips to memory: at most 128 registers.)
+template <int MB>
+__global__ void __launch_bounds__(WD_WAVES * KA_WAVE) __attribute__((amdgpu_waves_per_eu(4, 4)))
+skinny_wide_kernel(WideArgs p) {
+    constexpr int ROWS = MB * 16;
+    constexpr int XL = ROWS / 2 / WD_WAVES;            // loads of two rows per wave and chunk
+    static_assert(XL * 2 * WD_WAVES == ROWS, "the rows of a chunk divide over the waves' loads");
+    __shared__ __attribute__((aligned(16))) unsigned char xs[2][ROWS * WD_ROW_BYTES];
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / KA_WAVE), lane = threadIdx.x % KA_WAVE;
+    const int r = lane % 16, g = lane / 16;
+    const int M = p.M, N = p.N;
+    const int split = blockIdx.y;
+    const int n0 = (blockIdx.x * WD_WAVES + wave) * SK_STRIP;
+    const int koff = (r / 8) * 32 + g * 8;
+    const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+    const int K0 = sk_pinned(p.K[0]), K1 = sk_pinned(p.K[1]);
+
+    // this part's k-blocks of each segment, and its chunks: segment 0's first
+    int kb_lo[2], kb_hi[2], chunks[2];
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+        const int nb = p.A[s] ? ((s ? K1 : K0) + SK_KBLOCK - 1) / SK_KBLOCK : 0;
+        const int per = (nb + p.splits - 1) / p.splits;
+        kb_lo[s] = min(split * per, nb);
+        kb_hi[s] = min(kb_lo[s] + per, nb);
+        chunks[s] = (kb_hi[s] - kb_lo[s] + WD_CB - 1) / WD_CB;
+    }
+    const int n_chunks = chunks[0] + chunks[1];
+
+    const size_t wrow = (size_t)min(n0 + r % 8, N - 1);
+    const bf16_t* const wrow0 = p.W[0] + wrow * p.ldw[0];
+    const bf16_t* const wrow1 = p.A[1] ? p.W[1] + wrow * p.ldw[1] : wrow0;
+    // what this lane brings of a chunk's activations: of the two rows 2 * (wave * XL + i) + lane / 32
+    // the unit lane % 32, which goes to place unit ^ (row & 15)
+    const bf16_t* const a0 = sk_pinned(p.A[0]);
+    const bf16_t* const a1 = sk_pinned(p.A[1] ? p.A[1] : p.A[0]);
+    const long lda0 = sk_pinned(p.lda[0]), lda1 = sk_pinned(p.A[1] ? p.lda[1] : p.lda[0]);
+    int xm[XL], xplace[XL];
+#pragma unroll
+    for (int i = 0; i < XL; ++i) {
+        const int m = (wave * XL + i) * 2 + lane / 32;
+        xplace[i] = m * WD_ROW_BYTES + (((lane % 32) ^ (m & 15)) * 16);
+        xm[i] = min(m, M - 1);
+    }
+
+    // Where chunk c lies: first k-block, end of the part, segment. A chunk past the end is the
+    // last one again: every load below is issued in every round, under no condition, so that the
+    // compiler's counts of loads in flight are exact.
+    auto chunk_of = [&](int c, int& kb, int& kb_end, int& seg) {
+        const int cc = max(min(c, n_chunks - 1), 0);
+        seg = chunks[1] > 0 && cc >= chunks[0];
+        kb = kb_lo[seg] + (seg ? cc - chunks[0] : cc) * WD_CB;
+        kb_end = c < n_chunks ? kb_hi[seg] : kb;
+    };
+    bf16x8 xr[XL];
+    auto fetch_x = [&](int c) {
+        int kb, kb_end, seg;
+        chunk_of(c, kb, kb_end, seg);
+        const int Ks = seg ? K1 : K0;
+#pragma unroll
+        for (int i = 0; i < XL; ++i)
+            xr[i] = sk_load8((seg ? a1 : a0) + ((size_t)xm[i] * (seg ? lda1 : lda0) + min(kb * SK_KBLOCK + (lane % 32) * 8, Ks - 8)));
+    };
+    // activations past the part's end or past the end of K go to LDS as zeros (the weights that
+    // meet them are then some other place of their row)
+    auto store_x = [&](int buf, int c) {
+        int kb, kb_end, seg;
+        chunk_of(c, kb, kb_end, seg);
+        const int k = kb * SK_KBLOCK + (lane % 32) * 8;
+        const bool ok = k < min(kb_end * SK_KBLOCK, seg ? K1 : K0);
+#pragma unroll
+        for (int i = 0; i < XL; ++i) *reinterpret_cast<bf16x8*>(xs[buf] + xplace[i]) = ok ? xr[i] : zero;
+    };
+    bf16x8 w[WD_DEPTH][WD_CB];
+    auto fetch_w = [&](int slot, int c) {
+        int kb, kb_end, seg;
+        chunk_of(c, kb, kb_end, seg);
+        const int Ks = seg ? K1 : K0;
+        const bf16_t* wp = seg ? wrow1 : wrow0;
+#pragma unroll
+        for (int j = 0; j < WD_CB; ++j) w[slot][j] = sk_load8_stream(wp + min((kb + j) * SK_KBLOCK + koff, Ks - 8));
+    };
+
+    floatx4 lo[MB], hi[MB];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+        lo[mb] = floatx4{0.f, 0.f, 0.f, 0.f};
+        hi[mb] = floatx4{0.f, 0.f, 0.f, 0.f};
+    }
+    auto compute = [&](int buf, int slot) {
+        const unsigned char* base = xs[buf];
+#pragma unroll
+        for (int j = 0; j < WD_CB; ++j) {
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb) {
+                const int m = mb * 16 + r;
+                const bf16x8 xlo = *reinterpret_cast<const bf16x8*>(base + m * WD_ROW_BYTES + (((j * 8 + g) ^ r) * 16));
+                const bf16x8 xhi = *reinterpret_cast<const bf16x8*>(base + m * WD_ROW_BYTES + (((j * 8 + 4 + g) ^ r) * 16));
+                lo[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[slot][j], xlo, lo[mb], 0, 0, 0);
+                hi[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w[slot][j], xhi, hi[mb], 0, 0, 0);
+            }
+        }
+    };
+    // LDS writes of this wave done, then everybody's: what the barrier of __syncthreads() would
+    // do too, but that one also waits for every load in flight
+    auto lds_barrier = [&]() {
+        __builtin_amdgcn_s_waitcnt(0xc07f);      // lgkmcnt(0), the other counters at their maximum
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+    };
+
+    // Weights run up to WD_DEPTH chunks ahead (in registers), activations one (in registers
+    // during the products of the chunk before, then in the LDS buffer that those products have
+    // left: the barrier at the head of the round says that all waves have).
+    fetch_x(0);
+#pragma unroll
+    for (int d = 0; d < WD_DEPTH; ++d) fetch_w(d, d);
+    store_x(0, 0);
+    for (int c = 0; c < n_chunks; c += WD_DEPTH) {
+#pragma unroll
+        for (int d = 0; d < WD_DEPTH; ++d) {
+            if (c + d >= n_chunks) break;                 // (uniform; no load stands behind it)
+            lds_barrier();
+            fetch_x(c + d + 1);
+            compute((c + d) & 1, d);
+            fetch_w(d, c + d + WD_DEPTH);
+            store_x((c + d + 1) & 1, c + d + 1);
+        }
+    }
+
+    // rows 0..7 of the strip are in lo of the lanes g < 2, rows 8..15 (the other half of every
+    // k-block) in hi of the lanes g >= 2: they meet in the lanes g < 2
+    float* mine = p.partial + (size_t)split * M * N;
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+        floatx4 v = g < 2 ? lo[mb] : hi[mb];
+        floatx4 o;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o[i] = __shfl_xor(v[i], 32, KA_WAVE);
+        const int m = mb * 16 + r, n = n0 + g * 4;
+        if (g < 2 && m < M) {
+            v += o;
+            float* dst = mine + (size_t)m * N + n;
+            if (n + 3 < N && (N % 4) == 0) *reinterpret_cast<floatx4*>(dst) = v;
+            else
+                for (int i = 0; i < 4 && n + i < N; ++i) dst[i] = v[i];
+        }
+    }
+}
+
+// out = act(sum of the parts + biases) (+ out): one thread per four neighbouring outputs
+__global__ void __launch_bounds__(256)
+skinny_wide_finish_kernel(const float* __restrict__ partial, int splits, const float* __restrict__ bias,
+                          const float* __restrict__ bias2, void* __restrict__ out, int out_dtype, long ldo, int M,
+                          int N, int act, int accumulate) {
+    const int quads = (N + 3) / 4;
+    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= M * quads) return;
+    const int m = idx / quads, n = (idx % quads) * 4;
+    const bool whole = n + 3 < N && N % 4 == 0;
+    float s[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int sp = 0; sp < splits; ++sp) {
+        const float* src = partial + ((size_t)sp * M + m) * N + n;
+        if (whole) {
+            floatx4 v = *reinterpret_cast<const floatx4*>(src);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) s[i] += v[i];
+        } else {
+            for (int i = 0; i < 4 && n + i < N; ++i) s[i] += src[i];
+        }
+    }
+    for (int i = 0; i < 4 && n + i < N; ++i) {
+        float x = s[i] + (bias ? bias[n + i] : 0.f) + (bias2 ? bias2[n + i] : 0.f);
+        if (act == 1) x = ka_gelu_tanh_fast(x);
+        const size_t o = (size_t)m * ldo + n + i;
+        if (out_dtype == KA_F32) {
+            float* op = reinterpret_cast<float*>(out) + o;
+            *op = accumulate ? *op + x : x;
+        } else {
+            reinterpret_cast<bf16_t*>(out)[o] = (bf16_t)x;
+        }
+    }
+}
+
+// ----------------------------------------------------------------------------
 // Host side
 // ----------------------------------------------------------------------------
 static int sk_compute_units() {
@@ -554,6 +767,12 @@ static int sk_compute_units() {
 // tests of the split kernel on sizes that it otherwise never sees.
 static int sk_persistent_enabled = 1;
 KA_API void ka_skinny_set_persistent(int enabled) { sk_persistent_enabled = enabled; }
+// The wide kernel (17 to 64 rows, activations through LDS, parts of K in scratch memory): 1 where
+// it was measured faster, which is with two K-segments (a K too long for the persistent kernel's
+// registers: 30 against 48 us for Moondream 2's output projection + fc2 at 64 rows; one segment
+// of 2048: 21 against 15 us), 2 wherever it can run (for tests), 0 nowhere.
+static int sk_wide_enabled = 1;
+KA_API void ka_skinny_set_wide(int enabled) { sk_wide_enabled = enabled; }
 
 template <int PER, int MB, bool HALF, bool LN>
 static int launch_persistent_one(int grid, size_t dyn, int strips, hipStream_t stream, const SkinnyArgs& args) {
@@ -648,7 +867,7 @@ KA_API int ka_linear_skinny_fused(const void* A1, long lda1, int K1, const void*
                                   long ldwa, const float* biasa, void* outa, int out_dtype_a, long ldoa, int Na,
                                   int acta, int accumulate_a, const void* Wb, long ldwb, const float* biasb,
                                   void* outb, int out_dtype_b, long ldob, int Nb, int actb, int M,
-                                  int target_waves, hipStream_t stream) {
+                                  int target_waves, float* partials, long partial_floats, hipStream_t stream) {
     const char* who = "ka_linear_skinny_fused";
     KA_CHECK(M > 0 && M <= 64, "%s: M=%d outside 1..64", who, M);
     KA_CHECK(K1 > 0 && K1 % 8 == 0, "%s: K=%d must be a positive multiple of 8", who, K1);
@@ -693,6 +912,32 @@ KA_API int ka_linear_skinny_fused(const void* A1, long lda1, int K1, const void*
         KA_LAUNCH_CHECK();
         return 0;
     }
+    if (M > 16 && !Wb && partials && (sk_wide_enabled >= 2 || (sk_wide_enabled && A2))) {
+        WideArgs wide = {};
+        wide.A[0] = args.A[0]; wide.lda[0] = args.lda[0]; wide.W[0] = args.a.W; wide.ldw[0] = args.a.ldw; wide.K[0] = K1;
+        if (A2) { wide.A[1] = args.A[1]; wide.lda[1] = args.lda[1]; wide.W[1] = args.W2; wide.ldw[1] = args.ldw2; wide.K[1] = K2; }
+        wide.M = M; wide.N = Na; wide.partial = partials;
+        // parts of K: two workgroups per CU where K is long enough for that, every part at least two chunks
+        const int groups = ka_cdiv(Na, WD_WAVES * SK_STRIP);
+        int splits = ka_cdiv(2 * sk_compute_units(), groups);
+        if (splits > ka_cdiv(kblocks, 2 * WD_CB)) splits = ka_cdiv(kblocks, 2 * WD_CB);
+        while (splits > 1 && (long)splits * M * Na > partial_floats) --splits;
+        if ((long)splits * M * Na <= partial_floats) {
+            wide.splits = splits;
+            dim3 grid(groups, splits);
+            switch (MB) {
+                case 2: hipLaunchKernelGGL(skinny_wide_kernel<2>, grid, dim3(WD_WAVES * KA_WAVE), 0, stream, wide); break;
+                case 3: hipLaunchKernelGGL(skinny_wide_kernel<3>, grid, dim3(WD_WAVES * KA_WAVE), 0, stream, wide); break;
+                default: hipLaunchKernelGGL(skinny_wide_kernel<4>, grid, dim3(WD_WAVES * KA_WAVE), 0, stream, wide); break;
+            }
+            KA_LAUNCH_CHECK();
+            const int quads = M * ka_cdiv(Na, 4);
+            hipLaunchKernelGGL(skinny_wide_finish_kernel, dim3(ka_cdiv(quads, 256)), dim3(256), 0, stream, partials, splits,
+                               biasa, A2 ? bias2 : nullptr, outa, out_dtype_a, ldoa, M, Na, acta, accumulate_a);
+            KA_LAUNCH_CHECK();
+            return 0;
+        }
+    }
     if (!A2 && !accumulate_a && sk_persistent_enabled && persistent_fits(M, kblocks, args)) {
         if (launch_persistent(strips, M, kblocks, false, 0, stream, args)) return -1;
         KA_LAUNCH_CHECK();
@@ -718,8 +963,9 @@ KA_API int ka_linear_skinny_fused(const void* A1, long lda1, int K1, const void*
 // One input, one weight matrix, one output.
 KA_API int ka_linear_skinny_bf16(const void* A, long lda, const void* W, long ldw, const float* bias,
                                  void* out, int out_dtype, long ldo, int M, int N, int K, int act,
-                                 int accumulate, int target_waves, hipStream_t stream) {
+                                 int accumulate, int target_waves, float* partials, long partial_floats,
+                                 hipStream_t stream) {
     return ka_linear_skinny_fused(A, lda, K, nullptr, 0, 0, nullptr, 0, nullptr, nullptr, nullptr, nullptr, 0.f, W,
                                   ldw, bias, out, out_dtype, ldo, N, act, accumulate, nullptr, 0, nullptr, nullptr, 0,
-                                  0, 0, 0, M, target_waves, stream);
+                                  0, 0, 0, M, target_waves, partials, partial_floats, stream);
 }

@@ -18,14 +18,14 @@ _c_void_p, _c_int, _c_long, _c_float = ctypes.c_void_p, ctypes.c_int, ctypes.c_l
 
 _SIGNATURES = {
     "ka_linear_skinny_bf16": [_c_void_p, _c_long, _c_void_p, _c_long, _c_void_p, _c_void_p, _c_int, _c_long, _c_int,
-                              _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
+                              _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_long, _c_void_p],
     "ka_linear_skinny_fused": [
         _c_void_p, _c_long, _c_int,                                   # A1, lda1, K1
         _c_void_p, _c_long, _c_int, _c_void_p, _c_long, _c_void_p,    # A2, lda2, K2, W2, ldw2, bias2
         _c_void_p, _c_void_p, _c_void_p, _c_float,                    # ln_x, gamma, beta, eps
         _c_void_p, _c_long, _c_void_p, _c_void_p, _c_int, _c_long, _c_int, _c_int, _c_int,   # target a
         _c_void_p, _c_long, _c_void_p, _c_void_p, _c_int, _c_long, _c_int, _c_int,           # target b
-        _c_int, _c_int, _c_void_p],                                   # M, target_waves, stream
+        _c_int, _c_int, _c_void_p, _c_long, _c_void_p],               # M, target_waves, partial sums and how many, stream
     "ka_linear_tiled_bf16": [_c_void_p, _c_long, _c_void_p, _c_long, _c_void_p, _c_void_p, _c_int, _c_long, _c_int,
                              _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
     "ka_attention_prefill_bf16": [_c_void_p, _c_long, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p,
@@ -55,8 +55,11 @@ TILED_CONFIG = 0
 SKINNY_TARGET_WAVES = 2048
 SCRATCH_FLOATS = 8 << 20
 SCRATCH_COUNTERS = 1 << 16
+WIDE_FLOATS = 8 << 20              # 32 MB of partial sums for skinny linears of 17 to 64 rows
+_wide_scratch = {}
 # Keys of one row a workgroup of the decode attention kernel takes before the row is split.
 DECODE_KEYS_PER_WORKGROUP = 4096
+DECODE_WAVE_SLOTS = 4096            # waves of the decode attention kernel that the chip holds at once
 
 _lib = None
 _scratch: Dict[torch.device, tuple] = {}
@@ -88,6 +91,13 @@ def set_skinny_persistent(enabled: int) -> None:
     lib().ka_skinny_set_persistent(int(enabled))
 
 
+def set_skinny_wide(enabled: int) -> None:
+    """Where skinny linears of 17 to 64 rows use the kernel that shares the activations through
+    LDS: 1 (the default) with two K-segments, where it was measured faster, 2 wherever it can run
+    (for tests), 0 nowhere."""
+    lib().ka_skinny_set_wide(int(enabled))
+
+
 def _check(status: int) -> None:
     if status != 0:
         raise KernelError(lib().ka_last_error().decode())
@@ -101,6 +111,19 @@ def scratch(device: torch.device):
         _scratch[key] = (torch.zeros(SCRATCH_FLOATS, dtype=torch.float32, device=device),
                          torch.zeros(SCRATCH_COUNTERS, dtype=torch.int32, device=device))
     return _scratch[key]
+
+
+def _wide_args(device: torch.device, rows: int):
+    """Scratch memory for the parts of K of a skinny linear of more than 16 rows: fp32 partial
+    sums, one buffer per device, made at the first such call. Calls on one device must not
+    overlap."""
+    if rows <= 16:
+        return None, 0
+    key = torch.device(device)
+    if key not in _wide_scratch:
+        _wide_scratch[key] = torch.empty(WIDE_FLOATS, dtype=torch.float32, device=device)
+    buf = _wide_scratch[key]
+    return buf.data_ptr(), buf.numel()
 
 
 def _operand_ok(t: torch.Tensor, k: int) -> bool:
@@ -134,7 +157,7 @@ def linear_bf16(a, weight, bias, out, act, accumulate) -> bool:
     if m <= SKINNY_MAX_ROWS:
         _check(handle.ka_linear_skinny_bf16(a.data_ptr(), a.stride(0), weight.data_ptr(), weight.stride(0), _ptr(bias),
                                             out.data_ptr(), _OUT_CODE[out.dtype], out.stride(0), m, n, k, act,
-                                            int(accumulate), SKINNY_TARGET_WAVES, stream_ptr()))
+                                            int(accumulate), SKINNY_TARGET_WAVES, *_wide_args(a.device, m), stream_ptr()))
     else:
         _check(handle.ka_linear_tiled_bf16(a.data_ptr(), a.stride(0), weight.data_ptr(), weight.stride(0), _ptr(bias),
                                            out.data_ptr(), _OUT_CODE[out.dtype], out.stride(0), m, n, k, act,
@@ -157,7 +180,7 @@ def linear_pair_accumulate(a1, w1, b1, a2, w2, b2, out) -> bool:
         a1.data_ptr(), a1.stride(0), k1, a2.data_ptr(), a2.stride(0), k2, w2.data_ptr(), w2.stride(0), _ptr(b2),
         None, None, None, 0.0,
         w1.data_ptr(), w1.stride(0), _ptr(b1), out.data_ptr(), KA_F32, out.stride(0), n, 0, 1,
-        None, 0, None, None, 0, 0, 0, 0, m, SKINNY_TARGET_WAVES, stream_ptr()))
+        None, 0, None, None, 0, 0, 0, 0, m, SKINNY_TARGET_WAVES, *_wide_args(a1.device, m), stream_ptr()))
     return True
 
 
@@ -175,7 +198,7 @@ def linear_two_outputs(a, wa, ba, out_a, act_a, wb, bb, out_b, act_b) -> bool:
         None, None, None, 0.0,
         wa.data_ptr(), wa.stride(0), _ptr(ba), out_a.data_ptr(), _OUT_CODE[out_a.dtype], out_a.stride(0), na, act_a, 0,
         wb.data_ptr(), wb.stride(0), _ptr(bb), out_b.data_ptr(), _OUT_CODE[out_b.dtype], out_b.stride(0), nb, act_b,
-        m, SKINNY_TARGET_WAVES, stream_ptr()))
+        m, SKINNY_TARGET_WAVES, None, 0, stream_ptr()))
     return True
 
 
@@ -209,7 +232,7 @@ def layernorm_linear(x, gamma, beta, eps, wa, ba, out_a, act_a, wb=None, bb=None
         wa.data_ptr(), wa.stride(0), _ptr(ba), out_a.data_ptr(), _OUT_CODE[out_a.dtype], out_a.stride(0), na, act_a, 0,
         _ptr(wb), wb.stride(0) if two else 0, _ptr(bb) if two else None, _ptr(out_b),
         _OUT_CODE[out_b.dtype] if two else 0, out_b.stride(0) if two else 0, nb, act_b,
-        m, SKINNY_TARGET_WAVES, stream_ptr()))
+        m, SKINNY_TARGET_WAVES, None, 0, stream_ptr()))
     return True
 
 
@@ -217,14 +240,18 @@ def layernorm_linear_pair(x, gamma, beta, eps, wa, ba, out_a, act_a, wb, bb, out
     return layernorm_linear(x, gamma, beta, eps, wa, ba, out_a, act_a, wb, bb, out_b, act_b)
 
 
-def decode_shape(max_kv: int):
+def decode_shape(max_kv: int, workgroups: int = 1):
     """``(splits, waves)`` of the decode attention kernel: a workgroup of up to 16 waves takes a
     64-key tile per wave and round; rows longer than 4096 keys are cut into splits that meet
-    through scratch memory."""
+    through scratch memory. With many workgroups (rows x heads) each gets fewer waves, so that
+    they all fit on the chip at once (measured at 1024 keys: 16 waves up to 256 workgroups, 8 at
+    512 and 1024, 4 from 2048 on)."""
     splits = max(1, -(-max_kv // DECODE_KEYS_PER_WORKGROUP))
     tiles = -(-max_kv // (64 * splits))
     waves = 4 if tiles <= 4 else 8 if tiles <= 8 else 16
-    return splits, waves
+    groups = workgroups * splits
+    fit = 16 if groups <= DECODE_WAVE_SLOTS // 16 else 8 if groups <= DECODE_WAVE_SLOTS // 4 else 4
+    return splits, min(waves, fit)
 
 
 def _attention_operands_ok(q, out) -> bool:
@@ -243,7 +270,7 @@ def attention_decode_bf16(q, k_cache, v_cache, block_table, token_row, kv_lo, kv
     if batch is None or not batch.decode_only or not _attention_operands_ok(q, out) \
             or not handle.ka_attention_decode_supported(head_dim, page_size):
         return False
-    splits, waves = decode_shape(batch.max_kv)
+    splits, waves = decode_shape(batch.max_kv, n * n_heads)
     partial, counters = scratch(q.device)
     if n * n_heads * splits * (head_dim + 2) > partial.numel() or n * n_heads > counters.numel():
         return False

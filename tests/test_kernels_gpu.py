@@ -120,17 +120,22 @@ def test_linear_generic(shape):
     _linear_case(core.linear_generic, m, n, k, f32, f32, f32, 0, False, lda=k + 5)      # strided rows
 
 
-@pytest.mark.parametrize("persistent", [1, 0])
+@pytest.mark.parametrize("persistent,wide", [(1, 0), (0, 0), (1, 2)])
 @pytest.mark.parametrize("shape", [(1, 48, 64), (8, 2048, 2048), (5, 100, 200), (16, 6144, 2048), (33, 77, 8192),
                                    (64, 51200, 512), (17, 2048, 8192), (3, 16, 8), (9, 20000, 1032), (40, 4100, 2048),
                                    (8, 1000, 4096), (12, 515, 3000), (64, 9000, 1024)])
-def test_linear_skinny_bf16(shape, persistent):
+def test_linear_skinny_bf16(shape, persistent, wide):
     """The weight-streaming MFMA kernels: the persistent one (activations in registers, workgroups
-    walk over strips; a form of its own for at most 8 rows) and the one with K-splits that takes
-    the rest, which is tested on the same shapes with the persistent one switched off."""
+    walk over strips; a form of its own for at most 8 rows), the one with K-splits that takes
+    the rest, which is tested on the same shapes with the persistent one switched off, and the
+    wide one for 17 rows and more, which the engine uses with two K-segments only and which
+    mode 2 sends these shapes to."""
     from kestrel_amd.ops import fast
 
     m, n, k = shape
+    if m <= 16 and wide:
+        pytest.skip("the wide kernel takes 17 rows and more")
+    fast.set_skinny_wide(wide)
     bf, f32 = torch.bfloat16, torch.float32
 
     def fn(a, w, bias, out, act, accumulate):
@@ -143,6 +148,7 @@ def test_linear_skinny_bf16(shape, persistent):
         _linear_case(fn, m, n, k, bf, bf, bf, 0, False, lda=k + 16)
     finally:
         fast.set_skinny_persistent(1)
+        fast.set_skinny_wide(1)
 
 
 def test_linear_skinny_is_the_same_on_every_run():
@@ -497,13 +503,19 @@ def test_masks_before_sampling_and_logprobs_after():
     assert torch.allclose(out.cpu().double(), torch.tensor(ref, dtype=torch.float64), atol=2e-5, rtol=1e-5)
 
 
+@pytest.mark.parametrize("wide", [1, 0])
 @pytest.mark.parametrize("shape", [(8, 2048, 2048, 8192), (1, 40, 64, 200), (16, 2048, 2048, 8192), (33, 96, 120, 320),
-                                   (64, 256, 8, 72)])
-def test_two_segment_skinny_linear(shape):
-    """out += a1 w1^T + b1 + a2 w2^T + b2 in one launch."""
+                                   (64, 256, 8, 72), (64, 2048, 2048, 8192), (17, 515, 1032, 40), (48, 100, 264, 2056)])
+def test_two_segment_skinny_linear(shape, wide):
+    """out += a1 w1^T + b1 + a2 w2^T + b2 in one launch (17 rows and more: by the kernel that
+    shares the activations through LDS and cuts K into parts, and, with that one switched off,
+    by the one that takes fewer rows too)."""
     from kestrel_amd.ops import fast
 
     m, n, k1, k2 = shape
+    if m <= 16 and not wide:
+        pytest.skip("the wide kernel takes no part below 17 rows")
+    fast.set_skinny_wide(wide)
     torch.manual_seed(20)
     a1, a2 = torch.randn(m, k1).bfloat16().to(DEV), torch.randn(m, k2).bfloat16().to(DEV)
     w1 = (torch.randn(n, k1) / k1 ** 0.5).bfloat16().to(DEV)
@@ -517,6 +529,10 @@ def test_two_segment_skinny_linear(shape):
     out2 = start.clone()
     assert fast.linear_pair_accumulate(a1, w1, None, a2, w2, None, out2)
     _close(out2, ref - b1.double() - b2.double(), torch.float32, scale=200)
+    out3 = start.clone()
+    assert fast.linear_pair_accumulate(a1, w1, None, a2, w2, None, out3)
+    assert torch.equal(out2, out3)                      # the same bits on every run
+    fast.set_skinny_wide(1)
 
 
 @pytest.mark.parametrize("shape", [(8, 2048, 6144, 8192), (1, 64, 40, 24), (16, 320, 100, 200), (5, 2048, 48, 8),
