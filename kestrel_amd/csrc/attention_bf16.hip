@@ -628,6 +628,132 @@ static int check_common(const char* who, const void* q, long q_row_stride, const
     return 0;
 }
 
+// ----------------------------------------------------------------------------------------------
+// rotary encoding + cache write, a page's worth of tokens per workgroup
+// ----------------------------------------------------------------------------------------------
+// A workgroup takes 16 consecutive tokens of the packed batch. Queries are rotated in place and
+// keys rotated into the cache with 16-byte loads and stores (8 channels of a head and their 8
+// partners in the other half of the rotated part per thread). Values: the cache keeps a page
+// transposed, [channel][16 tokens]; when the 16 tokens fill one page in order (which they do
+// inside a prompt that starts on a page boundary) a thread gathers 8 channels of all 16 tokens
+// and stores 8 rows of 32 bytes, 256 contiguous bytes; other tokens are stored one by one.
+constexpr int RC_TOKENS = AT_PAGE;
+constexpr int RC_THREADS = 256;
+
+__global__ void __launch_bounds__(RC_THREADS)
+rope_cache_pages_kernel(bf16_t* __restrict__ qkv, long row_stride, const int* __restrict__ positions,
+                        const int* __restrict__ slots, const float* __restrict__ table,
+                        bf16_t* __restrict__ k_cache, bf16_t* __restrict__ v_cache, int n, int H, int Hkv,
+                        int hd, int rot) {
+    const int t0 = blockIdx.x * RC_TOKENS;
+    const int n_here = min(RC_TOKENS, n - t0);
+    const int half = rot / 2;
+    const int pair_units = half / 8;                  // per head: 8 channels + their 8 partners
+    const int plain_units = (hd - rot) / 8;           // per head: 8 channels that are not rotated
+    const size_t page_elems = (size_t)Hkv * AT_PAGE * hd;
+
+    // queries and keys: (token, head, unit); heads 0..H-1 are queries, H..H+Hkv-1 keys
+    const int units = pair_units + plain_units;
+    const int per_token = (H + Hkv) * units;
+    // (the work of a group of tokens is dealt out over gridDim.y workgroups: there are few groups)
+    const int lane_id = blockIdx.y * RC_THREADS + threadIdx.x, lanes = gridDim.y * RC_THREADS;
+    for (int idx = lane_id; idx < n_here * per_token; idx += lanes) {
+        const int i = idx / per_token, rest = idx % per_token;
+        const int head = rest / units, u = rest % units;
+        const int t = t0 + i;
+        const bool is_key = head >= H;
+        const int slot = is_key && slots ? slots[t] : -1;
+        if (is_key && slot < 0) continue;                       // nothing is cached for this token
+        bf16_t* src = qkv + (size_t)t * row_stride + (size_t)head * hd;     // the keys follow the queries
+        bf16_t* kdst = nullptr;
+        if (is_key) kdst = k_cache + (size_t)(slot / AT_PAGE) * page_elems + ((size_t)(head - H) * AT_PAGE + slot % AT_PAGE) * hd;
+        if (u < pair_units) {
+            const int c0 = u * 8;
+            bf16x8 a = at_load8(src + c0), b = at_load8(src + half + c0);
+            const float* cs = table + (size_t)positions[t] * rot;
+            floatx4 c[2] = {*reinterpret_cast<const floatx4*>(cs + c0), *reinterpret_cast<const floatx4*>(cs + c0 + 4)};
+            floatx4 sn[2] = {*reinterpret_cast<const floatx4*>(cs + half + c0), *reinterpret_cast<const floatx4*>(cs + half + c0 + 4)};
+            bf16x8 ra, rb;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                float x = (float)a[j], y = (float)b[j], cc = c[j / 4][j % 4], ss = sn[j / 4][j % 4];
+                ra[j] = (bf16_t)(x * cc - y * ss);
+                rb[j] = (bf16_t)(y * cc + x * ss);
+            }
+            bf16_t* dst = is_key ? kdst : src;
+            *reinterpret_cast<bf16x8*>(dst + c0) = ra;
+            *reinterpret_cast<bf16x8*>(dst + half + c0) = rb;
+        } else if (is_key) {
+            const int c0 = rot + (u - pair_units) * 8;
+            *reinterpret_cast<bf16x8*>(kdst + c0) = at_load8(src + c0);
+        }
+    }
+    if (!slots) return;
+
+    // values
+    const int first = slots[t0];
+    bool whole_page = n_here == RC_TOKENS && first >= 0 && first % AT_PAGE == 0;
+    if (whole_page) {
+        for (int i = 1; i < RC_TOKENS; ++i) whole_page = whole_page && slots[t0 + i] == first + i;   // (the same for all threads)
+    }
+    const int vwidth = Hkv * hd;
+    const bf16_t* vsrc = qkv + (size_t)t0 * row_stride + (size_t)(H + Hkv) * hd;
+    if (whole_page) {
+        bf16_t* vpage = v_cache + (size_t)(first / AT_PAGE) * page_elems;
+        for (int c0 = lane_id * 8; c0 < vwidth; c0 += lanes * 8) {
+            bf16x8 v[RC_TOKENS];
+#pragma unroll
+            for (int i = 0; i < RC_TOKENS; ++i) v[i] = at_load8(vsrc + (size_t)i * row_stride + c0);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                bf16x8 lo, hi;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    lo[i] = v[i][j];
+                    hi[i] = v[8 + i][j];
+                }
+                // channel c0 + j = (head, d): its 16 tokens are one row of the page
+                bf16_t* dst = vpage + (size_t)(c0 + j) * AT_PAGE;
+                *reinterpret_cast<bf16x8*>(dst) = lo;
+                *reinterpret_cast<bf16x8*>(dst + 8) = hi;
+            }
+        }
+    } else {
+        for (int idx = lane_id; idx < n_here * vwidth; idx += lanes) {
+            const int i = idx / vwidth, c = idx % vwidth;
+            const int slot = slots[t0 + i];
+            if (slot < 0) continue;
+            v_cache[(size_t)(slot / AT_PAGE) * page_elems + (size_t)c * AT_PAGE + slot % AT_PAGE] = vsrc[(size_t)i * row_stride + c];
+        }
+    }
+}
+
+// Rotates q in place (the first `rot` channels of every head, halves paired) and writes rotated
+// keys and the values into the paged cache (slots null: rotates q only; a slot < 0: that token is
+// not cached). bf16, pages of 16, head size and rot / 2 multiples of 8, rows 16-byte aligned.
+KA_API int ka_rope_cache_pages_supported(int hd, int rot, int page_size) {
+    return page_size == AT_PAGE && hd % 8 == 0 && rot > 0 && rot % 16 == 0 && rot <= hd;
+}
+
+KA_API int ka_rope_cache_pages_bf16(void* qkv, long row_stride, const int* positions, const int* slots,
+                                    const float* table, int table_rows, void* k_cache, void* v_cache, int n, int H,
+                                    int Hkv, int hd, int rot, int page_size, hipStream_t stream) {
+    const char* who = "ka_rope_cache_pages_bf16";
+    KA_CHECK(n >= 0 && H > 0 && Hkv > 0, "%s: bad sizes", who);
+    KA_CHECK(ka_rope_cache_pages_supported(hd, rot, page_size), "%s: head size %d, rotary size %d, page size %d not covered", who, hd, rot, page_size);
+    KA_CHECK(row_stride >= (long)(H + 2 * Hkv) * hd && row_stride % 8 == 0 && (uintptr_t)qkv % 16 == 0, "%s: rows must be 16-byte aligned and hold q, k and v", who);
+    KA_CHECK(table && table_rows > 0 && (uintptr_t)table % 16 == 0, "%s: rotary table missing or not 16-byte aligned", who);
+    KA_CHECK(!slots || (k_cache && v_cache && (uintptr_t)k_cache % 16 == 0 && (uintptr_t)v_cache % 16 == 0), "%s: cache tensors missing or not 16-byte aligned", who);
+    if (n == 0) return 0;
+    const int groups = ka_cdiv(n, RC_TOKENS);
+    int parts = ka_cdiv(2048, groups);           // enough workgroups for the chip, whatever the number of tokens
+    if (parts > 16) parts = 16;
+    hipLaunchKernelGGL(rope_cache_pages_kernel, dim3(groups, parts), dim3(RC_THREADS), 0, stream, (bf16_t*)qkv,
+                       row_stride, positions, slots, table, (bf16_t*)k_cache, (bf16_t*)v_cache, n, H, Hkv, hd, rot);
+    KA_LAUNCH_CHECK();
+    return 0;
+}
+
 KA_API int ka_attention_prefill_supported(int hd, int page_size) {
     return page_size == AT_PAGE && (hd == 32 || hd == 64 || hd == 96 || hd == 128);
 }

@@ -31,6 +31,8 @@ _SIGNATURES = {
     "ka_attention_prefill_bf16": [_c_void_p, _c_long, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p,
                                   _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_long, _c_float,
                                   _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
+    "ka_rope_cache_pages_bf16": [_c_void_p, _c_long, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p,
+                                 _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
     "ka_attention_decode_bf16": [_c_void_p, _c_long, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p,
                                  _c_void_p, _c_void_p, _c_long, _c_float, _c_int, _c_int, _c_int, _c_int, _c_int,
                                  _c_int, _c_int, _c_void_p, _c_long, _c_void_p, _c_int,
@@ -77,6 +79,8 @@ def lib():
         handle.ka_last_error.restype = ctypes.c_char_p
         handle.ka_skinny_set_persistent.argtypes = [_c_int]
         handle.ka_skinny_set_persistent.restype = None
+        handle.ka_rope_cache_pages_supported.argtypes = [_c_int, _c_int, _c_int]
+        handle.ka_rope_cache_pages_supported.restype = _c_int
         for name in ("ka_attention_prefill_supported", "ka_attention_decode_supported"):
             getattr(handle, name).argtypes = [_c_int, _c_int]
             getattr(handle, name).restype = _c_int
@@ -238,6 +242,24 @@ def layernorm_linear(x, gamma, beta, eps, wa, ba, out_a, act_a, wb=None, bb=None
 
 def layernorm_linear_pair(x, gamma, beta, eps, wa, ba, out_a, act_a, wb, bb, out_b, act_b) -> bool:
     return layernorm_linear(x, gamma, beta, eps, wa, ba, out_a, act_a, wb, bb, out_b, act_b)
+
+
+def rope_cache_bf16(qkv, positions, slots, table, k_cache, v_cache, n_heads, n_kv_heads, head_dim, page_size) -> bool:
+    """Rotary encoding of q (in place) and k, and the cache write of k and v, a page's worth of
+    tokens per workgroup (``ops.core.rope_cache`` says what the operands are). False: not covered
+    (another page size, a rotary size that is no multiple of 16, rows that are not 16-byte aligned)."""
+    if table is None or qkv.dtype != torch.bfloat16 or qkv.stride(1) != 1 or qkv.stride(0) % 8 or qkv.data_ptr() % 16:
+        return False
+    rot = int(table.shape[1])
+    handle = lib()
+    if not handle.ka_rope_cache_pages_supported(head_dim, rot, page_size) or table.data_ptr() % 16:
+        return False
+    if slots is not None and (k_cache.data_ptr() % 16 or v_cache.data_ptr() % 16):
+        return False
+    _check(handle.ka_rope_cache_pages_bf16(qkv.data_ptr(), qkv.stride(0), positions.data_ptr(), _ptr(slots), table.data_ptr(),
+                                           int(table.shape[0]), _ptr(k_cache), _ptr(v_cache), qkv.shape[0], n_heads,
+                                           n_kv_heads, head_dim, rot, page_size, stream_ptr()))
+    return True
 
 
 def decode_shape(max_kv: int, workgroups: int = 1):

@@ -81,8 +81,15 @@ class PagedAttention(Mixer):
                                           batch.kv_hi, out, self.scale, spec.n_heads, spec.n_kv_heads, spec.head_dim,
                                           batch, fuse=(k_new, v_new, self._table, group.slots)):
                 return out
-        core.rope_cache(qkv, batch.positions, group.slots if cache.writes else None, self._table, cache.k, cache.v,
-                        spec.n_heads, spec.n_kv_heads, spec.head_dim, group.page_size)
+        slots = group.slots if cache.writes else None
+        done = False
+        if qkv.dtype == torch.bfloat16:
+            from ..ops import fast
+            done = fast.rope_cache_bf16(qkv, batch.positions, slots, self._table, cache.k, cache.v, spec.n_heads,
+                                        spec.n_kv_heads, spec.head_dim, group.page_size)
+        if not done:
+            core.rope_cache(qkv, batch.positions, slots, self._table, cache.k, cache.v, spec.n_heads, spec.n_kv_heads,
+                            spec.head_dim, group.page_size)
         paged_attention(qkv, cache.k, cache.v, group.block_table, batch.token_row, group.kv_lo, batch.kv_hi, out,
                         self.scale, spec.n_heads, spec.n_kv_heads, spec.head_dim, batch)
         return out

@@ -248,6 +248,57 @@ def test_rope_and_cache_write(heads, dtype):
             assert float(k_cache[slot // ps, :, slot % ps, :].abs().max()) == 0.0
 
 
+@pytest.mark.parametrize("heads", [(4, 4, 64, 32), (6, 2, 48, 16), (3, 1, 128, 128), (2, 2, 80, 32)])
+def test_rope_and_cache_write_by_pages(heads):
+    """The bf16 kernel that takes 16 tokens per workgroup: tokens that fill whole pages in order
+    (the fast way to store the values), a run that starts in the middle of a page, a token that
+    is not cached, scattered slots and a ragged end; and with no slots at all, q alone."""
+    from kestrel_amd.ops import fast
+
+    h, hkv, hd, rot = heads
+    bf = torch.bfloat16
+    torch.manual_seed(14)
+    ps, pages = 16, 12
+    # tokens 0..31: pages 5 and 2 in order; 32..47: page 7 from offset 3 on, running into page 9;
+    # 48..63: scattered, one not cached; 64..70: a ragged tail on page 0
+    slots = list(range(5 * ps, 6 * ps)) + list(range(2 * ps, 3 * ps))
+    slots += list(range(7 * ps + 3, 8 * ps)) + list(range(9 * ps, 9 * ps + 3))
+    scattered = (torch.randperm(2 * ps)[:16] + 10 * ps).tolist()
+    scattered[4] = -1
+    slots += scattered + list(range(0, 7))
+    n = len(slots)
+    positions = torch.randint(0, 200, (n,), dtype=torch.int32)
+    qkv = torch.randn(n, (h + 2 * hkv) * hd).to(bf)
+    table = plain.rotary_table(rot, 256, 777.0, torch.float32)
+    k_cache = torch.zeros(pages, hkv, ps, hd, dtype=bf, device=DEV)
+    v_cache = torch.zeros(pages, hkv, hd, ps, dtype=bf, device=DEV)
+    dev = qkv.to(DEV)
+    slots_t = torch.tensor(slots, dtype=torch.int32)
+    assert fast.rope_cache_bf16(dev, positions.to(DEV), slots_t.to(DEV), table.to(DEV), k_cache, v_cache, h, hkv, hd, ps)
+    t64 = plain.rotary_table(rot, 256, 777.0)
+    q = plain.apply_rotary(qkv[:, :h * hd].double().view(n, h, hd), positions, t64)
+    k = plain.apply_rotary(qkv[:, h * hd:(h + hkv) * hd].double().view(n, hkv, hd), positions, t64)
+    v = qkv[:, (h + hkv) * hd:].view(n, hkv, hd)
+    _close(dev[:, :h * hd].view(n, h, hd), q, bf)
+    assert torch.equal(dev[:, h * hd:].cpu(), qkv[:, h * hd:])          # k and v rows themselves stay as they were
+    for t in range(n):
+        if slots[t] < 0:
+            continue
+        page, off = slots[t] // ps, slots[t] % ps
+        _close(k_cache[page, :, off, :], k[t], bf)
+        assert torch.equal(v_cache[page, :, :, off].cpu(), v[t])
+    written = {s for s in slots if s >= 0}
+    for slot in range(pages * ps):
+        if slot not in written:
+            assert float(k_cache[slot // ps, :, slot % ps, :].abs().max()) == 0.0
+            assert float(v_cache[slot // ps, :, :, slot % ps].abs().max()) == 0.0
+    only_q = qkv.to(DEV)
+    assert fast.rope_cache_bf16(only_q, positions.to(DEV), None, table.to(DEV), None, None, h, hkv, hd, ps)
+    assert torch.equal(only_q[:, :h * hd], dev[:, :h * hd]) and torch.equal(only_q[:, h * hd:].cpu(), qkv[:, h * hd:])
+    assert not fast.rope_cache_bf16(qkv.to(DEV), positions.to(DEV), None, torch.zeros(256, 24, device=DEV), None, None,
+                                    h, hkv, hd, ps)               # a rotary size that is no multiple of 16
+
+
 class PagedCase:
     """Rows of cached keys and values scattered over shuffled pages, and packed query tokens."""
 
