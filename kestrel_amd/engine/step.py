@@ -18,6 +18,7 @@ from __future__ import annotations
 from dataclasses import dataclass
 from typing import Dict, List, Optional, Sequence, Tuple
 
+import numpy as np
 import torch
 
 from ..cache.manager import CacheManager
@@ -64,6 +65,38 @@ def graph_buckets(max_batch: int) -> List[int]:
     return sizes
 
 
+class _Column:
+    """The int32 values of one section of a step's metadata, gathered piece by piece: lists from
+    rows of a few tokens, arrays from prompt portions (thousands of tokens, which are never
+    turned into Python integers)."""
+
+    def __init__(self) -> None:
+        self.pieces: list = []
+        self.count = 0
+
+    def __len__(self) -> int:
+        return self.count
+
+    def extend(self, values) -> None:
+        if isinstance(values, np.ndarray):
+            self.pieces.append(values)
+        else:
+            values = list(values)
+            if self.pieces and isinstance(self.pieces[-1], list):
+                self.pieces[-1].extend(values)
+            else:
+                self.pieces.append(values)
+        self.count += len(values)
+
+    def append(self, value: int) -> None:
+        self.extend((value,))
+
+    def write(self, host: np.ndarray, offset: int) -> None:
+        for piece in self.pieces:
+            host[offset:offset + len(piece)] = piece
+            offset += len(piece)
+
+
 class _GraphState:
     """A captured decode step of one bucket size: its metadata, scratch and graph."""
 
@@ -78,6 +111,7 @@ class ModelRunner:
     """Owns the model, its cache and the scratch memory; ``step`` is the only way in."""
 
     STAGING_RING = 4
+    SCALAR_ROW = 16          # rows of at most this many tokens are laid out token by token, longer ones as arrays
     QUERY_BLOCK = 32         # queries of one row a workgroup of the prompt attention kernel takes
 
     def __init__(self, model: DecoderModel, cache: CacheManager, device: torch.device,
@@ -165,53 +199,78 @@ class ModelRunner:
             cache.ensure(e.slot, start + len(e.tokens))
 
         n_groups = len(cache.groups)
-        ids: List[int] = []
-        positions: List[int] = []
-        token_row: List[int] = []
-        kv_hi: List[int] = []
+        ids, positions, token_row, kv_hi = _Column(), _Column(), _Column(), _Column()
+        blocks: List[Tuple[int, int, int]] = []      # of queries: row, first token, most keys any of them sees
         logit_rows: List[int] = []
         given_rows: List[int] = []
         given: List[torch.Tensor] = []
         row_slot: List[int] = []
         cu_q = [0]
         kv_len: List[int] = []
-        slots: List[List[int]] = [[] for _ in range(n_groups)]
-        kv_lo: List[Optional[List[int]]] = [[] if g.spec.window is not None else None for g in cache.groups]
+        slots = [_Column() for _ in range(n_groups)]
+        kv_lo = [_Column() if g.spec.window is not None else None for g in cache.groups]
         max_pages = max(1, fixed_pages)
         max_q = max_kv = 1
         causal_only = True
         for r, (e, start) in enumerate(zip(entries, starts)):
             q = len(e.tokens)
             base = len(ids)
-            hi = [start + i + 1 for i in range(q)]
             for lo_b, hi_b in e.bidirectional:
                 if not (start <= lo_b < hi_b <= start + q):
                     raise ValueError(f"slot {e.slot}: the bidirectional block [{lo_b}, {hi_b}) must lie inside one "
                                      f"portion, this one covers [{start}, {start + q})")
-                for p in range(lo_b, hi_b):
-                    hi[p - start] = max(hi[p - start], hi_b)
                 causal_only = False
-            n_given = 0
-            for i, tok in enumerate(e.tokens):
-                tok = int(tok)
-                if tok == PENDING_TOKEN:
-                    tok = PENDING_TOKEN - e.slot      # the embedding kernel reads pending[slot]
-                elif tok < 0:
-                    given_rows.append(base + i)
-                    n_given += 1
-                    tok = -1
-                elif tok >= plan.vocab_size:
-                    raise ValueError(f"slot {e.slot}: token id {tok} outside the vocabulary of {plan.vocab_size}")
-                ids.append(tok)
+            if q <= self.SCALAR_ROW:
+                hi = [start + i + 1 for i in range(q)]
+                for lo_b, hi_b in e.bidirectional:
+                    for p in range(lo_b, hi_b):
+                        hi[p - start] = max(hi[p - start], hi_b)
+                row_ids, row_given = [], []
+                for i, tok in enumerate(e.tokens):
+                    tok = int(tok)
+                    if tok == PENDING_TOKEN:
+                        tok = PENDING_TOKEN - e.slot      # the embedding kernel reads pending[slot]
+                    elif tok < 0:
+                        row_given.append(base + i)
+                        tok = -1
+                    elif tok >= plan.vocab_size:
+                        raise ValueError(f"slot {e.slot}: token id {tok} outside the vocabulary of {plan.vocab_size}")
+                    row_ids.append(tok)
+            else:
+                # a prompt portion has thousands of tokens: a loop over them in Python would take
+                # longer than some of the kernels that follow
+                hi_a = np.arange(start + 1, start + q + 1, dtype=np.int64)
+                for lo_b, hi_b in e.bidirectional:
+                    np.maximum(hi_a[lo_b - start:hi_b - start], hi_b, out=hi_a[lo_b - start:hi_b - start])
+                tok_a = np.asarray(e.tokens, dtype=np.int64).reshape(-1)
+                pending = tok_a == PENDING_TOKEN
+                is_given = (tok_a < 0) & ~pending
+                too_large = tok_a >= plan.vocab_size
+                if too_large.any():
+                    raise ValueError(f"slot {e.slot}: token id {int(tok_a[too_large][0])} outside the vocabulary of "
+                                     f"{plan.vocab_size}")
+                tok_a[pending] = PENDING_TOKEN - e.slot
+                tok_a[is_given] = -1
+                row_given = (base + np.nonzero(is_given)[0]).tolist()
+                row_ids, hi = tok_a, hi_a
+            n_given = len(row_given)
+            given_rows.extend(row_given)
+            ids.extend(row_ids)
             if n_given:
                 if e.embeds is None or e.embeds.dim() != 2 or tuple(e.embeds.shape) != (n_given, plan.dim):
                     raise ValueError(f"slot {e.slot}: {n_given} places need embeddings of shape [{n_given}, {plan.dim}]")
                 given.append(e.embeds)
             elif e.embeds is not None and e.embeds.numel():
                 raise ValueError(f"slot {e.slot}: embeddings given but no token id is -1")
-            positions.extend(range(start, start + q))
-            token_row.extend([r] * q)
+            if q <= self.SCALAR_ROW:
+                positions.extend(range(start, start + q))
+                token_row.extend([r] * q)
+            else:
+                positions.extend(np.arange(start, start + q, dtype=np.int64))
+                token_row.extend(np.full(q, r, dtype=np.int64))
             kv_hi.extend(hi)
+            for first in range(0, q, self.QUERY_BLOCK):
+                blocks.append((r, base + first, int(max(hi[first:first + self.QUERY_BLOCK]))))
             for w in e.want:
                 if not 0 <= int(w) < q:
                     raise ValueError(f"slot {e.slot}: wanted place {w} outside its {q} tokens")
@@ -225,7 +284,11 @@ class ModelRunner:
                 if fixed_pages and len(table) > fixed_pages:
                     raise ValueError(f"slot {e.slot}: {len(table)} pages exceed the fixed table width {fixed_pages}")
                 max_pages = max(max_pages, len(table))
-                slots[g].extend(table[p // ps] * ps + p % ps for p in range(start, start + q))
+                if q <= self.SCALAR_ROW:
+                    slots[g].extend(table[p // ps] * ps + p % ps for p in range(start, start + q))
+                else:
+                    places = np.arange(start, start + q, dtype=np.int64)
+                    slots[g].extend(np.asarray(table, dtype=np.int64)[places // ps] * ps + places % ps)
                 if kv_lo[g] is not None:
                     kv_lo[g].extend(cache.window_start(g, p) for p in range(start, start + q))
         n_real = len(entries)
@@ -234,6 +297,7 @@ class ModelRunner:
             positions.append(0)
             token_row.append(r)
             kv_hi.append(0)
+            blocks.append((r, len(ids) - 1, 0))
             logit_rows.append(len(ids) - 1)
             cu_q.append(len(ids))
             kv_len.append(0)
@@ -247,14 +311,13 @@ class ModelRunner:
 
         qblk_row: List[int] = []
         qblk_tok: List[int] = []
-        blocks = [(r, first) for r in range(n_rows) for first in range(cu_q[r], cu_q[r + 1], self.QUERY_BLOCK)]
         # the blocks that see the most keys first: a launch then ends with short ones
-        blocks.sort(key=lambda b: -max(kv_hi[b[1]:min(b[1] + self.QUERY_BLOCK, cu_q[b[0] + 1])]))
-        for r, first in blocks:
+        blocks.sort(key=lambda b: -b[2])
+        for r, first, _ in blocks:
             qblk_row.append(r)
             qblk_tok.append(first)
         # one packed int32 buffer, every section starting on a 16-byte boundary
-        sections: List[Tuple[str, List[int]]] = [
+        sections: List[Tuple[str, object]] = [
             ("ids", ids), ("positions", positions), ("token_row", token_row), ("kv_hi", kv_hi),
             ("row_slot", row_slot), ("cu_q", cu_q), ("kv_len", kv_len), ("logit_rows", logit_rows),
             ("given_rows", given_rows), ("qblk_row", qblk_row), ("qblk_tok", qblk_tok),
@@ -279,7 +342,9 @@ class ModelRunner:
         host = staging.numpy()
         for name, values in sections:
             off, count = offsets[name]
-            if count:
+            if count and isinstance(values, _Column):
+                values.write(host, off)
+            elif count:
                 host[off:off + count] = values
         if meta is None:
             if self._meta_device is None or self._meta_device.numel() < total:
