@@ -49,7 +49,7 @@ SKINNY_LN_MAX_WIDTH = 2048
 # the persistent kernel then repeats the LayerNorm of all rows once; with a few hundred workgroups
 # that is cheaper than a launch of its own (measured on MI355X: 3 % of a decode step at batch 8).
 FUSE_LAYERNORM_PROLOGUE = True
-# Tile of the tiled kernels: 0 lets them choose by size; 221, 211 (any K), 12222, 23212, 22224, 13122
+# Tile of the tiled kernels: 0 lets them choose by size; 221, 211 (any K), 12222, 23212, 22224, 22232, 13122
 # (K in steps of 64 or 32, loads straight into LDS) force one (for measurements and tests).
 TILED_CONFIG = 0
 # Waves the split weight-streaming kernel aims to have on the chip: 8 per workgroup at 256 strips

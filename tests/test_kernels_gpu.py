@@ -182,7 +182,7 @@ def test_linear_tiled_bf16(shape):
     _linear_case(fn, m, n, k, bf, bf, bf, 0, False, lda=k + 8)
 
 
-@pytest.mark.parametrize("config", [12222, 23212, 22224, 13122])
+@pytest.mark.parametrize("config", [12222, 23212, 22224, 22232, 13122])
 @pytest.mark.parametrize("shape", [(65, 128, 64), (300, 333, 512), (513, 700, 192), (2048, 512, 1024), (100, 2048, 2048), (70, 90, 32)])
 def test_linear_large_tile_bf16(shape, config, monkeypatch):
     """The kernel that loads straight into LDS, at every wave tile, with ragged edges in M and N
