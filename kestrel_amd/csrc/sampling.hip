@@ -191,6 +191,180 @@ sample_kernel(const float* __restrict__ logits, long ld, const float* __restrict
     if (threadIdx.x == 0) ka_store_token(out, pending, r, found_idx >= 0 ? found_idx : greedy);
 }
 
+// The same selection for rows of at most R * 1024 logits, each read once: a thread keeps its R
+// logits (then probabilities) in registers. The threshold of the nucleus is bisected between 0
+// and the largest probability and the search ends as soon as no probability lies between its
+// bounds (the set {p >= threshold} is then settled); the draw is located by wave sums of the
+// groups of 64 neighbouring tokens, one scan of those, and one scan inside the group found.
+// sample_kernel above passes over the row about 35 times (300 us at a vocabulary of 51200: a
+// quarter of a decode step); this one takes about a tenth of that.
+template <int R>
+__global__ void __launch_bounds__(SM_THREADS)
+sample_regs_kernel(const float* __restrict__ logits, long ld, const float* __restrict__ temps,
+                   const float* __restrict__ top_ps, const unsigned long long* __restrict__ rng_key,
+                   const int* __restrict__ rng_counter, int* __restrict__ out, int V,
+                   PendingTable pending) {
+    __shared__ float sf[SM_WAVES];
+    __shared__ int si[SM_WAVES];
+    __shared__ float group_sum[R * SM_WAVES];       // of tokens (j * 1024 + wave * 64) .. + 64, in that order
+    __shared__ int found_group;
+    __shared__ float found_before;
+    const int r = blockIdx.x, tid = threadIdx.x;
+    const int lane = tid % KA_WAVE, wave = tid / KA_WAVE;
+    const float* row = logits + (size_t)r * ld;
+    const float T = temps[r];
+    // (every load unconditional, from a place moved inside the row: a load under a branch would
+    // make the compiler wait for each one before the next is asked for)
+    float x[R];
+#pragma unroll
+    for (int j = 0; j < R; ++j) x[j] = row[min(j * SM_THREADS + tid, V - 1)];
+#pragma unroll
+    for (int j = 0; j < R; ++j)
+        if (j * SM_THREADS + tid >= V) x[j] = -INFINITY;
+    // the maximum and its first index
+    float best = -INFINITY;
+    int best_i = 0x7fffffff;
+#pragma unroll
+    for (int j = 0; j < R; ++j) {
+        const int i = j * SM_THREADS + tid;
+        if (i < V && x[j] > best) { best = x[j]; best_i = i; }      // j rises with i: the first of equals stays
+    }
+#pragma unroll
+    for (int off = KA_WAVE / 2; off > 0; off >>= 1) {
+        float ov = __shfl_xor(best, off, KA_WAVE);
+        int oi = __shfl_xor(best_i, off, KA_WAVE);
+        if (ov > best || (ov == best && oi < best_i)) { best = ov; best_i = oi; }
+    }
+    if (lane == 0) { sf[wave] = best; si[wave] = best_i; }
+    __syncthreads();
+    best = sf[0]; best_i = si[0];
+    for (int w = 1; w < SM_WAVES; ++w) {
+        float ov = sf[w]; int oi = si[w];
+        if (ov > best || (ov == best && oi < best_i)) { best = ov; best_i = oi; }
+    }
+    const int greedy = best_i == 0x7fffffff ? 0 : best_i;
+    if (!(T > SM_GREEDY_EPS)) {
+        if (tid == 0) ka_store_token(out, pending, r, greedy);
+        return;
+    }
+    const float inv_t = 1.0f / T, mx = best;
+    float z = 0.f;
+#pragma unroll
+    for (int j = 0; j < R; ++j) {
+        x[j] = expf((x[j] - mx) * inv_t);              // exp(-inf) = 0: masked tokens and the places past V
+        z += x[j];
+    }
+    z = block_reduce_sum(z, sf);
+    const float inv_z = 1.0f / z;
+#pragma unroll
+    for (int j = 0; j < R; ++j) x[j] *= inv_z;
+    const float top_p = top_ps ? top_ps[r] : 1.0f;
+    float thresh = 0.f, mass = 1.0f;
+    if (top_p < 1.0f) {
+        // f(t) = mass of {p >= t} falls with t; keep the largest t with f(t) >= top_p
+        float lo = 0.f, hi = inv_z * (1.0f + 1e-6f) + 1e-30f;      // just above the largest probability
+        for (int it = 0; it < 32; ++it) {
+            const float mid = 0.5f * (lo + hi);
+            // the mass at and above mid, and how many probabilities lie in [lo, hi)
+            float f = 0.f, between = 0.f;
+#pragma unroll
+            for (int j = 0; j < R; ++j) {
+                f += x[j] >= mid ? x[j] : 0.f;
+                between += (x[j] >= lo && x[j] < hi && x[j] > 0.f) ? 1.f : 0.f;
+            }
+            // both sums at once: two values per wave through LDS
+            f = ka_wave_sum(f);
+            between = ka_wave_sum(between);
+            __syncthreads();
+            if (lane == 0) { sf[wave] = f; group_sum[wave] = between; }
+            __syncthreads();
+            f = 0.f; between = 0.f;
+#pragma unroll
+            for (int w = 0; w < SM_WAVES; ++w) { f += sf[w]; between += group_sum[w]; }
+            const bool exhausted = !(mid > lo && mid < hi);          // no float left between the bounds
+            if (f >= top_p) lo = mid; else hi = mid;
+            // f(lo) >= top_p > f(hi) throughout. With at most one probability in [lo, hi) the
+            // tokens above hi do not reach top_p, so that one is needed: {p >= lo} is the nucleus,
+            // the same set for the old and the new bounds. (Tracking the least and the greatest
+            // probability between the bounds instead, which also ends the search on equal
+            // probabilities, costs more per round than it saves: 172 against 115 us per step.)
+            if (between <= 1.f || exhausted) break;
+        }
+        thresh = lo;
+        float f = 0.f;
+#pragma unroll
+        for (int j = 0; j < R; ++j) {
+            if (x[j] < thresh) x[j] = 0.f;
+            f += x[j];
+        }
+        mass = block_reduce_sum(f, sf);
+    }
+    const float u = ka_uniform(rng_key[r], (unsigned long long)(unsigned)rng_counter[r]);
+    const float target = u * mass;
+    // Inversion in index order: the first token whose cumulative mass exceeds the target.
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < R; ++j) {
+        float g = ka_wave_sum(x[j]);
+        if (lane == 0) group_sum[j * SM_WAVES + wave] = g;
+    }
+    if (tid == 0) found_group = -1;
+    __syncthreads();
+    if (wave == 0) {
+        // one wave walks over the R * 16 group sums, 64 at a time
+        float running = 0.f;
+        for (int base = 0; base < R * SM_WAVES; base += KA_WAVE) {
+            const int gi = base + lane;
+            const float v = gi < R * SM_WAVES ? group_sum[gi] : 0.f;
+            float scan = v;
+#pragma unroll
+            for (int off = 1; off < KA_WAVE; off <<= 1) {
+                float o = __shfl_up(scan, off, KA_WAVE);
+                if (lane >= off) scan += o;
+            }
+            // sums only grow along the lanes: the first one past the target is the group (its own
+            // sum is then positive: the one before was not past it)
+            const float incl = running + scan;
+            const unsigned long long hit = __ballot(incl > target && v > 0.f);
+            if (hit) {
+                const int first = __ffsll((long long)hit) - 1;
+                if (lane == first) { found_group = gi; found_before = incl - v; }
+                break;
+            }
+            running += __shfl(scan, KA_WAVE - 1, KA_WAVE);
+        }
+    }
+    __syncthreads();
+    const int grp = found_group;
+    int token = greedy;
+    if (grp >= 0) {
+        const int j = grp / SM_WAVES, w = grp % SM_WAVES;
+        if (wave == w) {
+            float p = 0.f;
+#pragma unroll
+            for (int jj = 0; jj < R; ++jj)
+                if (jj == j) p = x[jj];
+            float scan = p;
+#pragma unroll
+            for (int off = 1; off < KA_WAVE; off <<= 1) {
+                float o = __shfl_up(scan, off, KA_WAVE);
+                if (lane >= off) scan += o;
+            }
+            const float incl = found_before + scan;
+            const unsigned long long past = __ballot(p > 0.f && incl > target);
+            const unsigned long long any = __ballot(p > 0.f);
+            // the first token past the target; if the two ways of summing disagree in the last
+            // bit and none is, the group's last token with any mass
+            int pick = -1;
+            if (past) pick = __ffsll((long long)past) - 1;
+            else if (any) pick = 63 - __clzll((long long)any);
+            if (lane == (pick < 0 ? 0 : pick)) ka_store_token(out, pending, r, pick < 0 ? greedy : j * SM_THREADS + w * KA_WAVE + pick);
+        }
+        return;
+    }
+    if (tid == 0) ka_store_token(out, pending, r, token);
+}
+
 KA_API int ka_argmax(const float* logits, long ld, int* out, int rows, int V, int* pending,
                      const int* pending_at, int n_pending, hipStream_t stream) {
     KA_CHECK(!pending || (pending_at && n_pending > 0), "ka_argmax: a pending table needs its places");
@@ -202,6 +376,8 @@ KA_API int ka_argmax(const float* logits, long ld, int* out, int rows, int V, in
     return 0;
 }
 
+static int sm_passes_only = 0;
+
 KA_API int ka_sample(const float* logits, long ld, const float* temps, const float* top_ps,
                      const unsigned long long* rng_key, const int* rng_counter, int* out, int rows,
                      int V, int* pending, const int* pending_at, int n_pending, hipStream_t stream) {
@@ -209,11 +385,28 @@ KA_API int ka_sample(const float* logits, long ld, const float* temps, const flo
     KA_CHECK(!pending || (pending_at && n_pending > 0), "ka_sample: a pending table needs its places");
     KA_CHECK(temps && rng_key && rng_counter, "ka_sample: temperatures and generator state are required");
     if (rows == 0) return 0;
-    hipLaunchKernelGGL(sample_kernel, dim3(rows), dim3(SM_THREADS), 0, stream, logits, ld, temps, top_ps, rng_key,
-                       rng_counter, out, V, PendingTable{pending, pending_at, n_pending});
+    const PendingTable table{pending, pending_at, n_pending};
+    const int per_thread = ka_cdiv(V, SM_THREADS);
+#define KA_SAMPLE_REGS(RV)                                                                                        \
+    hipLaunchKernelGGL(sample_regs_kernel<RV>, dim3(rows), dim3(SM_THREADS), 0, stream, logits, ld, temps, top_ps, \
+                       rng_key, rng_counter, out, V, table)
+    if (sm_passes_only || per_thread > 64)
+        hipLaunchKernelGGL(sample_kernel, dim3(rows), dim3(SM_THREADS), 0, stream, logits, ld, temps, top_ps, rng_key,
+                           rng_counter, out, V, table);
+    else if (per_thread <= 8) KA_SAMPLE_REGS(8);
+    else if (per_thread <= 16) KA_SAMPLE_REGS(16);
+    else if (per_thread <= 32) KA_SAMPLE_REGS(32);
+    else if (per_thread <= 40) KA_SAMPLE_REGS(40);
+    else if (per_thread <= 52) KA_SAMPLE_REGS(52);
+    else KA_SAMPLE_REGS(64);
+#undef KA_SAMPLE_REGS
     KA_LAUNCH_CHECK();
     return 0;
 }
+
+// 1: every row goes through the kernel that passes over the row many times, whatever its length
+// (otherwise rows longer than 65536 only): for tests of that kernel.
+KA_API void ka_sample_set_passes_only(int on) { sm_passes_only = on; }
 
 // ----------------------------------------------------------------------------
 // Masks before sampling (kestrel/scheduler/scheduler.py:2563-2604,2854-2927): tokens a request

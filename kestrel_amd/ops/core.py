@@ -57,6 +57,8 @@ def lib():
         handle.ka_last_error.restype = ctypes.c_char_p
         handle.ka_uniform_host.argtypes = [ctypes.c_ulonglong, ctypes.c_ulonglong]
         handle.ka_uniform_host.restype = _c_float
+        handle.ka_sample_set_passes_only.argtypes = [_c_int]
+        handle.ka_sample_set_passes_only.restype = None
         _lib = handle
     return _lib
 
@@ -256,6 +258,12 @@ def sample(logits: torch.Tensor, temps: torch.Tensor, top_ps: Optional[torch.Ten
     _check(lib().ka_sample(logits.data_ptr(), logits.stride(0), temps.data_ptr(), _ptr(top_ps), rng_key.data_ptr(),
                            rng_counter.data_ptr(), out.data_ptr(), rows, vocab,
                            *_pending_args("sample", rows, pending, pending_at), stream_ptr()))
+
+
+def set_sample_passes_only(on: bool) -> None:
+    """Sends every row through the sampling kernel that passes over the row many times (it
+    otherwise serves rows of more than 65536 logits only): for tests."""
+    lib().ka_sample_set_passes_only(int(bool(on)))
 
 
 def _logit_rows(who: str, logits: torch.Tensor):

@@ -500,6 +500,49 @@ def test_argmax_and_sampling():
     assert 0.0 <= core.uniform(mix_key(5, 42), 7) < 1.0
 
 
+@pytest.mark.parametrize("passes_only", [False, True])
+@pytest.mark.parametrize("vocab", [51200, 1003, 40000, 70000])
+def test_every_draw_is_the_inversion_of_the_nucleus(vocab, passes_only):
+    """The token drawn is the first, in index order, whose cumulative mass in the plain
+    implementation's nucleus distribution exceeds the request's uniform number: for peaked and
+    flat rows, masked tokens, equal logits; by the kernel that keeps a row in registers and by
+    the one that passes over it (which alone takes rows of more than 65536)."""
+    from kestrel_amd.ops import core
+    from kestrel_amd.sampling import Sampler, mix_key
+
+    torch.manual_seed(31)
+    rows = 24
+    logits = torch.randn(rows, vocab)
+    logits[:8] *= 4.0                                  # peaked rows
+    logits[8:12] *= 0.02                               # almost flat rows
+    logits[12, 100:200] = float("-inf")                # masked tokens
+    logits[13, :] = 0.5                                # all equal
+    logits[14, 7] = logits[14, 900] = 9.0              # two equal leaders
+    temps = [0.7] * 8 + [1.0] * 8 + [1.3] * 8
+    tops = ([0.9, 0.5, 0.99, 0.3] * 6)
+    tops[13] = 1.0                                     # (equal probabilities at the nucleus's edge are all kept by the
+                                                       # kernels and taken in index order by the plain implementation)
+    seeds, counters = list(range(100, 100 + rows)), list(range(rows))
+    sampler = Sampler(torch.device(DEV), seed=9)
+    core.set_sample_passes_only(passes_only)
+    try:
+        ids = sampler.sample(logits.to(DEV), temps, tops, seeds, counters).cpu().tolist()
+    finally:
+        core.set_sample_passes_only(False)
+    exact = 0
+    for r in range(rows):
+        probs = plain.nucleus_probs(logits[r], temps[r], tops[r])
+        u = core.uniform(mix_key(9, seeds[r]), counters[r])
+        cdf = torch.cumsum(probs, dim=0)
+        want = int(torch.searchsorted(cdf, torch.tensor(u, dtype=torch.float64), right=True))
+        assert probs[ids[r]] > 0, (r, ids[r])                     # never outside the nucleus
+        if ids[r] == want:
+            exact += 1
+        else:                                    # fp32 sums against fp64: off by a sliver of mass at most
+            assert abs(float(cdf[ids[r]] - cdf[want])) < 3e-4, (r, ids[r], want)    # tens of thousands of fp32 additions
+    assert exact >= rows - 6
+
+
 def test_masks_before_sampling_and_logprobs_after():
     """Vectors of the reference's own tests (``tests/scheduler/test_logprobs.py``): suppression
     composes with an allow-list (``:923-939``); the log-probability of the chosen token follows the
