@@ -132,6 +132,12 @@ class GenerationScheduler:
         left = request.prompt_length - seq.fed
         take = min(left, budget)
         block = request.block_length
+        if take < left:
+            # cut on a page boundary where that is possible, so that the next portion starts on one
+            page = self.runner.cache.page_size
+            aligned = (seq.fed + take) // page * page - seq.fed
+            if aligned > 0 and not (seq.fed < block and seq.fed + aligned < block):
+                take = aligned
         if seq.fed < block and seq.fed + take < block:
             return 0                      # the block must go in whole
         return take
@@ -200,6 +206,10 @@ class GenerationScheduler:
         for seq in admitted:
             self.waiting.remove(seq)
             self.prefilling.append(seq)
+        # prompt portions first in the packed batch: a portion that starts on a page boundary then
+        # also starts on a multiple of 16 tokens, which is what lets the cache write store whole
+        # pages of values at once
+        plan.rows.sort(key=lambda row: row.kind != "prefill")
         return plan
 
     # ------------------------------------------------------------------ running

@@ -87,6 +87,21 @@ def test_prompt_is_cut_under_the_token_budget_and_then_decoded():
     assert runner.cache.groups[0].pool.free_count == 16 and runner.cache.free_slots == 4
 
 
+def test_portions_end_on_page_boundaries():
+    """A portion that does not finish its prompt is cut back to a page boundary (pages of 4 here),
+    so that the next one starts on a fresh page; the last portion takes what is left."""
+    sched, runner = _scheduler(budget=10)
+    sched.enqueue_request(_req(0, 23, 1))
+    sched.run_until_done()
+    portions = [(p, n) for step in runner.steps for _s, p, n, _w in step if n > 1]
+    assert portions == [(0, 8), (8, 8), (16, 7)]
+    # a budget smaller than a page still makes progress
+    sched, runner = _scheduler(budget=3)
+    sched.enqueue_request(_req(0, 9, 1))
+    sched.run_until_done()
+    assert [(p, n) for step in runner.steps for _s, p, n, _w in step][:4] == [(0, 3), (3, 1), (4, 3), (7, 2)]
+
+
 def test_decodes_ride_beside_prompt_portions():
     sched, runner = _scheduler(budget=8)
     sched.enqueue_request(_req(0, 4, 6))
@@ -94,9 +109,11 @@ def test_decodes_ride_beside_prompt_portions():
     sched.enqueue_request(_req(1, 20, 2))
     sched.advance()
     step = runner.steps[-1]
-    assert [(n, want) for _s, _p, n, want in step] == [(1, [0]), (7, [])]   # decode first, prompt gets the rest
+    # the decoding request has its token first, the prompt gets the rest of the budget, cut down to a
+    # page boundary (pages of 4: 4 of the 7 places left); in the packed batch the portion stands first
+    assert [(n, want) for _s, _p, n, want in step] == [(4, []), (1, [0])]
     sched.advance()
-    assert [n for _s, _p, n, _w in runner.steps[-1]] == [1, 7]
+    assert [(p, n) for _s, p, n, _w in runner.steps[-1]][0] == (4, 4)      # the next portion starts on that boundary
     results = sched.run_until_done()
     assert sorted(r.request_id for r in results) == [0, 1]
 
@@ -161,8 +178,8 @@ def test_a_bidirectional_block_goes_in_one_portion():
     sched.enqueue_request(GenerationRequest(1, [5, 6, 7, 8, 9, 10], 2, prefix_embeds=embeds, prefix_ids=[0]))
     sched.advance()
     step = runner.steps[-1]
-    # 1 decode + 11 budget: block of 8 (BOS + 7 rows) and 3 text tokens
-    assert [(n, w) for _s, _p, n, w in step] == [(1, [0]), (11, [])]
+    # 1 decode + 11 budget: block of 8 (BOS + 7 rows) and 3 text tokens, cut back to the page boundary at 8
+    assert [(n, w) for _s, _p, n, w in step] == [(8, []), (1, [0])]
     sched.run_until_done()
     # a block larger than what is left of the budget waits for a step with room; it is never split
     sched, runner = _scheduler(budget=9, n_pages=32)
