@@ -19,7 +19,7 @@
 // Decode kernel. One query per row: a bandwidth problem. The keys of a row are cut into splits
 // (grid z) and 64-key tiles (waves); 16-byte loads are fully coalesced for keys (8 lanes per key
 // row at hd 64) and values (2 lanes per channel row of a page). Waves merge through LDS, splits
-// through scratch memory by the last workgroup to arrive, always in the same order.
+// through scratch memory in a second kernel, always in the same order.
 #include "ka_common.h"
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
@@ -362,7 +362,7 @@ attn_decode_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t
                    const bf16_t* __restrict__ v_cache, const int* __restrict__ block_table, int max_pages,
                    const int* __restrict__ token_row, const int* __restrict__ kv_lo,
                    const int* __restrict__ kv_hi, bf16_t* __restrict__ out, long out_row_stride, float scale,
-                   int H, int Hkv, float* __restrict__ partial, unsigned* __restrict__ counters, DecodeFuse fz) {
+                   int H, int Hkv, float* __restrict__ partial, DecodeFuse fz) {
     constexpr int LPK = HD / 8;            // lanes per key row
     constexpr int KPI = KA_WAVE / LPK;     // keys per load instruction
     constexpr int VU = HD * 2 / KA_WAVE;   // 16-byte value loads per lane and page
@@ -580,36 +580,47 @@ attn_decode_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t
             int d = e * KA_WAVE + lane;
             if (d < HD) mine[2 + d] = od[e];
         }
-        __threadfence();
-        unsigned seen = 0;
-        if (lane == 0) seen = atomicAdd(&counters[t * H + h], 1u);
-        seen = __shfl(seen, 0, KA_WAVE);
-        if (seen != (unsigned)(S - 1)) return;
-        if (lane == 0) atomicExch(&counters[t * H + h], 0u);
-        __threadfence();
-        const float* all = partial + (size_t)(t * H + h) * S * REC;
-        M = -INFINITY;
-        for (int s = 0; s < S; ++s)
-            M = fmaxf(M, __hip_atomic_load(all + s * REC, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
-        L = 0.f;
-#pragma unroll
-        for (int e = 0; e < (HD + KA_WAVE - 1) / KA_WAVE; ++e) od[e] = 0.f;
-        for (int s = 0; s < S; ++s) {
-            float ms = __hip_atomic_load(all + s * REC, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            float f = ms == -INFINITY ? 0.f : exp2f(ms - M);
-            L += __hip_atomic_load(all + s * REC + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) * f;
-#pragma unroll
-            for (int e = 0; e < (HD + KA_WAVE - 1) / KA_WAVE; ++e) {
-                int d = e * KA_WAVE + lane;
-                if (d < HD) od[e] += __hip_atomic_load(all + s * REC + 2 + d, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) * f;
-            }
-        }
+        return;            // the parts meet in attn_decode_merge_kernel
     }
     float inv = L > 0.f ? 1.0f / L : 0.f;
     bf16_t* op = out + (size_t)t * out_row_stride + (size_t)h * HD;
 #pragma unroll
     for (int e = 0; e < (HD + KA_WAVE - 1) / KA_WAVE; ++e) {
         int d = e * KA_WAVE + lane;
+        if (d < HD) op[d] = (bf16_t)(od[e] * inv);
+    }
+}
+
+// The parts of a row's keys meet here, in the order of the parts: one wave per (token, head).
+// A kernel of its own and no arrival counter inside the first: a workgroup that waits for the
+// others' sums to become visible has to flush and refill its XCD's L2 (tens of microseconds).
+template <int HD>
+__global__ void __launch_bounds__(KA_WAVE)
+attn_decode_merge_kernel(const float* __restrict__ partial, int S, bf16_t* __restrict__ out, long out_row_stride, int H) {
+    constexpr int REC = HD + 2;
+    constexpr int E = (HD + KA_WAVE - 1) / KA_WAVE;
+    const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+    const float* all = partial + (size_t)(t * H + h) * S * REC;
+    float M = -INFINITY;
+    for (int s = 0; s < S; ++s) M = fmaxf(M, all[s * REC]);
+    float L = 0.f, od[E];
+#pragma unroll
+    for (int e = 0; e < E; ++e) od[e] = 0.f;
+    for (int s = 0; s < S; ++s) {
+        const float ms = all[s * REC];
+        const float f = ms == -INFINITY ? 0.f : exp2f(ms - M);
+        L += all[s * REC + 1] * f;
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+            const int d = e * KA_WAVE + lane;
+            if (d < HD) od[e] += all[s * REC + 2 + d] * f;
+        }
+    }
+    const float inv = L > 0.f ? 1.0f / L : 0.f;
+    bf16_t* op = out + (size_t)t * out_row_stride + (size_t)h * HD;
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+        const int d = e * KA_WAVE + lane;
         if (d < HD) op[d] = (bf16_t)(od[e] * inv);
     }
 }
@@ -813,7 +824,7 @@ KA_API int ka_attention_decode_bf16(const void* q, long q_row_stride, const void
                                     const int* block_table, int max_pages, const int* token_row, const int* kv_lo,
                                     const int* kv_hi, void* out, long out_row_stride, float scale, int n, int H,
                                     int Hkv, int hd, int page_size, int splits, int waves, float* partial,
-                                    long partial_floats, unsigned* counters, int n_counters, const void* k_new,
+                                    long partial_floats, const void* k_new,
                                     const void* v_new, long new_stride, const float* table, int rot,
                                     const int* slots, void* k_cache_w, void* v_cache_w, hipStream_t stream) {
     if (check_common("ka_attention_decode_bf16", q, q_row_stride, out, out_row_stride, n, H, Hkv, hd, page_size,
@@ -822,10 +833,9 @@ KA_API int ka_attention_decode_bf16(const void* q, long q_row_stride, const void
     KA_CHECK(ka_attention_decode_supported(hd, page_size), "ka_attention_decode_bf16: head size %d not covered", hd);
     KA_CHECK(splits >= 1 && splits <= 65535, "ka_attention_decode_bf16: bad split count %d", splits);
     if (splits > 1) {
-        KA_CHECK(partial && counters, "ka_attention_decode_bf16: scratch missing");
+        KA_CHECK(partial, "ka_attention_decode_bf16: scratch missing");
         KA_CHECK(ka_attention_decode_partial_floats(n, H, hd, splits) <= partial_floats,
                  "ka_attention_decode_bf16: scratch too small");
-        KA_CHECK((long)n * H <= n_counters, "ka_attention_decode_bf16: too few counters");
     }
     KA_CHECK(waves == 4 || waves == 8 || waves == 16, "ka_attention_decode_bf16: waves must be 4, 8 or 16");
     DecodeFuse fz = {};
@@ -841,7 +851,7 @@ KA_API int ka_attention_decode_bf16(const void* q, long q_row_stride, const void
 #define KA_AD(HDV, WV)                                                                                              \
     hipLaunchKernelGGL((attn_decode_kernel<HDV, WV>), grid, block, 0, stream, (const bf16_t*)q, q_row_stride,      \
                        (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, max_pages, token_row, kv_lo,   \
-                       kv_hi, (bf16_t*)out, out_row_stride, scale, H, Hkv, partial, counters, fz)
+                       kv_hi, (bf16_t*)out, out_row_stride, scale, H, Hkv, partial, fz)
     if (hd == 64) {
         if (waves == 4) KA_AD(64, 4); else if (waves == 8) KA_AD(64, 8); else KA_AD(64, 16);
     } else {
@@ -849,5 +859,10 @@ KA_API int ka_attention_decode_bf16(const void* q, long q_row_stride, const void
     }
 #undef KA_AD
     KA_LAUNCH_CHECK();
+    if (splits > 1) {
+        if (hd == 64) hipLaunchKernelGGL(attn_decode_merge_kernel<64>, dim3(n, H), dim3(KA_WAVE), 0, stream, partial, splits, (bf16_t*)out, out_row_stride, H);
+        else hipLaunchKernelGGL(attn_decode_merge_kernel<128>, dim3(n, H), dim3(KA_WAVE), 0, stream, partial, splits, (bf16_t*)out, out_row_stride, H);
+        KA_LAUNCH_CHECK();
+    }
     return 0;
 }

@@ -35,7 +35,7 @@ _SIGNATURES = {
                                  _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
     "ka_attention_decode_bf16": [_c_void_p, _c_long, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p,
                                  _c_void_p, _c_void_p, _c_long, _c_float, _c_int, _c_int, _c_int, _c_int, _c_int,
-                                 _c_int, _c_int, _c_void_p, _c_long, _c_void_p, _c_int,
+                                 _c_int, _c_int, _c_void_p, _c_long,
                                  _c_void_p, _c_void_p, _c_long, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p,
                                  _c_void_p],
 }
@@ -56,7 +56,6 @@ TILED_CONFIG = 0
 # (measured best for the output projection + second feed-forward linear of Moondream 2).
 SKINNY_TARGET_WAVES = 2048
 SCRATCH_FLOATS = 8 << 20
-SCRATCH_COUNTERS = 1 << 16
 WIDE_FLOATS = 8 << 20              # 32 MB of partial sums for skinny linears of 17 to 64 rows
 _wide_scratch = {}
 # Keys of one row a workgroup of the decode attention kernel takes before the row is split.
@@ -107,13 +106,12 @@ def _check(status: int) -> None:
         raise KernelError(lib().ka_last_error().decode())
 
 
-def scratch(device: torch.device):
-    """Partial results and arrival counters that splits of a long row meet through (one pair per
-    device; the kernels leave the counters at zero). Calls on one device must not overlap."""
+def scratch(device: torch.device) -> torch.Tensor:
+    """Partial results that the parts of a row's keys meet through in decode attention (one
+    buffer per device). Calls on one device must not overlap."""
     key = torch.device(device)
     if key not in _scratch:
-        _scratch[key] = (torch.zeros(SCRATCH_FLOATS, dtype=torch.float32, device=device),
-                         torch.zeros(SCRATCH_COUNTERS, dtype=torch.int32, device=device))
+        _scratch[key] = torch.zeros(SCRATCH_FLOATS, dtype=torch.float32, device=device)
     return _scratch[key]
 
 
@@ -264,8 +262,9 @@ def rope_cache_bf16(qkv, positions, slots, table, k_cache, v_cache, n_heads, n_k
 
 def decode_shape(max_kv: int, workgroups: int = 1):
     """``(splits, waves)`` of the decode attention kernel: a workgroup of up to 16 waves takes a
-    64-key tile per wave and round; rows longer than 4096 keys are cut into splits that meet
-    through scratch memory. With many workgroups (rows x heads) each gets fewer waves, so that
+    64-key tile per wave and round; rows longer than 4096 keys are cut into parts whose sums
+    a second kernel merges (cutting the keys of a few short rows further, to put more CUs to
+    work, was measured and changes nothing: 0.887 ms a step at batch 1 either way). With many workgroups (rows x heads) each gets fewer waves, so that
     they all fit on the chip at once (measured at 1024 keys: 16 waves up to 256 workgroups, 8 at
     512 and 1024, 4 from 2048 on)."""
     splits = max(1, -(-max_kv // DECODE_KEYS_PER_WORKGROUP))
@@ -293,8 +292,8 @@ def attention_decode_bf16(q, k_cache, v_cache, block_table, token_row, kv_lo, kv
             or not handle.ka_attention_decode_supported(head_dim, page_size):
         return False
     splits, waves = decode_shape(batch.max_kv, n * n_heads)
-    partial, counters = scratch(q.device)
-    if n * n_heads * splits * (head_dim + 2) > partial.numel() or n * n_heads > counters.numel():
+    partial = scratch(q.device)
+    if n * n_heads * splits * (head_dim + 2) > partial.numel():
         return False
     k_new = v_new = table = slots = None
     new_stride = rot = 0
@@ -302,14 +301,14 @@ def attention_decode_bf16(q, k_cache, v_cache, block_table, token_row, kv_lo, kv
         k_new, v_new, table, slots = fuse
         rot = int(table.shape[1])
         new_stride = k_new.stride(0)
-        if rot % 16 or rot > head_dim or splits != 1 or k_new.data_ptr() % 16 or v_new.data_ptr() % 16 \
+        if rot % 16 or rot > head_dim or k_new.data_ptr() % 16 or v_new.data_ptr() % 16 \
                 or new_stride % 8 or v_new.stride(0) != new_stride:
             return False
     _check(handle.ka_attention_decode_bf16(
         q.data_ptr(), q.stride(0), k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(),
         block_table.shape[1], token_row.data_ptr(), _ptr(kv_lo), kv_hi.data_ptr(), out.data_ptr(), out.stride(0),
         float(scale), n, n_heads, n_kv_heads, head_dim, page_size, splits, waves, partial.data_ptr(), partial.numel(),
-        counters.data_ptr(), counters.numel(), _ptr(k_new), _ptr(v_new), new_stride, _ptr(table), rot, _ptr(slots),
+        _ptr(k_new), _ptr(v_new), new_stride, _ptr(table), rot, _ptr(slots),
         k_cache.data_ptr(), v_cache.data_ptr(), stream_ptr()))
     return True
 

@@ -691,7 +691,7 @@ def test_decode_attention_that_rotates_and_stores(shape):
 
 
 def test_decode_attention_splits_long_rows(monkeypatch):
-    """Rows longer than a workgroup's share are cut into splits that meet through scratch memory."""
+    """Rows longer than a workgroup's share are cut into parts that a second kernel merges."""
     from kestrel_amd.ops import fast
 
     monkeypatch.setattr(fast, "DECODE_KEYS_PER_WORKGROUP", 256)
@@ -699,5 +699,5 @@ def test_decode_attention_splits_long_rows(monkeypatch):
     bf = torch.bfloat16
     case = PagedCase([1000, 3, 257, 700], [1, 1, 1, 1], h, hkv, hd, 16, bf, seed=24)
     assert fast.decode_shape(case.batch.max_kv)[0] == 4
-    for _ in range(2):                                   # twice: the counters must be left at zero
+    for _ in range(2):                                   # twice: nothing of the first run may be left in the way
         _close(_run_attention(case, "fast", hd ** -0.5), case.reference(hd ** -0.5), bf)
