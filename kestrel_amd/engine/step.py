@@ -269,8 +269,14 @@ class ModelRunner:
                 positions.extend(np.arange(start, start + q, dtype=np.int64))
                 token_row.extend(np.full(q, r, dtype=np.int64))
             kv_hi.extend(hi)
-            for first in range(0, q, self.QUERY_BLOCK):
-                blocks.append((r, base + first, int(max(hi[first:first + self.QUERY_BLOCK]))))
+            if isinstance(hi, np.ndarray):
+                # most keys any query of a block sees: the blocks' maxima in one go
+                pad = (-q) % self.QUERY_BLOCK
+                tops = np.pad(hi, (0, pad)).reshape(-1, self.QUERY_BLOCK).max(axis=1).tolist()
+                blocks.extend((r, base + i * self.QUERY_BLOCK, top) for i, top in enumerate(tops))
+            else:
+                for first in range(0, q, self.QUERY_BLOCK):
+                    blocks.append((r, base + first, max(hi[first:first + self.QUERY_BLOCK])))
             for w in e.want:
                 if not 0 <= int(w) < q:
                     raise ValueError(f"slot {e.slot}: wanted place {w} outside its {q} tokens")
