@@ -129,12 +129,23 @@ layernorm_regs_kernel(const float* __restrict__ x, const int* __restrict__ rows,
     int i = blockIdx.x;
     const float* src = x + (size_t)(rows ? rows[i] : i) * dim;
     TOut* dst = out + (size_t)i * dim;
-    floatx4 v[ITEMS];
+    // (every load unconditional, from a place moved inside the row; a load under a branch would
+    // make the compiler wait for each before the next is asked for)
+    floatx4 v[ITEMS], g[ITEMS], b[ITEMS];
     float s = 0.f;
+    const bool beta_vec = beta && (reinterpret_cast<uintptr_t>(beta) % 16 == 0);
+#pragma unroll
+    for (int j = 0; j < ITEMS; ++j) {
+        int d = min((j * LN_THREADS + (int)threadIdx.x) * 4, dim - 4);
+        v[j] = *reinterpret_cast<const floatx4*>(src + d);
+        g[j] = *reinterpret_cast<const floatx4*>(gamma + d);
+        b[j] = beta_vec ? *reinterpret_cast<const floatx4*>(beta + d) : floatx4{0.f, 0.f, 0.f, 0.f};
+    }
 #pragma unroll
     for (int j = 0; j < ITEMS; ++j) {
         int d = (j * LN_THREADS + threadIdx.x) * 4;
-        v[j] = d < dim ? *reinterpret_cast<const floatx4*>(src + d) : floatx4{0.f, 0.f, 0.f, 0.f};
+        if (d >= dim) v[j] = floatx4{0.f, 0.f, 0.f, 0.f};
+        if (beta && !beta_vec && d < dim) b[j] = floatx4{beta[d], beta[d + 1], beta[d + 2], beta[d + 3]};
         s += (v[j][0] + v[j][1]) + (v[j][2] + v[j][3]);
     }
     float mean = block_sum_256(s, smem) / (float)dim;
@@ -148,16 +159,20 @@ layernorm_regs_kernel(const float* __restrict__ x, const int* __restrict__ rows,
         }
     }
     float rstd = 1.0f / sqrtf(block_sum_256(q, smem) / (float)dim + eps);
+    const bool out_vec = reinterpret_cast<uintptr_t>(dst) % (4 * sizeof(TOut)) == 0;      // (dim is a multiple of 4)
 #pragma unroll
     for (int j = 0; j < ITEMS; ++j) {
         int d = (j * LN_THREADS + threadIdx.x) * 4;
         if (d < dim) {
-            floatx4 g = *reinterpret_cast<const floatx4*>(gamma + d);
+            TOut y[4];
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                float y = (v[j][e] - mean) * rstd * g[e];
-                if (beta) y += beta[d + e];
-                dst[d + e] = ka_from_float<TOut>(y);
+            for (int e = 0; e < 4; ++e) y[e] = ka_from_float<TOut>((v[j][e] - mean) * rstd * g[j][e] + b[j][e]);
+            if (out_vec) {
+                typedef TOut __attribute__((ext_vector_type(4))) out4;
+                *reinterpret_cast<out4*>(dst + d) = out4{y[0], y[1], y[2], y[3]};
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) dst[d + e] = y[e];
             }
         }
     }
