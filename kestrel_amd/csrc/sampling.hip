@@ -97,6 +97,43 @@ __device__ int block_argmax(const float* __restrict__ row, int V, float* smem_f,
     return best_i;
 }
 
+// The same for rows of at most R * 1024 logits, all of a thread's loads in flight at once (a row
+// is then one trip to memory; block_argmax asks for eight values a thread and round).
+template <int R>
+__global__ void __launch_bounds__(SM_THREADS)
+argmax_regs_kernel(const float* __restrict__ logits, long ld, int* __restrict__ out, int V,
+                   PendingTable pending) {
+    __shared__ float sf[SM_WAVES];
+    __shared__ int si[SM_WAVES];
+    const int r = blockIdx.x, tid = threadIdx.x;
+    const float* row = logits + (size_t)r * ld;
+    float x[R];
+#pragma unroll
+    for (int j = 0; j < R; ++j) x[j] = row[min(j * SM_THREADS + tid, V - 1)];
+    float best = -INFINITY;
+    int best_i = 0x7fffffff;
+#pragma unroll
+    for (int j = 0; j < R; ++j) {
+        const int i = j * SM_THREADS + tid;
+        if (i < V && x[j] > best) { best = x[j]; best_i = i; }      // j rises with i: the first of equals stays
+    }
+#pragma unroll
+    for (int off = KA_WAVE / 2; off > 0; off >>= 1) {
+        float ov = __shfl_xor(best, off, KA_WAVE);
+        int oi = __shfl_xor(best_i, off, KA_WAVE);
+        if (ov > best || (ov == best && oi < best_i)) { best = ov; best_i = oi; }
+    }
+    if (tid % KA_WAVE == 0) { sf[tid / KA_WAVE] = best; si[tid / KA_WAVE] = best_i; }
+    __syncthreads();
+    if (tid != 0) return;
+    best = sf[0]; best_i = si[0];
+    for (int w = 1; w < SM_WAVES; ++w) {
+        float ov = sf[w]; int oi = si[w];
+        if (ov > best || (ov == best && oi < best_i)) { best = ov; best_i = oi; }
+    }
+    ka_store_token(out, pending, r, best_i == 0x7fffffff ? 0 : best_i);
+}
+
 __global__ void __launch_bounds__(SM_THREADS)
 argmax_kernel(const float* __restrict__ logits, long ld, int* __restrict__ out, int V,
               PendingTable pending) {
@@ -370,8 +407,14 @@ KA_API int ka_argmax(const float* logits, long ld, int* out, int rows, int V, in
     KA_CHECK(!pending || (pending_at && n_pending > 0), "ka_argmax: a pending table needs its places");
     KA_CHECK(rows >= 0 && V > 0 && ld >= V, "ka_argmax: bad sizes rows=%d V=%d ld=%ld", rows, V, ld);
     if (rows == 0) return 0;
-    hipLaunchKernelGGL(argmax_kernel, dim3(rows), dim3(SM_THREADS), 0, stream, logits, ld, out, V,
-                       PendingTable{pending, pending_at, n_pending});
+    const PendingTable table{pending, pending_at, n_pending};
+    const int per_thread = ka_cdiv(V, SM_THREADS);
+    if (per_thread <= 16)
+        hipLaunchKernelGGL(argmax_regs_kernel<16>, dim3(rows), dim3(SM_THREADS), 0, stream, logits, ld, out, V, table);
+    else if (per_thread <= 52)
+        hipLaunchKernelGGL(argmax_regs_kernel<52>, dim3(rows), dim3(SM_THREADS), 0, stream, logits, ld, out, V, table);
+    else
+        hipLaunchKernelGGL(argmax_kernel, dim3(rows), dim3(SM_THREADS), 0, stream, logits, ld, out, V, table);
     KA_LAUNCH_CHECK();
     return 0;
 }
