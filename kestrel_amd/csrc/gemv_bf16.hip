@@ -724,13 +724,25 @@ skinny_wide_finish_kernel(const float* __restrict__ partial, int splits, const f
     const int m = idx / quads, n = (idx % quads) * 4;
     const bool whole = n + 3 < N && N % 4 == 0;
     float s[4] = {0.f, 0.f, 0.f, 0.f};
-    for (int sp = 0; sp < splits; ++sp) {
-        const float* src = partial + ((size_t)sp * M + m) * N + n;
-        if (whole) {
-            floatx4 v = *reinterpret_cast<const floatx4*>(src);
+    if (whole) {
+        // eight parts' sums are asked for at once (a part past the last is the last again, and
+        // left out of the sum), then added in the order of the parts
+        for (int sp0 = 0; sp0 < splits; sp0 += 8) {
+            floatx4 v[8];
 #pragma unroll
-            for (int i = 0; i < 4; ++i) s[i] += v[i];
-        } else {
+            for (int u = 0; u < 8; ++u)
+                v[u] = *reinterpret_cast<const floatx4*>(partial + ((size_t)min(sp0 + u, splits - 1) * M + m) * N + n);
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                if (sp0 + u < splits) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) s[i] += v[u][i];
+                }
+            }
+        }
+    } else {
+        for (int sp = 0; sp < splits; ++sp) {
+            const float* src = partial + ((size_t)sp * M + m) * N + n;
             for (int i = 0; i < 4 && n + i < N; ++i) s[i] += src[i];
         }
     }
