@@ -45,7 +45,13 @@ __device__ __forceinline__ void at_wave_sync() {
 // ----------------------------------------------------------------------------------------------
 constexpr int AP_WAVES = 4;                 // waves of a workgroup: all on the same 32 queries, keys interleaved
 constexpr int AP_QBLOCK = 32;               // queries per workgroup
-constexpr int AP_MAX_TABLE = 24576;         // block table entries of one row that fit in LDS beside the merge (393k keys)
+constexpr int AP_MAX_TABLE = 24576;         // most block table entries of one row kept in LDS (393k keys)
+constexpr int ap_merge_floats(int hd) { return (hd + 31) / 32 * 16 + 2; }
+// block table entries of one row that fit in LDS beside the merge at head size hd
+constexpr int ap_max_table(int hd) {
+    int left = (160 * 1024 - (AP_WAVES - 1) * ap_merge_floats(hd) * KA_WAVE * 4 - 256) / 4;
+    return left < AP_MAX_TABLE ? left : AP_MAX_TABLE;
+}
 
 // (At least two waves per SIMD, except at head size 128, which needs more registers: with 256 registers a lane the compiler lets the MFMAs write
 // ordinary registers. Left to itself it puts their results in accumulator registers and then
@@ -58,9 +64,13 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_
                     const int* __restrict__ cu_q, const int* __restrict__ kv_len,
                     const int* __restrict__ kv_lo, const int* __restrict__ kv_hi, bf16_t* __restrict__ out,
                     long out_row_stride, float scale, int H, int Hkv, int table_entries) {
+    static_assert(HD % 16 == 0 && HD >= 16 && HD <= 256, "head sizes in steps of 16 up to 256");
     constexpr int QC = HD / 16;          // 16-byte chunks of half a head row = MFMA steps of the score product
-    constexpr int DB = HD / 32;          // 32-channel blocks of the output
-    constexpr int REC = DB * 16 + 2;     // floats a lane hands over at the merge: its outputs, m and l
+    constexpr int DB = (HD + 31) / 32;   // 32-channel blocks of the output
+    // A head size that is no multiple of 32 leaves the last block half used: its lanes 16..31
+    // load the channels of lanes 0..15 once more, and what they compute is never stored.
+    constexpr bool HALF_BLOCK = HD % 32 != 0;
+    constexpr int REC = ap_merge_floats(HD);   // floats a lane hands over at the merge: its outputs, m and l
     __shared__ float mrg[AP_WAVES - 1][REC][KA_WAVE];
     extern __shared__ int pages[];       // the row's block table: `table_entries` of them
     // Heads are the fast index of the grid: the workgroups that run side by side then have the
@@ -123,6 +133,7 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_
     const size_t page_stride = (size_t)Hkv * AT_PAGE * HD;           // elements of a page, keys or values
     const unsigned k_lane = (unsigned)(kvh * AT_PAGE * HD + lg * (HD / 2));
     const unsigned v_lane = (unsigned)((kvh * HD + li) * AT_PAGE + lg * 8);
+    const unsigned v_lane_half = (unsigned)((kvh * HD + (DB - 1) * 32 + (li & 15)) * AT_PAGE + lg * 8);
 
     // half a key row of tile `key0` for this lane's (permuted) key
     auto load_keys = [&](int key0, bf16x8* dst) {
@@ -142,7 +153,8 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_
             unsigned page = (unsigned)__builtin_amdgcn_readfirstlane(pages[kbase / AT_PAGE]);
             const bf16_t* vp = v_cache + (size_t)page * page_stride;
 #pragma unroll
-            for (int db = 0; db < DB; ++db) dst[pg][db] = at_load8(vp + (v_lane + db * 32 * AT_PAGE));
+            for (int db = 0; db < DB; ++db)
+                dst[pg][db] = at_load8(vp + (HALF_BLOCK && db == DB - 1 ? v_lane_half : v_lane + db * 32 * AT_PAGE));
         }
     };
     // what of them may be used: nothing of a page outside the wave's keys (another page was
@@ -278,6 +290,7 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_
     for (int db = 0; db < DB; ++db)
 #pragma unroll
         for (int qd = 0; qd < 4; ++qd) {
+            if (db * 32 + qd * 8 >= HD) continue;          // the unused half of the last block
             int d = db * 32 + qd * 8 + lg * 4;
             bf16x4 r = {(bf16_t)(o[db][qd * 4 + 0] * inv), (bf16_t)(o[db][qd * 4 + 1] * inv),
                         (bf16_t)(o[db][qd * 4 + 2] * inv), (bf16_t)(o[db][qd * 4 + 3] * inv)};
@@ -289,6 +302,7 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_
 // decode kernel
 // ----------------------------------------------------------------------------------------------
 constexpr int AD_TILE = 64;               // keys per wave tile
+constexpr int ad_lanes_per_key(int hd) { int l = 1; while (l * 8 < hd) l *= 2; return l; }
 
 // What the decode kernel needs to take over the rotary encoding and the cache write of the
 // step's own token (slots null: that work was done before, and the token's key is in the cache).
@@ -363,9 +377,14 @@ attn_decode_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t
                    const int* __restrict__ token_row, const int* __restrict__ kv_lo,
                    const int* __restrict__ kv_hi, bf16_t* __restrict__ out, long out_row_stride, float scale,
                    int H, int Hkv, float* __restrict__ partial, DecodeFuse fz) {
-    constexpr int LPK = HD / 8;            // lanes per key row
+    static_assert(HD % 16 == 0 && HD >= 16 && HD <= 256, "head sizes in steps of 16 up to 256");
+    constexpr int CPK = HD / 8;            // 16-byte chunks of a key row
+    constexpr int LPK = ad_lanes_per_key(HD);   // lanes per key row: the chunks, rounded up to a power of two
     constexpr int KPI = KA_WAVE / LPK;     // keys per load instruction
-    constexpr int VU = HD * 2 / KA_WAVE;   // 16-byte value loads per lane and page
+    constexpr int KL = AD_TILE / KPI;      // key loads per lane and tile
+    constexpr int VU = (HD + 31) / 32;     // 16-byte value loads per lane and page (a lane takes channel u * 32 + lane / 2)
+    // Where the head size is no power of two, the lanes past a key row's chunks, and past the
+    // channels of a value page, ask for what another lane asks for and add nothing.
     constexpr int TP = AD_TILE / AT_PAGE;  // pages of a tile
     constexpr int REC = HD + 2;            // floats of a partial result: m, l, o[HD]
     __shared__ float ps[WAVES][AD_TILE];
@@ -382,7 +401,9 @@ attn_decode_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t
     const int lo_tile = lo & ~(AD_TILE - 1);      // tiles start on page boundaries; keys below lo are masked
     const int chunk = ((hi - lo_tile + S - 1) / S + AD_TILE - 1) / AD_TILE * AD_TILE;
     const int s_lo = lo_tile + split * chunk, s_hi = min(hi, s_lo + chunk);
-    const int ks = lane / LPK, dg = lane % LPK;
+    const int ks = lane / LPK, dg_lane = lane % LPK;
+    const bool chunk_live = dg_lane < CPK;             // this lane holds a chunk of the key row
+    const int dg = chunk_live ? dg_lane : 0;
     const float sl2 = scale * AT_LOG2E;
     const bool takes_new = fused && wave == 0 && split == 0;     // this wave adds the token's own key and value
 
@@ -403,7 +424,7 @@ attn_decode_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t
         kr = at_fetch_rotary(fz.k_new + (size_t)t * fz.stride + (size_t)kvh * HD, dg, fz.rot);
         const bf16_t* vrow = fz.v_new + (size_t)t * fz.stride + (size_t)kvh * HD;
 #pragma unroll
-        for (int u = 0; u < VU; ++u) vnew[u] = vrow[u * 32 + lane / 2];
+        for (int u = 0; u < VU; ++u) vnew[u] = vrow[min(u * 32 + lane / 2, HD - 1)];
     }
 
     const int* bt = block_table + (size_t)row * max_pages;
@@ -423,7 +444,7 @@ attn_decode_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t
         for (int j = 0; j < 8; ++j) qf[j] = (float)qplain[j];
     }
 #pragma unroll
-    for (int j = 0; j < 8; ++j) qf[j] *= sl2;
+    for (int j = 0; j < 8; ++j) qf[j] = chunk_live ? qf[j] * sl2 : 0.f;
     float m_i = -INFINITY, l_i = 0.f;
     float acc[VU];
 #pragma unroll
@@ -436,7 +457,7 @@ attn_decode_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t
         const int slot = fz.slots[t];
         if (slot >= 0 && h % (H / Hkv) == 0) {
             const size_t page = slot / AT_PAGE, off = slot % AT_PAGE;
-            if (ks == 0) {
+            if (ks == 0 && chunk_live) {
                 bf16x8 kb;
 #pragma unroll
                 for (int j = 0; j < 8; ++j) kb[j] = (bf16_t)kn[j];
@@ -446,7 +467,7 @@ attn_decode_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t
 #pragma unroll
                 for (int u = 0; u < VU; ++u) {
                     int d = u * 32 + lane / 2;
-                    fz.v_cache[((page * Hkv + kvh) * HD + d) * AT_PAGE + off] = vnew[u];
+                    if (d < HD) fz.v_cache[((page * Hkv + kvh) * HD + d) * AT_PAGE + off] = vnew[u];
                 }
             }
         }
@@ -465,19 +486,19 @@ attn_decode_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t
         // All key loads of the tile go out before any arithmetic, and none stands under a
         // condition: a place outside [lo, s_hi) is moved to one inside and masked afterwards. The
         // compiler can then wait for exactly the register it needs instead of for everything.
-        bf16x8 kreg[LPK];
+        bf16x8 kreg[KL];
 #pragma unroll
-        for (int i = 0; i < LPK; ++i) {
+        for (int i = 0; i < KL; ++i) {
             int key = tile0 + i * KPI + ks;
             int kc = max(min(key, s_hi - 1), lo);   // a place that holds data (pages below lo may be gone)
             int page = bt[kc / AT_PAGE];
             kreg[i] = at_load8(k_cache + (((size_t)page * Hkv + kvh) * AT_PAGE + kc % AT_PAGE) * HD + dg * 8);
         }
         __builtin_amdgcn_sched_barrier(0);     // all of them, before the first is used
-        float sc[LPK];
+        float sc[KL];
         float mx = -INFINITY;
 #pragma unroll
-        for (int i = 0; i < LPK; ++i) {
+        for (int i = 0; i < KL; ++i) {
             int key = tile0 + i * KPI + ks;
             bool ok = key >= lo && key < s_hi;
             float dot = 0.f;
@@ -501,7 +522,7 @@ attn_decode_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t
             int page = bt[kc / AT_PAGE];
 #pragma unroll
             for (int u = 0; u < VU; ++u) {
-                int d = u * 32 + lane / 2;
+                int d = min(u * 32 + lane / 2, HD - 1);
                 vreg[pg][u] = at_load8(v_cache + (((size_t)page * Hkv + kvh) * HD + d) * AT_PAGE + (lane & 1) * 8);
             }
         }
@@ -510,10 +531,10 @@ attn_decode_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t
         float rowsum = 0.f;
         at_wave_sync();                        // the previous tile's probabilities have been read
 #pragma unroll
-        for (int i = 0; i < LPK; ++i) {
+        for (int i = 0; i < KL; ++i) {
             float p = exp2f(sc[i] - m_new);
             rowsum += p;
-            if (dg == 0) ps[wave][i * KPI + ks] = p;
+            if (dg_lane == 0) ps[wave][i * KPI + ks] = p;
         }
 #pragma unroll
         for (int off = LPK; off < KA_WAVE; off <<= 1) rowsum += __shfl_xor(rowsum, off, KA_WAVE);
@@ -549,7 +570,8 @@ attn_decode_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t
     if (lane == 0) { merge[wave][0] = m_i; merge[wave][1] = l_i; }
     if ((lane & 1) == 0) {
 #pragma unroll
-        for (int u = 0; u < VU; ++u) merge[wave][2 + u * 32 + lane / 2] = acc[u];
+        for (int u = 0; u < VU; ++u)
+            if (u * 32 + lane / 2 < HD) merge[wave][2 + u * 32 + lane / 2] = acc[u];
     }
     __syncthreads();
     if (wave != 0) return;
@@ -765,12 +787,22 @@ KA_API int ka_rope_cache_pages_bf16(void* qkv, long row_stride, const int* posit
     return 0;
 }
 
+// Head sizes in steps of 16 up to 128 and in steps of 32 up to 256.
+static bool at_head_size_covered(int hd) {
+    return hd >= 16 && hd <= 256 && hd % 16 == 0 && (hd <= 128 || hd % 32 == 0);
+}
+
 KA_API int ka_attention_prefill_supported(int hd, int page_size) {
-    return page_size == AT_PAGE && (hd == 32 || hd == 64 || hd == 96 || hd == 128);
+    return page_size == AT_PAGE && at_head_size_covered(hd);
+}
+
+// Keys of one row that the prompt kernel takes at this head size (its block table lies in LDS).
+KA_API int ka_attention_prefill_max_keys(int hd) {
+    return at_head_size_covered(hd) ? ap_max_table(hd) * AT_PAGE : 0;
 }
 
 KA_API int ka_attention_decode_supported(int hd, int page_size) {
-    return page_size == AT_PAGE && (hd == 64 || hd == 128);
+    return page_size == AT_PAGE && at_head_size_covered(hd);
 }
 
 KA_API int ka_attention_prefill_bf16(const void* q, long q_row_stride, const void* k_cache, const void* v_cache,
@@ -787,8 +819,8 @@ KA_API int ka_attention_prefill_bf16(const void* q, long q_row_stride, const voi
     // width of the block table is kept in LDS)
     int table_entries = max_pages;
     if (longest_row > 0 && ka_cdiv(longest_row, AT_PAGE) < max_pages) table_entries = ka_cdiv(longest_row, AT_PAGE);
-    KA_CHECK(table_entries <= AP_MAX_TABLE, "ka_attention_prefill_bf16: a row of %d keys is longer than the %d this kernel takes",
-             table_entries * AT_PAGE, AP_MAX_TABLE * AT_PAGE);
+    KA_CHECK(table_entries <= ap_max_table(hd), "ka_attention_prefill_bf16: a row of %d keys is longer than the %d this kernel takes at head size %d",
+             table_entries * AT_PAGE, ap_max_table(hd) * AT_PAGE, hd);
     const size_t table_bytes = (size_t)table_entries * sizeof(int);
     KA_CHECK(n_qblocks <= 65535, "ka_attention_prefill_bf16: more than 65535 blocks of queries in one launch");
     dim3 grid(H, n_qblocks), block(KA_WAVE * AP_WAVES);
@@ -797,7 +829,7 @@ KA_API int ka_attention_prefill_bf16(const void* q, long q_row_stride, const voi
         static bool configured = false;                                                                             \
         if (!configured) {                                                                                          \
             hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(attn_prefill_kernel<HDV>),             \
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, AP_MAX_TABLE * sizeof(int)); \
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, ap_max_table(HDV) * sizeof(int)); \
             KA_CHECK(e == hipSuccess, "ka_attention_prefill_bf16: cannot reserve LDS: %s", hipGetErrorString(e));   \
             configured = true;                                                                                      \
         }                                                                                                           \
@@ -806,10 +838,18 @@ KA_API int ka_attention_prefill_bf16(const void* q, long q_row_stride, const voi
                        (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, max_pages, qblk_row, qblk_tok,  \
                        cu_q, kv_len, kv_lo, kv_hi, (bf16_t*)out, out_row_stride, scale, H, Hkv, table_entries)
     switch (hd) {
+        case 16: KA_AP(16); break;
         case 32: KA_AP(32); break;
+        case 48: KA_AP(48); break;
         case 64: KA_AP(64); break;
+        case 80: KA_AP(80); break;
         case 96: KA_AP(96); break;
-        default: KA_AP(128); break;
+        case 112: KA_AP(112); break;
+        case 128: KA_AP(128); break;
+        case 160: KA_AP(160); break;
+        case 192: KA_AP(192); break;
+        case 224: KA_AP(224); break;
+        default: KA_AP(256); break;
     }
 #undef KA_AP
     KA_LAUNCH_CHECK();
@@ -846,22 +886,40 @@ KA_API int ka_attention_decode_bf16(const void* q, long q_row_stride, const void
         KA_CHECK(new_stride % 8 == 0 && (uintptr_t)k_new % 16 == 0 && (uintptr_t)v_new % 16 == 0, "ka_attention_decode_bf16: new key rows must be 16-byte aligned");
         fz = DecodeFuse{(const bf16_t*)k_new, (const bf16_t*)v_new, new_stride, table, rot, slots, (bf16_t*)k_cache_w, (bf16_t*)v_cache_w};
     }
-    if (hd == 128 && waves == 16) waves = 8;   // 16 waves leave 128 registers a lane: too few for a tile's loads
+    if (hd > 64 && waves == 16) waves = 8;   // 16 waves leave 128 registers a lane: too few for a tile's loads (measured at head size 80: 26.4 against 23.6 us)
     dim3 grid(n, H, splits), block(KA_WAVE * waves);
 #define KA_AD(HDV, WV)                                                                                              \
     hipLaunchKernelGGL((attn_decode_kernel<HDV, WV>), grid, block, 0, stream, (const bf16_t*)q, q_row_stride,      \
                        (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, max_pages, token_row, kv_lo,   \
                        kv_hi, (bf16_t*)out, out_row_stride, scale, H, Hkv, partial, fz)
-    if (hd == 64) {
-        if (waves == 4) KA_AD(64, 4); else if (waves == 8) KA_AD(64, 8); else KA_AD(64, 16);
-    } else {
-        if (waves == 4) KA_AD(128, 4); else KA_AD(128, 8);
+#define KA_AD_SMALL(HDV)                                                                                            \
+    case HDV:                                                                                                       \
+        if (waves == 4) KA_AD(HDV, 4); else if (waves == 8) KA_AD(HDV, 8); else KA_AD(HDV, 16);                     \
+        break
+#define KA_AD_LARGE(HDV)                                                                                            \
+    case HDV:                                                                                                       \
+        if (waves == 4) KA_AD(HDV, 4); else KA_AD(HDV, 8);                                                          \
+        break
+    switch (hd) {
+        KA_AD_SMALL(16); KA_AD_SMALL(32); KA_AD_SMALL(48); KA_AD_SMALL(64);
+        KA_AD_LARGE(80); KA_AD_LARGE(96); KA_AD_LARGE(112); KA_AD_LARGE(128);
+        KA_AD_LARGE(160); KA_AD_LARGE(192); KA_AD_LARGE(224); KA_AD_LARGE(256);
     }
+#undef KA_AD_SMALL
+#undef KA_AD_LARGE
 #undef KA_AD
     KA_LAUNCH_CHECK();
     if (splits > 1) {
-        if (hd == 64) hipLaunchKernelGGL(attn_decode_merge_kernel<64>, dim3(n, H), dim3(KA_WAVE), 0, stream, partial, splits, (bf16_t*)out, out_row_stride, H);
-        else hipLaunchKernelGGL(attn_decode_merge_kernel<128>, dim3(n, H), dim3(KA_WAVE), 0, stream, partial, splits, (bf16_t*)out, out_row_stride, H);
+#define KA_ADM(HDV)                                                                                                 \
+    case HDV:                                                                                                       \
+        hipLaunchKernelGGL(attn_decode_merge_kernel<HDV>, dim3(n, H), dim3(KA_WAVE), 0, stream, partial, splits,    \
+                           (bf16_t*)out, out_row_stride, H);                                                        \
+        break
+        switch (hd) {
+            KA_ADM(16); KA_ADM(32); KA_ADM(48); KA_ADM(64); KA_ADM(80); KA_ADM(96); KA_ADM(112); KA_ADM(128);
+            KA_ADM(160); KA_ADM(192); KA_ADM(224); KA_ADM(256);
+        }
+#undef KA_ADM
         KA_LAUNCH_CHECK();
     }
     return 0;

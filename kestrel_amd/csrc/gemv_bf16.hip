@@ -849,13 +849,14 @@ static int launch_persistent(int strips, int M, int kblocks, bool ln, size_t dyn
 
 template <int MB, bool HALF>
 static int launch_split(int waves, int strips, hipStream_t stream, const SkinnyArgs& args) {
-    if (waves >= 16) {
+    // (rounded to the nearest of 4, 8 and 16)
+    if (waves >= 12) {
         if constexpr (HALF) {      // 16 waves leave 128 registers a lane: enough only for the half-column form
             hipLaunchKernelGGL((skinny_split_kernel<MB, 16, HALF>), dim3(strips), dim3(16 * KA_WAVE), 0, stream, args);
             return 0;
         }
     }
-    if (waves >= 8) hipLaunchKernelGGL((skinny_split_kernel<MB, 8, HALF>), dim3(strips), dim3(8 * KA_WAVE), 0, stream, args);
+    if (waves >= 6) hipLaunchKernelGGL((skinny_split_kernel<MB, 8, HALF>), dim3(strips), dim3(8 * KA_WAVE), 0, stream, args);
     else hipLaunchKernelGGL((skinny_split_kernel<MB, 4, HALF>), dim3(strips), dim3(4 * KA_WAVE), 0, stream, args);
     return 0;
 }

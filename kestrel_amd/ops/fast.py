@@ -83,6 +83,8 @@ def lib():
         for name in ("ka_attention_prefill_supported", "ka_attention_decode_supported"):
             getattr(handle, name).argtypes = [_c_int, _c_int]
             getattr(handle, name).restype = _c_int
+        handle.ka_attention_prefill_max_keys.argtypes = [_c_int]
+        handle.ka_attention_prefill_max_keys.restype = _c_int
         _lib = handle
     return _lib
 
@@ -325,7 +327,10 @@ def attention_bf16(q, k_cache, v_cache, block_table, token_row, kv_lo, kv_hi, ou
                              n_kv_heads, head_dim, batch):
         return True
     handle = lib()
-    if handle.ka_attention_prefill_supported(head_dim, page_size) and batch.qblk_row is not None:
+    # the longest row's block table must fit in LDS (the whole table's width where the length is not known)
+    longest = int(batch.max_kv) if batch.max_kv > 1 else block_table.shape[1] * page_size
+    if handle.ka_attention_prefill_supported(head_dim, page_size) and batch.qblk_row is not None \
+            and longest <= handle.ka_attention_prefill_max_keys(head_dim):
         _check(handle.ka_attention_prefill_bf16(
             q.data_ptr(), q.stride(0), k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(),
             block_table.shape[1], batch.qblk_row.data_ptr(), batch.qblk_tok.data_ptr(), int(batch.qblk_row.numel()),

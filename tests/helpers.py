@@ -25,15 +25,21 @@ TINY_D = {"text": {"dim": 128, "ff_dim": 136, "n_layers": 2, "vocab_size": 300, 
                    "n_kv_heads": 1, "rope_theta": 10000.0, "prefix_attn": 9, "layer_norm_eps": 1e-5}}
 TINY_E = {"text": {"dim": 256, "ff_dim": 264, "n_layers": 2, "vocab_size": 411, "max_context": 192, "n_heads": 2,
                    "n_kv_heads": 2, "rope_theta": 2500.0, "rotary_dim": 32, "prefix_attn": 6, "layer_norm_eps": 2e-6}}
+# A head size that is no power of two on the MFMA kernels (80, as in Phi-2: ten 16-byte chunks a key row, two
+# and a half blocks of 32 output channels), grouped kv heads, a rotary part of 32 channels.
+TINY_F = {"text": {"dim": 160, "ff_dim": 168, "n_layers": 2, "vocab_size": 333, "max_context": 256, "n_heads": 4,
+                   "n_kv_heads": 2, "head_dim": 80, "rotary_dim": 32, "rope_theta": 10000.0, "prefix_attn": 7,
+                   "layer_norm_eps": 1e-5}}
 RECIPES = {
     "A": InitRecipe(std=0.02),
     "B": InitRecipe(std=0.03, gain_std=0.02, shift_std=0.02),
     "C": InitRecipe(std=0.05, bias_std=0.1, gain_std=0.1, shift_std=0.05),
     "D": InitRecipe(std=0.04, gain_std=0.05, shift_std=0.05),
     "E": InitRecipe(std=0.03, bias_std=0.05, gain_std=0.05, shift_std=0.02),
+    "F": InitRecipe(std=0.04, bias_std=0.03, gain_std=0.05, shift_std=0.03),
 }
-CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D, "E": TINY_E}
-SEEDS = {"A": 0, "B": 1, "C": 2, "D": 3, "E": 4}
+CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D, "E": TINY_E, "F": TINY_F}
+SEEDS = {"A": 0, "B": 1, "C": 2, "D": 3, "E": 4, "F": 5}
 
 
 @functools.lru_cache(maxsize=None)

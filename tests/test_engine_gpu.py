@@ -17,7 +17,7 @@ pytestmark = pytest.mark.gpu
 
 DTYPES = [torch.float32, torch.bfloat16]
 DTYPE_IDS = ["fp32", "bf16"]
-NAMES = ["A", "B", "C", "D", "E"]
+NAMES = ["A", "B", "C", "D", "E", "F"]
 
 
 def _runner(name, dtype, n_pages=64, page_size=16, max_requests=8):
@@ -110,7 +110,7 @@ def test_mixed_batches_with_page_reuse(name, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=DTYPE_IDS)
-@pytest.mark.parametrize("name", ["B", "C", "D", "E"])
+@pytest.mark.parametrize("name", ["B", "C", "D", "E", "F"])
 def test_prefix_embeddings_bidirectional(name, dtype):
     """Given embeddings as one bidirectional block, then text; the block in one portion, the
     rest cut into portions and decoded; two such requests mixed."""
@@ -134,7 +134,7 @@ def test_split_bidirectional_block_is_refused():
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=DTYPE_IDS)
-@pytest.mark.parametrize("name", ["B", "D"])
+@pytest.mark.parametrize("name", ["B", "D", "F"])
 def test_long_decoding(name, dtype):
     """A short prompt, then every further token one by one up to the context length."""
     length = helpers.flat_config(name)["max_context"]

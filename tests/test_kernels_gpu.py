@@ -391,7 +391,8 @@ def test_attention_generic(shape, dtype):
     _close(_run_attention(block, "generic", hd ** -0.5), block.reference(hd ** -0.5), dtype)
 
 
-@pytest.mark.parametrize("shape", [(4, 4, 64), (6, 2, 32), (3, 1, 96), (4, 2, 128), (32, 32, 64)])
+@pytest.mark.parametrize("shape", [(4, 4, 64), (6, 2, 32), (3, 1, 96), (4, 2, 128), (32, 32, 64), (2, 2, 16), (6, 3, 48),
+                                   (4, 4, 80), (3, 1, 112), (2, 1, 160), (2, 2, 192), (2, 1, 224), (1, 1, 256)])
 def test_attention_prompt_kernel(shape):
     """Whole prompts, portions that continue a cache, single tokens in a mixed batch, a block that
     sees both ways, a window; query counts that do not fill a wave."""
@@ -405,7 +406,8 @@ def test_attention_prompt_kernel(shape):
     _close(_run_attention(windowed, "fast", 0.2), windowed.reference(0.2), bf)
 
 
-@pytest.mark.parametrize("shape", [(4, 4, 64), (6, 2, 128), (32, 32, 64), (8, 1, 64)])
+@pytest.mark.parametrize("shape", [(4, 4, 64), (6, 2, 128), (32, 32, 64), (8, 1, 64), (2, 2, 16), (4, 1, 32), (6, 3, 48),
+                                   (4, 4, 80), (3, 1, 96), (2, 2, 112), (2, 1, 160), (2, 2, 192), (2, 1, 224), (1, 1, 256)])
 def test_attention_decode_kernel(shape):
     """One token per row, contexts from one key to many splits' worth, with and without a window."""
     h, hkv, hd = shape
@@ -653,7 +655,8 @@ def test_layernorm_prologue_skinny_linear(shape):
                                           torch.empty(17, nb, dtype=torch.bfloat16, device=DEV), 1)
 
 
-@pytest.mark.parametrize("shape", [(4, 4, 64, 32), (6, 2, 128, 64), (8, 1, 64, 16)])
+@pytest.mark.parametrize("shape", [(4, 4, 64, 32), (6, 2, 128, 64), (8, 1, 64, 16), (2, 2, 16, 16), (4, 2, 48, 32), (4, 4, 80, 32),
+                                   (2, 1, 112, 48), (2, 2, 160, 80), (1, 1, 256, 128)])
 def test_decode_attention_that_rotates_and_stores(shape):
     """The decode kernel with rotary encoding and cache write fused in, against the rotary kernel
     followed by the plain decode kernel: same outputs, same cache."""
