@@ -925,7 +925,20 @@ KA_API int ka_linear_skinny_fused(const void* A1, long lda1, int K1, const void*
         KA_LAUNCH_CHECK();
         return 0;
     }
-    if (M > 16 && !Wb && partials && (sk_wide_enabled >= 2 || (sk_wide_enabled && A2))) {
+    // More than 16 rows of a K too long for the persistent kernel's registers: the split kernel
+    // would read all activations from L2 once per strip (78 us for 48 rows, K = 2560, N = 17920;
+    // the wide kernel shares them through LDS). Two targets go one after the other.
+    const bool persistent_ok = !A2 && !accumulate_a && sk_persistent_enabled && persistent_fits(M, kblocks, args);
+    if (M > 16 && Wb && partials && sk_wide_enabled && !persistent_ok) {
+        int rc = ka_linear_skinny_fused(A1, lda1, K1, nullptr, 0, 0, nullptr, 0, nullptr, nullptr, nullptr, nullptr, 0.f,
+                                        Wa, ldwa, biasa, outa, out_dtype_a, ldoa, Na, acta, accumulate_a, nullptr, 0,
+                                        nullptr, nullptr, 0, 0, 0, 0, M, target_waves, partials, partial_floats, stream);
+        if (rc) return rc;
+        return ka_linear_skinny_fused(A1, lda1, K1, nullptr, 0, 0, nullptr, 0, nullptr, nullptr, nullptr, nullptr, 0.f,
+                                      Wb, ldwb, biasb, outb, out_dtype_b, ldob, Nb, actb, 0, nullptr, 0, nullptr,
+                                      nullptr, 0, 0, 0, 0, M, target_waves, partials, partial_floats, stream);
+    }
+    if (M > 16 && !Wb && partials && (sk_wide_enabled >= 2 || (sk_wide_enabled && (A2 || !persistent_ok)))) {
         WideArgs wide = {};
         wide.A[0] = args.A[0]; wide.lda[0] = args.lda[0]; wide.W[0] = args.a.W; wide.ldw[0] = args.a.ldw; wide.K[0] = K1;
         if (A2) { wide.A[1] = args.A[1]; wide.lda[1] = args.lda[1]; wide.W[1] = args.W2; wide.ldw[1] = args.ldw2; wide.K[1] = K2; }
@@ -951,7 +964,7 @@ KA_API int ka_linear_skinny_fused(const void* A1, long lda1, int K1, const void*
             return 0;
         }
     }
-    if (!A2 && !accumulate_a && sk_persistent_enabled && persistent_fits(M, kblocks, args)) {
+    if (persistent_ok) {
         if (launch_persistent(strips, M, kblocks, false, 0, stream, args)) return -1;
         KA_LAUNCH_CHECK();
         return 0;

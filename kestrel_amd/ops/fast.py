@@ -202,7 +202,7 @@ def linear_two_outputs(a, wa, ba, out_a, act_a, wb, bb, out_b, act_b) -> bool:
         None, None, None, 0.0,
         wa.data_ptr(), wa.stride(0), _ptr(ba), out_a.data_ptr(), _OUT_CODE[out_a.dtype], out_a.stride(0), na, act_a, 0,
         wb.data_ptr(), wb.stride(0), _ptr(bb), out_b.data_ptr(), _OUT_CODE[out_b.dtype], out_b.stride(0), nb, act_b,
-        m, SKINNY_TARGET_WAVES, None, 0, stream_ptr()))
+        m, SKINNY_TARGET_WAVES, *_wide_args(a.device, m), stream_ptr()))
     return True
 
 
