@@ -938,7 +938,11 @@ KA_API int ka_linear_skinny_fused(const void* A1, long lda1, int K1, const void*
                                       Wb, ldwb, biasb, outb, out_dtype_b, ldob, Nb, actb, 0, nullptr, 0, nullptr,
                                       nullptr, 0, 0, 0, 0, M, target_waves, partials, partial_floats, stream);
     }
-    if (M > 16 && !Wb && partials && (sk_wide_enabled >= 2 || (sk_wide_enabled && (A2 || !persistent_ok)))) {
+    // Up to 16 rows of two segments: where there are more strips than CUs the split kernel,
+    // which gives a strip to a workgroup, takes about twice the time that it takes with one
+    // strip a CU (N = 2560, K = 2560 + 10240, 16 rows: 40 us; 25 us here).
+    const bool crowded = A2 && strips > sk_compute_units() && M > 4;      // (a single row: 19 us against 24)
+    if (!Wb && partials && ((sk_wide_enabled && (M > 16 ? (A2 || !persistent_ok) : crowded)) || sk_wide_enabled >= 2)) {
         WideArgs wide = {};
         wide.A[0] = args.A[0]; wide.lda[0] = args.lda[0]; wide.W[0] = args.a.W; wide.ldw[0] = args.a.ldw; wide.K[0] = K1;
         if (A2) { wide.A[1] = args.A[1]; wide.lda[1] = args.lda[1]; wide.W[1] = args.W2; wide.ldw[1] = args.ldw2; wide.K[1] = K2; }
@@ -952,6 +956,7 @@ KA_API int ka_linear_skinny_fused(const void* A1, long lda1, int K1, const void*
             wide.splits = splits;
             dim3 grid(groups, splits);
             switch (MB) {
+                case 1: hipLaunchKernelGGL(skinny_wide_kernel<1>, grid, dim3(WD_WAVES * KA_WAVE), 0, stream, wide); break;
                 case 2: hipLaunchKernelGGL(skinny_wide_kernel<2>, grid, dim3(WD_WAVES * KA_WAVE), 0, stream, wide); break;
                 case 3: hipLaunchKernelGGL(skinny_wide_kernel<3>, grid, dim3(WD_WAVES * KA_WAVE), 0, stream, wide); break;
                 default: hipLaunchKernelGGL(skinny_wide_kernel<4>, grid, dim3(WD_WAVES * KA_WAVE), 0, stream, wide); break;

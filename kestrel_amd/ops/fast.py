@@ -56,7 +56,7 @@ TILED_CONFIG = 0
 # (measured best for the output projection + second feed-forward linear of Moondream 2).
 SKINNY_TARGET_WAVES = 2048
 SCRATCH_FLOATS = 8 << 20
-WIDE_FLOATS = 8 << 20              # 32 MB of partial sums for skinny linears of 17 to 64 rows
+WIDE_FLOATS = 8 << 20              # 32 MB of partial sums for the wide skinny kernel
 _wide_scratch = {}
 # Keys of one row a workgroup of the decode attention kernel takes before the row is split.
 DECODE_KEYS_PER_WORKGROUP = 4096
@@ -118,11 +118,9 @@ def scratch(device: torch.device) -> torch.Tensor:
 
 
 def _wide_args(device: torch.device, rows: int):
-    """Scratch memory for the parts of K of a skinny linear of more than 16 rows: fp32 partial
-    sums, one buffer per device, made at the first such call. Calls on one device must not
-    overlap."""
-    if rows <= 16:
-        return None, 0
+    """Scratch memory for the parts of K of a skinny linear that goes to the wide kernel: fp32
+    partial sums, one buffer per device, made at the first skinny call (a step's first run is
+    never inside a graph capture). Calls on one device must not overlap."""
     key = torch.device(device)
     if key not in _wide_scratch:
         _wide_scratch[key] = torch.empty(WIDE_FLOATS, dtype=torch.float32, device=device)
