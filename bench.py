@@ -24,6 +24,13 @@ if ROOT not in sys.path:
 # Layer sizes of the benchmark model (Moondream 2 text decoder) and its workload.
 MODEL = {"dim": 2048, "ff_dim": 8192, "n_layers": 24, "vocab_size": 51200, "max_context": 2048, "n_heads": 32,
          "n_kv_heads": 32, "rope_theta": 10000.0, "prefix_attn": 730, "layer_norm_eps": 1e-5}
+# Another member of the family for measurements beside the default: Phi-2's layer sizes (head size 80).
+SIZES = {
+    "moondream2": MODEL,
+    "phi2": {"dim": 2560, "ff_dim": 10240, "n_layers": 32, "vocab_size": 51200, "max_context": 2048, "n_heads": 32,
+             "n_kv_heads": 32, "rope_theta": 10000.0, "prefix_attn": 0, "layer_norm_eps": 1e-5, "rotary_dim": 32},
+}
+LABELS = {"moondream2": ("Moondream 2 text decoder sizes", "moondream2-text"), "phi2": ("Phi-2 layer sizes", "phi2-sizes")}
 CONTEXT = 1024          # tokens each request holds when decoding starts (730 prefix + 294 text)
 PREFILL_TOKENS = 2048
 PAGE_SIZE = 16
@@ -32,7 +39,7 @@ PEAK_HBM = 8.0e12
 PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
 
 
-def build_model(layers: int, dtype, device):
+def build_model(layers: int, dtype, device, sizes=None):
     """The benchmark model with random weights drawn on the GPU (nothing is read from disk)."""
     import torch
 
@@ -41,7 +48,7 @@ def build_model(layers: int, dtype, device):
     from kestrel_amd.weights import InitRecipe, random_tensor
 
     spec = get_spec("moondream2")
-    typed = spec.read_config({"text": dict(MODEL, n_layers=layers)})
+    typed = spec.read_config({"text": dict(sizes or MODEL, n_layers=layers)})
     net = DecoderModel(spec.build_plan(typed))
     recipe = InitRecipe(std=0.02)
     store = torch.bfloat16
@@ -192,7 +199,8 @@ def main() -> int:
     parser.add_argument("--steps", type=int, default=128)
     parser.add_argument("--warmup", type=int, default=8)
     parser.add_argument("--batch", type=int, default=8)
-    parser.add_argument("--layers", type=int, default=MODEL["n_layers"], help="fewer layers than the model has (named in config)")
+    parser.add_argument("--sizes", default="moondream2", choices=sorted(SIZES), help="layer sizes (the default is the benchmark's)")
+    parser.add_argument("--layers", type=int, default=None, help="fewer layers than the model has (named in config)")
     parser.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     parser.add_argument("--skip-points", action="store_true", help="only the default batch (no batch 1 / 64, no prefill)")
     parser.add_argument("--only-prefill", action="store_true", help="only the 2,048-token prefill (for profiling)")
@@ -209,7 +217,10 @@ def main() -> int:
     torch.cuda.set_device(device)
     dtype = torch.bfloat16 if args.dtype == "bf16" else torch.float32
     size = 2 if dtype == torch.bfloat16 else 4
-    net, typed = build_model(args.layers, dtype, device)
+    sizes = SIZES[args.sizes]
+    if args.layers is None:
+        args.layers = sizes["n_layers"]
+    net, typed = build_model(args.layers, dtype, device, sizes)
     weights = model_bytes(net, size)
 
     if args.only_prefill:
@@ -222,12 +233,12 @@ def main() -> int:
     step_bytes = weights + kv_bytes * (size / 2) + args.batch * typed.dim * size
     achieved = step_bytes / (elapsed / args.steps)
     record = {
-        "metric": f"decode tok/s (Moondream 2 text decoder sizes, batch {args.batch}, context {CONTEXT})",
+        "metric": f"decode tok/s ({LABELS[args.sizes][0]}, batch {args.batch}, context {CONTEXT})",
         "value": round(value, 1),
         "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": args.dtype, "data": "synthetic (seeded random token ids and prefix embeddings, random weights N(0,0.02))",
-        "config": {"model": "moondream2-text", "n_layers": args.layers, "n_layers_full": MODEL["n_layers"],
+        "config": {"model": LABELS[args.sizes][1], "n_layers": args.layers, "n_layers_full": sizes["n_layers"],
                    "dim": typed.dim, "ff_dim": typed.ff_dim, "n_heads": typed.n_heads, "n_kv_heads": typed.n_kv_heads,
                    "head_dim": typed.head_dim, "rotary_dim": typed.rotary_dim, "vocab_size": typed.vocab_size,
                    "global_batch": args.batch, "seq_len": CONTEXT, "prefix_attn": typed.prefix_attn,
