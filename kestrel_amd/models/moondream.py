@@ -28,6 +28,10 @@ from ..parts.specs import (AttentionSpec, DenseFeedForwardSpec, LayerSpec, Model
 _PRESET = Path(__file__).resolve().parent / "presets" / "moondream2.json"
 _REQUIRED = ("dim", "ff_dim", "n_layers", "vocab_size", "max_context", "n_heads", "n_kv_heads", "rope_theta")
 _OPTIONAL = ("prefix_attn", "group_size", "moe", "tau_attn", "head_dim", "rotary_dim", "layer_norm_eps")
+# Other spellings of the three values that the reference fixes in code and of its rotary base.
+_ALIASES = {"layer_norm_eps": ("layernorm_eps", "ln_eps", "norm_eps", "eps", "layer_norm_epsilon"),
+            "rotary_dim": ("rot_dim", "rope_dim", "rotary_ndims"),
+            "rope_theta": ("theta", "rotary_theta", "rope_base")}
 
 
 def _preset() -> Dict[str, Any]:
@@ -57,10 +61,18 @@ class MoondreamTextConfig:
         preset = _preset()
         text = config.get("text")
         if text is None:
-            flat = {k: config[k] for k in _REQUIRED + _OPTIONAL if k in config}
+            spellings = _REQUIRED + _OPTIONAL + tuple(o for others in _ALIASES.values() for o in others)
+            flat = {k: config[k] for k in spellings if k in config}
             text = flat if flat else preset["text"]
         if not isinstance(text, dict):
             raise ValueError("config.json: 'text' must be an object")
+        text = dict(text)
+        for key, others in _ALIASES.items():
+            given = [o for o in others if o in text]
+            if given and (key in text or len(given) > 1):
+                raise ValueError(f"config.json: {[key] * (key in text) + given} name the same value")
+            if given:
+                text[key] = text.pop(given[0])
         unknown = sorted(set(text) - set(_REQUIRED) - set(_OPTIONAL))
         if unknown:
             raise ValueError(f"config.json: unknown text keys {unknown}; known: {sorted(_REQUIRED + _OPTIONAL)}")
@@ -148,7 +160,8 @@ def build_plan(cfg: MoondreamTextConfig) -> ModelPlan:
 
 def _claims(config: Dict[str, Any]) -> bool:
     text = config.get("text", config)
-    return isinstance(text, dict) and all(k in text for k in ("dim", "ff_dim", "n_layers", "n_heads", "rope_theta"))
+    return isinstance(text, dict) and all(k in text for k in ("dim", "ff_dim", "n_layers", "n_heads")) \
+        and any(k in text for k in ("rope_theta",) + _ALIASES["rope_theta"])
 
 
 register(ModelSpec(

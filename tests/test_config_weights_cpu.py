@@ -56,6 +56,22 @@ def test_config_errors(change, message):
         MoondreamTextConfig.from_dict({"text": text})
 
 
+def test_other_spellings_of_the_added_keys():
+    from kestrel_amd.config import get_spec
+    from kestrel_amd.config.registry import resolve
+
+    base = {k: v for k, v in helpers.flat_config("C").items() if k not in ("layer_norm_eps", "rotary_dim", "rope_theta")}
+    spelled = dict(base, eps=3e-5, rope_dim=12, theta=1234.5)
+    for config in (spelled, {"text": spelled}):
+        assert resolve(config).name == "moondream2"
+        cfg = get_spec("moondream2").read_config(config)
+        assert (cfg.layer_norm_eps, cfg.rotary_dim, cfg.rope_theta) == (3e-5, 12, 1234.5)
+    with pytest.raises(ValueError, match="name the same value"):
+        get_spec("moondream2").read_config(dict(spelled, ln_eps=1e-5))
+    with pytest.raises(ValueError, match="name the same value"):
+        get_spec("moondream2").read_config(dict(spelled, layer_norm_eps=1e-5))
+
+
 def test_quantized_config_is_refused():
     text = dict(helpers.TINY_A["text"], group_size=128)
     with pytest.raises(NotImplementedError):
