@@ -38,7 +38,8 @@ typedef __attribute__((ext_vector_type(4))) float floatx4;
 constexpr int SK_STRIP = 8;        // weight rows per strip
 constexpr int SK_KBLOCK = 64;      // k per wave and step
 constexpr int SK_LN_ROWS = 16;     // most rows the LayerNorm prologue takes
-constexpr int SK_XV = 8;           // float4 per lane of a row kept in registers (rows up to 2048 wide)
+constexpr int SK_XV = 8;           // float4 per lane of a row kept in registers: rows up to 2048 wide
+constexpr int SK_XV_WIDE = 16;     // ... and up to 4096 wide, then without the scale and shift beside them
 constexpr int SK_PAD = 8;          // bf16 of padding per LDS row (keeps 16-byte reads off each other's banks)
 constexpr int SP_WAVES = 8;        // waves of a persistent workgroup
 constexpr int SP_MAX_PER = 8;      // most k-blocks per wave it keeps activations for
@@ -155,34 +156,41 @@ __device__ __forceinline__ void sk_finish(const floatx4 (*red)[MB][KA_WAVE], con
 // A row to be normalised, with the scale and shift that meet it: fetched in one trip to memory
 // (sk_fetch_row) and turned into bf16 in LDS later (sk_normalise_row), so that other loads can
 // be issued in between without standing in front of these in the wave's queue.
+// (XV float4 per lane; EARLY: scale and shift come with the row, else they are read when the row
+// is normalised: a second trip, to L2 by then, that rows of more than 2048 pay for their registers)
+template <int XV, bool EARLY>
 struct RowOperands {
-    floatx4 x[SK_XV], gamma[SK_XV], beta[SK_XV];
+    floatx4 x[XV], gamma[EARLY ? XV : 1], beta[EARLY ? XV : 1];
 };
 
-__device__ __forceinline__ void sk_fetch_row(const SkinnyArgs& p, int m, int lane, RowOperands& row) {
+template <int XV, bool EARLY>
+__device__ __forceinline__ void sk_fetch_row(const SkinnyArgs& p, int m, int lane, RowOperands<XV, EARLY>& row) {
     const int K = p.K[0];
     const float* src = p.ln_x + (size_t)m * K;
 #pragma unroll
-    for (int j = 0; j < SK_XV; ++j) {
+    for (int j = 0; j < XV; ++j) {
         const int k = min((j * KA_WAVE + lane) * 4, K - 4);
         row.x[j] = *reinterpret_cast<const floatx4*>(src + k);
-        row.gamma[j] = *reinterpret_cast<const floatx4*>(p.ln_gamma + k);
-        row.beta[j] = p.ln_beta ? *reinterpret_cast<const floatx4*>(p.ln_beta + k) : floatx4{0.f, 0.f, 0.f, 0.f};
+        if constexpr (EARLY) {
+            row.gamma[j] = *reinterpret_cast<const floatx4*>(p.ln_gamma + k);
+            row.beta[j] = p.ln_beta ? *reinterpret_cast<const floatx4*>(p.ln_beta + k) : floatx4{0.f, 0.f, 0.f, 0.f};
+        }
     }
 }
 
-__device__ __forceinline__ void sk_normalise_row(const SkinnyArgs& p, bf16_t* xs, int m, int lane, RowOperands& row) {
+template <int XV, bool EARLY>
+__device__ __forceinline__ void sk_normalise_row(const SkinnyArgs& p, bf16_t* xs, int m, int lane, RowOperands<XV, EARLY>& row) {
     const int K = p.K[0], ld = K + SK_PAD;
     float s = 0.f;
 #pragma unroll
-    for (int j = 0; j < SK_XV; ++j) {
+    for (int j = 0; j < XV; ++j) {
         if ((j * KA_WAVE + lane) * 4 >= K) row.x[j] = floatx4{0.f, 0.f, 0.f, 0.f};
         s += (row.x[j][0] + row.x[j][1]) + (row.x[j][2] + row.x[j][3]);
     }
     float mean = ka_wave_sum(s) / (float)K;
     float q = 0.f;
 #pragma unroll
-    for (int j = 0; j < SK_XV; ++j) {
+    for (int j = 0; j < XV; ++j) {
         if ((j * KA_WAVE + lane) * 4 < K) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) q += (row.x[j][i] - mean) * (row.x[j][i] - mean);
@@ -190,12 +198,20 @@ __device__ __forceinline__ void sk_normalise_row(const SkinnyArgs& p, bf16_t* xs
     }
     float rstd = 1.0f / sqrtf(ka_wave_sum(q) / (float)K + p.ln_eps);
 #pragma unroll
-    for (int j = 0; j < SK_XV; ++j) {
+    for (int j = 0; j < XV; ++j) {
         const int k = (j * KA_WAVE + lane) * 4;
         if (k < K) {
+            floatx4 gm, bt;
+            if constexpr (EARLY) {
+                gm = row.gamma[j];
+                bt = row.beta[j];
+            } else {
+                gm = *reinterpret_cast<const floatx4*>(p.ln_gamma + k);
+                bt = p.ln_beta ? *reinterpret_cast<const floatx4*>(p.ln_beta + k) : floatx4{0.f, 0.f, 0.f, 0.f};
+            }
             bf16x4 y;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) y[i] = (bf16_t)((row.x[j][i] - mean) * rstd * row.gamma[j][i] + row.beta[j][i]);
+            for (int i = 0; i < 4; ++i) y[i] = (bf16_t)((row.x[j][i] - mean) * rstd * gm[i] + bt[i]);
             *reinterpret_cast<bf16x4*>(xs + m * ld + k) = y;
         }
     }
@@ -263,7 +279,7 @@ skinny_persistent_kernel(SkinnyArgs p, int total_strips) {
     // The first strips' weights are on their way while the activations come in. A wave's loads
     // come back in the order in which it asked, so the row that it is to normalise is asked for
     // before the weights: the LayerNorm would otherwise wait for them.
-    RowOperands row;
+    RowOperands<PER <= 4 ? SK_XV : SK_XV_WIDE, PER <= 4> row;
     if constexpr (LN) {
         if (wave < M) sk_fetch_row(p, wave, lane, row);
         __builtin_amdgcn_sched_barrier(0);
@@ -789,7 +805,7 @@ KA_API void ka_skinny_set_wide(int enabled) { sk_wide_enabled = enabled; }
 template <int PER, int MB, bool HALF, bool LN>
 static int launch_persistent_one(int grid, size_t dyn, int strips, hipStream_t stream, const SkinnyArgs& args) {
     // two strips ahead where one workgroup has a CU (and its registers) to itself
-    constexpr int DEPTH = LN ? 3 : 2;
+    constexpr int DEPTH = LN && PER <= 4 ? 3 : 2;
     if (dyn > 0) {
         static size_t reserved = 0;
         if (dyn > reserved) {
@@ -809,8 +825,7 @@ static int launch_persistent_per(int per, int grid, size_t dyn, int strips, hipS
     if (per <= 1) return launch_persistent_one<1, MB, HALF, LN>(grid, dyn, strips, stream, args);
     if (per <= 2) return launch_persistent_one<2, MB, HALF, LN>(grid, dyn, strips, stream, args);
     if (per <= 4) return launch_persistent_one<4, MB, HALF, LN>(grid, dyn, strips, stream, args);
-    // (the LayerNorm prologue takes rows of at most 2048: four blocks per wave)
-    if constexpr (MB == 1 && !LN) return launch_persistent_one<8, MB, HALF, LN>(grid, dyn, strips, stream, args);
+    if constexpr (MB == 1) return launch_persistent_one<8, MB, HALF, LN>(grid, dyn, strips, stream, args);
     return 1;
 }
 
@@ -892,7 +907,7 @@ KA_API int ka_linear_skinny_fused(const void* A1, long lda1, int K1, const void*
     const bool ln = ln_x != nullptr;
     if (ln) {
         KA_CHECK(M <= SK_LN_ROWS, "%s: the LayerNorm prologue takes at most %d rows", who, SK_LN_ROWS);
-        KA_CHECK(K1 <= SK_XV * KA_WAVE * 4, "%s: the LayerNorm prologue takes rows of at most %d", who, SK_XV * KA_WAVE * 4);
+        KA_CHECK(K1 <= SK_XV_WIDE * KA_WAVE * 4, "%s: the LayerNorm prologue takes rows of at most %d", who, SK_XV_WIDE * KA_WAVE * 4);
         KA_CHECK(ln_gamma && ln_eps >= 0.f && (uintptr_t)ln_x % 16 == 0 && (uintptr_t)ln_gamma % 16 == 0 &&
                      (uintptr_t)ln_beta % 16 == 0, "%s: LayerNorm operands must be 16-byte aligned", who);
         KA_CHECK(A2 == nullptr && !accumulate_a, "%s: no second segment and no accumulation with a LayerNorm prologue", who);

@@ -44,7 +44,7 @@ _SIGNATURES = {
 SKINNY_MAX_ROWS = 64
 # Rows (and their width) up to which the weight-streaming kernel can normalise its input itself.
 SKINNY_LN_MAX_ROWS = 16
-SKINNY_LN_MAX_WIDTH = 2048
+SKINNY_LN_MAX_WIDTH = 4096
 # Whether blocks let the weight-streaming kernel normalise its input itself. Every workgroup of
 # the persistent kernel then repeats the LayerNorm of all rows once; with a few hundred workgroups
 # that is cheaper than a launch of its own (measured on MI355X: 3 % of a decode step at batch 8).
@@ -207,7 +207,7 @@ def linear_two_outputs(a, wa, ba, out_a, act_a, wb, bb, out_b, act_b) -> bool:
 def layernorm_linear(x, gamma, beta, eps, wa, ba, out_a, act_a, wb=None, bb=None, out_b=None, act_b=0) -> bool:
     """``h = LayerNorm(x)``; ``out_a = act_a(h @ wa.T + ba)`` and, if a second target is given,
     ``out_b = act_b(h @ wb.T + bb)`` in one launch: the kernel normalises the fp32 rows itself
-    (at most 16 of them, at most 2048 wide)."""
+    (at most 16 of them, at most 4096 wide, and no more than fit in 96 KB of LDS as bf16)."""
     m, k = x.shape
     if not (0 < m <= SKINNY_LN_MAX_ROWS) or k % 8 or k > SKINNY_LN_MAX_WIDTH or x.dtype != torch.float32 \
             or not x.is_contiguous():

@@ -632,7 +632,8 @@ def test_two_segment_skinny_linear(shape, wide):
 
 
 @pytest.mark.parametrize("shape", [(8, 2048, 6144, 8192), (1, 64, 40, 24), (16, 320, 100, 200), (5, 2048, 48, 8),
-                                   (12, 1000, 24, 20000), (3, 2048, 8192, 16384)])
+                                   (12, 1000, 24, 20000), (3, 2048, 8192, 16384), (8, 2560, 7680, 10240), (16, 2560, 64, 40),
+                                   (1, 4096, 100, 200), (11, 3080, 48, 24), (5, 2056, 8, 16)])
 def test_layernorm_prologue_skinny_linear(shape):
     """LayerNorm, then two linears from the normalised rows, in one launch."""
     from kestrel_amd.ops import fast
