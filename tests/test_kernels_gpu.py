@@ -128,13 +128,11 @@ def test_linear_skinny_bf16(shape, persistent, wide):
     """The weight-streaming MFMA kernels: the persistent one (activations in registers, workgroups
     walk over strips; a form of its own for at most 8 rows), the one with K-splits that takes
     the rest, which is tested on the same shapes with the persistent one switched off, and the
-    wide one for 17 rows and more, which the engine uses with two K-segments only and which
-    mode 2 sends these shapes to."""
+    wide one, which the engine uses where the others do badly and which mode 2 sends all of these
+    shapes to."""
     from kestrel_amd.ops import fast
 
     m, n, k = shape
-    if m <= 16 and wide:
-        pytest.skip("the wide kernel takes 17 rows and more")
     fast.set_skinny_wide(wide)
     bf, f32 = torch.bfloat16, torch.float32
 
@@ -168,7 +166,8 @@ def test_linear_skinny_is_the_same_on_every_run():
 @pytest.mark.parametrize("shape", [(65, 128, 64), (200, 2048, 2048), (129, 100, 200), (300, 333, 520),
                                    (2048, 512, 1024), (128, 6144, 2048), (70, 8, 8)])
 def test_linear_tiled_bf16(shape):
-    """The tiled MFMA kernel with ragged edges in M, N and K."""
+    """More than 64 rows with ragged edges in M, N and K: the tiled MFMA kernel, or, up to 256 rows
+    of few tiles, the weight-streaming kernel in parts."""
     from kestrel_amd.ops import fast
 
     m, n, k = shape
@@ -599,18 +598,18 @@ def test_masks_before_sampling_and_logprobs_after():
     assert torch.allclose(out.cpu().double(), torch.tensor(ref, dtype=torch.float64), atol=2e-5, rtol=1e-5)
 
 
-@pytest.mark.parametrize("wide", [1, 0])
+@pytest.mark.parametrize("wide", [1, 0, 2])
 @pytest.mark.parametrize("shape", [(8, 2048, 2048, 8192), (1, 40, 64, 200), (16, 2048, 2048, 8192), (33, 96, 120, 320),
-                                   (64, 256, 8, 72), (64, 2048, 2048, 8192), (17, 515, 1032, 40), (48, 100, 264, 2056)])
+                                   (64, 256, 8, 72), (64, 2048, 2048, 8192), (17, 515, 1032, 40), (48, 100, 264, 2056),
+                                   (8, 2560, 64, 136), (16, 4104, 72, 40)])
 def test_two_segment_skinny_linear(shape, wide):
-    """out += a1 w1^T + b1 + a2 w2^T + b2 in one launch (17 rows and more: by the kernel that
-    shares the activations through LDS and cuts K into parts, and, with that one switched off,
-    by the one that takes fewer rows too)."""
+    """out += a1 w1^T + b1 + a2 w2^T + b2 in one launch: by the kernel that shares the activations
+    through LDS and cuts K into parts where the engine uses it (1: 17 rows and more, and fewer rows
+    of more strips than CUs), nowhere (0: the kernel that gives a strip to a workgroup) and
+    everywhere (2)."""
     from kestrel_amd.ops import fast
 
     m, n, k1, k2 = shape
-    if m <= 16 and not wide:
-        pytest.skip("the wide kernel takes no part below 17 rows")
     fast.set_skinny_wide(wide)
     torch.manual_seed(20)
     a1, a2 = torch.randn(m, k1).bfloat16().to(DEV), torch.randn(m, k2).bfloat16().to(DEV)
