@@ -12,6 +12,7 @@
 // That kernel takes any K (in steps of 8); where K is a multiple of 64 the large-tile kernel
 // further down, which loads straight into LDS, is used instead.
 #include "ka_common.h"
+#include "ka_partials.h"
 
 #include <stdlib.h>
 
@@ -209,8 +210,18 @@ __global__ void __launch_bounds__(KA_WAVE * GN * GM)
     __attribute__((amdgpu_waves_per_eu(GN * GM / 4, (WN * WM > 8 ? 1 : 2) * (GN * GM / 4))))
 gemm_dma_kernel(const bf16_t* __restrict__ A, long lda, const bf16_t* __restrict__ W, long ldw,
                 const float* __restrict__ bias, void* __restrict__ out, int out_dtype, long ldo, int M,
-                int N, int K, int act, int accumulate, int tiles_n, int tiles_m) {
+                int N, int K, int act, int accumulate, int tiles_n, int tiles_m, int k_per) {
     static_assert(BK == 32 || BK == 64, "K-steps of 32 or 64");
+    // K cut into parts (grid y): part p multiplies the k_per columns from p * k_per on and writes
+    // its sums as fp32 [M, N] of its own (the host passes the partial buffer as `out`, no bias,
+    // no activation; a finishing kernel adds the parts up)
+    if (k_per > 0) {
+        const int part = blockIdx.y;
+        A += (size_t)part * k_per;
+        W += (size_t)part * k_per;
+        K = min(k_per, K - part * k_per);
+        out = reinterpret_cast<float*>(out) + (size_t)part * M * ldo;
+    }
     static_assert(NS >= 2 && NS <= 4, "two to four stages");
     static_assert(GN * GM == 4 || GN * GM == 8, "four or eight waves");
     constexpr int WAVES = GN * GM;
@@ -371,7 +382,8 @@ gemm_dma_kernel(const bf16_t* __restrict__ A, long lda, const bf16_t* __restrict
 
 template <int WN, int WM, int GN, int GM, int BK, int NS>
 static int launch_dma(const bf16_t* A, long lda, const bf16_t* W, long ldw, const float* bias, void* out,
-                      int out_dtype, long ldo, int M, int N, int K, int act, int accumulate, hipStream_t stream) {
+                      int out_dtype, long ldo, int M, int N, int K, int act, int accumulate, hipStream_t stream,
+                      int parts = 1, int k_per = 0) {
     static bool configured = false;
     constexpr int BN = 32 * WN * GN, BM = 32 * WM * GM;
     constexpr int smem = gd_smem(BN, BM, BK, NS);
@@ -386,8 +398,8 @@ static int launch_dma(const bf16_t* A, long lda, const bf16_t* W, long ldw, cons
     long total = (long)tiles_n * tiles_m;
     long launched = ((total + 7) / 8) * 8;
     KA_CHECK(launched < (1L << 31), "ka_linear_tiled_bf16: too many tiles");
-    hipLaunchKernelGGL((gemm_dma_kernel<WN, WM, GN, GM, BK, NS>), dim3((unsigned)launched), dim3(KA_WAVE * GN * GM), smem,
-                       stream, A, lda, W, ldw, bias, out, out_dtype, ldo, M, N, K, act, accumulate, tiles_n, tiles_m);
+    hipLaunchKernelGGL((gemm_dma_kernel<WN, WM, GN, GM, BK, NS>), dim3((unsigned)launched, parts), dim3(KA_WAVE * GN * GM), smem,
+                       stream, A, lda, W, ldw, bias, out, out_dtype, ldo, M, N, K, act, accumulate, tiles_n, tiles_m, k_per);
     return 0;
 }
 
@@ -412,10 +424,13 @@ static int launch_config(const bf16_t* A, long lda, const bf16_t* W, long ldw, c
     return 0;
 }
 
-// `config`: 0 chooses by size; other values force a tile (for measurements and tests).
+// `config`: 0 chooses by size; other values force a tile (for measurements and tests), with
+// 1000000 * parts added to force K to be cut into that many parts as well. `partials`: scratch
+// memory for the sums of such parts (null: K is never cut).
 KA_API int ka_linear_tiled_bf16(const void* A, long lda, const void* W, long ldw, const float* bias,
                                 void* out, int out_dtype, long ldo, int M, int N, int K, int act,
-                                int accumulate, int config, hipStream_t stream) {
+                                int accumulate, int config, float* partials, long partial_floats,
+                                hipStream_t stream) {
     KA_CHECK(M > 0 && N > 0 && K > 0 && K % 8 == 0, "ka_linear_tiled_bf16: M=%d N=%d K=%d (K must be a multiple of 8)", M, N, K);
     KA_CHECK(lda % 8 == 0 && ldw % 8 == 0 && lda >= K && ldw >= K, "ka_linear_tiled_bf16: row strides must be multiples of 8 and >= K");
     KA_CHECK(((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0), "ka_linear_tiled_bf16: operands must be 16-byte aligned");
@@ -424,6 +439,8 @@ KA_API int ka_linear_tiled_bf16(const void* A, long lda, const void* W, long ldw
     KA_CHECK(out_dtype == KA_F32 || out_dtype == KA_BF16, "ka_linear_tiled_bf16: bad output type");
     KA_CHECK(!(accumulate && out_dtype != KA_F32), "ka_linear_tiled_bf16: accumulate needs an fp32 output");
     KA_CHECK((uintptr_t)out % 16 == 0, "ka_linear_tiled_bf16: output must be 16-byte aligned");
+    int parts = config >= 1000000 ? config / 1000000 : 0;      // 0: chosen below
+    config %= 1000000;
     if (config == 0) {
         if (K % 64 == 0) {
             // Tiles of 128 x 128 read 64 flops' worth of operands per byte from L2, which is what
@@ -442,8 +459,16 @@ KA_API int ka_linear_tiled_bf16(const void* A, long lda, const void* W, long ldw
             long rounds192 = (t192 + cus - 1) / cus;
             if (t192 * 10 >= rounds192 * cus * 7 && t192 * rounds * 10 > t256 * rounds192 * 11) config = 22232;
             else if (t256 * 10 >= rounds * cus * 7) config = 22224;
-            else if (t128 <= cus) config = 23212;
-            else config = 12222;
+            else if (t128 <= cus) {
+                config = 23212;
+                // Few tiles (a few hundred rows of a narrow output): K is cut into parts so that
+                // about every CU gets a workgroup; a second kernel adds the parts up.
+                if (parts == 0 && partials && t128 * 2 <= cus && K >= 1024) {
+                    parts = (int)(cus / t128);
+                    if (parts > K / 512) parts = K / 512;
+                    if (parts > 8) parts = 8;
+                }
+            } else config = 12222;
         } else {
             long t22 = (long)ka_cdiv(N, 128) * ka_cdiv(M, 128);
             config = t22 >= 512 ? 221 : 211;
@@ -452,6 +477,20 @@ KA_API int ka_linear_tiled_bf16(const void* A, long lda, const void* W, long ldw
     const bf16_t* a = (const bf16_t*)A;
     const bf16_t* w = (const bf16_t*)W;
     int rc;
+    if (parts >= 2 && config == 23212 && K % 64 == 0) {
+        int k_per = ka_cdiv(ka_cdiv(K, parts), 64) * 64;
+        parts = ka_cdiv(K, k_per);
+        if (parts >= 2 && partials && (long)parts * M * N <= partial_floats) {
+            rc = launch_dma<1, 2, 4, 2, 64, 3>(a, lda, w, ldw, nullptr, partials, KA_F32, N, M, N, K, 0, 0, stream, parts, k_per);
+            if (rc) return rc;
+            KA_LAUNCH_CHECK();
+            const int quads = M * ka_cdiv(N, 4);
+            hipLaunchKernelGGL(ka_partials_finish_kernel, dim3(ka_cdiv(quads, 256)), dim3(256), 0, stream, partials, parts,
+                               bias, (const float*)nullptr, out, out_dtype, ldo, M, N, act, accumulate);
+            KA_LAUNCH_CHECK();
+            return 0;
+        }
+    }
     switch (config) {
         case 221: rc = launch_config<2, 2, 64>(a, lda, w, ldw, bias, out, out_dtype, ldo, M, N, K, act, accumulate, stream); break;
         case 211: rc = launch_config<2, 1, 64>(a, lda, w, ldw, bias, out, out_dtype, ldo, M, N, K, act, accumulate, stream); break;

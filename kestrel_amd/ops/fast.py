@@ -27,7 +27,7 @@ _SIGNATURES = {
         _c_void_p, _c_long, _c_void_p, _c_void_p, _c_int, _c_long, _c_int, _c_int,           # target b
         _c_int, _c_int, _c_void_p, _c_long, _c_void_p],               # M, target_waves, partial sums and how many, stream
     "ka_linear_tiled_bf16": [_c_void_p, _c_long, _c_void_p, _c_long, _c_void_p, _c_void_p, _c_int, _c_long, _c_int,
-                             _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
+                             _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_long, _c_void_p],
     "ka_attention_prefill_bf16": [_c_void_p, _c_long, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p,
                                   _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_long, _c_float,
                                   _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
@@ -42,7 +42,6 @@ _SIGNATURES = {
 
 # Rows up to which the weight-streaming kernel is used instead of the tiled one.
 SKINNY_MAX_ROWS = 64
-FEW_ROWS_MAX = 128                 # rows up to which a block runs on the weight-streaming kernels, 64 at a time (measured at a width of 2048: 17.5k against 14.7k tok/s at 128 rows, 18.3k against 19.7k at 256)
 # Rows (and their width) up to which the weight-streaming kernel can normalise its input itself.
 SKINNY_LN_MAX_ROWS = 16
 SKINNY_LN_MAX_WIDTH = 4096
@@ -157,23 +156,14 @@ def linear_bf16(a, weight, bias, out, act, accumulate) -> bool:
     if accumulate and out.dtype != torch.float32:
         raise KernelError("linear: accumulate needs an fp32 output")
     handle = lib()
-    # up to FEW_ROWS_MAX rows whose tiles of 128 x 128 would leave most CUs idle: the
-    # weight-streaming kernel, SKINNY_MAX_ROWS rows at a time
-    few = m <= SKINNY_MAX_ROWS or (TILED_CONFIG == 0 and m <= FEW_ROWS_MAX and -(-m // 128) * -(-n // 128) < 128)
-    if few:
-        parts = -(-m // SKINNY_MAX_ROWS)
-        size = -(-m // parts)
-        for lo in range(0, m, size):
-            rows = min(size, m - lo)
-            _check(handle.ka_linear_skinny_bf16(a.data_ptr() + lo * a.stride(0) * 2, a.stride(0), weight.data_ptr(),
-                                                weight.stride(0), _ptr(bias),
-                                                out.data_ptr() + lo * out.stride(0) * out.element_size(),
-                                                _OUT_CODE[out.dtype], out.stride(0), rows, n, k, act, int(accumulate),
-                                                SKINNY_TARGET_WAVES, *_wide_args(a.device, rows), stream_ptr()))
+    if m <= SKINNY_MAX_ROWS:
+        _check(handle.ka_linear_skinny_bf16(a.data_ptr(), a.stride(0), weight.data_ptr(), weight.stride(0), _ptr(bias),
+                                            out.data_ptr(), _OUT_CODE[out.dtype], out.stride(0), m, n, k, act,
+                                            int(accumulate), SKINNY_TARGET_WAVES, *_wide_args(a.device, m), stream_ptr()))
     else:
         _check(handle.ka_linear_tiled_bf16(a.data_ptr(), a.stride(0), weight.data_ptr(), weight.stride(0), _ptr(bias),
                                            out.data_ptr(), _OUT_CODE[out.dtype], out.stride(0), m, n, k, act,
-                                           int(accumulate), TILED_CONFIG, stream_ptr()))
+                                           int(accumulate), TILED_CONFIG, *_wide_args(a.device, m), stream_ptr()))
     return True
 
 

@@ -18,7 +18,7 @@ def _parallel_few_rows(block: "Block", x, batch, cache) -> bool:
     from ..ops.linear import linear
 
     n = x.shape[0]
-    if block.dtype != torch.bfloat16 or n > fast.FEW_ROWS_MAX:
+    if block.dtype != torch.bfloat16 or n > fast.SKINNY_MAX_ROWS:
         return False
     m_in, f_in = block.mixer.input_projection(), block.feed_forward.input_projection()
     m_out, f_out = block.mixer.output_projection(), block.feed_forward.output_projection()
@@ -28,30 +28,20 @@ def _parallel_few_rows(block: "Block", x, batch, cache) -> bool:
     projected = ws.get("block.mixer_in", (n, m_in[2]), block.dtype)
     hidden = ws.get("block.ff_hidden", (n, f_in[2]), block.dtype)
     norm = block.norm
-    # More rows than the weight-streaming kernels take at once go through them in equal parts:
-    # a tiled product of so few rows would put a handful of CUs to work (16 tiles of 128 x 128 at
-    # 128 rows and a width of 2048), and the weights of a layer, read once from HBM, come from
-    # the memory-side cache for the parts after the first.
-    parts = -(-n // fast.SKINNY_MAX_ROWS)
-    size = -(-n // parts)
-    spans = [(lo, min(lo + size, n)) for lo in range(0, n, size)]
     fused = False
-    if parts == 1 and fast.FUSE_LAYERNORM_PROLOGUE and getattr(norm.spec, "kind", None) == "layernorm":
+    if fast.FUSE_LAYERNORM_PROLOGUE and getattr(norm.spec, "kind", None) == "layernorm":
         fused = fast.layernorm_linear_pair(x, norm.weight, norm.bias, norm.spec.eps, m_in[0], m_in[1], projected, 0,
                                            f_in[0], f_in[1], hidden, f_in[3])
     if not fused:
         h = ws.get("block.h", tuple(x.shape), block.dtype)
         norm.forward(x, h)
-        for lo, hi in spans:
-            if not fast.linear_two_outputs(h[lo:hi], m_in[0], m_in[1], projected[lo:hi], 0, f_in[0], f_in[1],
-                                           hidden[lo:hi], f_in[3]):
-                linear(h[lo:hi], m_in[0], m_in[1], projected[lo:hi])
-                linear(h[lo:hi], f_in[0], f_in[1], hidden[lo:hi], act=f_in[3])
+        if not fast.linear_two_outputs(h, m_in[0], m_in[1], projected, 0, f_in[0], f_in[1], hidden, f_in[3]):
+            linear(h, m_in[0], m_in[1], projected)
+            linear(h, f_in[0], f_in[1], hidden, act=f_in[3])
     mixed = block.mixer.attend(projected, batch, cache)
-    for lo, hi in spans:
-        if not fast.linear_pair_accumulate(mixed[lo:hi], m_out[0], m_out[1], hidden[lo:hi], f_out[0], f_out[1], x[lo:hi]):
-            linear(mixed[lo:hi], m_out[0], m_out[1], x[lo:hi], accumulate=True)
-            linear(hidden[lo:hi], f_out[0], f_out[1], x[lo:hi], accumulate=True)
+    if not fast.linear_pair_accumulate(mixed, m_out[0], m_out[1], hidden, f_out[0], f_out[1], x):
+        linear(mixed, m_out[0], m_out[1], x, accumulate=True)
+        linear(hidden, f_out[0], f_out[1], x, accumulate=True)
     return True
 
 

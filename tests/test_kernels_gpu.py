@@ -164,10 +164,9 @@ def test_linear_skinny_is_the_same_on_every_run():
 
 
 @pytest.mark.parametrize("shape", [(65, 128, 64), (200, 2048, 2048), (129, 100, 200), (300, 333, 520),
-                                   (2048, 512, 1024), (128, 6144, 2048), (70, 8, 8)])
+                                   (2048, 512, 1024), (128, 6144, 2048), (70, 8, 8), (520, 2048, 8192), (300, 200, 1088)])
 def test_linear_tiled_bf16(shape):
-    """More than 64 rows with ragged edges in M, N and K: the tiled MFMA kernel, or, up to 256 rows
-    of few tiles, the weight-streaming kernel in parts."""
+    """The tiled MFMA kernel with ragged edges in M, N and K (K cut into parts where there are few tiles)."""
     from kestrel_amd.ops import fast
 
     m, n, k = shape
@@ -181,16 +180,16 @@ def test_linear_tiled_bf16(shape):
     _linear_case(fn, m, n, k, bf, bf, bf, 0, False, lda=k + 8)
 
 
-@pytest.mark.parametrize("config", [12222, 23212, 22224, 22232, 13122])
+@pytest.mark.parametrize("config", [12222, 23212, 22224, 22232, 13122, 2023212, 5023212])
 @pytest.mark.parametrize("shape", [(65, 128, 64), (300, 333, 512), (513, 700, 192), (2048, 512, 1024), (100, 2048, 2048), (70, 90, 32)])
 def test_linear_large_tile_bf16(shape, config, monkeypatch):
     """The kernel that loads straight into LDS, at every wave tile, with ragged edges in M and N
-    (K in steps of 64)."""
+    (K in steps of 64); the last two with K cut into two and five parts."""
     from kestrel_amd.ops import fast
 
     m, n, k = shape
     bf, f32 = torch.bfloat16, torch.float32
-    if k % (32 * (config // 100 % 10)):
+    if k % (32 * (config % 1000000 // 100 % 10)):
         pytest.skip("K is no multiple of this tile's K-step")
     monkeypatch.setattr(fast, "TILED_CONFIG", config)
 
