@@ -110,6 +110,33 @@ def test_mixed_batches_with_page_reuse(name, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=DTYPE_IDS)
+@pytest.mark.parametrize("name", ["D", "F"])
+def test_many_requests_decoded_together(name, dtype):
+    """More rows than the weight-streaming kernels take (70 and 130): short prompts fed together in
+    one step, then decoded side by side, one token each a step."""
+    for count in (70, 130):
+        runner = _runner(name, dtype, n_pages=2 * count + 8, max_requests=count)
+        reqs = {f"r{i}": _request(name, f"r{i}", 900 + i, 6 + i % 9) for i in range(count)}
+        steps = [[(tag, 3 + int(tag[1:]) % 4) for tag in reqs]]
+        while True:
+            fed = steps_fed(steps)
+            rest = [(tag, 1) for tag, r in reqs.items() if fed.get(tag, 0) < r.length]
+            if not rest:
+                break
+            steps.append(rest)
+        got = helpers.replay(runner, reqs, steps)
+        _check(name, dtype, reqs, got)
+
+
+def steps_fed(steps):
+    fed = {}
+    for step in steps:
+        for tag, count in step:
+            fed[tag] = fed.get(tag, 0) + count
+    return fed
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=DTYPE_IDS)
 @pytest.mark.parametrize("name", ["B", "C", "D", "E", "F"])
 def test_prefix_embeddings_bidirectional(name, dtype):
     """Given embeddings as one bidirectional block, then text; the block in one portion, the
