@@ -30,6 +30,9 @@ TINY_E = {"text": {"dim": 256, "ff_dim": 264, "n_layers": 2, "vocab_size": 411, 
 TINY_F = {"text": {"dim": 160, "ff_dim": 168, "n_layers": 2, "vocab_size": 333, "max_context": 256, "n_heads": 4,
                    "n_kv_heads": 2, "head_dim": 80, "rotary_dim": 32, "rope_theta": 10000.0, "prefix_attn": 7,
                    "layer_norm_eps": 1e-5}}
+# A long context (rows of more than 4096 keys are cut into parts by the decode attention kernel), one layer.
+TINY_G = {"text": {"dim": 64, "ff_dim": 72, "n_layers": 1, "vocab_size": 211, "max_context": 6144, "n_heads": 2,
+                   "n_kv_heads": 1, "rope_theta": 50000.0, "prefix_attn": 0, "layer_norm_eps": 1e-5}}
 RECIPES = {
     "A": InitRecipe(std=0.02),
     "B": InitRecipe(std=0.03, gain_std=0.02, shift_std=0.02),
@@ -37,9 +40,10 @@ RECIPES = {
     "D": InitRecipe(std=0.04, gain_std=0.05, shift_std=0.05),
     "E": InitRecipe(std=0.03, bias_std=0.05, gain_std=0.05, shift_std=0.02),
     "F": InitRecipe(std=0.04, bias_std=0.03, gain_std=0.05, shift_std=0.03),
+    "G": InitRecipe(std=0.08, bias_std=0.05, gain_std=0.05, shift_std=0.03),
 }
-CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D, "E": TINY_E, "F": TINY_F}
-SEEDS = {"A": 0, "B": 1, "C": 2, "D": 3, "E": 4, "F": 5}
+CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "D": TINY_D, "E": TINY_E, "F": TINY_F, "G": TINY_G}
+SEEDS = {"A": 0, "B": 1, "C": 2, "D": 3, "E": 4, "F": 5, "G": 6}
 
 
 @functools.lru_cache(maxsize=None)

@@ -171,6 +171,19 @@ def test_long_decoding(name, dtype):
     _check(name, dtype, reqs, got)
 
 
+@pytest.mark.parametrize("dtype", DTYPES, ids=DTYPE_IDS)
+def test_a_context_of_thousands(dtype):
+    """4,300 tokens: most in two portions, the rest one by one (the decode attention kernel cuts a
+    row of more than 4096 keys into parts), beside a short request."""
+    name = "G"
+    runner = _runner(name, dtype, n_pages=300, max_requests=2)
+    reqs = {"long": _request(name, "long", 950, 4300), "short": _request(name, "short", 951, 40)}
+    steps = [[("long", 3000)], [("long", 1090), ("short", 30)]] + [[("long", 1), ("short", 1)] for _ in range(10)] \
+        + [[("long", 1)] for _ in range(200)]
+    got = helpers.replay(runner, reqs, steps)
+    _check(name, dtype, reqs, got)
+
+
 @pytest.mark.parametrize("page_size", [1, 4, 64])
 def test_other_page_sizes(page_size):
     runner = _runner("A", torch.float32, n_pages=512 // page_size, page_size=page_size)
