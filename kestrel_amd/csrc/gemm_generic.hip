@@ -61,6 +61,52 @@ gemm_generic_kernel(const TA* __restrict__ A, long lda, const TW* __restrict__ W
     }
 }
 
+// Few rows in fp32 (decoding on the 32-bit path): the tile above would put a sixteenth of its
+// threads to work and read every weight through LDS. Here a wave owns one output column: its
+// lanes walk over K with 16-byte loads of the weight row and of each activation row, every lane
+// adds up its own k in their order, and the lanes' sums meet in a fixed tree. Plain fp32 FMA as
+// above; the order of a sum is another than the tile's, the same for every M and N.
+constexpr int GV_ROWS = 16;      // most rows
+constexpr int GV_WAVES = 4;      // output columns per workgroup
+
+typedef __attribute__((ext_vector_type(4))) float gv_float4;
+
+__global__ void __launch_bounds__(GV_WAVES * KA_WAVE)
+gemv_f32_kernel(const float* __restrict__ A, long lda, const float* __restrict__ W, long ldw,
+                const float* __restrict__ bias, float* __restrict__ out, long ldo, int M, int N, int K, int act,
+                int accumulate) {
+    const int wave = threadIdx.x / KA_WAVE, lane = threadIdx.x % KA_WAVE;
+    const int n = blockIdx.x * GV_WAVES + wave;
+    if (n >= N) return;
+    const float* wrow = W + (size_t)n * ldw;
+    float acc[GV_ROWS];
+#pragma unroll
+    for (int m = 0; m < GV_ROWS; ++m) acc[m] = 0.f;
+    for (int k = lane * 4; k < K; k += KA_WAVE * 4) {
+        const gv_float4 w = *reinterpret_cast<const gv_float4*>(wrow + k);
+#pragma unroll
+        for (int m = 0; m < GV_ROWS; ++m) {
+            if (m < M) {
+                const gv_float4 a = *reinterpret_cast<const gv_float4*>(A + (size_t)m * lda + k);
+                acc[m] = fmaf(a[3], w[3], fmaf(a[2], w[2], fmaf(a[1], w[1], fmaf(a[0], w[0], acc[m]))));
+            }
+        }
+    }
+#pragma unroll
+    for (int m = 0; m < GV_ROWS; ++m) {
+        if (m >= M) break;
+        float v = acc[m];
+#pragma unroll
+        for (int off = KA_WAVE / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, KA_WAVE);
+        if (lane == 0) {
+            v += bias ? bias[n] : 0.f;
+            if (act == 1) v = ka_gelu_tanh(v);
+            const size_t o = (size_t)m * ldo + n;
+            out[o] = accumulate ? out[o] + v : v;
+        }
+    }
+}
+
 template <typename TA, typename TW, typename TOut>
 static void launch(const void* A, long lda, const void* W, long ldw, const float* bias, void* out,
                    long ldo, int M, int N, int K, int act, int accumulate, hipStream_t stream) {
@@ -82,6 +128,13 @@ KA_API int ka_linear_generic(const void* A, int a_dtype, long lda, const void* W
     KA_CHECK(ka_cdiv(M, GT) <= 65535, "ka_linear_generic: M=%d too large for one launch", M);
     if (M == 0) return 0;
     int key = a_dtype * 4 + w_dtype * 2 + out_dtype;
+    if (key == 0 && M <= GV_ROWS && K % 4 == 0 && lda % 4 == 0 && ldw % 4 == 0 && (uintptr_t)A % 16 == 0 &&
+        (uintptr_t)W % 16 == 0) {
+        hipLaunchKernelGGL(gemv_f32_kernel, dim3(ka_cdiv(N, GV_WAVES)), dim3(GV_WAVES * KA_WAVE), 0, stream,
+                           (const float*)A, lda, (const float*)W, ldw, bias, (float*)out, ldo, M, N, K, act, accumulate);
+        KA_LAUNCH_CHECK();
+        return 0;
+    }
 #define KA_CASE(k, TA, TW, TO) \
     case k: launch<TA, TW, TO>(A, lda, W, ldw, bias, out, ldo, M, N, K, act, accumulate, stream); break;
     switch (key) {

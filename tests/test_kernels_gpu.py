@@ -106,7 +106,8 @@ def _linear_case(fn, m, n, k, a_dtype, w_dtype, out_dtype, act, accumulate, seed
     _close(out, ref, worst, scale=2)
 
 
-@pytest.mark.parametrize("shape", [(1, 37, 19), (65, 130, 200), (7, 64, 96), (130, 77, 333)])
+@pytest.mark.parametrize("shape", [(1, 37, 19), (65, 130, 200), (7, 64, 96), (130, 77, 333), (16, 51, 2048), (3, 1000, 260),
+                                   (17, 40, 64)])
 def test_linear_generic(shape):
     from kestrel_amd.ops import core
 
