@@ -61,6 +61,77 @@ gemm_generic_kernel(const TA* __restrict__ A, long lda, const TW* __restrict__ W
     }
 }
 
+// Many rows in fp32 (prompts on the 32-bit path): the same sums, k in ascending order for every
+// output, from a tile of 128 x 128 x 8 with 8 x 8 outputs a thread, 16-byte loads (rows and K
+// must allow them: the host sends everything else to the kernel above) and two LDS stages.
+constexpr int GF = 128;   // tile edge in M and N
+constexpr int GFK = 8;    // tile depth
+
+__global__ void __launch_bounds__(256)
+gemm_f32_kernel(const float* __restrict__ A, long lda, const float* __restrict__ W, long ldw,
+                const float* __restrict__ bias, float* __restrict__ out, long ldo, int M, int N, int K, int act,
+                int accumulate) {
+    typedef __attribute__((ext_vector_type(4))) float f4;
+    __shared__ __attribute__((aligned(16))) float As[2][GFK][GF + 4];
+    __shared__ __attribute__((aligned(16))) float Ws[2][GFK][GF + 4];
+    const int tx = threadIdx.x % 16, ty = threadIdx.x / 16;
+    const int m0 = blockIdx.y * GF, n0 = blockIdx.x * GF;
+    // each thread brings four consecutive k of one row of each operand tile (rows past the end
+    // are the last row again: their outputs are never stored)
+    const int lr = threadIdx.x / 2, lk = (threadIdx.x % 2) * 4;
+    const float* arow = A + (size_t)min(m0 + lr, M - 1) * lda + lk;
+    const float* wrow = W + (size_t)min(n0 + lr, N - 1) * ldw + lk;
+    const f4 zero = {0.f, 0.f, 0.f, 0.f};
+    auto fetch = [&](int k0, f4& ra, f4& rw) {
+        const bool ok = k0 + lk < K;             // K is a multiple of 4
+        ra = ok ? *reinterpret_cast<const f4*>(arow + k0) : zero;
+        rw = ok ? *reinterpret_cast<const f4*>(wrow + k0) : zero;
+    };
+    auto stash = [&](int buf, const f4& ra, const f4& rw) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            As[buf][lk + j][lr] = ra[j];
+            Ws[buf][lk + j][lr] = rw[j];
+        }
+    };
+    float acc[8][8] = {};
+    f4 ra, rw;
+    fetch(0, ra, rw);
+    stash(0, ra, rw);
+    __syncthreads();
+    const int steps = (K + GFK - 1) / GFK;
+    for (int s = 0; s < steps; ++s) {
+        const int buf = s & 1;
+        if (s + 1 < steps) fetch((s + 1) * GFK, ra, rw);
+#pragma unroll
+        for (int k = 0; k < GFK; ++k) {
+            const f4 a0 = *reinterpret_cast<const f4*>(&As[buf][k][ty * 8]), a1 = *reinterpret_cast<const f4*>(&As[buf][k][ty * 8 + 4]);
+            const f4 w0 = *reinterpret_cast<const f4*>(&Ws[buf][k][tx * 8]), w1 = *reinterpret_cast<const f4*>(&Ws[buf][k][tx * 8 + 4]);
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+#pragma unroll
+                for (int j = 0; j < 8; ++j)
+                    acc[i][j] = fmaf(i < 4 ? a0[i] : a1[i - 4], j < 4 ? w0[j] : w1[j - 4], acc[i][j]);
+        }
+        if (s + 1 < steps) stash(buf ^ 1, ra, rw);
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const int m = m0 + ty * 8 + i;
+        if (m >= M) continue;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int n = n0 + tx * 8 + j;
+            if (n >= N) continue;
+            float v = acc[i][j] + (bias ? bias[n] : 0.f);
+            if (act == 1) v = ka_gelu_tanh(v);
+            const size_t o = (size_t)m * ldo + n;
+            out[o] = accumulate ? out[o] + v : v;
+        }
+    }
+}
+
 // Few rows in fp32 (decoding on the 32-bit path): the tile above would put a sixteenth of its
 // threads to work and read every weight through LDS. Here a wave owns one output column: its
 // lanes walk over K with 16-byte loads of the weight row and of each activation row, every lane
@@ -128,8 +199,15 @@ KA_API int ka_linear_generic(const void* A, int a_dtype, long lda, const void* W
     KA_CHECK(ka_cdiv(M, GT) <= 65535, "ka_linear_generic: M=%d too large for one launch", M);
     if (M == 0) return 0;
     int key = a_dtype * 4 + w_dtype * 2 + out_dtype;
-    if (key == 0 && M <= GV_ROWS && K % 4 == 0 && lda % 4 == 0 && ldw % 4 == 0 && (uintptr_t)A % 16 == 0 &&
-        (uintptr_t)W % 16 == 0) {
+    const bool vectors = key == 0 && K % 4 == 0 && lda % 4 == 0 && ldw % 4 == 0 && (uintptr_t)A % 16 == 0 &&
+                         (uintptr_t)W % 16 == 0;
+    if (vectors && M > GV_ROWS && ka_cdiv(M, GF) <= 65535) {
+        hipLaunchKernelGGL(gemm_f32_kernel, dim3(ka_cdiv(N, GF), ka_cdiv(M, GF)), dim3(256), 0, stream, (const float*)A, lda,
+                           (const float*)W, ldw, bias, (float*)out, ldo, M, N, K, act, accumulate);
+        KA_LAUNCH_CHECK();
+        return 0;
+    }
+    if (vectors && M <= GV_ROWS) {
         hipLaunchKernelGGL(gemv_f32_kernel, dim3(ka_cdiv(N, GV_WAVES)), dim3(GV_WAVES * KA_WAVE), 0, stream,
                            (const float*)A, lda, (const float*)W, ldw, bias, (float*)out, ldo, M, N, K, act, accumulate);
         KA_LAUNCH_CHECK();
