@@ -181,8 +181,12 @@ def test_linear_tiled_bf16(shape):
     _linear_case(fn, m, n, k, bf, bf, bf, 0, False, lda=k + 8)
 
 
-@pytest.mark.parametrize("config", [12222, 23212, 22224, 22232, 13122, 2023212, 5023212])
-@pytest.mark.parametrize("shape", [(65, 128, 64), (300, 333, 512), (513, 700, 192), (2048, 512, 1024), (100, 2048, 2048), (70, 90, 32)])
+_LARGE_TILE_SHAPES = [(65, 128, 64), (300, 333, 512), (513, 700, 192), (2048, 512, 1024), (100, 2048, 2048), (70, 90, 32)]
+_LARGE_TILE_CONFIGS = [12222, 23212, 22224, 22232, 13122, 2023212, 5023212]
+
+
+@pytest.mark.parametrize("shape,config", [(sh, c) for sh in _LARGE_TILE_SHAPES for c in _LARGE_TILE_CONFIGS
+                                          if sh[2] % (32 * (c % 1000000 // 100 % 10)) == 0])   # K in the tile's K-steps
 def test_linear_large_tile_bf16(shape, config, monkeypatch):
     """The kernel that loads straight into LDS, at every wave tile, with ragged edges in M and N
     (K in steps of 64); the last two with K cut into two and five parts."""
@@ -190,8 +194,6 @@ def test_linear_large_tile_bf16(shape, config, monkeypatch):
 
     m, n, k = shape
     bf, f32 = torch.bfloat16, torch.float32
-    if k % (32 * (config % 1000000 // 100 % 10)):
-        pytest.skip("K is no multiple of this tile's K-step")
     monkeypatch.setattr(fast, "TILED_CONFIG", config)
 
     def fn(a, w, bias, out, act, accumulate):
