@@ -97,7 +97,7 @@ class DecodeBench:
         self.torch, self.StepEntry, self.PENDING = torch, StepEntry, PENDING_TOKEN
         self.net, self.typed, self.batch, self.context = net, typed, batch, context
         pages_per_request = -(-(context + steps_total + 1) // PAGE_SIZE)
-        self.runner = make_runner(net, PAGE_SIZE, batch * pages_per_request, batch, max_tokens_per_step=4096,
+        self.runner = make_runner(net, PAGE_SIZE, batch * pages_per_request, batch, max_tokens_per_step=max(4096, context),
                                   enable_graphs=True)
         self.sampler = Sampler(net.device, pending=self.runner.pending)
         self.host = [torch.empty(batch, dtype=torch.int32, pin_memory=True) for _ in range(2)]
@@ -202,6 +202,8 @@ def main() -> int:
     parser.add_argument("--sizes", default="moondream2", choices=sorted(SIZES), help="layer sizes (the default is the benchmark's)")
     parser.add_argument("--layers", type=int, default=None, help="fewer layers than the model has (named in config)")
     parser.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
+    parser.add_argument("--context", type=int, default=CONTEXT, help="tokens each request holds when decoding starts")
+    parser.add_argument("--prefill-tokens", type=int, default=PREFILL_TOKENS, help="length of the timed prompt")
     parser.add_argument("--skip-points", action="store_true", help="only the default batch (no batch 1 / 64, no prefill)")
     parser.add_argument("--only-prefill", action="store_true", help="only the 2,048-token prefill (for profiling)")
     args = parser.parse_args()
@@ -217,23 +219,25 @@ def main() -> int:
     torch.cuda.set_device(device)
     dtype = torch.bfloat16 if args.dtype == "bf16" else torch.float32
     size = 2 if dtype == torch.bfloat16 else 4
-    sizes = SIZES[args.sizes]
+    sizes = dict(SIZES[args.sizes])
+    # a longer context than the model's own is measured with its position table made longer
+    sizes["max_context"] = max(sizes["max_context"], args.context + max(args.steps, 16) + args.warmup + 8, args.prefill_tokens)
     if args.layers is None:
         args.layers = sizes["n_layers"]
     net, typed = build_model(args.layers, dtype, device, sizes)
     weights = model_bytes(net, size)
 
     if args.only_prefill:
-        seconds = time_prefill(net, typed, PREFILL_TOKENS)
-        print(json.dumps({"prefill_ms": round(seconds * 1e3, 3), "tokens": PREFILL_TOKENS, "dtype": args.dtype}))
+        seconds = time_prefill(net, typed, args.prefill_tokens)
+        print(json.dumps({"prefill_ms": round(seconds * 1e3, 3), "tokens": args.prefill_tokens, "dtype": args.dtype}))
         return 0
-    elapsed, kv_bytes = time_decode(net, typed, args.batch, CONTEXT, args.steps, args.warmup)
+    elapsed, kv_bytes = time_decode(net, typed, args.batch, args.context, args.steps, args.warmup)
     ms_per_step = elapsed / args.steps * 1e3
     value = args.batch * args.steps / elapsed
     step_bytes = weights + kv_bytes * (size / 2) + args.batch * typed.dim * size
     achieved = step_bytes / (elapsed / args.steps)
     record = {
-        "metric": f"decode tok/s ({LABELS[args.sizes][0]}, batch {args.batch}, context {CONTEXT})",
+        "metric": f"decode tok/s ({LABELS[args.sizes][0]}, batch {args.batch}, context {args.context})",
         "value": round(value, 1),
         "unit": "tok/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
@@ -241,19 +245,19 @@ def main() -> int:
         "config": {"model": LABELS[args.sizes][1], "n_layers": args.layers, "n_layers_full": sizes["n_layers"],
                    "dim": typed.dim, "ff_dim": typed.ff_dim, "n_heads": typed.n_heads, "n_kv_heads": typed.n_kv_heads,
                    "head_dim": typed.head_dim, "rotary_dim": typed.rotary_dim, "vocab_size": typed.vocab_size,
-                   "global_batch": args.batch, "seq_len": CONTEXT, "prefix_attn": typed.prefix_attn,
+                   "global_batch": args.batch, "seq_len": args.context, "prefix_attn": typed.prefix_attn,
                    "page_size": PAGE_SIZE, "parallelism": "single-gpu"},
         "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": PEAK_HBM / 1e9, "unit": "GB/s",
                      "frac": round(achieved / PEAK_HBM, 4)},
     }
     if not args.skip_points:
-        seconds = time_prefill(net, typed, PREFILL_TOKENS)
-        flops = prefill_flops(typed, PREFILL_TOKENS, min(typed.prefix_attn, PREFILL_TOKENS - 1))
-        record["prefill"] = {"value": round(PREFILL_TOKENS / seconds, 1), "tokens": PREFILL_TOKENS,
+        seconds = time_prefill(net, typed, args.prefill_tokens)
+        flops = prefill_flops(typed, args.prefill_tokens, min(typed.prefix_attn, args.prefill_tokens - 1))
+        record["prefill"] = {"value": round(args.prefill_tokens / seconds, 1), "tokens": args.prefill_tokens,
                              "ms": round(seconds * 1e3, 3), "frac": round(flops / seconds / PEAK_FLOPS[args.dtype], 4)}
         points = {}
         for batch, steps in ((1, args.steps), (64, max(16, args.steps // 4))):
-            e, _ = time_decode(net, typed, batch, CONTEXT, steps, min(args.warmup, 4))
+            e, _ = time_decode(net, typed, batch, args.context, steps, min(args.warmup, 4))
             points[f"decode_b{batch}"] = round(batch * steps / e, 1)
         record["points"] = points
     print(json.dumps(record))
