@@ -230,3 +230,75 @@ def test_trace_run_program(tmp_path, dtype):
     helpers.assert_close(load(2, 1), exp_b[[36]], tdtype, "step 2")
     helpers.assert_close(load(3, 1), exp_a[[48]], tdtype, "step 3")
     helpers.assert_close(load(4, 1), exp_a[[49]], tdtype, "step 4")
+
+
+def _random_configuration(rng):
+    """A small configuration drawn at random: head sizes in steps of 16 (in steps of 32 above 128),
+    grouped heads, widths and vocabularies that are no power of two, every rotary width."""
+    while True:
+        hd = rng.choice([16, 32, 48, 64, 80, 96, 112, 128, 160, 192, 256])
+        hkv = rng.choice([1, 2, 3])
+        heads = hkv * rng.choice([1, 2, 3])
+        if heads * hd <= 640:
+            break
+    explicit = rng.random() < 0.5
+    cfg = {"dim": rng.choice([40, 72, 100, 136, 200, 264]) if explicit else heads * hd,
+           "ff_dim": rng.choice([24, 56, 136, 200, 320]), "n_layers": rng.choice([1, 2, 3]),
+           "vocab_size": rng.choice([97, 300, 777, 1000]), "max_context": 512, "n_heads": heads, "n_kv_heads": hkv,
+           "rope_theta": rng.choice([100.0, 5000.0, 10000.0, 1.5e6]), "prefix_attn": 0,
+           "layer_norm_eps": rng.choice([1e-5, 1e-6, 3e-4])}
+    if explicit:
+        cfg["head_dim"] = hd
+    rotary = rng.choice([None, None, hd, 2, max(hd // 2 - 2, 2), 0])
+    if rotary is not None:
+        cfg["rotary_dim"] = rotary - rotary % 2
+    return cfg
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=DTYPE_IDS)
+@pytest.mark.parametrize("seed", range(8))
+def test_configurations_drawn_at_random(seed, dtype, tmp_path):
+    """Six requests of a random configuration, up to four live, cut at random into portions and
+    single tokens, some with a block of given embeddings, in a pool that makes pages come back."""
+    import random
+
+    from kestrel_amd.engine.loading import load_model, make_runner
+    from kestrel_amd.weights import InitRecipe, write_random_model
+
+    rng = random.Random(1000 + seed)
+    cfg = _random_configuration(rng)
+    folder = str(tmp_path / "model")
+    write_random_model(folder, {"text": cfg}, seed, InitRecipe(std=0.04, bias_std=0.04, gain_std=0.1, shift_std=0.05))
+    weights = helpers.stored_weights(folder)
+    net = load_model(folder, dtype, torch.device("cuda:0"))
+    lengths = [rng.choice([3, 17, 33, 64, 65, 130, 257]) for _ in range(6)]
+    pages = sum(sorted(-(-n // 16) for n in lengths)[-4:]) + 2
+    runner = make_runner(net, 16, pages, 4)
+    helpers.poison_cache(runner)
+    reqs = {}
+    for i, n in enumerate(lengths):
+        n_prefix = rng.choice([0, 0, 5, 17]) if n > 20 else 0
+        prefix = torch.randn(n_prefix, cfg["dim"], generator=torch.Generator().manual_seed(seed * 100 + i)) if n_prefix else None
+        reqs[f"r{i}"] = Request(f"r{i}", helpers.random_ids(seed * 10 + i, n - n_prefix, cfg["vocab_size"]), prefix)
+    waiting, live, steps, fed = list(reqs), [], [], {tag: 0 for tag in reqs}
+    while waiting or live:
+        while waiting and len(live) < 4 and (not live or rng.random() < 0.7):
+            live.append(waiting.pop(0))
+        step = []
+        for tag in list(live):
+            if rng.random() < 0.2 and len(live) > 1:
+                continue                                   # left out of this step
+            req = reqs[tag]
+            count = rng.choice([1, 1, 2, 3, 7, 16, 31, 64, 100, 1000])
+            if fed[tag] == 0 and req.n_prefix:
+                count = max(count, req.n_prefix)
+            count = min(count, req.length - fed[tag])
+            fed[tag] += count
+            step.append((tag, count))
+            if fed[tag] == req.length:
+                live.remove(tag)
+        if step:
+            steps.append(step)
+    got = helpers.replay(runner, reqs, steps, poison=True)
+    for tag, req in reqs.items():
+        helpers.assert_close(got[tag], plain.forward(cfg, weights, req.ids, req.prefix), dtype, f"{cfg} request {tag}")
