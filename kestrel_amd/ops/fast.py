@@ -50,7 +50,8 @@ SKINNY_LN_MAX_WIDTH = 4096
 # that is cheaper than a launch of its own (measured on MI355X: 3 % of a decode step at batch 8).
 FUSE_LAYERNORM_PROLOGUE = True
 # Tile of the tiled kernels: 0 lets them choose by size; 221, 211 (any K), 12222, 23212, 22224, 22232, 13122
-# (K in steps of 64 or 32, loads straight into LDS) force one (for measurements and tests).
+# (K in steps of 64 or 32, loads straight into LDS) force one, and 1000000 * parts + 23212 forces K to be cut into
+# that many parts as well (for measurements and tests).
 TILED_CONFIG = 0
 # Waves the split weight-streaming kernel aims to have on the chip: 8 per workgroup at 256 strips
 # (measured best for the output projection + second feed-forward linear of Moondream 2).
@@ -97,9 +98,10 @@ def set_skinny_persistent(enabled: int) -> None:
 
 
 def set_skinny_wide(enabled: int) -> None:
-    """Where skinny linears of 17 to 64 rows use the kernel that shares the activations through
-    LDS: 1 (the default) with two K-segments, where it was measured faster, 2 wherever it can run
-    (for tests), 0 nowhere."""
+    """Where skinny linears use the kernel that shares the activations through LDS and cuts K
+    into parts: 1 (the default) where it was measured faster (two K-segments at 17 to 64 rows or
+    with more strips than CUs at 5 to 16 rows; one segment too long for the persistent kernel's
+    registers at 17 to 64 rows), 2 wherever it can run (for tests), 0 nowhere."""
     lib().ka_skinny_set_wide(int(enabled))
 
 
