@@ -267,13 +267,13 @@ def decode_shape(max_kv: int, workgroups: int = 1):
     64-key tile per wave and round; rows longer than 4096 keys are cut into parts whose sums
     a second kernel merges (cutting the keys of a few short rows further, to put more CUs to
     work, was measured and changes nothing: 0.887 ms a step at batch 1 either way). With many workgroups (rows x heads) each gets fewer waves, so that
-    they all fit on the chip at once (measured at 1024 keys: 16 waves up to 256 workgroups, 8 at
-    512 and 1024, 4 from 2048 on)."""
+    they all fit on the chip at once (measured at 1024 keys: 16 waves up to 256 workgroups, 8 up to
+    512, 4 beyond: workgroups of four waves fit five to a CU)."""
     splits = max(1, -(-max_kv // DECODE_KEYS_PER_WORKGROUP))
     tiles = -(-max_kv // (64 * splits))
     waves = 4 if tiles <= 4 else 8 if tiles <= 8 else 16
     groups = workgroups * splits
-    fit = 16 if groups <= DECODE_WAVE_SLOTS // 16 else 8 if groups <= DECODE_WAVE_SLOTS // 4 else 4
+    fit = 16 if groups <= DECODE_WAVE_SLOTS // 16 else 8 if groups <= DECODE_WAVE_SLOTS // 8 else 4
     return splits, min(waves, fit)
 
 
