@@ -1,9 +1,10 @@
-"""Command line: ``python -m kestrel_amd <generate | random-weights | replay>``.
+"""Command line: ``python -m kestrel_amd <generate | random-weights | replay | profile-decode>``.
 
 Option names follow the reference's ``RuntimeConfig`` fields (``kestrel/config.py:155-179``:
 ``--model-path --dtype --max-batch-size --page-size --kv-cache-pages``) and its request
 settings (``temperature``, ``top_p``, ``max_tokens``; ``kestrel/engine/core.py:1161-1174``).
-Prompts are token ids: the tokenizer is outside this engine.
+Prompts are token ids: the tokenizer is outside this engine. ``profile-decode`` takes the options
+of the reference's decode profiling script (``scripts/profile_decode.py:243-256``).
 """
 
 from __future__ import annotations
@@ -101,6 +102,74 @@ def _random_weights(args) -> int:
     return 0
 
 
+def _profile_decode(args) -> int:
+    """Steady-state decode steps of one batch, timed one by one: what the reference's
+    ``scripts/profile_decode.py`` measures (``:309-470``: a batch of equal prompts is fed, the
+    decode step is warmed up, the last ``--profile-iters`` of ``--decode-iters`` steps are timed
+    with events and summarised in one ``PROFILE:`` line)."""
+    import torch
+
+    from .config.runtime import parse_dtype
+    from .engine.loading import load_model, make_runner
+    from .engine.step import PENDING_TOKEN, StepEntry
+    from .sampling import Sampler
+
+    device = torch.device(args.device)
+    if device.index is None:
+        device = torch.device("cuda", torch.cuda.current_device())
+    print(f"Loading model from {args.weights}...")
+    net = load_model(args.weights, parse_dtype(args.dtype), device)
+    plan = net.plan
+    print(f"Model loaded. Config: {len(plan.layers)} layers, hidden={plan.dim}")
+    total = max(1, args.decode_iters)
+    profiled = max(1, min(args.profile_iters, total))
+    batch, prompt_len = args.batch_size, max(1, args.prompt_len)
+    if prompt_len + args.warmup + total + 1 > plan.max_positions:
+        print(f"profile-decode: {prompt_len} + {args.warmup + total} tokens exceed the model's context of "
+              f"{plan.max_positions}", file=sys.stderr)
+        return 2
+    pages = -(-(prompt_len + args.warmup + total + 1) // args.page_size)
+    runner = make_runner(net, args.page_size, batch * pages, batch, max_tokens_per_step=max(4096, prompt_len),
+                         enable_graphs=True)
+    sampler = Sampler(device, pending=runner.pending)
+    # the prompt: the first token id of the model, then ids counting up (taken into the vocabulary)
+    prompt = [plan.bos_token_id] + [(100 + i) % plan.vocab_size for i in range(prompt_len - 1)]
+    slots = []
+    for _ in range(batch):
+        slot = runner.admit()
+        logits = runner.step([StepEntry(slot, prompt, want=[prompt_len - 1])])
+        sampler.greedy(logits, slots=[slot])
+        slots.append(slot)
+
+    def run_decode():
+        logits = runner.step([StepEntry(slot, [PENDING_TOKEN], want=[0]) for slot in slots])
+        sampler.greedy(logits, slots=slots)
+
+    print(f"Running {args.warmup} warmup decode iterations...")
+    for _ in range(args.warmup):
+        run_decode()
+    torch.cuda.synchronize(device)
+    print(f"Running profiled decode iterations (HIP graph replay)... total={total}, profiled={profiled}")
+    starts = [torch.cuda.Event(enable_timing=True) for _ in range(profiled)]
+    ends = [torch.cuda.Event(enable_timing=True) for _ in range(profiled)]
+    at = 0
+    for i in range(total):
+        timed = i >= total - profiled
+        if timed:
+            starts[at].record()
+        run_decode()
+        if timed:
+            ends[at].record()
+            at += 1
+    torch.cuda.synchronize(device)
+    times = sorted(a.elapsed_time(b) for a, b in zip(starts, ends))
+    avg = sum(times) / len(times)
+    p50, p90 = times[len(times) // 2], times[max(0, int(0.9 * (len(times) - 1)))]
+    print(f"PROFILE: batch={batch}, prompt_len={prompt_len}, profile_iters={profiled}, avg_ms={avg:.3f}, "
+          f"p50_ms={p50:.3f}, p90_ms={p90:.3f}, min_ms={times[0]:.3f}, max_ms={times[-1]:.3f}")
+    return 0
+
+
 def main(argv=None) -> int:
     parser = argparse.ArgumentParser(prog="kestrel_amd", description="MI355X inference engine")
     sub = parser.add_subparsers(dest="command", required=True)
@@ -130,6 +199,18 @@ def main(argv=None) -> int:
     rw.add_argument("--shift-std", type=float, default=0.0)
     rw.add_argument("--store-dtype", default="bfloat16", choices=["bfloat16", "float32"])
     rw.set_defaults(run=_random_weights)
+
+    pd = sub.add_parser("profile-decode", help="time steady-state decode steps of one batch")
+    pd.add_argument("--weights", required=True, help="folder with config.json and model.safetensors")
+    pd.add_argument("--batch-size", type=int, default=33, help="decode batch size")
+    pd.add_argument("--prompt-len", type=int, default=740, help="prompt length (prefill tokens)")
+    pd.add_argument("--warmup", type=int, default=5, help="warmup decode iterations")
+    pd.add_argument("--decode-iters", type=int, default=50, help="total decode iterations")
+    pd.add_argument("--profile-iters", type=int, default=20, help="steady-state decode iterations that are timed (the last N)")
+    pd.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    pd.add_argument("--page-size", type=int, default=16)
+    pd.add_argument("--device", default="cuda")
+    pd.set_defaults(run=_profile_decode)
 
     rp = sub.add_parser("replay", help="trace replay (the same program as bin/trace_run)", add_help=False)
     rp.set_defaults(run=None)

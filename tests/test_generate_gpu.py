@@ -208,3 +208,18 @@ def test_command_line(tmp_path):
     stop = cfg.get("eos_id", 0)
     expected = tokens[:tokens.index(stop) + 1] if stop in tokens else tokens
     _assert_greedy(record["tokens"], expected, margins, 1e-4, "command line")
+
+
+def test_profile_decode_command(tmp_path):
+    """The decode timing command with the reference script's options: one PROFILE line."""
+    env = dict(os.environ, PYTHONPATH=ROOT)
+    done = subprocess.run([sys.executable, "-m", "kestrel_amd", "profile-decode", "--weights", helpers.model_dir("D"),
+                           "--batch-size", "3", "--prompt-len", "20", "--warmup", "2", "--decode-iters", "6",
+                           "--profile-iters", "4"], capture_output=True, text=True, env=env, cwd=ROOT, timeout=300)
+    assert done.returncode == 0, done.stderr
+    line = [l for l in done.stdout.splitlines() if l.startswith("PROFILE:")]
+    assert len(line) == 1 and "batch=3, prompt_len=20, profile_iters=4, avg_ms=" in line[0]
+    too_long = subprocess.run([sys.executable, "-m", "kestrel_amd", "profile-decode", "--weights", helpers.model_dir("D"),
+                               "--prompt-len", "250", "--decode-iters", "50"], capture_output=True, text=True, env=env,
+                              cwd=ROOT, timeout=300)
+    assert too_long.returncode == 2 and "exceed the model's context" in too_long.stderr
