@@ -314,3 +314,58 @@ def test_a_layer_may_read_another_layers_cache():
         o = plain.attention_core(q, kv0[0], kv0[1], allowed, hd ** -0.5).reshape(20, nh * hd)
         x = x + plain.linear(o, w[p + "attn.proj.weight"], w[p + "attn.proj.bias"]) + plain.mlp(xn, w, p)
     helpers.assert_close(whole, plain.head(x, w, cfg), torch.float32, "shared cache against plain")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+def test_a_windowed_layer_beside_a_full_one(dtype):
+    """The second layer of a tiny Moondream plan is given a window of 24 keys: its keys and values
+    live in a group with a pool of its own, which gives pages back as the window passes them, while
+    the first layer keeps all keys. Two requests in portions and single tokens, against the plain
+    model with the window in the second layer's mask."""
+    from dataclasses import replace
+
+    from kestrel_amd.config import get_spec
+    from kestrel_amd.engine.loading import make_runner
+    from kestrel_amd.models import DecoderModel
+    from tests.helpers import Request
+
+    name, window = "D", 24
+    spec = get_spec("moondream2")
+    plan = spec.build_plan(spec.read_config(helpers.CONFIGS[name]))
+    layers = list(plan.layers)
+    layers[1] = replace(layers[1], mixer=replace(layers[1].mixer, window=window))
+    model = DecoderModel(replace(plan, layers=tuple(layers)))
+    stored = helpers.stored_weights(helpers.model_dir(name))
+    model.bind(dict(stored), dtype, DEV)
+    runner = make_runner(model, 16, 12, 2)
+    assert len(runner.cache.groups) == 2 and [g.spec.window for g in runner.cache.groups] == [None, window]
+    helpers.poison_cache(runner)
+    cfg = helpers.flat_config(name)
+    reqs = {"a": Request("a", helpers.random_ids(60, 100, cfg["vocab_size"])),
+            "b": Request("b", helpers.random_ids(61, 58, cfg["vocab_size"]))}
+    steps = [[("a", 37)], [("a", 30), ("b", 20)], [("a", 1), ("b", 33)]] + [[("a", 1), ("b", 1)] for _ in range(5)] \
+        + [[("a", 1)] for _ in range(27)]
+    held = []
+    original = runner.step
+
+    def step_and_count(entries):
+        out = original(entries)
+        held.append(runner.cache.n_pages - runner.cache.groups[1].pool.free_count)
+        return out
+
+    runner.step = step_and_count
+    got = helpers.replay(runner, reqs, steps, poison=True)
+    # the windowed group never holds more than the window and a portion's worth of pages per request
+    assert max(held) <= 2 * (-(-(window + 37) // 16) + 1) and held[-1] <= -(-window // 16) + 1
+    assert all(g.pool.free_count == runner.cache.n_pages for g in runner.cache.groups)
+    for tag, req in reqs.items():
+        n = req.length
+        w = {k: v.double() for k, v in stored.items()}
+        x = w["text.wte"][torch.tensor(req.ids)]
+        positions = torch.arange(n)
+        causal = plain.visibility(positions, None)
+        near = causal & (positions.unsqueeze(1) - positions.unsqueeze(0) < window)
+        table = plain.rotary_table(plain.rotary_dim_of(cfg), n, cfg["rope_theta"])
+        x = plain.block(x, w, 0, cfg, positions, causal, table)
+        x = plain.block(x, w, 1, cfg, positions, near, table)
+        helpers.assert_close(got[tag], plain.head(x, w, cfg), dtype, f"windowed layer, request {tag}")
