@@ -12,6 +12,15 @@
 
 constexpr int ATT_MAX_HD = 512;
 
+// Four neighbouring elements with one load (the address must be a multiple of 4 elements).
+template <typename T>
+__device__ __forceinline__ void att_load4(const T* p, float v[4]) {
+    typedef __attribute__((ext_vector_type(4))) T vec4;
+    const vec4 x = *reinterpret_cast<const vec4*>(p);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) v[i] = ka_to_float(x[i]);
+}
+
 template <typename T>
 __global__ void __launch_bounds__(KA_WAVE)
 attention_generic_kernel(const T* __restrict__ q, long q_row_stride, const T* __restrict__ k_cache,
@@ -31,6 +40,8 @@ attention_generic_kernel(const T* __restrict__ q, long q_row_stride, const T* __
     for (int d = lane; d < hd; d += KA_WAVE) qs[d] = ka_to_float(qp[d]) * scale;
     __syncthreads();
     const int* bt = block_table + (size_t)row * max_pages;
+    const bool k_vectors = hd % 4 == 0 && reinterpret_cast<uintptr_t>(k_cache) % (4 * sizeof(T)) == 0;
+    const bool v_vectors = page_size % 4 == 0 && reinterpret_cast<uintptr_t>(v_cache) % (4 * sizeof(T)) == 0;
     float m = -INFINITY, l = 0.f;
     float o[ATT_MAX_HD / KA_WAVE];
 #pragma unroll
@@ -45,7 +56,17 @@ attention_generic_kernel(const T* __restrict__ q, long q_row_stride, const T* __
             const T* kp = k_cache + (((long)page * Hkv + kvh) * page_size + key % page_size) * hd;
             off = ((long)page * Hkv + kvh) * hd * page_size + key % page_size;
             float acc = 0.f;
-            for (int d = 0; d < hd; ++d) acc = fmaf(qs[d], ka_to_float(kp[d]), acc);
+            if (k_vectors) {
+                // four channels with one load, added in the same order as one by one
+                for (int d = 0; d < hd; d += 4) {
+                    float k4[4];
+                    att_load4(kp + d, k4);
+#pragma unroll
+                    for (int u = 0; u < 4; ++u) acc = fmaf(qs[d + u], k4[u], acc);
+                }
+            } else {
+                for (int d = 0; d < hd; ++d) acc = fmaf(qs[d], ka_to_float(kp[d]), acc);
+            }
             s = acc;
         }
         float m_new = fmaxf(m, ka_wave_max(s));
@@ -63,7 +84,20 @@ attention_generic_kernel(const T* __restrict__ q, long q_row_stride, const T* __
             int d = lane + i * KA_WAVE;
             if (d < hd) {
                 float acc = o[i] * corr;
-                for (int j = 0; j < count; ++j) acc = fmaf(ps[j], ka_to_float(v_cache[offs[j] + (long)d * page_size]), acc);
+                const T* vd = v_cache + (long)d * page_size;
+                int j = 0;
+                // A chunk that starts on a multiple of four keys: every four keys from there lie in
+                // one page, their values side by side in the cache: one load, added in the same
+                // order as one by one.
+                if (v_vectors && (base & 3) == 0) {
+                    for (; j + 3 < count; j += 4) {
+                        float v4[4];
+                        att_load4(vd + offs[j], v4);
+#pragma unroll
+                        for (int u = 0; u < 4; ++u) acc = fmaf(ps[j + u], v4[u], acc);
+                    }
+                }
+                for (; j < count; ++j) acc = fmaf(ps[j], ka_to_float(vd[offs[j]]), acc);
                 o[i] = acc;
             }
         }
