@@ -67,19 +67,24 @@ gemm_generic_kernel(const TA* __restrict__ A, long lda, const TW* __restrict__ W
 constexpr int GF = 128;   // tile edge in M and N
 constexpr int GFK = 8;    // tile depth
 
+// (RM: output rows a thread holds, 8 or 4: tiles of 128 or 64 rows; the lower tile doubles the
+// workgroups of a narrow output that would otherwise leave CUs with one or none)
+template <int RM>
 __global__ void __launch_bounds__(256)
 gemm_f32_kernel(const float* __restrict__ A, long lda, const float* __restrict__ W, long ldw,
                 const float* __restrict__ bias, float* __restrict__ out, long ldo, int M, int N, int K, int act,
                 int accumulate) {
     typedef __attribute__((ext_vector_type(4))) float f4;
-    __shared__ __attribute__((aligned(16))) float As[2][GFK][GF + 4];
+    constexpr int TM = 16 * RM;
+    __shared__ __attribute__((aligned(16))) float As[2][GFK][TM + 4];
     __shared__ __attribute__((aligned(16))) float Ws[2][GFK][GF + 4];
     const int tx = threadIdx.x % 16, ty = threadIdx.x / 16;
-    const int m0 = blockIdx.y * GF, n0 = blockIdx.x * GF;
+    const int m0 = blockIdx.y * TM, n0 = blockIdx.x * GF;
     // each thread brings four consecutive k of one row of each operand tile (rows past the end
     // are the last row again: their outputs are never stored)
     const int lr = threadIdx.x / 2, lk = (threadIdx.x % 2) * 4;
-    const float* arow = A + (size_t)min(m0 + lr, M - 1) * lda + lk;
+    const bool brings_a = lr < TM;
+    const float* arow = A + (size_t)min(m0 + min(lr, TM - 1), M - 1) * lda + lk;
     const float* wrow = W + (size_t)min(n0 + lr, N - 1) * ldw + lk;
     const f4 zero = {0.f, 0.f, 0.f, 0.f};
     auto fetch = [&](int k0, f4& ra, f4& rw) {
@@ -90,11 +95,11 @@ gemm_f32_kernel(const float* __restrict__ A, long lda, const float* __restrict__
     auto stash = [&](int buf, const f4& ra, const f4& rw) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            As[buf][lk + j][lr] = ra[j];
+            if (brings_a) As[buf][lk + j][lr] = ra[j];
             Ws[buf][lk + j][lr] = rw[j];
         }
     };
-    float acc[8][8] = {};
+    float acc[RM][8] = {};
     f4 ra, rw;
     fetch(0, ra, rw);
     stash(0, ra, rw);
@@ -105,20 +110,25 @@ gemm_f32_kernel(const float* __restrict__ A, long lda, const float* __restrict__
         if (s + 1 < steps) fetch((s + 1) * GFK, ra, rw);
 #pragma unroll
         for (int k = 0; k < GFK; ++k) {
-            const f4 a0 = *reinterpret_cast<const f4*>(&As[buf][k][ty * 8]), a1 = *reinterpret_cast<const f4*>(&As[buf][k][ty * 8 + 4]);
+            float a[RM];
+#pragma unroll
+            for (int i = 0; i < RM; i += 4) {
+                const f4 v = *reinterpret_cast<const f4*>(&As[buf][k][ty * RM + i]);
+#pragma unroll
+                for (int u = 0; u < 4; ++u) a[i + u] = v[u];
+            }
             const f4 w0 = *reinterpret_cast<const f4*>(&Ws[buf][k][tx * 8]), w1 = *reinterpret_cast<const f4*>(&Ws[buf][k][tx * 8 + 4]);
 #pragma unroll
-            for (int i = 0; i < 8; ++i)
+            for (int i = 0; i < RM; ++i)
 #pragma unroll
-                for (int j = 0; j < 8; ++j)
-                    acc[i][j] = fmaf(i < 4 ? a0[i] : a1[i - 4], j < 4 ? w0[j] : w1[j - 4], acc[i][j]);
+                for (int j = 0; j < 8; ++j) acc[i][j] = fmaf(a[i], j < 4 ? w0[j] : w1[j - 4], acc[i][j]);
         }
         if (s + 1 < steps) stash(buf ^ 1, ra, rw);
         __syncthreads();
     }
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        const int m = m0 + ty * 8 + i;
+    for (int i = 0; i < RM; ++i) {
+        const int m = m0 + ty * RM + i;
         if (m >= M) continue;
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
@@ -201,9 +211,13 @@ KA_API int ka_linear_generic(const void* A, int a_dtype, long lda, const void* W
     int key = a_dtype * 4 + w_dtype * 2 + out_dtype;
     const bool vectors = key == 0 && K % 4 == 0 && lda % 4 == 0 && ldw % 4 == 0 && (uintptr_t)A % 16 == 0 &&
                          (uintptr_t)W % 16 == 0;
-    if (vectors && M > GV_ROWS && ka_cdiv(M, GF) <= 65535) {
-        hipLaunchKernelGGL(gemm_f32_kernel, dim3(ka_cdiv(N, GF), ka_cdiv(M, GF)), dim3(256), 0, stream, (const float*)A, lda,
-                           (const float*)W, ldw, bias, (float*)out, ldo, M, N, K, act, accumulate);
+    if (vectors && M > GV_ROWS && ka_cdiv(M, 64) <= 65535) {
+        if ((long)ka_cdiv(N, GF) * ka_cdiv(M, GF) >= 512)
+            hipLaunchKernelGGL(gemm_f32_kernel<8>, dim3(ka_cdiv(N, GF), ka_cdiv(M, GF)), dim3(256), 0, stream, (const float*)A, lda,
+                               (const float*)W, ldw, bias, (float*)out, ldo, M, N, K, act, accumulate);
+        else
+            hipLaunchKernelGGL(gemm_f32_kernel<4>, dim3(ka_cdiv(N, GF), ka_cdiv(M, 64)), dim3(256), 0, stream, (const float*)A, lda,
+                               (const float*)W, ldw, bias, (float*)out, ldo, M, N, K, act, accumulate);
         KA_LAUNCH_CHECK();
         return 0;
     }

@@ -107,7 +107,7 @@ def _linear_case(fn, m, n, k, a_dtype, w_dtype, out_dtype, act, accumulate, seed
 
 
 @pytest.mark.parametrize("shape", [(1, 37, 19), (65, 130, 200), (7, 64, 96), (130, 77, 333), (16, 51, 2048), (3, 1000, 260),
-                                   (17, 40, 64), (300, 257, 1028), (129, 128, 12), (2048, 100, 520)])
+                                   (17, 40, 64), (300, 257, 1028), (129, 128, 12), (2048, 100, 520), (2050, 4100, 36)])
 def test_linear_generic(shape):
     from kestrel_amd.ops import core
 
