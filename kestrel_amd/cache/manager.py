@@ -138,7 +138,9 @@ class CacheManager:
                                   dtype=self.dtype, device=self.device)
         for entry, (_c, state_spec, _r) in enumerate(self.needs):
             if state_spec is not None:
-                self.states[entry] = torch.zeros((self.max_requests, *state_spec.shape),
+                # one row more than there are slots: the last one is a spare that rows without a
+                # request (slot -1, the rows that pad a captured batch) may read and write
+                self.states[entry] = torch.zeros((self.max_requests + 1, *state_spec.shape),
                                                  dtype=getattr(torch, state_spec.dtype), device=self.device)
 
     def bytes_per_page(self) -> int:

@@ -17,6 +17,7 @@ import threading
 import time
 from concurrent.futures import Future
 from dataclasses import dataclass
+from collections.abc import Mapping, Sequence as Sequence_abc
 from typing import AsyncIterator, Dict, List, Optional, Sequence
 
 import torch
@@ -25,7 +26,7 @@ from ..config.runtime import RuntimeConfig
 from ..sampling.sampler import Sampler
 from .loading import load_model, make_runner
 from .scheduler import GenerationScheduler
-from .types import GenerationRequest, SchedulerResult
+from .types import GeneratedPrefix, GenerationRequest, SchedulerResult
 
 
 @dataclass
@@ -61,6 +62,36 @@ class StreamUpdate:
 class _Pending:
     def __init__(self, request: GenerationRequest, future: Future, stream: Optional["queue.Queue"]) -> None:
         self.request, self.future, self.stream = request, future, stream
+
+
+def _generated_prefix(raw) -> GeneratedPrefix:
+    """``None``, a ``GeneratedPrefix`` or a mapping with ``tokens`` and optionally ``logprobs``
+    (``kestrel/engine/core.py:1260-1294``)."""
+    if raw is None:
+        return GeneratedPrefix()
+    if isinstance(raw, GeneratedPrefix):
+        tokens, logprobs = raw.tokens, raw.logprobs
+    else:
+        if not isinstance(raw, Mapping):
+            raise TypeError("_generated_prefix must be a mapping or None")
+        extra = set(raw) - {"tokens", "logprobs"}
+        if extra:
+            raise TypeError(f"_generated_prefix has unsupported key(s): {', '.join(sorted(map(str, extra)))}")
+        if "tokens" not in raw:
+            raise ValueError("_generated_prefix.tokens is required")
+        tokens, logprobs = raw["tokens"], raw.get("logprobs")
+    if tokens is None:
+        tokens = ()
+    if isinstance(tokens, (str, bytes)) or not isinstance(tokens, (Sequence_abc, torch.Tensor)):
+        raise TypeError("_generated_prefix.tokens must be a sequence of token ids")
+    tokens = tuple(int(t) for t in tokens)
+    if logprobs is not None:
+        if isinstance(logprobs, (str, bytes)) or not isinstance(logprobs, (Sequence_abc, torch.Tensor)):
+            raise TypeError("_generated_prefix.logprobs must be a sequence of floats or None")
+        logprobs = tuple(float(v) for v in logprobs)
+        if len(logprobs) != len(tokens):
+            raise ValueError("_generated_prefix.logprobs must have the same length as generated prefix tokens")
+    return GeneratedPrefix(tokens, logprobs)
 
 
 def _normalise(temperature, top_p):
@@ -209,7 +240,7 @@ class InferenceEngine:
     # ------------------------------------------------------------------ requests
     def _make_request(self, prompt_ids, max_new_tokens, temperature, top_p, prefix_embeds, prefix_ids, stop_ids, seed,
                       on_token, return_logprobs=False, suppress_next_token_ids=(), suppressed_token_ids=(),
-                      allowed_token_ids=None) -> GenerationRequest:
+                      allowed_token_ids=None, generated_prefix=None) -> GenerationRequest:
         if self._fatal is not None:
             raise RuntimeError("the engine has stopped after an error") from self._fatal
         if self._thread is None:
@@ -226,16 +257,20 @@ class InferenceEngine:
                                  suppress_next_token_ids=tuple(int(t) for t in suppress_next_token_ids or ()),
                                  suppressed_token_ids=tuple(int(t) for t in suppressed_token_ids or ()),
                                  allowed_token_ids=None if allowed_token_ids is None
-                                 else tuple(int(t) for t in allowed_token_ids))
+                                 else tuple(int(t) for t in allowed_token_ids),
+                                 generated_prefix=_generated_prefix(generated_prefix))
 
     def submit_sync(self, prompt_ids: Sequence[int], *, max_new_tokens: int, temperature: Optional[float] = None,
                     top_p: Optional[float] = None, prefix_embeds: Optional[torch.Tensor] = None,
                     prefix_ids: Sequence[int] = (), stop_ids: Optional[Sequence[int]] = None,
                     seed: Optional[int] = None, _stream: Optional["queue.Queue"] = None, **sampling) -> Future:
         """Queue a request; the returned future resolves to an ``EngineResult``. ``sampling`` takes
-        ``return_logprobs``, ``suppress_next_token_ids``, ``suppressed_token_ids`` and
-        ``allowed_token_ids`` (``kestrel/engine/core.py:556-597``)."""
-        unknown = set(sampling) - {"return_logprobs", "suppress_next_token_ids", "suppressed_token_ids", "allowed_token_ids"}
+        ``return_logprobs``, ``suppress_next_token_ids``, ``suppressed_token_ids``,
+        ``allowed_token_ids`` and ``generated_prefix`` (tokens the request generated before: they are
+        fed after the prompt, count against ``max_new_tokens`` and head the result)
+        (``kestrel/engine/core.py:556-597``)."""
+        unknown = set(sampling) - {"return_logprobs", "suppress_next_token_ids", "suppressed_token_ids",
+                                   "allowed_token_ids", "generated_prefix"}
         if unknown:
             raise TypeError(f"unknown options: {sorted(unknown)}")
         on_token = None
@@ -267,7 +302,8 @@ class InferenceEngine:
 
     async def generate(self, prompt_ids: Sequence[int], *, settings: Optional[dict] = None, **options) -> EngineResult:
         """``settings`` takes the reference's keys: ``temperature``, ``top_p``, ``max_tokens`` and the
-        private ``_logprobs`` and ``_suppress_next_token_ids`` (``kestrel/engine/core.py:556-597``)."""
+        private ``_logprobs``, ``_suppress_next_token_ids`` and ``_generated_prefix``
+        (``kestrel/engine/core.py:556-597``)."""
         settings = dict(settings or {})
         if "max_tokens" in settings:
             options.setdefault("max_new_tokens", settings.pop("max_tokens"))
@@ -275,6 +311,8 @@ class InferenceEngine:
             options.setdefault("return_logprobs", bool(settings.pop("_logprobs")))
         if "_suppress_next_token_ids" in settings:
             options.setdefault("suppress_next_token_ids", settings.pop("_suppress_next_token_ids"))
+        if "_generated_prefix" in settings:
+            options.setdefault("generated_prefix", settings.pop("_generated_prefix"))
         for key in ("temperature", "top_p"):
             if key in settings:
                 options.setdefault(key, settings.pop(key))

@@ -39,9 +39,10 @@ from collections import deque
 from dataclasses import dataclass, field
 from typing import Deque, Dict, List, Optional, Tuple
 
+import numpy as np
 import torch
 
-from .step import PENDING_TOKEN, StepEntry
+from .step import PENDING_TOKEN, StepEntry, StepRefused
 from .types import GenerationRequest, RequestMetrics, RequestPhase, SchedulerResult, Sequence_
 
 
@@ -95,6 +96,7 @@ class GenerationScheduler:
         self.running: List[Sequence_] = []
         self.completed: List[SchedulerResult] = []
         self.steps = 0
+        self.failed_steps = 0
 
     # ------------------------------------------------------------------ intake
     def enqueue_request(self, request: GenerationRequest) -> None:
@@ -108,12 +110,41 @@ class GenerationScheduler:
             raise ValueError("an allow-list needs at least one token")
         if request.prompt_length == 0:
             raise ValueError("a request needs at least one prompt token or embedding")
-        if request.prompt_length >= self.max_positions:
-            raise ValueError(f"prompt of {request.prompt_length} tokens leaves no room in a context of {self.max_positions}")
+        if request.prefill_length >= self.max_positions:
+            raise ValueError(f"prompt of {request.prefill_length} tokens leaves no room in a context of {self.max_positions}")
+        self._check_contents(request)
         if request.block_length > self.max_num_batched_tokens:
             raise ValueError(f"the bidirectional block of {request.block_length} positions does not fit in one step "
                              f"of {self.max_num_batched_tokens} tokens")
         self.waiting.append(Sequence_(request))
+
+    def _check_contents(self, request: GenerationRequest) -> None:
+        """What a request brings must be what the step function takes, so that it is refused here,
+        alone, and not in the middle of a step that others share."""
+        plan = self.runner.model.plan
+        vocab = plan.vocab_size
+        for name, ids in (("prompt_ids", request.prompt_ids), ("prefix_ids", request.prefix_ids),
+                          ("generated_prefix.tokens", request.generated_prefix.tokens),
+                          ("suppress_next_token_ids", request.suppress_next_token_ids),
+                          ("suppressed_token_ids", request.suppressed_token_ids),
+                          ("allowed_token_ids", request.allowed_token_ids or ()),
+                          ("stop_ids", request.stop_ids or ())):
+            if len(ids) == 0:
+                continue
+            values = np.asarray(ids)
+            if values.ndim != 1 or values.dtype.kind not in "iu":
+                raise ValueError(f"{name} must be a flat sequence of integer token ids")
+            low, high = int(values.min()), int(values.max())
+            if low < 0 or high >= vocab:
+                bad = low if low < 0 else high
+                raise ValueError(f"{name}: token id {bad} outside the vocabulary of {vocab}")
+        embeds = request.prefix_embeds
+        if embeds is not None:
+            dim = getattr(plan, "dim", None)
+            if not isinstance(embeds, torch.Tensor) or embeds.dim() != 2 or not embeds.is_floating_point() \
+                    or (dim is not None and embeds.shape[1] != dim):
+                shape = tuple(embeds.shape) if isinstance(embeds, torch.Tensor) else type(embeds).__name__
+                raise ValueError(f"prefix_embeds must be a floating-point tensor [rows, {dim}], got {shape}")
 
     def has_pending_work(self) -> bool:
         return bool(self.waiting or self.prefilling or self.running or self._inflight)
@@ -129,7 +160,7 @@ class GenerationScheduler:
     def _portion(self, seq: Sequence_, budget: int) -> int:
         """Places of the prompt to feed next within ``budget`` (0: does not fit now)."""
         request = seq.request
-        left = request.prompt_length - seq.fed
+        left = request.prefill_length - seq.fed
         take = min(left, budget)
         block = request.block_length
         if take < left:
@@ -155,11 +186,14 @@ class GenerationScheduler:
             a, b = max(lo, n_ids) - n_ids, min(hi, n_ids + n_emb) - n_ids
             tokens.extend([-1] * (b - a))
             embeds = request.prefix_embeds[a:b]
-        for p in range(max(lo, n_ids + n_emb), hi):
+        n_prompt = request.prompt_length
+        for p in range(max(lo, n_ids + n_emb), min(hi, n_prompt)):
             tokens.append(int(request.prompt_ids[p - n_ids - n_emb]))
+        for p in range(max(lo, n_prompt), hi):       # what it had generated before follows the prompt
+            tokens.append(int(request.generated_prefix.tokens[p - n_prompt]))
         block = request.block_length
         bidirectional = [(0, block)] if block and lo == 0 else []
-        ends_prompt = hi == request.prompt_length
+        ends_prompt = hi == request.prefill_length
         return StepEntry(seq.slot, tokens, want=[take - 1] if ends_prompt else [], embeds=embeds,
                          bidirectional=bidirectional, start=lo)
 
@@ -227,9 +261,9 @@ class GenerationScheduler:
             did = True
         return did or self._fail_unfittable()
 
-    def _launch(self, plan: StepPlan) -> None:
-        self.steps += 1
-        logits = self.runner.step([row.entry for row in plan.rows])
+    def _sample(self, plan: StepPlan, logits: torch.Tensor):
+        """Queue the sampling of the rows that end a prompt or decode, and the copy of their
+        tokens to the host. Returns ``(ids, event, logprobs)``."""
         sampled_rows = [row for row in plan.rows if row.samples]
         ids = event = logprobs = None
         if sampled_rows:
@@ -238,10 +272,10 @@ class GenerationScheduler:
             tops = [r.top_p for r in requests]
             seeds = [r.seed if r.seed is not None else r.request_id for r in requests]
             indices = [row.seq.launched for row in sampled_rows]
-            # masks: what a request never wants, and what it does not want as its first token
+            # masks: what a request never wants, and what it does not want as its first new token
             suppress = [(i, int(t)) for i, r in enumerate(requests) for t in r.suppressed_token_ids]
             suppress += [(i, int(t)) for i, (row, r) in enumerate(zip(sampled_rows, requests))
-                         if row.seq.launched == 0 for t in r.suppress_next_token_ids]
+                         if row.seq.launched == r.generated_prefix_length for t in r.suppress_next_token_ids]
             allowed = [r.allowed_token_ids for r in requests]
             extras = {}
             if suppress:
@@ -260,6 +294,16 @@ class GenerationScheduler:
                 ids, event = self._to_host(ids)
                 if logprobs is not None:
                     logprobs, event = self._to_host(logprobs)
+        return ids, event, logprobs
+
+    def _launch(self, plan: StepPlan) -> None:
+        self.steps += 1
+        try:
+            logits = self.runner.step([row.entry for row in plan.rows])
+            ids, event, logprobs = self._sample(plan, logits)
+        except Exception as exc:
+            self._fail_rows(plan, exc)
+            return
         for row in plan.rows:
             seq = row.seq
             if row.kind == "prefill":
@@ -273,6 +317,22 @@ class GenerationScheduler:
                 self.running.append(seq)
                 seq.phase = RequestPhase.RUNNING
         self._inflight.append(LaunchedStep(plan.rows, ids, event, logprobs))
+
+    def _fail_rows(self, plan: StepPlan, exc: Exception) -> None:
+        """The step function raised. If it refused one entry (``StepRefused``: found before anything
+        ran or changed), that request fails alone and the others are planned again. Anything else
+        may have happened half-way through the step: every request of the step fails, the ones in
+        other queues go on (``kestrel/scheduler/scheduler.py:1576-1613,1696-1763``). Slots and pages
+        come back at once, or when a step of the request that is still in flight has been read."""
+        now = time.perf_counter()
+        if isinstance(exc, StepRefused) and 0 <= exc.entry_index < len(plan.rows):
+            rows = [plan.rows[exc.entry_index]]
+        else:
+            rows = list(plan.rows)
+        for row in rows:
+            if row.seq.finish_reason is None:
+                self._finish(row.seq, "error", now, f"{type(exc).__name__}: {exc}")
+        self.failed_steps += 1
 
     def _to_host(self, values: torch.Tensor):
         """Start the copy of a step's tokens (or their log-probabilities) into pinned memory; the
@@ -338,7 +398,8 @@ class GenerationScheduler:
         started = seq.prefill_started_at if seq.prefill_started_at is not None else seq.submitted_at
         first = seq.first_token_at if seq.first_token_at is not None else now
         metrics = RequestMetrics(
-            prompt_tokens=seq.request.prompt_length, decode_tokens=len(seq.tokens),
+            prompt_tokens=seq.request.prompt_length,
+            decode_tokens=max(0, len(seq.tokens) - seq.request.generated_prefix_length),
             prefill_time_ms=(first - started) * 1e3, ttft_ms=(first - seq.submitted_at) * 1e3,
             decode_time_ms=(now - first) * 1e3)
         self.completed.append(SchedulerResult(seq.request.request_id, list(seq.tokens), reason, metrics, error,

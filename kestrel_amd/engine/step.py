@@ -9,8 +9,10 @@ logits at the places asked for. The reference runs either padded whole prompts
 block table and key counts ``runtime.py:2283-2290``) is what is built here per token.
 
 Steps that hold one token per request are replayed as HIP graphs, one graph per batch
-size bucket (1, 2, 4, ... as in ``kestrel/runtime/decode_graph.py:20-25``): the metadata
-lives at fixed addresses, rows that pad the bucket see no keys and write nothing.
+size bucket (1, 2, 4, 8, 16, 32, 48, ... as in ``kestrel/runtime/decode_graph.py:18-23``): the
+metadata lives at fixed addresses, rows that pad the bucket see no keys and write nothing. A graph
+is captured, and run once before that, on padding rows alone: no live request is touched by
+anything but the replays, so a mixer that keeps state is advanced once a step.
 """
 
 from __future__ import annotations
@@ -27,6 +29,17 @@ from .batch import GroupBatch, StepBatch, Workspace
 
 
 PENDING_TOKEN = -2     # "the token that sampling last left for this request on the device"
+GIVEN_TOKEN = -1       # "the embedding of this place is given"
+
+
+class StepRefused(ValueError):
+    """An entry of a step is not what the step function takes. It is raised before any page is
+    taken or any kernel runs, so the other entries of the step can be run again without it;
+    ``entry_index`` names the entry."""
+
+    def __init__(self, entry_index: int, message: str) -> None:
+        super().__init__(message)
+        self.entry_index = entry_index
 
 
 @dataclass
@@ -55,14 +68,14 @@ def _align(n: int) -> int:
 
 
 def graph_buckets(max_batch: int) -> List[int]:
-    """Batch sizes graphs are captured for: powers of two up to ``max_batch``, and ``max_batch``
-    (``kestrel/runtime/decode_graph.py:20-25``; e.g. 33 -> 1, 2, 4, 8, 16, 32, 33)."""
-    sizes, size = [], 1
-    while size < max_batch:
-        sizes.append(size)
-        size *= 2
-    sizes.append(max_batch)
-    return sizes
+    """Batch sizes graphs are captured for: 1, 2, 4, 8, then every multiple of 16, then
+    ``max_batch`` itself (``kestrel/runtime/decode_graph.py:18-23``; 33 -> 1, 2, 4, 8, 16, 32, 33;
+    64 -> 1, 2, 4, 8, 16, 32, 48, 64)."""
+    max_batch = max(1, max_batch)
+    sizes = {size for size in (1, 2, 4, 8) if size <= max_batch}
+    sizes.update(range(16, max_batch + 1, 16))
+    sizes.add(max_batch)
+    return sorted(sizes)
 
 
 class _Column:
@@ -158,27 +171,59 @@ class ModelRunner:
         return buf, index
 
     def _check_entries(self, entries: Sequence[StepEntry]) -> List[int]:
+        """Everything that can be wrong with an entry is found here, before the step touches the
+        cache: its slot, its start, its token ids, its embeddings, its block and the places wanted.
+        Returns the entries' start positions."""
         plan = self.model.plan
-        if not entries:
-            raise ValueError("a step needs at least one entry")
         seen = set()
         starts: List[int] = []
         n_tokens = 0
-        for e in entries:
+        for index, e in enumerate(entries):
+            def refuse(message: str, index=index, e=e):
+                return StepRefused(index, f"slot {e.slot}: {message}")
             if e.slot in seen:
-                raise ValueError(f"slot {e.slot} appears twice in one step")
+                raise refuse("it appears twice in one step")
             seen.add(e.slot)
             if e.slot not in self.held:
-                raise ValueError(f"slot {e.slot} is not live")
-            if len(e.tokens) == 0:
-                raise ValueError(f"slot {e.slot}: an entry needs at least one token")
+                raise refuse("it is not live")
+            q = len(e.tokens)
+            if q == 0:
+                raise refuse("an entry needs at least one token")
             start = self.held[e.slot] if e.start is None else int(e.start)
             if start != self.held[e.slot]:
-                raise ValueError(f"slot {e.slot}: portion starts at {start} but the request holds {self.held[e.slot]} tokens")
-            if start + len(e.tokens) > plan.max_positions:
-                raise ValueError(f"slot {e.slot}: {start + len(e.tokens)} tokens exceed the model's {plan.max_positions} positions")
+                raise refuse(f"portion starts at {start} but the request holds {self.held[e.slot]} tokens")
+            if start + q > plan.max_positions:
+                raise refuse(f"{start + q} tokens exceed the model's {plan.max_positions} positions")
+            if q <= self.SCALAR_ROW:
+                n_given = 0
+                for tok in e.tokens:
+                    tok = int(tok)
+                    if tok >= plan.vocab_size or tok < PENDING_TOKEN:
+                        raise refuse(f"token id {tok} outside the vocabulary of {plan.vocab_size}")
+                    n_given += tok == GIVEN_TOKEN
+            else:
+                tok_a = np.asarray(e.tokens)
+                if tok_a.ndim != 1 or tok_a.dtype.kind not in "iu":
+                    raise refuse("token ids must be a flat sequence of integers")
+                bad = (tok_a >= plan.vocab_size) | (tok_a < PENDING_TOKEN)
+                if bad.any():
+                    raise refuse(f"token id {int(tok_a[bad][0])} outside the vocabulary of {plan.vocab_size}")
+                n_given = int((tok_a == GIVEN_TOKEN).sum())
+            if n_given:
+                if not isinstance(e.embeds, torch.Tensor) or e.embeds.dim() != 2 \
+                        or tuple(e.embeds.shape) != (n_given, plan.dim) or not e.embeds.is_floating_point():
+                    raise refuse(f"{n_given} places need floating-point embeddings of shape [{n_given}, {plan.dim}]")
+            elif e.embeds is not None and e.embeds.numel():
+                raise refuse("embeddings given but no token id is -1")
+            for lo_b, hi_b in e.bidirectional:
+                if not (start <= lo_b < hi_b <= start + q):
+                    raise refuse(f"the bidirectional block [{lo_b}, {hi_b}) must lie inside one portion, this one "
+                                 f"covers [{start}, {start + q})")
+            for w in e.want:
+                if not 0 <= int(w) < q:
+                    raise refuse(f"wanted place {w} outside its {q} tokens")
             starts.append(start)
-            n_tokens += len(e.tokens)
+            n_tokens += q
         if n_tokens > self.max_tokens_per_step:
             raise ValueError(f"{n_tokens} tokens in one step exceed the limit of {self.max_tokens_per_step}")
         return starts
@@ -194,6 +239,8 @@ class ModelRunner:
         """
         cache, plan = self.cache, self.model.plan
         ps = cache.page_size
+        if not entries and pad_rows <= 0:
+            raise ValueError("a step needs at least one entry")
         starts = self._check_entries(entries)
         for e, start in zip(entries, starts):
             cache.ensure(e.slot, start + len(e.tokens))
@@ -215,10 +262,7 @@ class ModelRunner:
         for r, (e, start) in enumerate(zip(entries, starts)):
             q = len(e.tokens)
             base = len(ids)
-            for lo_b, hi_b in e.bidirectional:
-                if not (start <= lo_b < hi_b <= start + q):
-                    raise ValueError(f"slot {e.slot}: the bidirectional block [{lo_b}, {hi_b}) must lie inside one "
-                                     f"portion, this one covers [{start}, {start + q})")
+            if e.bidirectional:
                 causal_only = False
             if q <= self.SCALAR_ROW:
                 hi = [start + i + 1 for i in range(q)]
@@ -230,11 +274,8 @@ class ModelRunner:
                     tok = int(tok)
                     if tok == PENDING_TOKEN:
                         tok = PENDING_TOKEN - e.slot      # the embedding kernel reads pending[slot]
-                    elif tok < 0:
+                    elif tok == GIVEN_TOKEN:
                         row_given.append(base + i)
-                        tok = -1
-                    elif tok >= plan.vocab_size:
-                        raise ValueError(f"slot {e.slot}: token id {tok} outside the vocabulary of {plan.vocab_size}")
                     row_ids.append(tok)
             else:
                 # a prompt portion has thousands of tokens: a loop over them in Python would take
@@ -242,26 +283,17 @@ class ModelRunner:
                 hi_a = np.arange(start + 1, start + q + 1, dtype=np.int64)
                 for lo_b, hi_b in e.bidirectional:
                     np.maximum(hi_a[lo_b - start:hi_b - start], hi_b, out=hi_a[lo_b - start:hi_b - start])
-                tok_a = np.asarray(e.tokens, dtype=np.int64).reshape(-1)
+                tok_a = np.array(e.tokens, dtype=np.int64).reshape(-1)     # a copy: it is edited below
                 pending = tok_a == PENDING_TOKEN
-                is_given = (tok_a < 0) & ~pending
-                too_large = tok_a >= plan.vocab_size
-                if too_large.any():
-                    raise ValueError(f"slot {e.slot}: token id {int(tok_a[too_large][0])} outside the vocabulary of "
-                                     f"{plan.vocab_size}")
+                is_given = tok_a == GIVEN_TOKEN
                 tok_a[pending] = PENDING_TOKEN - e.slot
-                tok_a[is_given] = -1
                 row_given = (base + np.nonzero(is_given)[0]).tolist()
                 row_ids, hi = tok_a, hi_a
             n_given = len(row_given)
             given_rows.extend(row_given)
             ids.extend(row_ids)
             if n_given:
-                if e.embeds is None or e.embeds.dim() != 2 or tuple(e.embeds.shape) != (n_given, plan.dim):
-                    raise ValueError(f"slot {e.slot}: {n_given} places need embeddings of shape [{n_given}, {plan.dim}]")
                 given.append(e.embeds)
-            elif e.embeds is not None and e.embeds.numel():
-                raise ValueError(f"slot {e.slot}: embeddings given but no token id is -1")
             if q <= self.SCALAR_ROW:
                 positions.extend(range(start, start + q))
                 token_row.extend([r] * q)
@@ -277,10 +309,7 @@ class ModelRunner:
             else:
                 for first in range(0, q, self.QUERY_BLOCK):
                     blocks.append((r, base + first, max(hi[first:first + self.QUERY_BLOCK])))
-            for w in e.want:
-                if not 0 <= int(w) < q:
-                    raise ValueError(f"slot {e.slot}: wanted place {w} outside its {q} tokens")
-                logit_rows.append(base + int(w))
+            logit_rows.extend(base + int(w) for w in e.want)
             cu_q.append(base + q)
             kv_len.append(start + q)
             row_slot.append(e.slot)
@@ -402,27 +431,31 @@ class ModelRunner:
         state = self._graphs.get(bucket)
         if state is None:
             state = self._graphs[bucket] = _GraphState(self.device)
-        if state.meta is None:
-            probe = self.build_batch(entries, pad_rows=bucket, fixed_pages=self._pages_cap)
-            state.meta = torch.empty(probe.host["meta_ints"], dtype=torch.int32, device=self.device)
-        batch = self.build_batch(entries, pad_rows=bucket, fixed_pages=self._pages_cap, meta=state.meta,
-                                 workspace=state.workspace)
-        # the decode attention kernel cuts a row's keys by the longest context of the batch: a
-        # graph must cut the same way on every replay, so it is captured for the longest possible
-        batch.max_kv = self.model.plan.max_positions
         if state.graph is None:
+            # Warm-up and capture on padding rows alone (no slot, no keys, nothing written): the
+            # layout of the metadata depends on the bucket only, and nothing of a live request,
+            # per-request state included, is touched before the first replay.
+            probe = self.build_batch([], pad_rows=bucket, fixed_pages=self._pages_cap)
+            state.meta = torch.empty(probe.host["meta_ints"], dtype=torch.int32, device=self.device)
+            blank = self.build_batch([], pad_rows=bucket, fixed_pages=self._pages_cap, meta=state.meta,
+                                     workspace=state.workspace)
+            # the decode attention kernel cuts a row's keys by the longest context of the batch: a
+            # graph must cut the same way on every replay, so it is captured for the longest possible
+            blank.max_kv = self.model.plan.max_positions
             current = torch.cuda.current_stream()
             side = torch.cuda.Stream()
             side.wait_stream(current)
             with torch.cuda.stream(side):          # first run outside capture: every buffer comes into being
-                self.model.forward(batch, self.layer_caches)
+                self.model.forward(blank, self.layer_caches)
             current.wait_stream(side)
             torch.cuda.synchronize()
             state.workspace.freeze()
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph):
-                state.logits = self.model.forward(batch, self.layer_caches)
+                state.logits = self.model.forward(blank, self.layer_caches)
             state.graph = graph
+        self.build_batch(entries, pad_rows=bucket, fixed_pages=self._pages_cap, meta=state.meta,
+                         workspace=state.workspace)
         state.graph.replay()
         self.graph_replays += 1
         return state.logits[:len(entries)]
@@ -433,6 +466,8 @@ class ModelRunner:
         """Run the entries as one batch. Returns fp32 logits ``[wanted, vocab]`` in the order of
         the entries and of their ``want``; the tensor is scratch memory and is overwritten by
         the next step."""
+        if not entries:
+            raise ValueError("a step needs at least one entry")
         bucket = self._graph_bucket(entries)
         if bucket is not None:
             logits = self._step_graph(entries, bucket)

@@ -15,6 +15,15 @@ from typing import Callable, List, Optional, Sequence, Tuple
 import torch
 
 
+@dataclass(frozen=True)
+class GeneratedPrefix:
+    """Tokens a request has already generated (``kestrel/scheduler/types.py:16-21``): they are fed
+    after the prompt, count against ``max_new_tokens`` and stand at the head of the result."""
+
+    tokens: Tuple[int, ...] = ()
+    logprobs: Optional[Tuple[float, ...]] = None
+
+
 class RequestPhase(enum.Enum):
     WAITING = "waiting"
     PREFILLING = "prefilling"
@@ -44,6 +53,17 @@ class GenerationRequest:
     suppress_next_token_ids: Sequence[int] = ()     # not to be the first generated token
     suppressed_token_ids: Sequence[int] = ()        # never to be generated
     allowed_token_ids: Optional[Sequence[int]] = None   # if given, the only tokens that may be generated
+    generated_prefix: GeneratedPrefix = field(default_factory=GeneratedPrefix)
+
+    def __post_init__(self) -> None:
+        # the checks of ``kestrel/scheduler/types.py:215-237``
+        prefix = self.generated_prefix
+        if prefix.logprobs is not None and len(prefix.logprobs) != len(prefix.tokens):
+            raise ValueError("generated_prefix.logprobs must have the same length as generated_prefix.tokens")
+        if prefix.tokens and len(prefix.tokens) >= self.max_new_tokens:
+            raise ValueError("generated_prefix.tokens must be shorter than max_new_tokens")
+        if prefix.tokens and self.return_logprobs and prefix.logprobs is None:
+            raise ValueError("generated_prefix.logprobs is required when return_logprobs is true")
 
     @property
     def block_length(self) -> int:
@@ -54,6 +74,16 @@ class GenerationRequest:
     def prompt_length(self) -> int:
         n = 0 if self.prefix_embeds is None else int(self.prefix_embeds.shape[0])
         return len(self.prefix_ids) + n + len(self.prompt_ids)
+
+    @property
+    def generated_prefix_length(self) -> int:
+        return len(self.generated_prefix.tokens)
+
+    @property
+    def prefill_length(self) -> int:
+        """Places that are fed before the first token is sampled: the prompt, then what the
+        request had generated before (``types.py:260-262``)."""
+        return self.prompt_length + len(self.generated_prefix.tokens)
 
 
 @dataclass
@@ -92,6 +122,14 @@ class Sequence_:
     first_token_at: Optional[float] = None
     prefill_started_at: Optional[float] = None
     finished_at: Optional[float] = None
+
+    def __post_init__(self) -> None:
+        # generated before: already part of the result, and of the count (``types.py:67-70``)
+        prefix = self.request.generated_prefix
+        self.tokens.extend(int(t) for t in prefix.tokens)
+        self.launched = len(prefix.tokens)
+        if self.request.return_logprobs and prefix.logprobs is not None:
+            self.logprobs.extend(float(v) for v in prefix.logprobs)
 
     @property
     def total_length(self) -> int:

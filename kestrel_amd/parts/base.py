@@ -54,7 +54,9 @@ class LayerCache:
     if the mixer keeps no keys and values; ``k``: ``[pages, Hkv, page_size, hd]``, ``v``:
     ``[pages, Hkv, hd, page_size]``;
     ``writes``: ``False`` when this run reads the cache of another run; ``state``:
-    ``[slots, *shape]`` per-request state, indexed by ``StepBatch.row_slot``.
+    ``[slots + 1, *shape]`` per-request state, indexed by ``StepBatch.row_slot``; its last row is
+    a spare for rows without a request (slot -1: what index -1 means to torch), whose content
+    nobody reads.
     """
 
     group: Optional[int] = None

@@ -90,6 +90,25 @@ def assert_close(actual: torch.Tensor, expected: torch.Tensor, dtype: torch.dtyp
                              f"error {err[idx]:.3g} > {bound[idx]:.3g}; max error {err.max():.3g}")
 
 
+def assert_greedy_follows(cfg: dict, weights, prompt: Sequence[int], tokens: Sequence[int], slack: float, what: str,
+                          prefix_embeds: Optional[torch.Tensor] = None) -> None:
+    """Every generated token must be the plain implementation's choice *after the engine's own
+    earlier tokens*: the plain model is run once over prompt + tokens and, at each place, the
+    engine's token may lie at most ``slack`` below the best logit. A near tie thus excuses one token
+    only and every later one is still checked."""
+    from tests.plain import moondream_plain as plain
+
+    tokens = list(tokens)
+    logits = plain.forward(cfg, weights, list(prompt) + tokens[:-1], prefix_embeds)
+    n_prefix = 0 if prefix_embeds is None else prefix_embeds.shape[0]
+    first = n_prefix + len(prompt) - 1
+    for i, token in enumerate(tokens):
+        row = logits[first + i]
+        gap = float(row.max() - row[token])
+        assert gap <= slack, (f"{what}: token {i} is {token}, the plain implementation gives {int(row.argmax())} "
+                              f"after the same tokens ({gap:.3g} better)")
+
+
 # ----------------------------------------------------------------------------
 # replaying requests through a runner in a given way of cutting
 # ----------------------------------------------------------------------------

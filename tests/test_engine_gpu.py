@@ -20,11 +20,11 @@ DTYPE_IDS = ["fp32", "bf16"]
 NAMES = ["A", "B", "C", "D", "E", "F"]
 
 
-def _runner(name, dtype, n_pages=64, page_size=16, max_requests=8):
+def _runner(name, dtype, n_pages=64, page_size=16, max_requests=8, graphs=False):
     from kestrel_amd.engine.loading import load_model, make_runner
 
     net = load_model(helpers.model_dir(name), dtype, torch.device("cuda:0"))
-    runner = make_runner(net, page_size, n_pages, max_requests)
+    runner = make_runner(net, page_size, n_pages, max_requests, enable_graphs=graphs)
     helpers.poison_cache(runner)
     return runner
 
@@ -184,6 +184,57 @@ def test_a_context_of_thousands(dtype):
     _check(name, dtype, reqs, got)
 
 
+@pytest.mark.parametrize("dtype", DTYPES, ids=DTYPE_IDS)
+@pytest.mark.parametrize("name", ["A", "D", "F"])
+def test_replayed_graphs_match_the_plain_implementation(name, dtype):
+    """Decode steps replayed as HIP graphs, compared logit by logit with the plain implementation:
+    one, three and five live requests (buckets of 1, 4 and 8, the last two with padding rows), across
+    page edges, with prompt steps (eager) between the replays, a request that ends and whose slot
+    and pages another takes, and a return to a bucket captured earlier."""
+    lengths = {"r0": 58, "r1": 41, "r2": 37, "r3": 50, "r4": 30, "r5": 44}
+    runner = _runner(name, dtype, n_pages=20, max_requests=8, graphs=True)
+    reqs = {tag: _request(name, tag, 1300 + i, n) for i, (tag, n) in enumerate(lengths.items())}
+    steps = [[("r0", 13)]]
+    steps += [[("r0", 1)]] * 5                                           # bucket 1, over the page edge at 16
+    steps += [[("r1", 30), ("r0", 1)], [("r2", 9), ("r0", 1), ("r1", 1)]]         # eager: prompts beside decoded tokens
+    steps += [[("r0", 1), ("r1", 1), ("r2", 1)]] * 6                     # bucket 4 with a padding row
+    steps += [[("r3", 29), ("r4", 15)]]
+    steps += [[("r0", 1), ("r1", 1), ("r2", 1), ("r3", 1), ("r4", 1)]] * 4        # bucket 8 with three padding rows; r1 ends
+    steps += [[("r5", 17), ("r2", 1)]]                                   # r5 takes r1's slot and pages
+    steps += [[("r4", 1), ("r5", 1), ("r0", 1), ("r2", 1), ("r3", 1)]] * 7        # bucket 8, other rows in other places
+    steps += [[("r0", 1), ("r3", 1), ("r5", 1)]] * 4                     # back to bucket 4
+    steps += [[("r0", 1)]] * 3                                           # and to bucket 1
+    fed = steps_fed(steps)
+    for tag, req in reqs.items():                                        # whatever is left, request by request (bucket 1)
+        steps += [[(tag, 1)]] * (req.length - fed[tag])
+    got = helpers.replay(runner, reqs, steps, poison=True)
+    assert all(r.done == r.length for r in reqs.values())
+    assert sorted(runner._graphs) == [1, 4, 8]
+    assert runner.graph_replays == sum(1 for step in steps if all(count == 1 for _tag, count in step))
+    _check(name, dtype, reqs, got)
+    assert runner.cache.groups[0].pool.free_count == 20
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=DTYPE_IDS)
+def test_replayed_graphs_over_a_long_context(dtype):
+    """A model whose context is longer than what one workgroup of the decode attention kernel takes
+    (4096 keys): a captured step is cut for the longest context there can be, so every replay goes
+    through the kernel that splits a row's keys and the one that merges the parts, with padding rows
+    that have no keys at all. A request is decoded across the 4096-key edge beside shorter ones."""
+    name = "G"
+    runner = _runner(name, dtype, n_pages=290, max_requests=3, graphs=True)
+    reqs = {"long": _request(name, "long", 1350, 4110), "mid": _request(name, "mid", 1351, 70),
+            "short": _request(name, "short", 1352, 21)}
+    steps = [[("long", 2500)], [("long", 1590), ("mid", 60)]]
+    steps += [[("long", 1), ("mid", 1)]] * 10                            # bucket 2: 4090 .. 4099
+    steps += [[("short", 12)]]
+    steps += [[("short", 1), ("long", 1)]] * 9                           # bucket 2, other rows
+    steps += [[("long", 1)]]                                             # bucket 1: the long one ends
+    got = helpers.replay(runner, reqs, steps)
+    assert sorted(runner._graphs) == [1, 2] and runner.graph_replays == 20
+    _check(name, dtype, reqs, got)
+
+
 @pytest.mark.parametrize("page_size", [1, 4, 64])
 def test_other_page_sizes(page_size):
     runner = _runner("A", torch.float32, n_pages=512 // page_size, page_size=page_size)
@@ -204,7 +255,7 @@ def test_trace_run_program(tmp_path, dtype):
         {"step": 1, "entries": [{"id": "a", "tokens": ids_a[18:48], "want": []},
                                 {"id": "b", "tokens": ids_b[:2], "want": [1]}], "end": []},
         {"step": 2, "entries": [{"id": "b", "tokens": ids_b[2:37], "want": [34]}], "end": ["b"]},
-        {"step": 3, "entries": [{"id": "a", "tokens": ids_a[48:49], "want": [0]}], "end": []},
+        {"step": 3, "entries": [{"id": "a", "tokens": ids_a[48:49], "want": []}], "end": []},
         {"step": 4, "entries": [{"id": "a", "tokens": ids_a[49:50], "want": [0]}], "end": ["a"]},
     ]
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
@@ -215,7 +266,7 @@ def test_trace_run_program(tmp_path, dtype):
         input="\n".join(json.dumps(l) for l in lines) + "\n", capture_output=True, text=True, timeout=300)
     assert done.returncode == 0, done.stderr
     assert [l for l in done.stdout.splitlines() if l.startswith("done")] == [f"done {i}" for i in range(5)]
-    assert not (out / "1.f32").exists() or True
+    assert sorted(f.name for f in out.iterdir()) == ["0.f32", "1.f32", "2.f32", "4.f32"]     # step 3 wanted nothing
     weights = helpers.stored_weights(helpers.model_dir(name))
     exp_a = plain.forward(cfg, weights, ids_a)
     exp_b = plain.forward(cfg, weights, ids_b)
@@ -228,7 +279,6 @@ def test_trace_run_program(tmp_path, dtype):
     helpers.assert_close(load(0, 2), exp_a[[0, 17]], tdtype, "step 0")
     helpers.assert_close(load(1, 1), exp_b[[1]], tdtype, "step 1")
     helpers.assert_close(load(2, 1), exp_b[[36]], tdtype, "step 2")
-    helpers.assert_close(load(3, 1), exp_a[[48]], tdtype, "step 3")
     helpers.assert_close(load(4, 1), exp_a[[49]], tdtype, "step 4")
 
 

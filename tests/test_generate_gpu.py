@@ -26,11 +26,14 @@ def _engine(name, dtype, **kw):
 
 
 def _assert_greedy(result_tokens, expected, margins, slack, what):
+    """For a path that must agree token by token (float32, where ``slack`` is far below any margin
+    the tests' prompts have)."""
+    assert len(result_tokens) == len(expected), what
     for i, (got, want) in enumerate(zip(result_tokens, expected)):
+        assert got == want or margins[i] < slack, \
+            f"{what}: token {i} is {got}, the plain implementation gives {want} (margin {margins[i]:.3g})"
         if got != want:
-            assert margins[i] < slack, f"{what}: token {i} is {got}, the plain implementation gives {want} (margin {margins[i]:.3g})"
-            return                                       # a near tie: later tokens follow another path
-    assert len(result_tokens) == len(expected)
+            return
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -43,7 +46,6 @@ def test_greedy_generation_matches_the_plain_implementation(name, dtype):
     weights = helpers.stored_weights(helpers.model_dir(name))
     prompts = [helpers.random_ids(900 + i, n, cfg["vocab_size"]) for i, n in enumerate([5, 17, 33, 70])]
     n_new = 16
-    expected = [plain.greedy_generate(cfg, weights, p, n_new) for p in prompts]
     slack = 1e-4 if dtype == "float32" else 5e-2
     for graphs, depth in ((False, 1), (True, 2), (False, 2)):
         engine = _engine(name, dtype, enable_graphs=graphs, pipeline_depth=depth)
@@ -53,9 +55,11 @@ def test_greedy_generation_matches_the_plain_implementation(name, dtype):
         finally:
             engine.shutdown_sync()
         assert (replays > 0) == graphs
-        for result, (tokens, margins) in zip(results, expected):
+        for prompt, result in zip(prompts, results):
             assert result.finish_reason == "length" and result.metrics.output_tokens == n_new
-            _assert_greedy(result.tokens, tokens, margins, slack, f"tiny {name} {dtype} graphs={graphs} depth={depth}")
+            assert len(result.tokens) == n_new
+            helpers.assert_greedy_follows(cfg, weights, prompt, result.tokens, slack,
+                                          f"tiny {name} {dtype} graphs={graphs} depth={depth}")
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -69,13 +73,14 @@ def test_generation_after_a_prefix_block(dtype):
     ids = helpers.random_ids(950, 11, cfg["vocab_size"])
     bos = weights["text.wte"][0].double().unsqueeze(0)
     prefix = torch.cat([bos, rows.double()])
-    tokens, margins = plain.greedy_generate(cfg, weights, ids, 12, prefix_embeds=prefix)
     engine = _engine(name, dtype)
     try:
         result = engine.generate_sync(ids, max_new_tokens=12, prefix_embeds=rows, prefix_ids=[0], stop_ids=())
     finally:
         engine.shutdown_sync()
-    _assert_greedy(result.tokens, tokens, margins, 1e-4 if dtype == "float32" else 5e-2, f"prefix {dtype}")
+    assert len(result.tokens) == 12
+    helpers.assert_greedy_follows(cfg, weights, ids, result.tokens, 1e-4 if dtype == "float32" else 5e-2,
+                                  f"prefix {dtype}", prefix_embeds=prefix)
 
 
 def test_sampling_is_reproducible_and_independent_of_the_batch():
@@ -146,6 +151,110 @@ def test_stop_ids_max_tokens_and_errors():
         assert engine.generate_sync(prompt, max_new_tokens=2, stop_ids=()).tokens == tokens[:2]
     finally:
         engine.shutdown_sync()
+
+
+@pytest.mark.parametrize("dtype,depth,graphs", [("float32", 1, False), ("bfloat16", 2, True)])
+def test_bad_requests_fail_alone_and_the_engine_goes_on(dtype, depth, graphs):
+    """Good and bad requests submitted together: an id beyond the vocabulary, an id of -1 with no
+    embedding behind it, the id that stands for "the pending token" inside the engine, embeddings
+    one column too wide. Each bad one raises for its caller only; the good ones give the plain
+    implementation's tokens; the engine serves a further request and every page and slot is back."""
+    name = "D"
+    cfg = helpers.flat_config(name)
+    weights = helpers.stored_weights(helpers.model_dir(name))
+    vocab, dim = cfg["vocab_size"], cfg["dim"]
+    good = [helpers.random_ids(1200 + i, n, vocab) for i, n in enumerate((21, 9, 30))]
+    slack = 1e-4 if dtype == "float32" else 5e-2
+    engine = _engine(name, dtype, pipeline_depth=depth, enable_graphs=graphs)
+    try:
+        futures = [
+            engine.submit_sync(good[0], max_new_tokens=8, stop_ids=()),
+            engine.submit_sync(good[1][:4] + [vocab] + good[1][4:], max_new_tokens=8, stop_ids=()),
+            engine.submit_sync(good[1][:4] + [-1] + good[1][4:], max_new_tokens=8, stop_ids=()),
+            engine.submit_sync([-2] + good[1], max_new_tokens=8, stop_ids=()),
+            engine.submit_sync(good[1], max_new_tokens=8, stop_ids=(), prefix_embeds=torch.zeros(5, dim + 1),
+                               prefix_ids=[0]),
+            engine.submit_sync(good[1], max_new_tokens=8, stop_ids=()),
+        ]
+        for bad in futures[1:5]:
+            with pytest.raises(ValueError):
+                bad.result(timeout=60)
+        for prompt, future in ((good[0], futures[0]), (good[1], futures[5])):
+            result = future.result(timeout=60)
+            assert len(result.tokens) == 8 and result.finish_reason == "length"
+            helpers.assert_greedy_follows(cfg, weights, prompt, result.tokens, slack, f"beside bad requests, {dtype}")
+        later = engine.generate_sync(good[2], max_new_tokens=6, stop_ids=())
+        helpers.assert_greedy_follows(cfg, weights, good[2], later.tokens, slack, f"after bad requests, {dtype}")
+        assert engine._fatal is None
+    finally:
+        engine.shutdown_sync()
+    cache = engine.runner.cache
+    cache.check()
+    assert cache.free_slots == cache.max_requests and not engine.runner.held
+    assert all(g.pool.free_count == g.pool.n_pages and g.pool.promised_unheld == 0 for g in cache.groups)
+
+
+@pytest.mark.parametrize("depth", [1, 2])
+def test_an_entry_the_step_function_refuses_fails_alone(depth):
+    """A request that got past the door (put into the queue by hand) with an id the step function
+    refuses: ``ModelRunner.step`` names the entry before it touches the cache, the scheduler fails
+    that request and runs the others of the step again without it."""
+    from kestrel_amd.engine.types import GenerationRequest, Sequence_
+
+    name = "A"
+    cfg = helpers.flat_config(name)
+    weights = helpers.stored_weights(helpers.model_dir(name))
+    prompts = [helpers.random_ids(1210 + i, n, cfg["vocab_size"]) for i, n in enumerate((13, 40, 7))]
+    engine = _engine(name, "float32", pipeline_depth=depth)
+    try:
+        sched, runner = engine.scheduler, engine.runner
+        engine.shutdown_sync()                      # the thread has ended: the scheduler is driven by hand
+        sched.enqueue_request(GenerationRequest(0, prompts[0], 6, stop_ids=()))
+        sched.advance()
+        sched.waiting.append(Sequence_(GenerationRequest(1, prompts[1][:20] + [cfg["vocab_size"] + 3] + prompts[1][20:],
+                                                         6, stop_ids=())))
+        sched.enqueue_request(GenerationRequest(2, prompts[2], 6, stop_ids=()))
+        results = {r.request_id: r for r in sched.run_until_done()}
+    finally:
+        engine.shutdown_sync()
+    assert results[1].finish_reason == "error" and "outside the vocabulary" in results[1].error
+    assert sched.failed_steps == 1
+    for i in (0, 2):
+        expected, margins = plain.greedy_generate(cfg, weights, prompts[i], 6)
+        _assert_greedy(results[i].tokens, expected, margins, 1e-4, f"request {i} beside a refused entry")
+    runner.cache.check()
+    assert runner.cache.free_slots == runner.cache.max_requests and not runner.held
+    assert all(g.pool.free_count == g.pool.n_pages and g.pool.promised_unheld == 0 for g in runner.cache.groups)
+
+
+@pytest.mark.parametrize("temperature", [0.0, 0.9])
+def test_a_request_resumed_with_its_generated_tokens_goes_on_as_before(temperature):
+    """``_generated_prefix`` (``kestrel/engine/core.py:556-597``): tokens generated before are fed
+    after the prompt, count against ``max_tokens`` and head the result. The draw of a token is keyed
+    by its index in the request, so a resumed request continues exactly as the unbroken one did."""
+    cfg = helpers.flat_config("B")
+    prompt = helpers.random_ids(1220, 23, cfg["vocab_size"])
+    engine = _engine("B", "float32")
+    try:
+        whole = engine.generate_sync(prompt, max_new_tokens=10, temperature=temperature, top_p=0.95, seed=5, stop_ids=(),
+                                     return_logprobs=True)
+
+        async def resume():
+            return await engine.generate(prompt, stop_ids=(), seed=5, settings={
+                "temperature": temperature, "top_p": 0.95, "max_tokens": 10, "_logprobs": True,
+                "_generated_prefix": {"tokens": whole.tokens[:4], "logprobs": whole.logprobs[:4]}})
+
+        resumed = asyncio.run(resume())
+        with pytest.raises(ValueError, match="shorter than max_new_tokens"):
+            engine.generate_sync(prompt, max_new_tokens=4, generated_prefix={"tokens": whole.tokens[:4]})
+        with pytest.raises(TypeError, match="unsupported key"):
+            engine.generate_sync(prompt, max_new_tokens=8, generated_prefix={"tokens": [1], "scores": [0.0]})
+    finally:
+        engine.shutdown_sync()
+    assert resumed.tokens == whole.tokens and resumed.finish_reason == "length"
+    assert resumed.metrics.output_tokens == 6 and resumed.metrics.input_tokens == len(prompt)
+    assert resumed.logprobs[:4] == whole.logprobs[:4]
+    assert max(abs(a - b) for a, b in zip(resumed.logprobs, whole.logprobs)) < 1e-4
 
 
 def test_a_request_too_large_for_the_cache_fails_alone():

@@ -479,8 +479,9 @@ def test_argmax_and_sampling():
         logits[2, 3] = logits[2, vocab - 1] = 50.0            # a tie: the first index wins
         out = torch.empty(5, dtype=torch.int32, device=DEV)
         core.argmax(logits, out)
-        assert out.tolist() == torch.argmax(logits.cpu(), dim=-1).tolist() or out[2].item() == 3
-        assert out[2].item() == 3
+        expected = torch.argmax(logits.cpu(), dim=-1).tolist()
+        expected[2] = 3                                       # whatever torch makes of the tie
+        assert out.tolist() == expected
     sampler = Sampler(torch.device(DEV), seed=5)
     logits = torch.tensor([[2.0, 1.0, 0.5, -1.0, -3.0, float("-inf")]] * 4000, device=DEV)
     # temperature -> 0 is argmax; top_p tiny keeps the best token only
@@ -660,8 +661,10 @@ def test_layernorm_prologue_skinny_linear(shape):
 @pytest.mark.parametrize("shape", [(4, 4, 64, 32), (6, 2, 128, 64), (8, 1, 64, 16), (2, 2, 16, 16), (4, 2, 48, 32), (4, 4, 80, 32),
                                    (2, 1, 112, 48), (2, 2, 160, 80), (1, 1, 256, 128)])
 def test_decode_attention_that_rotates_and_stores(shape):
-    """The decode kernel with rotary encoding and cache write fused in, against the rotary kernel
-    followed by the plain decode kernel: same outputs, same cache."""
+    """The decode kernel with rotary encoding and cache write fused in, against a float64
+    computation (the query and the new key rotated at the row's last position, the new key and value
+    behind the cached ones), and against the rotary kernel followed by the plain decode kernel: same
+    outputs, same cache."""
     from kestrel_amd.ops import core, fast
 
     h, hkv, hd, rot = shape
@@ -689,8 +692,24 @@ def test_decode_attention_that_rotates_and_stores(shape):
                                       h, hkv, hd, case.batch,
                                       fuse=(qkv[:, q_dim:q_dim + kv_dim], qkv[:, q_dim + kv_dim:], table, slots))
     _close(out_f, out_ref, bf)
+    # float64: rows of the fused q|k|v, rotated; keys and values that were cached before, then the new ones
+    table64 = plain.rotary_table(rot, 2048, 10000.0)
+    q64 = plain.apply_rotary(qkv[:, :q_dim].cpu().double().view(n, h, hd), positions.cpu(), table64)
+    k64 = plain.apply_rotary(qkv[:, q_dim:q_dim + kv_dim].cpu().double().view(n, hkv, hd), positions.cpu(), table64)
+    v64 = qkv[:, q_dim + kv_dim:].cpu().double().view(n, hkv, hd)
+    expected = torch.empty(n, h, hd, dtype=torch.float64)
+    for r, kv in enumerate(kv_lens):
+        for head in range(h):
+            g = head // (h // hkv)
+            keys = torch.cat([case.k[r][:kv - 1, g].double(), k64[r, g].to(bf).double().unsqueeze(0)])
+            vals = torch.cat([case.v[r][:kv - 1, g].double(), v64[r, g].unsqueeze(0)])
+            w = torch.softmax(keys @ q64[r, head] * hd ** -0.5, dim=0)
+            expected[r, head] = w @ vals
+    _close(out_f, expected.view(n, h * hd), bf)
     for r, kv in enumerate(kv_lens):
         page, off = int(slots[r]) // 16, int(slots[r]) % 16
+        _close(k_f[page, :, off, :], k64[r], bf)
+        assert torch.equal(v_f[page, :, :, off].cpu().double(), v64[r])
         assert torch.equal(k_f[page, :, off, :], k_ref[page, :, off, :])
         assert torch.equal(v_f[page, :, :, off], v_ref[page, :, :, off])
 

@@ -137,10 +137,21 @@ def _register_toys():
             self.w = tensors["w.weight"].to(device).float()
 
         def forward(self, h, batch, cache, residual):
-            # plain torch on the GPU: this toy shows the interfaces, not a kernel
+            # torch and the framework's plain linear on the GPU: this toy shows the interfaces, not a kernel
+            from kestrel_amd.ops.linear import linear
+
+            u = batch.workspace.get("toy.u", tuple(h.shape), torch.float32)
+            linear(h.float(), self.w, None, u)
+            if batch.decode_only:
+                # one token per row, nothing here looks at values on the host: this can be captured
+                # in a graph. Rows that pad the batch have slot -1, the state's spare last row.
+                slots = batch.row_slot.long()[batch.token_row.long()]
+                state = self.spec.decay * cache.state[slots] + u
+                cache.state[slots] = state
+                residual += state
+                return
             rows = batch.token_row.long()
             slots = batch.row_slot.long()
-            u = h.float() @ self.w.T
             for t in range(h.shape[0]):
                 slot = slots[rows[t]]
                 if slot < 0:
@@ -159,10 +170,17 @@ def _register_toys():
             self.t = {k: v.to(device).float() for k, v in tensors.items()}
 
         def forward(self, h, batch, residual):
+            from kestrel_amd.ops.linear import linear
+
             x = h.float()
-            choice = (x @ self.t["router.weight"].T).argmax(dim=-1)
-            both = torch.stack([x @ self.t["e0.weight"].T, x @ self.t["e1.weight"].T])
-            residual += both[choice, torch.arange(x.shape[0], device=x.device)]
+            n, d = x.shape
+            scores = batch.workspace.get("toy.router", (n, 2), torch.float32)     # fixed addresses: safe in a graph
+            both = batch.workspace.get("toy.experts", (2, n, d), torch.float32)
+            linear(x, self.t["router.weight"], None, scores)
+            linear(x, self.t["e0.weight"], None, both[0])
+            linear(x, self.t["e1.weight"], None, both[1])
+            second = (scores[:, 1] > scores[:, 0]).unsqueeze(1)                    # argmax of two, first wins a tie
+            residual += torch.where(second, both[1], both[0])
 
     class LearnedPosition(PositionEncoding):
         """Another position encoding: nothing to rotate, so no table."""
@@ -204,12 +222,9 @@ def _toy_reference(ids, w, decay, eps):
     return normed @ w["emb"].double().T          # tied head, no bias
 
 
-def test_toy_parts_build_and_step():
-    """A mixer with state, a routed feed-forward and another position encoding are registered
-    from here; a plan names a layer twice in its schedule; the generic decoder, the cache
-    manager and the step function run it in portions and match a plain computation."""
-    from kestrel_amd.cache import CacheManager
-    from kestrel_amd.engine.step import ModelRunner, StepEntry
+def _toy_model():
+    """The toy plan (a layer with a stateful mixer and a routed feed-forward, named twice around
+    an attention layer), its bound model and its weights."""
     from kestrel_amd.models import DecoderModel
     from kestrel_amd.parts import (AttentionSpec, DenseFeedForwardSpec, LayerSpec, ModelPlan, NormSpec, PositionSpec,
                                    ScheduleEntry)
@@ -242,6 +257,63 @@ def test_toy_parts_build_and_step():
         noise = torch.randn(spec.shape, generator=gen)
         weights[name] = (1 + 0.1 * noise) if spec.init == "gain" else 0.3 * noise
     model.bind(weights, torch.float32, DEV)
+    return model, weights, vocab, eps, decay
+
+
+def test_a_stateful_toy_mixer_is_stepped_once_per_replayed_step():
+    """The toy model with HIP graphs on: decode steps of two, then three live requests (buckets of
+    2 and 4, the second with a padding row) are replayed. A graph is captured and warmed up on
+    padding rows alone, so the state of a live request is advanced exactly once a step: every
+    replay's logits match the plain computation, with eager prompt steps between the replays."""
+    from kestrel_amd.cache import CacheManager
+    from kestrel_amd.engine.step import ModelRunner, StepEntry
+
+    model, weights, vocab, eps, decay = _toy_model()
+    cache = CacheManager(model.cache_needs(), 16, 12, 4, dtype=torch.float32, device=DEV)
+    runner = ModelRunner(model, cache, DEV, enable_graphs=True)
+    seqs = {name: helpers.random_ids(60 + i, n, vocab) for i, (name, n) in enumerate((("a", 30), ("b", 24), ("c", 19)))}
+    expected = {name: _toy_reference(ids, weights, decay, eps) for name, ids in seqs.items()}
+    slots, fed = {}, {}
+
+    def prompt(name, count):
+        slots[name] = runner.admit()
+        out = runner.step([StepEntry(slots[name], seqs[name][:count], want=[count - 1])]).clone()
+        fed[name] = count
+        helpers.assert_close(out[0], expected[name][count - 1], torch.float32, f"toy prompt {name}")
+
+    def decode(names, what):
+        entries = [StepEntry(slots[n], [seqs[n][fed[n]]], want=[0]) for n in names]
+        before = runner.graph_replays
+        out = runner.step(entries).clone()
+        assert runner.graph_replays == before + 1
+        for i, n in enumerate(names):
+            helpers.assert_close(out[i], expected[n][fed[n]], torch.float32, f"{what}: request {n} at {fed[n]}")
+            fed[n] += 1
+
+    prompt("a", 9)
+    prompt("b", 5)
+    for i in range(4):                       # bucket 2: the first of these steps captures the graph
+        decode(["a", "b"], f"bucket 2, replay {i}")
+    prompt("c", 7)                           # eager work between replays
+    for i in range(4):                       # bucket 4 with one padding row
+        decode(["c", "a", "b"], f"bucket 4, replay {i}")
+    runner.release(slots.pop("b"))
+    for i in range(3):                       # back to the first graph, other rows
+        decode(["a", "c"], f"bucket 2 again, replay {i}")
+    prompt("b", 11)                          # the freed slot is used again and starts from a zero state
+    for i in range(3):
+        decode(["b", "c", "a"], f"bucket 4 again, replay {i}")
+    assert sorted(runner._graphs) == [2, 4]
+
+
+def test_toy_parts_build_and_step():
+    """A mixer with state, a routed feed-forward and another position encoding are registered
+    from here; a plan names a layer twice in its schedule; the generic decoder, the cache
+    manager and the step function run it in portions and match a plain computation."""
+    from kestrel_amd.cache import CacheManager
+    from kestrel_amd.engine.step import ModelRunner, StepEntry
+
+    model, weights, vocab, eps, decay = _toy_model()
     needs = model.cache_needs()
     assert [n[0] is None for n in needs] == [True, False, True] and [n[1] is None for n in needs] == [False, True, False]
     cache = CacheManager(needs, 16, 8, 3, dtype=torch.float32, device=DEV)

@@ -14,13 +14,16 @@ from kestrel_amd.parts.specs import CacheSpec
 class FakeRunner:
     """Implements what the scheduler uses of ``ModelRunner``; records every step."""
 
-    def __init__(self, n_pages=16, page_size=4, max_requests=4, max_positions=64, vocab=32):
+    def __init__(self, n_pages=16, page_size=4, max_requests=4, max_positions=64, vocab=64):
         self.cache = CacheManager([(CacheSpec(1, 8, None), None, None)], page_size, n_pages, max_requests)
-        self.model = SimpleNamespace(plan=SimpleNamespace(max_positions=max_positions, vocab_size=vocab))
+        self.model = SimpleNamespace(plan=SimpleNamespace(max_positions=max_positions, vocab_size=vocab, dim=8))
         self.held = {}
         self.steps = []
         self.tokens = []
         self.vocab = vocab
+        self.refuse_token = None        # a step with this token in an entry is refused for that entry
+        self.break_at_step = None       # the step with this number fails as a whole
+        self.broken = []
 
     def admit(self, reserve_length=0, portion=1):
         slot = self.cache.admit(reserve_length, portion)
@@ -32,8 +35,16 @@ class FakeRunner:
         del self.held[slot]
 
     def step(self, entries):
+        from kestrel_amd.engine.step import StepRefused
+
         record = []
         wanted = 0
+        for i, e in enumerate(entries):            # refusals come before anything changes, as in ModelRunner
+            if self.refuse_token in list(e.tokens):
+                raise StepRefused(i, f"slot {e.slot}: token {self.refuse_token} is refused by this fake")
+        if self.break_at_step == len(self.steps) + len(self.broken):
+            self.broken.append([e.slot for e in entries])
+            raise RuntimeError("the device said no")
         for e in entries:
             start = self.held[e.slot] if e.start is None else e.start
             assert start == self.held[e.slot], "portions must follow each other"
@@ -206,6 +217,120 @@ def test_bad_requests_are_refused():
         sched.enqueue_request(_req(0, 64, 2))
 
 
+def test_what_the_step_function_would_refuse_is_refused_at_the_door():
+    sched, _ = _scheduler()
+    bad = [
+        (dict(prompt_ids=[1, 64]), "token id 64 outside the vocabulary"),
+        (dict(prompt_ids=[1, -1]), "token id -1 outside"),
+        (dict(prompt_ids=[-2, 3]), "token id -2 outside"),          # would otherwise read as "the pending token"
+        (dict(prompt_ids=[1], prefix_ids=[70], prefix_embeds=torch.zeros(2, 8)), "prefix_ids: token id 70"),
+        (dict(prompt_ids=[1], prefix_embeds=torch.zeros(2, 9)), "prefix_embeds"),
+        (dict(prompt_ids=[1], prefix_embeds=torch.zeros(2, 8, dtype=torch.int32)), "prefix_embeds"),
+        (dict(prompt_ids=[1], prefix_embeds=torch.zeros(16)), "prefix_embeds"),
+        (dict(prompt_ids=[1], suppressed_token_ids=(99,)), "suppressed_token_ids"),
+        (dict(prompt_ids=[1], suppress_next_token_ids=(-5,)), "suppress_next_token_ids"),
+        (dict(prompt_ids=[1], allowed_token_ids=(3, 64)), "allowed_token_ids"),
+        (dict(prompt_ids=[1.5, 2.0]), "integer token ids"),
+        (dict(prompt_ids=[[1, 2]]), "flat sequence"),
+    ]
+    for kwargs, message in bad:
+        with pytest.raises(ValueError, match=message):
+            sched.enqueue_request(GenerationRequest(0, max_new_tokens=2, **kwargs))
+    assert not sched.has_pending_work()
+
+
+@pytest.mark.parametrize("depth", [1, 2])
+def test_a_request_the_step_function_refuses_fails_alone(depth):
+    """Token 31 is inside the vocabulary, so the door lets it in; the (fake) step function refuses
+    the entry that holds it. The others of that step are planned again and finish as if it had
+    never been there."""
+    expected = {}
+    for with_bad in (False, True):
+        sched, runner = _scheduler(pipeline_depth=depth, budget=16, n_pages=32)
+        runner.refuse_token = 31
+        sched.enqueue_request(_req(0, 5, 4))
+        sched.advance()                                           # request 0 decodes when the bad one arrives
+        if with_bad:
+            sched.enqueue_request(GenerationRequest(1, [4, 31, 6], 3))
+        sched.enqueue_request(_req(2, 6, 3))
+        results = {r.request_id: r for r in sched.run_until_done()}
+        good = {i: (r.tokens, r.finish_reason) for i, r in results.items() if i != 1}
+        assert good == {0: ([10, 11, 12, 13], "length"), 2: ([10, 11, 12], "length")}
+        if with_bad:
+            assert results[1].finish_reason == "error" and "refused" in results[1].error
+            assert sched.failed_steps == 1
+        expected[with_bad] = good
+        runner.cache.check()
+        assert runner.cache.groups[0].pool.free_count == 32 and runner.cache.free_slots == 4 and not runner.held
+    assert expected[False] == expected[True]
+
+
+@pytest.mark.parametrize("depth", [1, 2])
+def test_a_step_that_breaks_takes_its_requests_only(depth):
+    """Step 2 raises something that names no entry: every request of that step fails, the ones
+    that wait are served afterwards, and every page and slot comes back."""
+    sched, runner = _scheduler(pipeline_depth=depth, budget=16, max_batch_size=2, n_pages=32)
+    runner.break_at_step = 2
+    for i in range(4):
+        sched.enqueue_request(_req(i, 5, 4))
+    results = {r.request_id: r for r in sched.run_until_done()}
+    assert len(runner.broken) == 1 and len(runner.broken[0]) == 2
+    failed = sorted(i for i, r in results.items() if r.finish_reason == "error")
+    assert failed == [0, 1] and all("the device said no" in results[i].error for i in failed)
+    assert all(results[i].tokens == [10, 11, 12, 13] and results[i].finish_reason == "length" for i in (2, 3))
+    runner.cache.check()
+    assert runner.cache.groups[0].pool.free_count == 32 and runner.cache.free_slots == 4 and not runner.held
+
+
+# ---------------------------------------------------------------------- tokens generated before
+def test_a_generated_prefix_is_fed_counted_and_returned():
+    """``kestrel/scheduler/types.py:215-263``; result and metrics as in the reference's
+    ``tests/scheduler/test_logprobs.py:177-202`` (tokens and logprobs keep the prefix at their head,
+    ``decode_tokens`` counts only what was decoded now)."""
+    from kestrel_amd.engine.types import GeneratedPrefix
+
+    sched, runner = _scheduler(budget=16)
+    request = GenerationRequest(7, [1], 4, return_logprobs=True, suppress_next_token_ids=(9,),
+                                generated_prefix=GeneratedPrefix((20, 21), (-0.1, -0.2)))
+    assert request.prompt_length == 1 and request.generated_prefix_length == 2 and request.prefill_length == 3
+    sched.enqueue_request(request)
+    (result,) = sched.run_until_done()
+    # fed: the prompt and the two old tokens in one portion; then one decode; 2 + 2 = max_new_tokens
+    assert runner.tokens[0] == [[1, 20, 21]] and [n for step in runner.steps for _s, _p, n, _w in step] == [3, 1]
+    assert result.tokens == [20, 21, 12, 13] and result.finish_reason == "length"
+    assert result.logprobs == [-0.1, -0.2, -1.5, -2.0]           # the fake sampler: -0.5 * (index + 1)
+    assert result.metrics.decode_tokens == 2 and result.metrics.prompt_tokens == 1
+    # the one-shot suppression applies to the first token after the prefix (index 2), not later
+    calls = sched.sampler.calls
+    assert calls[0]["indices"] == [2] and calls[0]["suppress"] == [(0, 9)] and calls[1]["suppress"] == []
+    assert runner.cache.groups[0].pool.free_count == 16
+
+
+def test_a_generated_prefix_is_checked():
+    from kestrel_amd.engine.types import GeneratedPrefix
+
+    with pytest.raises(ValueError, match="shorter"):
+        GenerationRequest(7, [1], 2, generated_prefix=GeneratedPrefix((10, 11)))
+    with pytest.raises(ValueError, match="same length"):
+        GenerationRequest(7, [1], 4, generated_prefix=GeneratedPrefix((10,), ()))
+    with pytest.raises(ValueError, match="return_logprobs"):
+        GenerationRequest(7, [1], 4, return_logprobs=True, generated_prefix=GeneratedPrefix((10,)))
+    sched, _ = _scheduler()
+    with pytest.raises(ValueError, match="generated_prefix.tokens: token id 70"):
+        sched.enqueue_request(GenerationRequest(7, [1], 4, generated_prefix=GeneratedPrefix((70,))))
+
+
+def test_a_generated_prefix_is_cut_like_a_prompt():
+    from kestrel_amd.engine.types import GeneratedPrefix
+
+    sched, runner = _scheduler(budget=4)
+    sched.enqueue_request(GenerationRequest(0, [1, 2, 3], 6, generated_prefix=GeneratedPrefix((20, 21, 22))))
+    (result,) = sched.run_until_done()
+    assert runner.tokens[0] == [[1, 2, 3, 20]] and runner.tokens[1] == [[21, 22]]
+    assert runner.steps[0][0][3] == [] and runner.steps[1][0][3] == [1]
+    assert result.tokens == [20, 21, 22, 13, 14, 15]
+
+
 def test_tokens_are_streamed_as_they_are_committed():
     sched, _ = _scheduler()
     seen = []
@@ -295,3 +420,17 @@ def test_masks_and_logprobs_reach_the_sampler(depth):
     assert results[1].logprobs is None and results[2].logprobs is None
     with pytest.raises(ValueError, match="allow-list"):
         sched.enqueue_request(_req(3, 2, 2, allowed_token_ids=()))
+
+
+# ---------------------------------------------------------------------- graph buckets
+def test_graph_buckets_follow_the_reference_rule():
+    """1, 2, 4, 8, every multiple of 16, and the largest batch itself: the reference's vectors
+    (``tests/test_decode_graph_manager.py:77-81``) and two sizes at which powers of two would differ."""
+    from kestrel_amd.engine.step import graph_buckets
+
+    assert graph_buckets(1) == [1]
+    assert graph_buckets(3) == [1, 2, 3]
+    assert graph_buckets(16) == [1, 2, 4, 8, 16]
+    assert graph_buckets(33) == [1, 2, 4, 8, 16, 32, 33]
+    assert graph_buckets(64) == [1, 2, 4, 8, 16, 32, 48, 64]
+    assert graph_buckets(100) == [1, 2, 4, 8, 16, 32, 48, 64, 80, 96, 100]
