@@ -21,6 +21,9 @@
 // row at hd 64) and values (2 lanes per channel row of a page). Waves merge through LDS, splits
 // through scratch memory in a second kernel, always in the same order.
 #include "ka_common.h"
+#include "ka_no_alloc.h"
+
+#include <mutex>
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
@@ -861,30 +864,30 @@ KA_API long ka_attention_decode_partial_floats(int n, int H, int hd, int splits)
     return (long)n * H * splits * (hd + 2);
 }
 
-KA_API int ka_attention_decode_bf16(const void* q, long q_row_stride, const void* k_cache, const void* v_cache,
-                                    const int* block_table, int max_pages, const int* token_row, const int* kv_lo,
-                                    const int* kv_hi, void* out, long out_row_stride, float scale, int n, int H,
-                                    int Hkv, int hd, int page_size, int splits, int waves, float* partial,
-                                    long partial_floats, const void* k_new,
-                                    const void* v_new, long new_stride, const float* table, int rot,
-                                    const int* slots, void* k_cache_w, void* v_cache_w, hipStream_t stream) {
-    if (check_common("ka_attention_decode_bf16", q, q_row_stride, out, out_row_stride, n, H, Hkv, hd, page_size,
+static int decode_launch(const char* who, const void* q, long q_row_stride, const void* k_cache, const void* v_cache,
+                         const int* block_table, int max_pages, const int* token_row, const int* kv_lo,
+                         const int* kv_hi, void* out, long out_row_stride, float scale, int n, int H,
+                         int Hkv, int hd, int page_size, int splits, int waves, float* partial,
+                         long partial_floats, const void* k_new,
+                         const void* v_new, long new_stride, const float* table, int rot,
+                         const int* slots, void* k_cache_w, void* v_cache_w, hipStream_t stream) {
+    if (check_common(who, q, q_row_stride, out, out_row_stride, n, H, Hkv, hd, page_size,
                      max_pages))
         return -1;
-    KA_CHECK(ka_attention_decode_supported(hd, page_size), "ka_attention_decode_bf16: head size %d not covered", hd);
-    KA_CHECK(splits >= 1 && splits <= 65535, "ka_attention_decode_bf16: bad split count %d", splits);
+    KA_CHECK(ka_attention_decode_supported(hd, page_size), "%s: head size %d not covered", who, hd);
+    KA_CHECK(splits >= 1 && splits <= 65535, "%s: bad split count %d", who, splits);
     if (splits > 1) {
-        KA_CHECK(partial, "ka_attention_decode_bf16: scratch missing");
+        KA_CHECK(partial, "%s: scratch missing", who);
         KA_CHECK(ka_attention_decode_partial_floats(n, H, hd, splits) <= partial_floats,
-                 "ka_attention_decode_bf16: scratch too small");
+                 "%s: scratch too small", who);
     }
-    KA_CHECK(waves == 4 || waves == 8 || waves == 16, "ka_attention_decode_bf16: waves must be 4, 8 or 16");
+    KA_CHECK(waves == 4 || waves == 8 || waves == 16, "%s: waves must be 4, 8 or 16", who);
     DecodeFuse fz = {};
     if (slots) {
         // the kernel rotates q and the new key itself and stores the token's key and value
-        KA_CHECK(k_new && v_new && k_cache_w && v_cache_w, "ka_attention_decode_bf16: fused mode needs the new key and value rows");
-        KA_CHECK(rot > 0 && rot <= hd && rot % 16 == 0 && table, "ka_attention_decode_bf16: fused mode needs a rotary width that is a multiple of 16 (got %d)", rot);
-        KA_CHECK(new_stride % 8 == 0 && (uintptr_t)k_new % 16 == 0 && (uintptr_t)v_new % 16 == 0, "ka_attention_decode_bf16: new key rows must be 16-byte aligned");
+        KA_CHECK(k_new && v_new && k_cache_w && v_cache_w, "%s: fused mode needs the new key and value rows", who);
+        KA_CHECK(rot > 0 && rot <= hd && rot % 16 == 0 && table, "%s: fused mode needs a rotary width that is a multiple of 16 (got %d)", who, rot);
+        KA_CHECK(new_stride % 8 == 0 && (uintptr_t)k_new % 16 == 0 && (uintptr_t)v_new % 16 == 0, "%s: new key rows must be 16-byte aligned", who);
         fz = DecodeFuse{(const bf16_t*)k_new, (const bf16_t*)v_new, new_stride, table, rot, slots, (bf16_t*)k_cache_w, (bf16_t*)v_cache_w};
     }
     if (hd > 64 && waves == 16) waves = 8;   // 16 waves leave 128 registers a lane: too few for a tile's loads (measured at head size 80: 26.4 against 23.6 us)
@@ -924,4 +927,71 @@ KA_API int ka_attention_decode_bf16(const void* q, long q_row_stride, const void
         KA_LAUNCH_CHECK();
     }
     return 0;
+}
+
+KA_API int ka_attention_decode_bf16(const void* q, long q_row_stride, const void* k_cache, const void* v_cache,
+                                    const int* block_table, int max_pages, const int* token_row, const int* kv_lo,
+                                    const int* kv_hi, void* out, long out_row_stride, float scale, int n, int H,
+                                    int Hkv, int hd, int page_size, int splits, int waves, float* partial,
+                                    long partial_floats, const void* k_new,
+                                    const void* v_new, long new_stride, const float* table, int rot,
+                                    const int* slots, void* k_cache_w, void* v_cache_w, hipStream_t stream) {
+    return decode_launch("ka_attention_decode_bf16", q, q_row_stride, k_cache, v_cache, block_table, max_pages, token_row,
+                         kv_lo, kv_hi, out, out_row_stride, scale, n, H, Hkv, hd, page_size, splits, waves, partial,
+                         partial_floats, k_new, v_new, new_stride, table, rot, slots, k_cache_w, v_cache_w, stream);
+}
+
+// ----------------------------------------------------------------------------------------------
+// the same without any memory from the caller beyond inputs and outputs (ka_no_alloc.h)
+// ----------------------------------------------------------------------------------------------
+// The partial results of the parts of a row's keys go through this array instead of a buffer the
+// caller allocated. Each GPU the library runs on holds its own copy until the process ends. In
+// host code the name stands for the symbol only; the address on a device is asked for once per
+// device (`static_scratch`) and only that pointer is ever handed to a kernel.
+static __device__ __align__(256) float scratch[KA_NO_ALLOC_SCRATCH_FLOATS];
+
+constexpr int KA_NO_ALLOC_MAX_DEVICES = 64;
+static float* g_scratch_ptr[KA_NO_ALLOC_MAX_DEVICES];
+static std::mutex g_scratch_lock;
+
+// The array's address on the current device, looked up at the first call on that device.
+static int static_scratch(float** ptr) {
+    int device = -1;
+    hipError_t e = hipGetDevice(&device);
+    KA_CHECK(e == hipSuccess, "ka_attention_decode_bf16_no_alloc: no current device: %s", hipGetErrorString(e));
+    KA_CHECK(device >= 0 && device < KA_NO_ALLOC_MAX_DEVICES, "ka_attention_decode_bf16_no_alloc: device %d beyond the %d this library keeps a scratch address for",
+             device, KA_NO_ALLOC_MAX_DEVICES);
+    std::lock_guard<std::mutex> hold(g_scratch_lock);
+    if (!g_scratch_ptr[device]) {
+        float* found = nullptr;
+        e = hipGetSymbolAddress((void**)&found, HIP_SYMBOL(scratch));
+        KA_CHECK(e == hipSuccess && found, "ka_attention_decode_bf16_no_alloc: cannot find the scratch array on device %d: %s", device,
+                 hipGetErrorString(e));
+        g_scratch_ptr[device] = found;
+    }
+    *ptr = g_scratch_ptr[device];
+    return 0;
+}
+
+KA_API int ka_attention_decode_bf16_no_alloc(const void* q, long q_row_stride, const void* k_cache, const void* v_cache,
+                                             const int* block_table, int max_pages, const int* token_row,
+                                             const int* kv_lo, const int* kv_hi, void* out, long out_row_stride,
+                                             float scale, int n, int H, int Hkv, int hd, int page_size, int splits,
+                                             int waves, const void* k_new, const void* v_new, long new_stride,
+                                             const float* table, int rot, const int* slots, void* k_cache_w,
+                                             void* v_cache_w, hipStream_t stream) {
+    const char* who = "ka_attention_decode_bf16_no_alloc";
+    KA_CHECK(n > 0 && H > 0 && hd > 0 && splits >= 1, "%s: bad sizes n=%d H=%d hd=%d splits=%d", who, n, H, hd, splits);
+    const long needed = splits > 1 ? ka_attention_decode_partial_floats(n, H, hd, splits) : 0;
+    KA_CHECK(needed <= KA_NO_ALLOC_SCRATCH_FLOATS,
+             "%s: %d tokens x %d heads x %d parts of the keys need %ld floats of scratch, the static array holds %ld "
+             "(fewer tokens a call, or ka_attention_decode_bf16 with a buffer of the caller's)",
+             who, n, H, splits, needed, (long)KA_NO_ALLOC_SCRATCH_FLOATS);
+    float* ptr = nullptr;
+    if (static_scratch(&ptr)) return -1;
+    // nothing in the array has to start at zero: every record that the merge reads was written by
+    // the kernel before it in this call (there are no counters or flags in it)
+    return decode_launch(who, q, q_row_stride, k_cache, v_cache, block_table, max_pages, token_row, kv_lo, kv_hi, out,
+                         out_row_stride, scale, n, H, Hkv, hd, page_size, splits, waves, ptr, KA_NO_ALLOC_SCRATCH_FLOATS,
+                         k_new, v_new, new_stride, table, rot, slots, k_cache_w, v_cache_w, stream);
 }

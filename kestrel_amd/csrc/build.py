@@ -30,7 +30,7 @@ LIBRARIES: Dict[str, List[str]] = {
     "core": ["ka_error.hip", "elementwise.hip", "gemm_generic.hip", "attention_generic.hip", "sampling.hip"],
     "fast": ["ka_error.hip", "gemm_bf16.hip", "gemv_bf16.hip", "attention_bf16.hip"],
 }
-HEADERS = ["ka_common.h", "ka_partials.h"]
+HEADERS = ["ka_common.h", "ka_partials.h", "ka_no_alloc.h"]
 
 HIPCC_FLAGS = [
     f"--offload-arch={ARCH}", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",
