@@ -189,8 +189,9 @@ def _as(w: Dict[str, Tensor], dtype) -> Dict[str, Tensor]:
 
 def forward(cfg: dict, weights: Dict[str, Tensor], ids: Sequence[int],
             prefix_embeds: Optional[Tensor] = None, block_ids: Optional[Sequence[int]] = None,
-            position_start: int = 0, dtype=torch.float64) -> Tensor:
-    """Logits ``[T, V]`` at every position of one sequence.
+            position_start: int = 0, dtype=torch.float64, rows: Optional[Sequence[int]] = None) -> Tensor:
+    """Logits ``[T, V]`` at every position of one sequence, or ``[len(rows), V]`` at the positions
+    ``rows`` (the rows are taken before the final norm and the head, ``runtime.py:2374-2379``).
 
     The sequence is ``prefix_embeds`` rows (given embeddings, used verbatim:
     ``runtime.py:2081-2115``) followed by the embeddings of ``ids``. ``block_ids`` has
@@ -215,6 +216,8 @@ def forward(cfg: dict, weights: Dict[str, Tensor], ids: Sequence[int],
     table = rotary_table(rotary_dim_of(cfg), position_start + total, float(cfg["rope_theta"]), dtype)
     for index in range(cfg["n_layers"]):
         x = block(x, w, index, cfg, positions, allowed, table)
+    if rows is not None:
+        x = x[torch.as_tensor(list(rows), dtype=torch.long)]
     return head(x, w, cfg)
 
 
