@@ -100,6 +100,49 @@ def test_sampling_is_reproducible_and_independent_of_the_batch():
     assert all(0 <= t < cfg["vocab_size"] for r in mixed for t in r.tokens)
 
 
+@pytest.mark.parametrize("depth,graphs", [(1, False), (2, True)])
+def test_sampled_generation_in_portions_beside_decodes_follows_the_plain_model(depth, graphs):
+    """Four requests, each a block of 17 positions (one id and 16 given embeddings, which see each
+    other both ways) and 3 to 40 ids, 24 tokens each at temperature 0.8 with a seed, under a token
+    budget of 24: the block goes in whole, the rest of a prompt in portions beside the decoded tokens
+    of the others. (A budget of 8 cannot hold the block, which may not be split; 24 is the nearest
+    that does.) Every token must be the one that the request's uniform number for that index picks,
+    by inversion in index order, from the plain implementation's softmax(logits / 0.8) after the
+    same earlier tokens."""
+    from kestrel_amd.ops import core
+    from kestrel_amd.sampling import mix_key
+
+    name, temperature, n_new, engine_seed = "B", 0.8, 24, 11
+    cfg = helpers.flat_config(name)
+    weights = helpers.stored_weights(helpers.model_dir(name))
+    bos = weights["text.wte"][0].double().unsqueeze(0)
+    requests = []
+    for i, n_ids in enumerate((3, 40, 11, 26)):
+        rows = torch.randn(cfg["prefix_attn"] - 1, cfg["dim"], generator=torch.Generator().manual_seed(40 + i))
+        requests.append((rows, helpers.random_ids(1230 + i, n_ids, cfg["vocab_size"]), 500 + i))
+    engine = _engine(name, "float32", max_num_batched_tokens=24, seed=engine_seed, pipeline_depth=depth,
+                     enable_graphs=graphs)
+    try:
+        futures = [engine.submit_sync(ids, max_new_tokens=n_new, temperature=temperature, top_p=1.0, seed=seed,
+                                      prefix_embeds=rows, prefix_ids=[0], stop_ids=()) for rows, ids, seed in requests]
+        results = [f.result(timeout=120) for f in futures]
+        steps = engine.scheduler.steps
+    finally:
+        engine.shutdown_sync()
+    assert steps < 4 * n_new, "the requests were decoded side by side"
+    for (rows, ids, seed), result in zip(requests, results):
+        assert len(result.tokens) == n_new and result.finish_reason == "length"
+        prefix = torch.cat([bos, rows.double()])
+        logits = plain.forward(cfg, weights, ids + result.tokens[:-1], prefix)
+        first = prefix.shape[0] + len(ids) - 1
+        for i, token in enumerate(result.tokens):
+            cdf = torch.cumsum(plain.nucleus_probs(logits[first + i], temperature, 1.0), dim=0)
+            u = core.uniform(mix_key(engine_seed, seed), i)
+            want = int(torch.searchsorted(cdf, torch.tensor(u, dtype=torch.float64), right=True))
+            assert token == want or abs(float(cdf[token] - cdf[want])) < 1e-4, \
+                f"request with seed {seed}, token {i}: {token}, the plain distribution and u = {u:.6f} give {want}"
+
+
 @pytest.mark.parametrize("depth", [1, 2])
 def test_masks_and_logprobs_through_the_entry_point(depth):
     """Greedy generation with the chosen tokens' log-probabilities, a token that may not come

@@ -421,10 +421,16 @@ def test_attention_decode_kernel(shape):
     _close(_run_attention(windowed, "fast", 0.25), windowed.reference(0.25), bf)
 
 
-def test_a_far_key_among_hundreds_is_found():
+EDGE_HEADS = [(4, 4, 64), (4, 2, 80), (2, 1, 128), (6, 3, 48), (4, 1, 16), (2, 2, 96), (2, 2, 256)]
+
+
+@pytest.mark.parametrize("heads", EDGE_HEADS)
+def test_a_far_key_among_hundreds_is_found(heads):
     """One query and one far key are scaled so that this key takes almost all the weight: a
-    kernel that loses it (a page's edge, a split's edge, a tile's edge) returns another value."""
-    h, hkv, hd = 4, 4, 64
+    kernel that loses it (a page's edge, a split's edge, a tile's edge) returns another value.
+    At every kind of head size the kernels treat differently (64 and below, no multiple of 32,
+    128, 256) and with grouped heads."""
+    h, hkv, hd = heads
     bf = torch.bfloat16
     for target in (0, 15, 16, 255, 256, 511, 777):
         case = PagedCase([900], [1], h, hkv, hd, 16, bf, seed=13)
@@ -447,11 +453,12 @@ def test_a_far_key_among_hundreds_is_found():
         _close(out[-1, :hd], prompt.v[0][target, 0].double(), bf)
 
 
-def test_a_windows_edge_is_kept():
+@pytest.mark.parametrize("heads", EDGE_HEADS)
+def test_a_windows_edge_is_kept(heads):
     """The key just outside a window lines up with the query far better than any other, the
     first key inside it second best: a kernel that lets the edge slip by one returns the wrong
     value. Edges on a page's first and last slot, on a tile's edge and in between."""
-    h, hkv, hd = 4, 4, 64
+    h, hkv, hd = heads
     bf = torch.bfloat16
     for window in (100, 101, 115, 132, 388, 389):
         for q_len in (1, 130):
