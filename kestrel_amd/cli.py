@@ -17,13 +17,14 @@ from typing import List
 
 
 def _add_runtime_options(parser: argparse.ArgumentParser) -> None:
-    parser.add_argument("--model-path", required=True, help="folder with config.json and model.safetensors")
+    parser.add_argument("--model-path", required=True, help="folder with config.json and model.safetensors (or a .pt checkpoint)")
     parser.add_argument("--model", default=None, help="architecture name (default: taken from config.json)")
     parser.add_argument("--device", default="cuda")
     parser.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     parser.add_argument("--max-batch-size", type=int, default=4)
     parser.add_argument("--page-size", type=int, default=16)
     parser.add_argument("--kv-cache-pages", type=int, default=None)
+    parser.add_argument("--kv-cache-bytes", type=int, default=None, help="size the cache pool by a byte budget instead")
     parser.add_argument("--max-num-batched-tokens", type=int, default=2048)
     parser.add_argument("--seed", type=int, default=0)
     parser.add_argument("--disable-graphs", action="store_true", help="do not replay decode steps as HIP graphs")
@@ -50,7 +51,8 @@ def _generate(args) -> int:
         prompts.extend([list(map(int, p)) for p in data])
     cfg = RuntimeConfig(model_path=args.model_path, model=args.model, device=args.device, dtype=args.dtype,
                         max_batch_size=args.max_batch_size, page_size=args.page_size,
-                        kv_cache_pages=args.kv_cache_pages, max_num_batched_tokens=args.max_num_batched_tokens,
+                        kv_cache_pages=args.kv_cache_pages, kv_cache_bytes=args.kv_cache_bytes,
+                        max_num_batched_tokens=args.max_num_batched_tokens,
                         seed=args.seed, enable_graphs=not args.disable_graphs, pipeline_depth=args.pipeline_depth)
     engine = InferenceEngine.create_sync(cfg)
     try:

@@ -34,8 +34,10 @@ class RuntimeConfig:
 
     ``model``: architecture name; ``None`` takes it from ``config.json``.
     ``max_batch_size``: most requests decoded together. ``page_size``: tokens per cache
-    page. ``kv_cache_pages``: pages of the pool; ``None`` sizes it from
-    ``kv_cache_tokens`` or, failing that, for ``max_batch_size`` full contexts.
+    page. The pool is sized by one of ``kv_cache_pages``, ``kv_cache_bytes`` (a byte budget as the
+    reference's ``KVMemoryPool`` takes, ``kestrel/kv_cache.py:52-86``) or ``kv_cache_tokens``; with
+    none of them, for ``max_batch_size`` full contexts. A pool that does not fit in the device's
+    free memory is refused at start with a ``MemoryError``.
     ``max_num_batched_tokens``: token budget of one step (prompt portions are cut to it).
     ``enable_graphs``: replay decode-only steps as captured HIP graphs.
     ``pipeline_depth``: 2 launches a step before the tokens of the one before have reached
@@ -50,6 +52,7 @@ class RuntimeConfig:
     page_size: int = 16
     kv_cache_pages: Optional[int] = None
     kv_cache_tokens: Optional[int] = None
+    kv_cache_bytes: Optional[int] = None
     max_num_batched_tokens: int = 2048
     enable_graphs: bool = True
     pipeline_depth: int = 2
@@ -67,6 +70,10 @@ class RuntimeConfig:
             raise ValueError("kv_cache_pages must be a positive integer")
         if self.kv_cache_tokens is not None and self.kv_cache_tokens <= 0:
             raise ValueError("kv_cache_tokens must be a positive integer")
+        if self.kv_cache_bytes is not None and self.kv_cache_bytes <= 0:
+            raise ValueError("kv_cache_bytes must be a positive integer")
+        if sum(v is not None for v in (self.kv_cache_pages, self.kv_cache_tokens, self.kv_cache_bytes)) > 1:
+            raise ValueError("give one of kv_cache_pages, kv_cache_tokens and kv_cache_bytes")
         if self.max_num_batched_tokens <= 0:
             raise ValueError("max_num_batched_tokens must be a positive integer")
         if self.pipeline_depth not in (1, 2):

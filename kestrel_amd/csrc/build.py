@@ -4,7 +4,9 @@ Each library is a group of ``.hip`` files linked into one shared object next to 
 sources (or, where that folder cannot be written, under a per-user temporary
 folder). ``load(name)`` loads what is built and compiles first only if nothing
 usable is there; ``build_all()`` always compiles. There is no fallback: a missing
-compiler with a missing library is an error.
+compiler with a missing library is an error, and so is a library that is older than
+its sources and cannot be rebuilt (``KESTREL_AMD_ALLOW_STALE=1`` loads it all the same,
+with a warning).
 """
 
 from __future__ import annotations
@@ -182,10 +184,16 @@ def load(name: str) -> ctypes.CDLL:
         if path is None or not fresh:
             try:
                 path = build(name)
-            except KernelBuildError:
+            except KernelBuildError as exc:
                 if path is None:
                     raise
-                _say(f"warning: {path.name} is older than its sources and could not be rebuilt; loading it as it is")
+                if os.environ.get("KESTREL_AMD_ALLOW_STALE") != "1":
+                    raise KernelBuildError(
+                        f"{path} is older than its sources and could not be rebuilt ({exc}); a stale library would run "
+                        f"other code than the sources say. Build it where hipcc is, or set KESTREL_AMD_ALLOW_STALE=1 "
+                        f"to load it as it is") from exc
+                _say(f"warning: {path.name} is older than its sources and could not be rebuilt; loading it as it is "
+                     f"(KESTREL_AMD_ALLOW_STALE=1)")
         try:
             lib = ctypes.CDLL(str(path))
         except OSError as exc:

@@ -201,10 +201,12 @@ KA_API int ka_layernorm(const float* x, const int* rows, const float* gamma, con
 }
 
 // ----------------------------------------------------------------------------
-// Rotary position encoding (non-interleaved halves of the first `rot` channels of
-// each head) applied in place to the q heads of a fused qkv row, and to the k heads
-// on their way into the paged cache together with v. The table row of position p is
-// [cos(p f_0..f_{rot/2-1}), sin(...)] in fp32; the rotation is computed in fp32.
+// Rotary position encoding of the first `rot` channels of each head, applied in place to
+// the q heads of a fused qkv row, and to the k heads on their way into the paged cache
+// together with v. The table row of position p is [cos(p f_0..f_{rot/2-1}), sin(...)] in
+// fp32; the rotation is computed in fp32. `interleaved` says which channels form the pair
+// that angle i turns: 0 = channel i with channel i + rot/2 (halves), 1 = channel 2i with
+// channel 2i + 1.
 //
 // qkv row: [H*hd q | Hkv*hd k | Hkv*hd v]. Key cache: [pages, Hkv, page_size, hd]; value cache:
 // [pages, Hkv, hd, page_size] (transposed inside the page, so that the MFMA attention kernels
@@ -217,7 +219,7 @@ __global__ void rope_cache_kernel(T* __restrict__ qkv, long row_stride,
                                   const int* __restrict__ positions, const int* __restrict__ slots,
                                   const float* __restrict__ table, T* __restrict__ k_cache,
                                   T* __restrict__ v_cache, int H, int Hkv, int hd, int rot,
-                                  int page_size, int rotate) {
+                                  int page_size, int rotate, int interleaved) {
     int t = blockIdx.x;
     T* row = qkv + (size_t)t * row_stride;
     int pos = positions[t];
@@ -228,10 +230,11 @@ __global__ void rope_cache_kernel(T* __restrict__ qkv, long row_stride,
         for (int idx = threadIdx.x; idx < H * half; idx += blockDim.x) {
             int h = idx / half, i = idx % half;
             T* p = row + h * hd;
-            float a = ka_to_float(p[i]), b = ka_to_float(p[i + half]);
+            const int ia = interleaved ? 2 * i : i, ib = interleaved ? 2 * i + 1 : i + half;
+            float a = ka_to_float(p[ia]), b = ka_to_float(p[ib]);
             float c = cs[i], s = cs[half + i];
-            p[i] = ka_from_float<T>(a * c - b * s);
-            p[i + half] = ka_from_float<T>(b * c + a * s);
+            p[ia] = ka_from_float<T>(a * c - b * s);
+            p[ib] = ka_from_float<T>(b * c + a * s);
         }
     }
     long slot = slots ? slots[t] : -1;
@@ -244,10 +247,11 @@ __global__ void rope_cache_kernel(T* __restrict__ qkv, long row_stride,
         size_t dst = (((size_t)page * Hkv + h) * page_size + off) * hd + d;
         float kv = ka_to_float(krow[idx]);
         if (rotate && d < rot) {
-            int i = d < half ? d : d - half;
-            float a = ka_to_float(krow[h * hd + i]), b = ka_to_float(krow[h * hd + i + half]);
+            const int i = interleaved ? d / 2 : (d < half ? d : d - half);
+            const int ia = interleaved ? 2 * i : i, ib = interleaved ? 2 * i + 1 : i + half;
+            float a = ka_to_float(krow[h * hd + ia]), b = ka_to_float(krow[h * hd + ib]);
             float c = cs[i], s = cs[half + i];
-            kv = d < half ? a * c - b * s : b * c + a * s;
+            kv = d == ia ? a * c - b * s : b * c + a * s;
         }
         k_cache[dst] = ka_from_float<T>(kv);
         size_t vdst = (((size_t)page * Hkv + h) * hd + d) * page_size + off;
@@ -258,8 +262,9 @@ __global__ void rope_cache_kernel(T* __restrict__ qkv, long row_stride,
 KA_API int ka_rope_cache(void* qkv, int dtype, long row_stride, const int* positions,
                          const int* slots, const float* table, int table_rows, void* k_cache,
                          void* v_cache, int n, int H, int Hkv, int hd, int rot, int page_size,
-                         hipStream_t stream) {
+                         int interleaved, hipStream_t stream) {
     KA_CHECK(n >= 0 && H > 0 && Hkv > 0 && hd > 0, "ka_rope_cache: bad sizes");
+    KA_CHECK(interleaved == 0 || interleaved == 1, "ka_rope_cache: pairing must be 0 (halves) or 1 (interleaved)");
     KA_CHECK(rot >= 0 && rot <= hd && rot % 2 == 0, "ka_rope_cache: rotary dim %d must be even and <= head dim %d", rot, hd);
     KA_CHECK(row_stride >= (long)(H + 2 * Hkv) * hd, "ka_rope_cache: row stride %ld too small", row_stride);
     KA_CHECK(page_size > 0, "ka_rope_cache: page size %d", page_size);
@@ -269,10 +274,10 @@ KA_API int ka_rope_cache(void* qkv, int dtype, long row_stride, const int* posit
     int rotate = rot > 0;
     if (dtype == KA_F32)
         hipLaunchKernelGGL(rope_cache_kernel<float>, grid, block, 0, stream, (float*)qkv, row_stride, positions, slots,
-                           table, (float*)k_cache, (float*)v_cache, H, Hkv, hd, rot, page_size, rotate);
+                           table, (float*)k_cache, (float*)v_cache, H, Hkv, hd, rot, page_size, rotate, interleaved);
     else if (dtype == KA_BF16)
         hipLaunchKernelGGL(rope_cache_kernel<bf16_t>, grid, block, 0, stream, (bf16_t*)qkv, row_stride, positions, slots,
-                           table, (bf16_t*)k_cache, (bf16_t*)v_cache, H, Hkv, hd, rot, page_size, rotate);
+                           table, (bf16_t*)k_cache, (bf16_t*)v_cache, H, Hkv, hd, rot, page_size, rotate, interleaved);
     else
         KA_CHECK(false, "ka_rope_cache: unsupported dtype %d", dtype);
     KA_LAUNCH_CHECK();

@@ -94,6 +94,30 @@ def _generated_prefix(raw) -> GeneratedPrefix:
     return GeneratedPrefix(tokens, logprobs)
 
 
+def pool_pages(cfg: RuntimeConfig, bytes_per_page: int, max_seq: int, free_bytes: Optional[int]) -> int:
+    """Pages of the cache pool (each group of layers gets that many), from the one knob that is set:
+    pages, a byte budget (``kestrel/kv_cache.py:52-136``), tokens, or by default ``max_batch_size``
+    full contexts. ``bytes_per_page``: what a page costs over all layers. ``free_bytes``: what the
+    device has free (``None``: not checked); a pool beyond it is refused here, before anything is
+    allocated, instead of failing somewhere inside the allocation."""
+    if cfg.kv_cache_pages is not None:
+        n_pages = cfg.kv_cache_pages
+    elif cfg.kv_cache_bytes is not None:
+        n_pages = cfg.kv_cache_bytes // max(bytes_per_page, 1)
+        if n_pages < 1:
+            raise MemoryError(f"kv_cache_bytes={cfg.kv_cache_bytes} holds less than one page of {bytes_per_page} bytes")
+    elif cfg.kv_cache_tokens is not None:
+        n_pages = -(-cfg.kv_cache_tokens // cfg.page_size)
+    else:
+        n_pages = cfg.max_batch_size * -(-max_seq // cfg.page_size)
+    needed = n_pages * bytes_per_page
+    if free_bytes is not None and needed > free_bytes:
+        gib = float(1 << 30)
+        raise MemoryError(f"the cache pool of {n_pages} pages needs {needed / gib:.1f} GiB, the device has "
+                          f"{free_bytes / gib:.1f} GiB free: lower kv_cache_pages / kv_cache_bytes / max_batch_size")
+    return n_pages
+
+
 def _normalise(temperature, top_p):
     temperature = 0.0 if temperature is None else float(temperature)
     top_p = 1.0 if top_p is None else float(top_p)
@@ -152,12 +176,11 @@ class InferenceEngine:
         net = load_model(cfg.model_path, cfg.dtype, device, cfg.model)
         self.plan = net.plan
         max_seq = min(cfg.max_seq_len or net.plan.max_positions, net.plan.max_positions)
-        if cfg.kv_cache_pages is not None:
-            n_pages = cfg.kv_cache_pages
-        elif cfg.kv_cache_tokens is not None:
-            n_pages = -(-cfg.kv_cache_tokens // cfg.page_size)
-        else:
-            n_pages = cfg.max_batch_size * -(-max_seq // cfg.page_size)
+        from ..cache.manager import CacheManager
+
+        sizing = CacheManager(net.cache_needs(), cfg.page_size, 1, 1, dtype=net.dtype)      # books only: no device memory
+        free_bytes, _total = torch.cuda.mem_get_info(device)
+        n_pages = pool_pages(cfg, sizing.bytes_per_page(), max_seq, free_bytes)
         self.runner = make_runner(net, cfg.page_size, n_pages, cfg.max_batch_size,
                                   max_tokens_per_step=cfg.max_num_batched_tokens, enable_graphs=cfg.enable_graphs)
         self.scheduler = GenerationScheduler(self.runner, Sampler(device, cfg.seed, pending=self.runner.pending),

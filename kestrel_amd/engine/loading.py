@@ -10,7 +10,7 @@ import torch
 from ..cache.manager import CacheManager
 from ..config.registry import read_model_dir
 from ..models.decoder import DecoderModel
-from ..weights.loader import load_tensors
+from ..weights.loader import find_weights, load_tensors
 from .step import ModelRunner
 
 
@@ -22,11 +22,17 @@ def require_gpu(device: torch.device) -> None:
 
 
 def load_model(model_dir, dtype: torch.dtype, device: torch.device, model: Optional[str] = None) -> DecoderModel:
-    """The model of ``model_dir`` (class chosen by its config.json) with its weights bound."""
+    """The model of ``model_dir`` (class chosen by its config.json) with its weights bound.
+    ``model_dir`` is a folder with ``config.json`` and the weights, or the weights file itself
+    (safetensors or a ``.pt`` checkpoint) with ``config.json`` beside it."""
     require_gpu(device)
+    model_dir = Path(model_dir)
+    weights_file = None
+    if model_dir.is_file():
+        weights_file, model_dir = model_dir, model_dir.parent
     spec, _typed, plan = read_model_dir(model_dir, model)
     net = DecoderModel(plan)
-    tensors = load_tensors(Path(model_dir) / spec.filename, net.params(), dtype, device=device,
+    tensors = load_tensors(weights_file or find_weights(model_dir, spec.filename), net.params(), dtype, device=device,
                            prefixes=spec.tensor_prefixes, foreign_prefixes=spec.foreign_prefixes)
     net.bind(tensors, dtype, device)
     return net

@@ -25,7 +25,7 @@ _SIGNATURES = {
     "ka_layernorm": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_float, _c_void_p, _c_int, _c_int, _c_int,
                      _c_void_p],
     "ka_rope_cache": [_c_void_p, _c_int, _c_long, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p,
-                      _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
+                      _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
     "ka_linear_generic": [_c_void_p, _c_int, _c_long, _c_void_p, _c_int, _c_long, _c_void_p, _c_void_p, _c_int,
                           _c_long, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
     "ka_attention_generic": [_c_void_p, _c_int, _c_long, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p,
@@ -154,15 +154,21 @@ def layernorm(x: torch.Tensor, gamma: torch.Tensor, beta: Optional[torch.Tensor]
                               code_of(out.dtype), n, dim, stream_ptr()))
 
 
+ROTARY_PAIRINGS = {"halves": 0, "interleaved": 1}
+
+
 def rope_cache(qkv: torch.Tensor, positions: torch.Tensor, slots: Optional[torch.Tensor],
                table: Optional[torch.Tensor], k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor],
-               n_heads: int, n_kv_heads: int, head_dim: int, page_size: int) -> None:
+               n_heads: int, n_kv_heads: int, head_dim: int, page_size: int, pairing: str = "halves") -> None:
     """Rotate q in place and write rotated k and v into the paged cache.
 
-    ``qkv``: ``[n, (H + 2 Hkv) hd]``; ``table``: fp32 ``[positions, R]`` or ``None`` for no
-    rotation; key cache ``[pages, Hkv, page_size, hd]``, value cache ``[pages, Hkv, hd, page_size]``;
+    ``qkv``: ``[n, (H + 2 Hkv) hd]``; ``table``: fp32 ``[positions, R]`` (the cosines of the R/2
+    angles of a position, then their sines) or ``None`` for no rotation; ``pairing``: which
+    channels angle ``i`` turns, ``"halves"`` (``i`` and ``i + R/2``) or ``"interleaved"`` (``2i`` and
+    ``2i + 1``); key cache ``[pages, Hkv, page_size, hd]``, value cache ``[pages, Hkv, hd, page_size]``;
     ``slots`` ``None`` writes nothing.
     """
+    _need(pairing in ROTARY_PAIRINGS, f"rope_cache: pairing {pairing!r} is not one of {sorted(ROTARY_PAIRINGS)}")
     _dev(qkv, positions, slots, table, k_cache, v_cache)
     n = qkv.shape[0]
     _need(qkv.dim() == 2 and qkv.stride(1) == 1 and qkv.shape[1] == (n_heads + 2 * n_kv_heads) * head_dim,
@@ -180,7 +186,7 @@ def rope_cache(qkv: torch.Tensor, positions: torch.Tensor, slots: Optional[torch
         _check_caches("rope_cache", k_cache, v_cache, qkv.dtype, n_kv_heads, page_size, head_dim)
     _check(lib().ka_rope_cache(qkv.data_ptr(), code_of(qkv.dtype), qkv.stride(0), positions.data_ptr(), _ptr(slots),
                                _ptr(table), rows, _ptr(k_cache), _ptr(v_cache), n, n_heads, n_kv_heads, head_dim,
-                               rot, page_size, stream_ptr()))
+                               rot, page_size, ROTARY_PAIRINGS[pairing], stream_ptr()))
 
 
 def linear_generic(a: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], out: torch.Tensor,

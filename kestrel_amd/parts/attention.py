@@ -23,6 +23,11 @@ class PagedAttention(Mixer):
     ``hd ** -0.5`` unless given (``text.py:158-185``); the output projection adds into the
     residual (``text.py:187-193``). Which keys a token sees comes with the batch
     (``kv_hi``, and the group's ``kv_lo`` for a window).
+
+    Positions: the part built from ``spec.position`` is asked for a ``Rotation`` (a cos|sin table
+    and the pairing of channels); ``None`` means q and k go into attention as they are. Nothing
+    else is understood here: an encoding that needs more (several axes, a learned table added to
+    the input) is refused when the weights are bound, not silently turned the rotary way.
     """
 
     def __init__(self, spec: AttentionSpec) -> None:
@@ -37,6 +42,7 @@ class PagedAttention(Mixer):
         self.qkv_weight = self.qkv_bias = self.proj_weight = self.proj_bias = None
         self.dtype: Optional[torch.dtype] = None
         self._table = None
+        self._pairing = "halves"
 
     def params(self) -> Dict[str, ParamSpec]:
         spec = self.spec
@@ -50,13 +56,28 @@ class PagedAttention(Mixer):
         return CacheSpec(self.spec.n_kv_heads, self.spec.head_dim, self.spec.window)
 
     def bind(self, tensors, dtype, device) -> None:
+        spec = self.spec
         self.dtype = dtype
         self.qkv_weight = tensors["qkv.weight"].to(device).contiguous()
         self.proj_weight = tensors["proj.weight"].to(device).contiguous()
         if self.spec.bias:
             self.qkv_bias = tensors["qkv.bias"].to(device=device, dtype=torch.float32).contiguous()
             self.proj_bias = tensors["proj.bias"].to(device=device, dtype=torch.float32).contiguous()
-        self._table = self.position.table(device)
+        rotation = self.position.rotation(device)
+        if rotation is None and callable(getattr(self.position, "table", None)) and self.position.table(device) is not None:
+            raise ValueError(f"the position encoding {getattr(spec.position, 'kind', '?')!r} holds a table but offers no "
+                             f"rotation(): attention would not know which channels to pair")
+        if rotation is not None:
+            table = rotation.table
+            if rotation.pairing not in core.ROTARY_PAIRINGS:
+                raise ValueError(f"attention cannot apply a rotation with pairing {rotation.pairing!r}; known: "
+                                 f"{', '.join(sorted(core.ROTARY_PAIRINGS))}")
+            if table.dtype != torch.float32 or table.dim() != 2 or table.shape[1] % 2 or table.shape[1] > self.spec.head_dim:
+                raise ValueError(f"a rotation's table must be fp32 [positions, R] with R even and at most the head size "
+                                 f"{self.spec.head_dim}, got {tuple(table.shape)} {table.dtype}")
+            self._table, self._pairing = table.to(device).contiguous(), rotation.pairing
+        else:
+            self._table, self._pairing = None, "halves"
 
     # The three stages are also offered one by one, so that a block may fuse the first with its
     # norm and the last with its feed-forward (see ``Mixer.input_projection``).
@@ -72,7 +93,8 @@ class PagedAttention(Mixer):
         n = qkv.shape[0]
         group = batch.groups[cache.group]
         out = batch.workspace.get("attn.out", (n, self.q_dim), self.dtype)
-        if qkv.dtype == torch.bfloat16 and batch.decode_only and cache.writes and self._table is not None:
+        halves = self._pairing == "halves"          # the MFMA-path kernels turn halves; the generic one any pairing
+        if qkv.dtype == torch.bfloat16 and batch.decode_only and cache.writes and self._table is not None and halves:
             # one token per row: the decode kernel rotates q and k and stores k and v itself
             from ..ops import fast
             k_new = qkv[:, self.q_dim:self.q_dim + self.kv_dim]
@@ -83,13 +105,13 @@ class PagedAttention(Mixer):
                 return out
         slots = group.slots if cache.writes else None
         done = False
-        if qkv.dtype == torch.bfloat16:
+        if qkv.dtype == torch.bfloat16 and halves:
             from ..ops import fast
             done = fast.rope_cache_bf16(qkv, batch.positions, slots, self._table, cache.k, cache.v, spec.n_heads,
                                         spec.n_kv_heads, spec.head_dim, group.page_size)
         if not done:
             core.rope_cache(qkv, batch.positions, slots, self._table, cache.k, cache.v, spec.n_heads, spec.n_kv_heads,
-                            spec.head_dim, group.page_size)
+                            spec.head_dim, group.page_size, self._pairing)
         paged_attention(qkv, cache.k, cache.v, group.block_table, batch.token_row, group.kv_lo, batch.kv_hi, out,
                         self.scale, spec.n_heads, spec.n_kv_heads, spec.head_dim, batch)
         return out

@@ -39,10 +39,26 @@ class Norm(Part):
         raise NotImplementedError
 
 
-class PositionEncoding(Part):
-    """Holds what a mixer needs to encode positions (for rotary: the angle table)."""
+@dataclass(frozen=True)
+class Rotation:
+    """A rotary encoding as the attention mixer and its kernels take it.
 
-    def table(self, device: torch.device) -> Optional[torch.Tensor]:
+    ``table``: fp32 ``[positions, R]``, row ``p`` = the cosines of the ``R / 2`` angles of position
+    ``p``, then their sines; the first ``R`` channels of every query and key head are turned.
+    ``pairing``: which two channels angle ``i`` turns: ``"halves"`` = ``i`` and ``i + R / 2``,
+    ``"interleaved"`` = ``2 i`` and ``2 i + 1``.
+    """
+
+    table: torch.Tensor
+    pairing: str = "halves"
+
+
+class PositionEncoding(Part):
+    """What a mixer needs to encode positions. An encoding that turns pairs of channels by angles
+    that grow with the position offers ``rotation``; one that offers nothing is applied nowhere
+    inside attention (order then comes from elsewhere, or from nowhere)."""
+
+    def rotation(self, device: torch.device) -> Optional[Rotation]:
         return None
 
 

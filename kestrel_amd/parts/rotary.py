@@ -6,7 +6,7 @@ from typing import Optional
 
 import torch
 
-from .base import PositionEncoding, register_position
+from .base import PositionEncoding, Rotation, register_position
 from .specs import PositionSpec
 
 
@@ -25,6 +25,10 @@ class NeoxRotary(PositionEncoding):
         if spec.rotary_dim and spec.max_positions <= 0:
             raise ValueError("a rotary encoding needs max_positions")
         self._table: Optional[torch.Tensor] = None
+
+    def rotation(self, device: torch.device) -> Optional[Rotation]:
+        table = self.table(device)
+        return None if table is None else Rotation(table, "halves")
 
     def table(self, device: torch.device) -> Optional[torch.Tensor]:
         spec = self.spec

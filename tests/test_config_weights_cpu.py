@@ -95,9 +95,29 @@ def test_runtime_config_checks():
     cfg = RuntimeConfig(model_path="x", dtype="float32", kv_cache_pages=8)
     assert cfg.dtype == torch.float32 and cfg.page_size == 16
     for bad in (dict(kv_cache_pages=0), dict(max_batch_size=0), dict(dtype="float16"), dict(device="cpu"),
-                dict(page_size=0), dict(max_num_batched_tokens=0)):
+                dict(page_size=0), dict(max_num_batched_tokens=0), dict(kv_cache_bytes=0),
+                dict(kv_cache_bytes=1 << 30, kv_cache_pages=8), dict(kv_cache_tokens=64, kv_cache_pages=8)):
         with pytest.raises(ValueError):
             RuntimeConfig(model_path="x", **bad)
+
+
+def test_the_cache_pool_is_sized_by_pages_tokens_or_bytes():
+    """``kv_cache_pages`` or ``kv_cache_bytes`` (``kestrel/kv_cache.py:52-136``: a byte budget, and
+    ``MemoryError`` beyond it), or tokens; the default is ``max_batch_size`` full contexts. A pool that
+    does not fit in what the device has free is refused before anything is allocated."""
+    from kestrel_amd.engine.engine import pool_pages
+
+    per_page = 3 * 1024 * 1024          # Moondream 2: 16 tokens x 196,608 bytes
+    assert pool_pages(RuntimeConfig(model_path="x", kv_cache_pages=40), per_page, 2048, None) == 40
+    assert pool_pages(RuntimeConfig(model_path="x", kv_cache_tokens=1000), per_page, 2048, None) == 63
+    assert pool_pages(RuntimeConfig(model_path="x", kv_cache_bytes=60 * 10 ** 9), per_page, 2048, None) == 19073
+    assert pool_pages(RuntimeConfig(model_path="x", max_batch_size=4), per_page, 2048, None) == 4 * 128
+    with pytest.raises(MemoryError, match="holds less than one page"):
+        pool_pages(RuntimeConfig(model_path="x", kv_cache_bytes=1000), per_page, 2048, None)
+    # 512 pages of 3 MiB do not fit in 1 GiB free
+    with pytest.raises(MemoryError, match="1.5 GiB.*1.0 GiB free"):
+        pool_pages(RuntimeConfig(model_path="x", max_batch_size=4), per_page, 2048, 1 << 30)
+    assert pool_pages(RuntimeConfig(model_path="x", max_batch_size=4), per_page, 2048, 4 << 30) == 512
 
 
 def test_random_model_folder_roundtrip(tmp_path):
@@ -170,6 +190,46 @@ def test_loader_reports_everything_at_once(tmp_path):
     assert "missing (2)" in text and "unexpected (2)" in text and "stored [8, 8], the model needs [256, 64]" in text
 
 
+def test_loader_reads_pt_checkpoints_with_the_same_report(tmp_path):
+    """A ``.pt`` file of tensors goes through the weights-only, memory-mapped loader
+    (``kestrel/models/moondream/weights.py:560-566``) and the same checks as safetensors."""
+    from kestrel_amd.weights.loader import find_weights
+
+    spec, params = _params()
+    stored = load_file(helpers.model_dir("A") + "/model.safetensors")
+    good = {"model." + k.replace("text.blocks", "text._orig_mod.blocks"): v for k, v in stored.items()}
+    torch.save(good, str(tmp_path / "model.pt"))
+    assert find_weights(tmp_path, "model.safetensors") == tmp_path / "model.pt"
+    got = load_tensors(tmp_path / "model.pt", params, torch.float32, prefixes=spec.tensor_prefixes)
+    want = load_tensors(helpers.model_dir("A") + "/model.safetensors", params, torch.float32, prefixes=spec.tensor_prefixes)
+    assert set(got) == set(want) and all(torch.equal(got[k], want[k]) for k in want)
+    bad = dict(stored)
+    del bad["text.lm_head.bias"]
+    bad["text.wte"] = torch.zeros(5, 5)
+    bad["stray"] = torch.zeros(1)
+    torch.save(bad, str(tmp_path / "bad.pt"))
+    with pytest.raises(WeightsError) as info:
+        load_tensors(tmp_path / "bad.pt", params, torch.bfloat16, prefixes=spec.tensor_prefixes)
+    assert info.value.missing == ["text.lm_head.bias"] and info.value.unexpected == ["stray"]
+    assert "text.wte: stored [5, 5]" in info.value.mismatched[0]
+    # a file that is not a mapping of tensors, and one that would have to run code to be read
+    torch.save([1, 2, 3], str(tmp_path / "list.pt"))
+    with pytest.raises(ValueError, match="mapping from tensor names"):
+        load_tensors(tmp_path / "list.pt", params, torch.bfloat16)
+    import pickle
+
+    class Runs:
+        def __reduce__(self):
+            return (print, ("this must never be printed",))
+
+    with open(tmp_path / "evil.pt", "wb") as handle:
+        pickle.dump({"text.wte": Runs()}, handle)
+    with pytest.raises(ValueError, match="weights-only loader"):
+        load_tensors(tmp_path / "evil.pt", params, torch.bfloat16)
+    with pytest.raises(FileNotFoundError, match="holds no weights"):
+        find_weights(tmp_path / "nowhere", "model.safetensors")
+
+
 def test_loader_refuses_integer_weights(tmp_path):
     spec, params = _params()
     stored = load_file(helpers.model_dir("A") + "/model.safetensors")
@@ -187,3 +247,28 @@ def test_missing_files(tmp_path):
     spec, params = _params()
     with pytest.raises(FileNotFoundError):
         load_tensors(tmp_path / "model.safetensors", params, torch.float32)
+
+
+def test_a_stale_library_that_cannot_be_rebuilt_is_an_error(tmp_path, monkeypatch):
+    """A built library whose stamp does not match the sources must not run silently where there is
+    no compiler: loading it is an error unless the environment says otherwise."""
+    from kestrel_amd.csrc import build
+
+    stale = tmp_path / "libka_core.so"
+    stale.write_bytes(b"not a library")
+
+    def no_compiler(name, verbose=True):
+        raise build.KernelBuildError("hipcc not found")
+
+    monkeypatch.setattr(build, "_find_built", lambda name: (stale, False))
+    monkeypatch.setattr(build, "build", no_compiler)
+    monkeypatch.setattr(build, "_loaded", {})
+    monkeypatch.delenv("KESTREL_AMD_ALLOW_STALE", raising=False)
+    with pytest.raises(build.KernelBuildError, match="older than its sources"):
+        build.load("core")
+    monkeypatch.setenv("KESTREL_AMD_ALLOW_STALE", "1")
+    with pytest.raises(build.KernelBuildError, match="cannot load"):       # it is tried, and is no library
+        build.load("core")
+    monkeypatch.setattr(build, "_find_built", lambda name: (None, False))
+    with pytest.raises(build.KernelBuildError, match="hipcc not found"):
+        build.load("core")

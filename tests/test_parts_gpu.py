@@ -54,7 +54,9 @@ def test_rotary_table_part():
     table = part.table(DEV)
     assert table.dtype == torch.float32 and tuple(table.shape) == (77, 12)
     torch.testing.assert_close(table.cpu().double(), plain.rotary_table(12, 77, 1234.5), atol=2e-5, rtol=0)
-    assert build_part("position", PositionSpec("none")).table(DEV) is None
+    assert build_part("position", PositionSpec("none")).rotation(DEV) is None
+    rotation = part.rotation(DEV)
+    assert rotation.pairing == "halves" and rotation.table is table
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
@@ -106,6 +108,67 @@ def test_attention_part(shape, dtype):
     ref = plain.attention(hs.double(), wd, "p.", cfg, positions, plain.visibility(positions, None),
                           plain.rotary_table(rot, 64, 500.0))
     helpers.assert_close(torch.cat(outs), ref, dtype, f"attention part {shape}")
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+@pytest.mark.parametrize("shape", [(4, 2, 32, 16), (2, 2, 64, 64), (3, 1, 48, 20)])
+def test_another_position_encoding_in_the_attention_mixer(shape, dtype):
+    """A rotary encoding that pairs neighbouring channels (2i with 2i + 1), registered from here:
+    the attention mixer takes its ``Rotation`` and the kernels turn the pairs it names. Turning
+    neighbours equals turning halves after moving the even channels of the rotated part of every
+    query and key head to the front, and scores do not change when queries and keys are permuted
+    alike: the plain implementation with the rows of the q|k weights permuted that way is the
+    reference. Also: an encoding that holds a table but offers no rotation is refused."""
+    from kestrel_amd.cache import CacheManager
+    from kestrel_amd.engine.step import ModelRunner, StepEntry
+    from kestrel_amd.parts import AttentionSpec, PositionEncoding, PositionSpec, Rotation, build_part, register_position
+
+    class PairsRotary(PositionEncoding):
+        def rotation(self, device):
+            spec = self.spec
+            return Rotation(plain.rotary_table(spec.rotary_dim, spec.max_positions, spec.theta, torch.float32).to(device),
+                            "interleaved")
+
+    class TableOnly(PositionEncoding):
+        def table(self, device):
+            return torch.zeros(4, 8, device=device)
+
+    register_position("toy_rotary_pairs", PairsRotary)
+    register_position("toy_table_only", TableOnly)
+    h, hkv, hd, rot = shape
+    dim = 40
+    spec = AttentionSpec("attention", dim, h, hkv, hd, PositionSpec("toy_rotary_pairs", rot, 300.0, 64), bias=True)
+    part = build_part("mixer", spec)
+    w = _tensors(part, dtype, 5, std=0.08)
+    part.bind(w, dtype, DEV)
+    cache = CacheManager([(part.cache_spec(), None, None)], 16, 8, 2, dtype=dtype, device=DEV)
+    fake_model = SimpleNamespace(plan=SimpleNamespace(max_positions=64, vocab_size=10, dim=dim))
+    runner = ModelRunner(fake_model, cache, DEV)
+    slot = runner.admit()
+    total = 39
+    hs = torch.randn(total, dim, generator=torch.Generator().manual_seed(8)).to(torch.bfloat16)
+    outs = []
+    for lo, hi in ((0, 18), (18, 35), (35, 36), (36, 37), (37, 39)):
+        batch = runner.build_batch([StepEntry(slot, [1] * (hi - lo))])
+        residual = torch.zeros(hi - lo, dim, device=DEV)
+        part.forward(hs[lo:hi].to(dtype).to(DEV), batch, runner.layer_caches[0], residual)
+        runner.held[slot] = hi
+        outs.append(residual.cpu())
+    order = list(range(0, rot, 2)) + list(range(1, rot, 2)) + list(range(rot, hd))     # evens of the rotated part first
+    rows = [head * hd + c for head in range(h + hkv) for c in order] + list(range((h + hkv) * hd, (h + 2 * hkv) * hd))
+    wd = {"p.attn." + k: v.double() for k, v in w.items()}
+    wd["p.attn.qkv.weight"], wd["p.attn.qkv.bias"] = wd["p.attn.qkv.weight"][rows], wd["p.attn.qkv.bias"][rows]
+    cfg = {"n_heads": h, "n_kv_heads": hkv, "head_dim": hd}
+    positions = torch.arange(total)
+    ref = plain.attention(hs.double(), wd, "p.", cfg, positions, plain.visibility(positions, None),
+                          plain.rotary_table(rot, 64, 300.0))
+    helpers.assert_close(torch.cat(outs), ref, dtype, f"attention with paired rotary {shape}")
+    halves = plain.attention(hs.double(), {"p.attn." + k: v.double() for k, v in w.items()}, "p.", cfg, positions,
+                             plain.visibility(positions, None), plain.rotary_table(rot, 64, 300.0))
+    assert (halves - ref).abs().max() > 0.02, "the two pairings must differ on this input, or the test shows nothing"
+    with pytest.raises(ValueError, match="offers no rotation"):
+        bad = build_part("mixer", AttentionSpec("attention", dim, h, hkv, hd, PositionSpec("toy_table_only", rot, 300.0, 64)))
+        bad.bind(_tensors(bad, dtype, 5), dtype, DEV)
 
 
 # ------------------------------------------------------------------------------------------------
