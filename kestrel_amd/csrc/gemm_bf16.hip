@@ -138,7 +138,7 @@ gemm_bf16_kernel(const bf16_t* __restrict__ A, long lda, const bf16_t* __restric
                 for (int i = 0; i < 4; ++i) {
                     float x = acc[a][b][q * 4 + i];
                     if (bias && n + i < N) x += bias[n + i];
-                    if (act == 1) x = ka_gelu_tanh_fast(x);
+                    if (act) x = ka_activate_fast(act, x);
                     v[i] = x;
                 }
                 size_t o = (size_t)m * ldo + n;
@@ -353,7 +353,7 @@ gemm_dma_kernel(const bf16_t* __restrict__ A, long lda, const bf16_t* __restrict
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     float x = acc[a][b][q * 4 + i] + bv[i];
-                    if (act == 1) x = ka_gelu_tanh_fast(x);
+                    if (act) x = ka_activate_fast(act, x);
                     v[i] = x;
                 }
                 size_t o = (size_t)m * ldo + n;
@@ -435,7 +435,7 @@ KA_API int ka_linear_tiled_bf16(const void* A, long lda, const void* W, long ldw
     KA_CHECK(lda % 8 == 0 && ldw % 8 == 0 && lda >= K && ldw >= K, "ka_linear_tiled_bf16: row strides must be multiples of 8 and >= K");
     KA_CHECK(((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0), "ka_linear_tiled_bf16: operands must be 16-byte aligned");
     KA_CHECK(ldo >= N, "ka_linear_tiled_bf16: output stride too small");
-    KA_CHECK(act == 0 || act == 1, "ka_linear_tiled_bf16: unknown activation %d", act);
+    KA_CHECK(ka_act_known(act), "ka_linear_tiled_bf16: unknown activation %d", act);
     KA_CHECK(out_dtype == KA_F32 || out_dtype == KA_BF16, "ka_linear_tiled_bf16: bad output type");
     KA_CHECK(!(accumulate && out_dtype != KA_F32), "ka_linear_tiled_bf16: accumulate needs an fp32 output");
     KA_CHECK((uintptr_t)out % 16 == 0, "ka_linear_tiled_bf16: output must be 16-byte aligned");

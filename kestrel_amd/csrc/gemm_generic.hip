@@ -53,7 +53,7 @@ gemm_generic_kernel(const TA* __restrict__ A, long lda, const TW* __restrict__ W
             int n = n0 + tx * 4 + j;
             if (n >= N) continue;
             float v = acc[i][j] + (bias ? bias[n] : 0.f);
-            if (act == 1) v = ka_gelu_tanh(v);
+            if (act) v = ka_activate(act, v);
             size_t o = (size_t)m * ldo + n;
             if (accumulate) v += ka_to_float(out[o]);
             out[o] = ka_from_float<TOut>(v);
@@ -135,7 +135,7 @@ gemm_f32_kernel(const float* __restrict__ A, long lda, const float* __restrict__
             const int n = n0 + tx * 8 + j;
             if (n >= N) continue;
             float v = acc[i][j] + (bias ? bias[n] : 0.f);
-            if (act == 1) v = ka_gelu_tanh(v);
+            if (act) v = ka_activate(act, v);
             const size_t o = (size_t)m * ldo + n;
             out[o] = accumulate ? out[o] + v : v;
         }
@@ -181,7 +181,7 @@ gemv_f32_kernel(const float* __restrict__ A, long lda, const float* __restrict__
         for (int off = KA_WAVE / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, KA_WAVE);
         if (lane == 0) {
             v += bias ? bias[n] : 0.f;
-            if (act == 1) v = ka_gelu_tanh(v);
+            if (act) v = ka_activate(act, v);
             const size_t o = (size_t)m * ldo + n;
             out[o] = accumulate ? out[o] + v : v;
         }
@@ -204,7 +204,7 @@ KA_API int ka_linear_generic(const void* A, int a_dtype, long lda, const void* W
                              int M, int N, int K, int act, int accumulate, hipStream_t stream) {
     KA_CHECK(M >= 0 && N > 0 && K > 0, "ka_linear_generic: bad sizes M=%d N=%d K=%d", M, N, K);
     KA_CHECK(lda >= K && ldw >= K && ldo >= N, "ka_linear_generic: strides too small");
-    KA_CHECK(act == 0 || act == 1, "ka_linear_generic: unknown activation %d", act);
+    KA_CHECK(ka_act_known(act), "ka_linear_generic: unknown activation %d", act);
     KA_CHECK(!(accumulate && out_dtype != KA_F32), "ka_linear_generic: accumulate needs an fp32 output");
     KA_CHECK(ka_cdiv(M, GT) <= 65535, "ka_linear_generic: M=%d too large for one launch", M);
     if (M == 0) return 0;

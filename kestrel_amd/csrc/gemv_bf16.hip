@@ -127,9 +127,9 @@ __device__ __forceinline__ void sk_finish(const floatx4 (*red)[MB][KA_WAVE], con
         for (int w = 0; w < NW; ++w) s += red[w][mb][lane] + red[w][mb][lane + OTHER];
         const int m = mb * 16 + r;
         if (m >= M) continue;
-        if (tg.act == 1) {
+        if (tg.act) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) s[i] = ka_gelu_tanh_fast(s[i]);
+            for (int i = 0; i < 4; ++i) s[i] = ka_activate_fast(tg.act, s[i]);
         }
         const size_t o = (size_t)m * tg.ldo + n;
         if (whole) {
@@ -835,7 +835,7 @@ static int check_target(const char* who, const SkinnyTarget& t, int K) {
     KA_CHECK(t.W && t.out, "%s: weight or output missing", who);
     KA_CHECK(t.N > 0 && t.ldw % 8 == 0 && t.ldw >= K && (uintptr_t)t.W % 16 == 0, "%s: weight rows must be 16-byte aligned and >= K", who);
     KA_CHECK(t.ldo >= t.N, "%s: output stride too small", who);
-    KA_CHECK(t.act == 0 || t.act == 1, "%s: unknown activation %d", who, t.act);
+    KA_CHECK(ka_act_known(t.act), "%s: unknown activation %d", who, t.act);
     KA_CHECK(t.out_dtype == KA_F32 || t.out_dtype == KA_BF16, "%s: bad output type", who);
     KA_CHECK(!(t.accumulate && t.out_dtype != KA_F32), "%s: accumulate needs an fp32 output", who);
     return 0;

@@ -80,4 +80,31 @@ __device__ __forceinline__ float ka_gelu_tanh_fast(float x) {
     return x * (1.0f - __fdividef(1.0f, 1.0f + e));   // 0.5 x (1 + tanh) = x (1 - 1 / (1 + e))
 }
 
+// Activations a linear kernel can apply in its epilogue. One table for every kernel family: a
+// further activation is a code here, a case in each of the two functions below, and its name in
+// the table of the Python face (ops/linear.py).
+enum KaAct : int { KA_ACT_NONE = 0, KA_ACT_GELU_TANH = 1, KA_ACT_RELU = 2, KA_ACT_SILU = 3, KA_ACT_COUNT = 4 };
+
+static inline bool ka_act_known(int act) { return act >= 0 && act < KA_ACT_COUNT; }
+
+// Library-exact forms: the 32-bit path.
+__device__ __forceinline__ float ka_activate(int act, float x) {
+    switch (act) {
+        case KA_ACT_GELU_TANH: return ka_gelu_tanh(x);
+        case KA_ACT_RELU: return fmaxf(x, 0.f);
+        case KA_ACT_SILU: return x / (1.0f + expf(-x));
+        default: return x;
+    }
+}
+
+// On the hardware's exponential and reciprocal: the kernels that write bf16 activations.
+__device__ __forceinline__ float ka_activate_fast(int act, float x) {
+    switch (act) {
+        case KA_ACT_GELU_TANH: return ka_gelu_tanh_fast(x);
+        case KA_ACT_RELU: return fmaxf(x, 0.f);
+        case KA_ACT_SILU: return x * __fdividef(1.0f, 1.0f + __expf(-x));
+        default: return x;
+    }
+}
+
 static inline int ka_cdiv(long a, long b) { return (int)((a + b - 1) / b); }

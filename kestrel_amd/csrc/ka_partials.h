@@ -43,7 +43,7 @@ ka_partials_finish_kernel(const float* __restrict__ partial, int splits, const f
     }
     for (int i = 0; i < 4 && n + i < N; ++i) {
         float x = s[i] + (bias ? bias[n + i] : 0.f) + (bias2 ? bias2[n + i] : 0.f);
-        if (act == 1) x = ka_gelu_tanh_fast(x);
+        if (act) x = ka_activate_fast(act, x);
         const size_t o = (size_t)m * ldo + n + i;
         if (out_dtype == KA_F32) {
             float* op = reinterpret_cast<float*>(out) + o;

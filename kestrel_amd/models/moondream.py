@@ -52,7 +52,8 @@ class MoondreamTextConfig:
     head_dim: int
     rotary_dim: int
     layer_norm_eps: float
-    prefix_attn: int = 0
+    prefix_attn: int = 0        # declared by the reference and never read there (``config.py:32,268``): the mask follows
+                                # the block a request brings; kept as the length measurements and tests give that block
     bos_id: int = 0
     eos_id: int = 0
 
@@ -154,7 +155,7 @@ def build_plan(cfg: MoondreamTextConfig) -> ModelPlan:
         names={"embedding": "text.wte", "final_norm.weight": "text.post_ln.weight",
                "final_norm.bias": "text.post_ln.bias", "head.weight": "text.lm_head.weight",
                "head.bias": "text.lm_head.bias"},
-        eos_token_ids=(cfg.eos_id,), bos_token_id=cfg.bos_id, default_prefix_attn=cfg.prefix_attn,
+        eos_token_ids=(cfg.eos_id,), bos_token_id=cfg.bos_id,
     )
 
 

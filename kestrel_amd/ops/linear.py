@@ -8,8 +8,10 @@ import torch
 
 from . import core
 
-ACT_NONE, ACT_GELU_TANH = 0, 1
-_ACTIVATIONS = {None: ACT_NONE, "none": ACT_NONE, "gelu_tanh": ACT_GELU_TANH}
+# The codes of ``KaAct`` in csrc/ka_common.h, which is where a further activation is added (every
+# linear kernel applies them through the same two functions there).
+ACT_NONE, ACT_GELU_TANH, ACT_RELU, ACT_SILU = 0, 1, 2, 3
+_ACTIVATIONS = {None: ACT_NONE, "none": ACT_NONE, "gelu_tanh": ACT_GELU_TANH, "relu": ACT_RELU, "silu": ACT_SILU}
 
 # Rows up to which the weight-streaming kernel is used instead of the tiled MFMA one.
 SKINNY_MAX_ROWS = 64
@@ -17,7 +19,7 @@ SKINNY_MAX_ROWS = 64
 
 def activation_code(name: Optional[str]) -> int:
     if name not in _ACTIVATIONS:
-        raise ValueError(f"unknown activation {name!r}; known: gelu_tanh, none")
+        raise ValueError(f"unknown activation {name!r}; known: {', '.join(sorted(k for k in _ACTIVATIONS if k))}")
     return _ACTIVATIONS[name]
 
 

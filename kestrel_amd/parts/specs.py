@@ -137,7 +137,6 @@ class ModelPlan:
     names: Mapping[str, str]  # "embedding", "final_norm.weight", "head.weight", ... -> tensor name
     eos_token_ids: Tuple[int, ...] = ()
     bos_token_id: Optional[int] = None
-    default_prefix_attn: int = 0
 
     def describe(self) -> Dict[str, object]:
         return {"architecture": self.architecture, "layers": len(self.layers), "schedule": len(self.schedule),

@@ -87,6 +87,9 @@ def test_layernorm(dim, out_dtype):
     _close(out, F.layer_norm(x.double()[[8, 0, 3]], (dim,), gamma.double(), None, 1e-6), out_dtype, scale=4)
 
 
+_ACTIVATE = {0: lambda x: x, 1: plain.gelu_tanh, 2: F.relu, 3: F.silu}       # the codes of kestrel_amd.ops.linear
+
+
 def _linear_case(fn, m, n, k, a_dtype, w_dtype, out_dtype, act, accumulate, seed=0, lda=None):
     torch.manual_seed(seed)
     lda = lda or k
@@ -98,8 +101,7 @@ def _linear_case(fn, m, n, k, a_dtype, w_dtype, out_dtype, act, accumulate, seed
     out = start.clone()
     fn(a, w, bias, out, act=act, accumulate=accumulate)
     ref = a.double() @ w.double().T + bias.double()
-    if act:
-        ref = plain.gelu_tanh(ref)
+    ref = _ACTIVATE[act](ref)
     if accumulate:
         ref = ref + start.double()
     worst = torch.float32 if (a_dtype == w_dtype == out_dtype == torch.float32) else torch.bfloat16
@@ -119,6 +121,44 @@ def test_linear_generic(shape):
                 continue
             _linear_case(core.linear_generic, m, n, k, a_dtype, w_dtype, out_dtype, act, accumulate)
     _linear_case(core.linear_generic, m, n, k, f32, f32, f32, 0, False, lda=k + 5)      # strided rows
+
+
+@pytest.mark.parametrize("name,code", [("gelu_tanh", 1), ("relu", 2), ("silu", 3)])
+def test_every_activation_in_every_linear_kernel(name, code):
+    """The activations come from one table that every kernel family applies in its epilogue: the
+    plain fp32 kernel, the weight-streaming ones (persistent, split, wide, with the norm in front),
+    the tiled one and the one that adds up parts of K."""
+    from kestrel_amd.ops import core, fast
+    from kestrel_amd.ops.linear import activation_code, linear
+
+    assert activation_code(name) == code and activation_code(None) == 0
+    with pytest.raises(ValueError, match="unknown activation"):
+        activation_code("swish-ish")
+    bf, f32 = torch.bfloat16, torch.float32
+    _linear_case(core.linear_generic, 19, 77, 130, f32, f32, f32, code, False)
+    _linear_case(core.linear_generic, 200, 136, 264, f32, f32, f32, code, False)       # the tiled fp32 form
+
+    def through_dispatch(a, w, bias, out, act, accumulate):
+        linear(a, w, bias, out, act=act, accumulate=accumulate)
+
+    for m, n, k in ((8, 2048, 2048), (40, 4100, 2048), (200, 333, 520), (520, 2048, 8192), (2048, 512, 1024)):
+        _linear_case(through_dispatch, m, n, k, bf, bf, bf, code, False)
+    for mode in (0, 2):                                      # the split kernel, then the wide one wherever it can run
+        fast.set_skinny_persistent(0 if mode == 0 else 1)
+        fast.set_skinny_wide(mode)
+        try:
+            _linear_case(through_dispatch, 12, 515, 3000, bf, bf, bf, code, False)
+        finally:
+            fast.set_skinny_persistent(1)
+            fast.set_skinny_wide(1)
+    torch.manual_seed(6)
+    x = (torch.randn(5, 264) * 2).to(DEV)
+    gamma, beta = (1 + 0.1 * torch.randn(264)).to(DEV), (0.1 * torch.randn(264)).to(DEV)
+    w = (torch.randn(72, 264) / 16).bfloat16().to(DEV)
+    out = torch.empty(5, 72, dtype=bf, device=DEV)
+    assert fast.layernorm_linear(x, gamma, beta, 1e-5, w, None, out, code)
+    h = F.layer_norm(x.double(), (264,), gamma.double(), beta.double(), 1e-5).to(bf).double()
+    _close(out, _ACTIVATE[code](h @ w.double().T), bf, scale=2)
 
 
 @pytest.mark.parametrize("persistent,wide", [(1, 0), (0, 0), (1, 2)])
