@@ -18,7 +18,7 @@ per-request state keyed by the row id: ``kestrel/runtime/uncached_paged.py:178-1
 
 from __future__ import annotations
 
-from dataclasses import dataclass
+from dataclasses import dataclass, field
 from typing import Dict, List, Optional, Sequence, Tuple
 
 import torch
@@ -74,8 +74,17 @@ class _Group:
     spec: CacheSpec
     entries: List[int]                 # schedule entries that own a cache in this group
     pool: PagePool
-    k: Optional[torch.Tensor] = None   # [len(entries), pages, Hkv, page_size, hd]
-    v: Optional[torch.Tensor] = None   # [len(entries), pages, Hkv, hd, page_size]
+    # per tensor the specification names: [len(entries), pages, *shape of a page]; for attention
+    # "k" [.., Hkv, page_size, hd] and "v" [.., Hkv, hd, page_size]
+    tensors: Dict[str, torch.Tensor] = field(default_factory=dict)
+
+    @property
+    def k(self) -> Optional[torch.Tensor]:
+        return self.tensors.get("k")
+
+    @property
+    def v(self) -> Optional[torch.Tensor]:
+        return self.tensors.get("v")
 
 
 class _SlotState:
@@ -130,12 +139,10 @@ class CacheManager:
     # ------------------------------------------------------------------ device memory
     def _allocate_device(self) -> None:
         for group in self.groups:
-            spec = group.spec
-            # values are kept transposed inside a page: eight consecutive keys of one channel are 16 bytes
-            group.k = torch.zeros((len(group.entries), self.n_pages, spec.n_kv_heads, self.page_size, spec.head_dim),
-                                  dtype=self.dtype, device=self.device)
-            group.v = torch.zeros((len(group.entries), self.n_pages, spec.n_kv_heads, spec.head_dim, self.page_size),
-                                  dtype=self.dtype, device=self.device)
+            # the layout of a page is the specification's business, not the manager's
+            for name, shape in group.spec.page_tensors(self.page_size).items():
+                group.tensors[name] = torch.zeros((len(group.entries), self.n_pages, *shape), dtype=self.dtype,
+                                                  device=self.device)
         for entry, (_c, state_spec, _r) in enumerate(self.needs):
             if state_spec is not None:
                 # one row more than there are slots: the last one is a spare that rows without a
@@ -145,19 +152,24 @@ class CacheManager:
 
     def bytes_per_page(self) -> int:
         size = torch.empty((), dtype=self.dtype).element_size()
-        return sum(2 * len(g.entries) * g.spec.n_kv_heads * self.page_size * g.spec.head_dim * size
-                   for g in self.groups)
+        total = 0
+        for g in self.groups:
+            for shape in g.spec.page_tensors(self.page_size).values():
+                count = 1
+                for extent in shape:
+                    count *= int(extent)
+                total += len(g.entries) * count * size
+        return total
 
     def layer_caches(self) -> List[LayerCache]:
         """One ``LayerCache`` per schedule entry."""
         out = []
         for entry, (cache_spec, _state, reads) in enumerate(self.needs):
             g = self._entry_group[entry]
-            k = v = None
-            if g is not None and self.groups[g].k is not None:
-                k = self.groups[g].k[self._entry_index[entry]]
-                v = self.groups[g].v[self._entry_index[entry]]
-            out.append(LayerCache(group=g, k=k, v=v, writes=reads is None, state=self.states[entry]))
+            tensors = {}
+            if g is not None:
+                tensors = {name: t[self._entry_index[entry]] for name, t in self.groups[g].tensors.items()}
+            out.append(LayerCache(group=g, tensors=tensors, writes=reads is None, state=self.states[entry]))
         return out
 
     # ------------------------------------------------------------------ sizes

@@ -11,7 +11,7 @@ name that its specification carries.
 
 from __future__ import annotations
 
-from dataclasses import dataclass
+from dataclasses import dataclass, field
 from typing import Callable, Dict, Optional
 
 import torch
@@ -67,19 +67,27 @@ class LayerCache:
     """What one run of a layer may touch of the cache manager's memory.
 
     ``group``: key into ``StepBatch.groups`` (block table, slots, window start) or ``None``
-    if the mixer keeps no keys and values; ``k``: ``[pages, Hkv, page_size, hd]``, ``v``:
-    ``[pages, Hkv, hd, page_size]``;
-    ``writes``: ``False`` when this run reads the cache of another run; ``state``:
+    if the mixer keeps nothing per token; ``tensors``: the paged tensors its cache
+    specification named, each ``[pages, *shape of a page]`` (for attention ``k``:
+    ``[pages, Hkv, page_size, hd]`` and ``v``: ``[pages, Hkv, hd, page_size]``, also reachable as
+    ``.k`` and ``.v``); ``writes``: ``False`` when this run reads the cache of another run; ``state``:
     ``[slots + 1, *shape]`` per-request state, indexed by ``StepBatch.row_slot``; its last row is
     a spare for rows without a request (slot -1: what index -1 means to torch), whose content
     nobody reads.
     """
 
     group: Optional[int] = None
-    k: Optional[torch.Tensor] = None
-    v: Optional[torch.Tensor] = None
+    tensors: Dict[str, torch.Tensor] = field(default_factory=dict)
     writes: bool = True
     state: Optional[torch.Tensor] = None
+
+    @property
+    def k(self) -> Optional[torch.Tensor]:
+        return self.tensors.get("k")
+
+    @property
+    def v(self) -> Optional[torch.Tensor]:
+        return self.tensors.get("v")
 
 
 class Mixer(Part):

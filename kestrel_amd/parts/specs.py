@@ -49,19 +49,31 @@ class PositionSpec:
 
 @dataclass(frozen=True)
 class CacheSpec:
-    """What a mixer keeps per token: keys and values of ``n_kv_heads`` x ``head_dim``.
+    """What an attention mixer keeps per token: keys and values of ``n_kv_heads`` x ``head_dim``.
 
     ``window`` = number of most recent positions a query reads (``None``: all), which
     lets the cache manager give back pages that have fallen out of it.
+
+    The cache manager asks a specification three things and nothing else, so a mixer that keeps
+    something other than keys and values per token (one latent, another layout) brings a
+    specification class of its own with the same three: ``window``; ``page_tensors(page_size)``,
+    the tensors of one page by name with their shapes (the manager allocates each as
+    ``[runs of layers, pages, *shape]`` and hands a layer its slice as ``LayerCache.tensors[name]``);
+    and ``group_key``, equal for layers that can share a block table and a pool of pages.
     """
 
     n_kv_heads: int
     head_dim: int
     window: Optional[int] = None
 
+    def page_tensors(self, page_size: int) -> Dict[str, Tuple[int, ...]]:
+        # values are kept transposed inside a page: eight consecutive keys of one channel are 16
+        # bytes, which is what the MFMA attention kernels load at a time
+        return {"k": (self.n_kv_heads, page_size, self.head_dim), "v": (self.n_kv_heads, self.head_dim, page_size)}
+
     @property
     def group_key(self) -> Tuple:
-        return (self.n_kv_heads, self.head_dim, self.window)
+        return ("kv", self.n_kv_heads, self.head_dim, self.window)
 
 
 @dataclass(frozen=True)

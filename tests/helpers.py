@@ -178,14 +178,13 @@ def replay(runner, requests: Dict[str, "Request"], steps, poison: bool = False) 
                 if poison:
                     for g, group in enumerate(runner.cache.groups):
                         if pages[g]:
-                            index = torch.tensor(pages[g], device=group.k.device)
-                            group.k[:, index] = float("nan")
-                            group.v[:, index] = float("nan")
+                            for tensor in group.tensors.values():
+                                tensor[:, torch.tensor(pages[g], device=tensor.device)] = float("nan")
         runner.cache.check()
     return {name: torch.cat(chunks, dim=0) for name, chunks in rows.items() if chunks}
 
 
 def poison_cache(runner) -> None:
     for group in runner.cache.groups:
-        group.k.fill_(float("nan"))
-        group.v.fill_(float("nan"))
+        for tensor in group.tensors.values():
+            tensor.fill_(float("nan"))

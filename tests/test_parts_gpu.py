@@ -404,6 +404,123 @@ def test_toy_parts_build_and_step():
     helpers.assert_close(out, _toy_reference(ids_b, weights, decay, eps), torch.float32, "toy c")
 
 
+@dataclass(frozen=True)
+class LatentCacheSpec:
+    """What the toy mixer below keeps per token: one vector, pages of ``[page_size, width]``."""
+
+    width: int
+    window: Optional[int] = None
+
+    def page_tensors(self, page_size):
+        return {"c": (page_size, self.width)}
+
+    @property
+    def group_key(self):
+        return ("latent", self.width, self.window)
+
+
+@dataclass(frozen=True)
+class LatentSpec:
+    kind: str
+    dim: int
+    width: int
+
+
+def test_a_mixer_with_a_cache_layout_of_its_own():
+    """A toy mixer that caches one latent per token (no keys, no values) in pages whose layout its
+    own specification names: the cache manager allocates what the specification says, gives the
+    layer its slice, and pages, block tables, slots and reuse work as for attention. The layer
+    stands beside an attention layer, which gets a group and a pool of its own."""
+    from kestrel_amd.cache import CacheManager
+    from kestrel_amd.engine.step import ModelRunner
+    from kestrel_amd.models import DecoderModel
+    from kestrel_amd.ops.linear import linear
+    from kestrel_amd.parts import (AttentionSpec, DenseFeedForwardSpec, LayerSpec, Mixer, ModelPlan, NormSpec, ParamSpec,
+                                   PositionSpec, ScheduleEntry, register_mixer)
+
+    class LatentMixer(Mixer):
+        """``c_t = h_t Wc`` is cached; the output at ``t`` is ``mean_{j <= t}(c_j) Wo``."""
+
+        def params(self):
+            return {"down.weight": ParamSpec((self.spec.width, self.spec.dim)), "up.weight": ParamSpec((self.spec.dim, self.spec.width))}
+
+        def cache_spec(self):
+            return LatentCacheSpec(self.spec.width)
+
+        def bind(self, tensors, dtype, device):
+            self.down, self.up = tensors["down.weight"].to(device).float(), tensors["up.weight"].to(device).float()
+
+        def forward(self, h, batch, cache, residual):
+            group = batch.groups[cache.group]
+            store = cache.tensors["c"]                              # [pages, page_size, width]
+            flat = store.view(-1, store.shape[-1])
+            n = h.shape[0]
+            latent = batch.workspace.get("toy.latent", (n, self.spec.width), torch.float32)
+            linear(h.float(), self.down, None, latent)
+            flat[group.slots.long()] = latent.to(flat.dtype)       # write before read, as attention does
+            means = torch.zeros(n, self.spec.width, device=h.device)
+            rows, hi = batch.token_row.tolist(), batch.kv_hi.tolist()
+            for t in range(n):
+                pages = group.block_table[rows[t], : -(-hi[t] // group.page_size)].long()
+                means[t] = store[pages].reshape(-1, store.shape[-1])[:hi[t]].float().mean(dim=0)
+            out = batch.workspace.get("toy.latent_out", (n, self.spec.dim), torch.float32)
+            linear(means, self.up, None, out)
+            residual += out
+
+    register_mixer("toy_latent", LatentMixer)
+    dim, vocab, eps, width = 32, 60, 1e-5, 12
+    norm = NormSpec("layernorm", dim, eps)
+    ff_names = {"feed_forward.fc1.weight": "{}.fc1.weight", "feed_forward.fc1.bias": "{}.fc1.bias",
+                "feed_forward.fc2.weight": "{}.fc2.weight", "feed_forward.fc2.bias": "{}.fc2.bias",
+                "norm.weight": "{}.ln.weight", "norm.bias": "{}.ln.bias"}
+    toy = LayerSpec("parallel", norm, LatentSpec("toy_latent", dim, width), DenseFeedForwardSpec("dense", dim, 40),
+                    names={**{k: v.format("l0") for k, v in ff_names.items()}, "mixer.down.weight": "l0.down", "mixer.up.weight": "l0.up"})
+    attn = LayerSpec("parallel", norm, AttentionSpec("attention", dim, 2, 1, 16, PositionSpec("rotary_neox", 8, 100.0, 96)),
+                     DenseFeedForwardSpec("dense", dim, 40),
+                     names={**{k: v.format("l1") for k, v in ff_names.items()}, "mixer.qkv.weight": "l1.attn.qkv.weight",
+                            "mixer.qkv.bias": "l1.attn.qkv.bias", "mixer.proj.weight": "l1.attn.proj.weight",
+                            "mixer.proj.bias": "l1.attn.proj.bias"})
+    plan = ModelPlan("toy-latent", vocab, dim, 96, (toy, attn), (ScheduleEntry(0), ScheduleEntry(1)), norm, head_bias=False,
+                     tied_head=True, names={"embedding": "emb", "final_norm.weight": "fn.weight", "final_norm.bias": "fn.bias"})
+    model = DecoderModel(plan)
+    gen = torch.Generator().manual_seed(9)
+    weights = {}
+    for name, spec in model.params().items():
+        noise = torch.randn(spec.shape, generator=gen)
+        weights[name] = (1 + 0.1 * noise) if spec.init == "gain" else 0.3 * noise
+    model.bind(weights, torch.float32, DEV)
+    cache = CacheManager(model.cache_needs(), 16, 9, 3, dtype=torch.float32, device=DEV)
+    assert len(cache.groups) == 2 and set(cache.groups[0].tensors) == {"c"} and set(cache.groups[1].tensors) == {"k", "v"}
+    assert tuple(cache.groups[0].tensors["c"].shape) == (1, 9, 16, width)
+    assert cache.bytes_per_page() == 4 * (16 * width + 2 * 16 * 16)
+    runner = ModelRunner(model, cache, DEV)
+    helpers.poison_cache(runner)
+
+    def reference(ids):
+        w = {k: v.double() for k, v in weights.items()}
+        x = w["emb"][torch.tensor(ids)]
+        positions = torch.arange(len(ids))
+        h = plain.layer_norm(x, w["l0.ln.weight"], w["l0.ln.bias"], eps)
+        latent = h @ w["l0.down"].T
+        means = torch.cumsum(latent, dim=0) / (positions + 1).unsqueeze(1)
+        x = x + means @ w["l0.up"].T + plain.mlp(h, {k.replace("l0.", "p.mlp."): v for k, v in w.items()}, "p.")
+        h = plain.layer_norm(x, w["l1.ln.weight"], w["l1.ln.bias"], eps)
+        wd = {k.replace("l1.", "p."): v for k, v in w.items() if k.startswith("l1.attn")}
+        wd.update({k.replace("l1.", "p.mlp."): v for k, v in w.items() if k.startswith("l1.fc")})
+        x = x + plain.attention(h, wd, "p.", {"n_heads": 2, "n_kv_heads": 1, "head_dim": 16}, positions,
+                                plain.visibility(positions, None), plain.rotary_table(8, 96, 100.0)) + plain.mlp(h, wd, "p.")
+        return plain.layer_norm(x, w["fn.weight"], w["fn.bias"], eps) @ w["emb"].T
+
+    lengths = {"a": 50, "b": 21, "c": 38, "d": 45}
+    reqs = {tag: helpers.Request(tag, helpers.random_ids(70 + i, n, vocab)) for i, (tag, n) in enumerate(lengths.items())}
+    steps = [[("a", 20), ("b", 3)], [("a", 1), ("b", 17), ("c", 30)], [("a", 29), ("b", 1), ("c", 1)],    # a and b end
+             [("c", 7), ("d", 33)], [("d", 1)], [("d", 11)]]        # d runs in pages a and b gave back (9 pages in all)
+    got = helpers.replay(runner, reqs, steps, poison=True)
+    for tag, req in reqs.items():
+        helpers.assert_close(got[tag], reference(req.ids), torch.float32, f"latent cache, request {tag}")
+    assert all(g.pool.free_count == 9 for g in cache.groups)
+
+
 def test_a_layer_may_read_another_layers_cache():
     """Schedule entry 1 keeps no keys and values and reads those of entry 0."""
     from kestrel_amd.config import get_spec
