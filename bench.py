@@ -6,7 +6,13 @@ prefix embeddings and text ids) through the engine's step function with greedy s
 on the GPU. The model has the layer sizes of the Moondream 2 text decoder with seeded
 random weights N(0, 0.02) in bf16; inputs are synthetic. Besides ``value`` (decoded tokens
 a second) the line carries a 2,048-token prefill, the decode step's HBM roofline and
-decode throughput at batch 1 and 64.
+decode throughput at batch 1 and 64. ``--peaks`` adds what this GPU reaches on a plain read stream
+and on a loop of matrix instructions beside the nominal peaks.
+
+``--workload waves256`` and ``--workload mixed48`` (the latter meant for ``--sizes phi2``) measure
+the whole engine instead: a model folder is written with seeded random weights, loaded through the
+loader, and requests go through ``InferenceEngine`` (scheduler, sampler, paged cache under
+pressure); the line then reports generated tokens a second.
 """
 
 from __future__ import annotations
@@ -193,6 +199,97 @@ def time_prefill(net, typed, tokens, repeats=3):
     return best
 
 
+def write_model_folder(sizes: dict, layers: int, seed: int) -> str:
+    """A model folder (config.json, model.safetensors) with seeded random weights N(0, 0.02)."""
+    import tempfile
+
+    from kestrel_amd.weights import InitRecipe, write_random_model
+
+    folder = tempfile.mkdtemp(prefix="kestrel_amd_bench_")
+    write_random_model(folder, {"text": dict(sizes, n_layers=layers)}, seed, InitRecipe(std=0.02))
+    return folder
+
+
+def run_workload(args, sizes: dict) -> dict:
+    """Requests through the entry point. ``waves256``: 256 requests in 4 waves, each a block of 730
+    given embeddings and 32 to 128 ids, 128 new tokens, half greedy and half at temperature 1, in
+    a cache pool of about 60 GB. ``mixed48``: 48 requests with prompts of 64 to 1,536 ids fed in
+    portions of at most 512 tokens beside the decoded tokens of the others, 128 new tokens each at
+    temperature 0.7."""
+    import random
+    import shutil
+
+    import torch
+
+    from kestrel_amd import InferenceEngine, RuntimeConfig
+
+    waves = args.workload == "waves256"
+    seed = 4 if waves else 3
+    started = time.perf_counter()
+    folder = write_model_folder(sizes, args.layers, seed)
+    written = time.perf_counter() - started
+    n_requests, n_new = (256, 128) if waves else (48, 128)
+    if waves:
+        cfg = RuntimeConfig(model_path=folder, dtype=args.dtype, max_batch_size=args.max_batch_size or 64,
+                            kv_cache_bytes=60 * 10 ** 9 * args.layers // sizes["n_layers"], max_seq_len=2048, seed=seed)
+    else:
+        cfg = RuntimeConfig(model_path=folder, dtype=args.dtype, max_batch_size=args.max_batch_size or 48,
+                            max_num_batched_tokens=512, max_seq_len=2048, seed=seed)
+    started = time.perf_counter()
+    engine = InferenceEngine.create_sync(cfg)
+    loaded = time.perf_counter() - started
+    try:
+        rng = random.Random(seed)
+        vocab, dim = sizes["vocab_size"], sizes["dim"]
+        prefix = torch.randn(730, dim, generator=torch.Generator().manual_seed(seed)).to("cuda:0") if waves else None
+
+        def submit(i):
+            if waves:
+                ids = [rng.randrange(0, vocab) for _ in range(rng.randint(32, 128))]
+                options = dict(temperature=1.0, top_p=1.0, seed=i) if i % 2 else {}
+                return engine.submit_sync(ids, max_new_tokens=n_new, prefix_embeds=prefix, stop_ids=(), **options)
+            ids = [rng.randrange(0, vocab) for _ in range(rng.randint(64, 1536))]
+            return engine.submit_sync(ids, max_new_tokens=n_new, temperature=0.7, top_p=1.0, seed=i, stop_ids=())
+
+        for future in [submit(1000 + i) for i in range(8 if waves else 4)]:      # warm-up: graphs, workspaces
+            future.result()
+        steps_before = engine.scheduler.steps
+        started = time.perf_counter()
+        futures = []
+        for wave in range(4 if waves else 1):
+            count = n_requests // 4 if waves else n_requests
+            futures += [submit(wave * count + j) for j in range(count)]
+            if waves:
+                time.sleep(0.05)
+        results = [f.result() for f in futures]
+        elapsed = time.perf_counter() - started
+        steps = engine.scheduler.steps - steps_before
+        pages = engine.runner.cache.n_pages
+    finally:
+        engine.shutdown_sync()
+        shutil.rmtree(folder, ignore_errors=True)
+    generated = sum(len(r.tokens) for r in results)
+    prompt = sum(r.metrics.input_tokens for r in results)
+    what = ("256 requests in 4 waves, 730 given embeddings + 32-128 ids each, 128 new tokens, half greedy half T=1" if waves
+            else "48 requests, prompts of 64-1536 ids in portions of at most 512 beside decodes, 128 new tokens at T=0.7")
+    return {
+        "metric": f"generated tok/s through the entry point ({LABELS[args.sizes][0]}; {what})",
+        "value": round(generated / elapsed, 1), "unit": "tok/s", "n_gpus": 1, "steps": steps, "warmup": 8 if waves else 4,
+        "ms_per_step": round(elapsed / max(steps, 1) * 1e3, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": args.dtype,
+        "data": "synthetic (seeded random token ids and prefix embeddings; a folder of random weights N(0,0.02) read by the loader)",
+        "config": {"model": LABELS[args.sizes][1], "workload": args.workload, "n_layers": args.layers,
+                   "n_layers_full": sizes["n_layers"], "dim": sizes["dim"], "ff_dim": sizes["ff_dim"],
+                   "n_heads": sizes["n_heads"], "vocab_size": sizes["vocab_size"], "requests": n_requests,
+                   "max_batch_size": cfg.max_batch_size, "max_num_batched_tokens": cfg.max_num_batched_tokens,
+                   "kv_cache_pages": pages, "page_size": PAGE_SIZE, "parallelism": "single-gpu"},
+        "seconds": round(elapsed, 3), "generated_tokens": generated, "prompt_tokens": prompt,
+        "all_tokens_per_second": round((generated + prompt) / elapsed, 1),
+        "finish_reasons": sorted({r.finish_reason for r in results}),
+        "setup_seconds": {"write_folder": round(written, 1), "load": round(loaded, 1)},
+    }
+
+
 def main() -> int:
     parser = argparse.ArgumentParser()
     parser.add_argument("--gpus", type=int, default=1)
@@ -206,6 +303,11 @@ def main() -> int:
     parser.add_argument("--prefill-tokens", type=int, default=PREFILL_TOKENS, help="length of the timed prompt")
     parser.add_argument("--skip-points", action="store_true", help="only the default batch (no batch 1 / 64, no prefill)")
     parser.add_argument("--only-prefill", action="store_true", help="only the 2,048-token prefill (for profiling)")
+    parser.add_argument("--peaks", action="store_true",
+                        help="also measure a plain read stream and a loop of matrix instructions on this GPU and report against them")
+    parser.add_argument("--workload", default="decode", choices=["decode", "waves256", "mixed48"],
+                        help="decode: the benchmark's decode step (default); the others run requests through InferenceEngine")
+    parser.add_argument("--max-batch-size", type=int, default=None, help="for the workloads through the entry point")
     args = parser.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -224,6 +326,9 @@ def main() -> int:
     sizes["max_context"] = max(sizes["max_context"], args.context + max(args.steps, 16) + args.warmup + 8, args.prefill_tokens)
     if args.layers is None:
         args.layers = sizes["n_layers"]
+    if args.workload != "decode":
+        print(json.dumps(run_workload(args, dict(SIZES[args.sizes]))))
+        return 0
     net, typed = build_model(args.layers, dtype, device, sizes)
     weights = model_bytes(net, size)
 
@@ -260,6 +365,15 @@ def main() -> int:
             e, _ = time_decode(net, typed, batch, args.context, steps, min(args.warmup, 4))
             points[f"decode_b{batch}"] = round(batch * steps / e, 1)
         record["points"] = points
+    if args.peaks:
+        from kestrel_amd.ops import core
+
+        peaks = core.measured_peaks(device)
+        record["roofline"]["peak_measured"] = round(peaks["hbm_read_gbs"], 1)
+        record["roofline"]["frac_measured"] = round(achieved / 1e9 / peaks["hbm_read_gbs"], 4)
+        if "prefill" in record and args.dtype == "bf16":
+            record["prefill"]["peak_measured"] = round(peaks["mfma_bf16_tflops"], 1)
+            record["prefill"]["frac_measured"] = round(flops / seconds / 1e12 / peaks["mfma_bf16_tflops"], 4)
     print(json.dumps(record))
     return 0
 

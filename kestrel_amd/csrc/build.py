@@ -29,7 +29,7 @@ ARCH = "gfx950"
 # library name -> its sources. "core" is all a float32 run needs; "fast" holds the
 # bf16 MFMA kernels of serving.
 LIBRARIES: Dict[str, List[str]] = {
-    "core": ["ka_error.hip", "elementwise.hip", "gemm_generic.hip", "attention_generic.hip", "sampling.hip"],
+    "core": ["ka_error.hip", "elementwise.hip", "gemm_generic.hip", "attention_generic.hip", "sampling.hip", "peaks.hip"],
     "fast": ["ka_error.hip", "gemm_bf16.hip", "gemv_bf16.hip", "attention_bf16.hip"],
 }
 HEADERS = ["ka_common.h", "ka_partials.h", "ka_no_alloc.h"]

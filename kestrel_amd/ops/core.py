@@ -105,6 +105,40 @@ def _check_caches(who: str, k_cache, v_cache, dtype, n_kv_heads: int, page_size:
           f"{who}: value cache must be [pages, Hkv, hd, page_size] of the activation type")
 
 
+def measured_peaks(device: torch.device, read_bytes: int = 2 << 30) -> dict:
+    """What this GPU reaches on a plain read stream of ``read_bytes`` (GB/s) and on a loop of bf16
+    matrix instructions that waits for nothing (TFLOP/s): the best of a few runs each."""
+    handle = lib()
+    for name, argtypes in (("ka_peak_read", [_c_void_p, _c_long, _c_int, _c_void_p, _c_void_p]),
+                           ("ka_peak_mfma_bf16", [_c_void_p, _c_int, _c_int, _c_void_p])):
+        getattr(handle, name).argtypes = argtypes
+        getattr(handle, name).restype = _c_int
+    sink = torch.zeros(16, dtype=torch.float32, device=device)
+    buffer = torch.ones(read_bytes // 4, dtype=torch.int32, device=device)
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+
+    def best_ms(launch, repeats=5):
+        launch()
+        torch.cuda.synchronize(device)
+        best = None
+        for _ in range(repeats):
+            start.record()
+            launch()
+            stop.record()
+            stop.synchronize()
+            ms = start.elapsed_time(stop)
+            best = ms if best is None else min(best, ms)
+        return best
+
+    read_ms = min(best_ms(lambda g=g: _check(handle.ka_peak_read(buffer.data_ptr(), read_bytes, g, sink.data_ptr(), stream_ptr())))
+                  for g in (2048, 4096, 8192))
+    workgroups, iters = 1024, 8000
+    mfma_ms = best_ms(lambda: _check(handle.ka_peak_mfma_bf16(sink.data_ptr(), workgroups, iters, stream_ptr())))
+    flops = workgroups * 4 * iters * 8 * 2 * 32 * 32 * 16
+    del buffer
+    return {"hbm_read_gbs": read_bytes / (read_ms * 1e-3) / 1e9, "mfma_bf16_tflops": flops / (mfma_ms * 1e-3) / 1e12}
+
+
 def uniform(key: int, counter: int) -> float:
     """The uniform number the sampling kernel draws for (key, counter)."""
     return float(lib().ka_uniform_host(key & (2 ** 64 - 1), counter))
