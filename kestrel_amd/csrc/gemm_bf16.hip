@@ -195,6 +195,22 @@ __device__ __forceinline__ void gd_wait_loads() {
     __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | 0x0f70);
 }
 
+// Waits until at most `younger` x LPW of this wave's loads are still in flight (the count of an
+// s_waitcnt is an immediate: one instruction per value that can occur, at most MAX).
+template <int LPW, int MAX>
+__device__ __forceinline__ void gd_wait_younger(int younger) {
+    static_assert(LPW * (MAX > 0 ? MAX : 0) <= 63, "more loads in flight than the counter holds");
+    if constexpr (MAX <= 0) {
+        gd_wait_loads<0>();
+    } else {
+        if (younger >= MAX) gd_wait_loads<LPW * MAX>();
+        else gd_wait_younger<LPW, MAX - 1>(younger);
+    }
+}
+
+// s_waitcnt lgkmcnt(0) alone: this wave's LDS reads have all arrived in its registers
+__device__ __forceinline__ void gd_wait_lds() { __builtin_amdgcn_s_waitcnt(0xc07f); }
+
 // The barrier alone, without the fence that __syncthreads() puts before it: that fence waits
 // for every load in flight, the younger stages' too. What must be ordered here is ordered by
 // hand: a wave has waited for its own loads of the stage (vmcnt) and for its LDS reads of the
@@ -205,7 +221,14 @@ __device__ __forceinline__ void gd_barrier() {
     asm volatile("" ::: "memory");
 }
 
-template <int WN, int WM, int GN, int GM, int BK, int NS>
+// Orders the LDS traffic of one wave: what its lanes wrote before is seen by its lanes after.
+__device__ __forceinline__ void at_epilogue_wave_sync() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+template <int WN, int WM, int GN, int GM, int BK, int NS, int SL>
 __global__ void __launch_bounds__(KA_WAVE * GN * GM)
     __attribute__((amdgpu_waves_per_eu(GN * GM / 4, (WN * WM > 8 ? 1 : 2) * (GN * GM / 4))))
 gemm_dma_kernel(const bf16_t* __restrict__ A, long lda, const bf16_t* __restrict__ W, long ldw,
@@ -222,7 +245,7 @@ gemm_dma_kernel(const bf16_t* __restrict__ A, long lda, const bf16_t* __restrict
         K = min(k_per, K - part * k_per);
         out = reinterpret_cast<float*>(out) + (size_t)part * M * ldo;
     }
-    static_assert(NS >= 2 && NS <= 4, "two to four stages");
+    static_assert(NS >= 2 && NS <= 8, "two to eight stages");
     static_assert(GN * GM == 4 || GN * GM == 8, "four or eight waves");
     constexpr int WAVES = GN * GM;
     constexpr int BN = 32 * WN * GN, BM = 32 * WM * GM;
@@ -295,92 +318,180 @@ gemm_dma_kernel(const bf16_t* __restrict__ A, long lda, const bf16_t* __restrict
     for (int b = 0; b < WM; ++b) xrow_off[b] = BN * ROW + (wm * 32 * WM + b * 32 + li) * ROW;
     const int swz = swizzle(li);
 
-    // NS - 1 stages are on their way while one is multiplied. A wave waits for its own loads of
-    // the stage it needs (the younger ones may stay in flight), the barrier then tells it that
-    // everybody's have landed and that the stage read last has been left by all.
+    // The K-steps' operands are read from LDS a group of SL k-slices (of 16) at a time, one group
+    // ahead of the group that is being multiplied, also across the edge of a K-step: the MFMAs of a
+    // stage's last group run while the first group of the next stage is on its way from LDS, so the
+    // matrix pipes do not stand still at every K-step while both waves of a SIMD wait for LDS
+    // together. For that the barrier of a K-step stands before the last group's MFMAs: a wave
+    // arrives when its own loads of the next stage have landed and its own reads of this stage are
+    // in its registers. After the barrier everybody's have, so the next stage may be read and this
+    // stage's memory may be written: the load of stage s + NS goes out, and has NS - 1 K-steps to land.
+    constexpr int G = BK / 16 / SL;                      // groups per K-step
+    static_assert(G * SL * 16 == BK, "the groups of slices do not divide a K-step");
     const int steps = K / BK;
+    // NS stages go out at once; the first has to be there before anything can be read
 #pragma unroll
-    for (int st = 0; st < NS - 1; ++st)
+    for (int st = 0; st < NS; ++st)
         if (st < steps) fetch(st, st * BK);
-    for (int s = 0; s < steps; ++s) {
-        const int younger = min(NS - 2, steps - 1 - s);          // stages asked for after stage s
-        if (NS >= 4 && younger >= 2) gd_wait_loads<2 * LPW>();
-        else if (NS >= 3 && younger >= 1) gd_wait_loads<LPW>();
-        else gd_wait_loads<0>();
+    {
+        const int younger = min(NS - 1, steps - 1);
+        gd_wait_younger<LPW, NS - 1>(younger);
         gd_barrier();
-        if (s + NS - 1 < steps) fetch((s + NS - 1) % NS, (s + NS - 1) * BK);
-        const unsigned char* base = gb_lds + (s % NS) * STAGE;
-        bf16x8 wa[2][WN], xb[2][WM];
-        auto operands = [&](int slot, int ks) {
-            const int place = ((ks * 2 + lg) ^ swz) * 16;
+    }
+    bf16x8 wa[2][SL][WN], xb[2][SL][WM];
+    auto operands = [&](auto slot_c, int stage, int g) {
+        constexpr int slot = decltype(slot_c)::value;
+        const unsigned char* base = gb_lds + (stage % NS) * STAGE;
 #pragma unroll
-            for (int a = 0; a < WN; ++a) wa[slot][a] = *reinterpret_cast<const bf16x8*>(base + wrow_off[a] + place);
+        for (int i = 0; i < SL; ++i) {
+            const int place = (((g * SL + i) * 2 + lg) ^ swz) * 16;
 #pragma unroll
-            for (int b = 0; b < WM; ++b) xb[slot][b] = *reinterpret_cast<const bf16x8*>(base + xrow_off[b] + place);
-        };
-        operands(0, 0);
+            for (int a = 0; a < WN; ++a) wa[slot][i][a] = *reinterpret_cast<const bf16x8*>(base + wrow_off[a] + place);
 #pragma unroll
-        for (int ks = 0; ks < BK / 16; ++ks) {
-            if (ks + 1 < BK / 16) operands((ks + 1) & 1, ks + 1);
+            for (int b = 0; b < WM; ++b) xb[slot][i][b] = *reinterpret_cast<const bf16x8*>(base + xrow_off[b] + place);
+        }
+    };
+    const int groups = steps * G;
+    // group t (stage t / G, its group t % G) is multiplied from the registers of slot t & 1
+    auto group = [&](auto slot_c, int t) {
+        constexpr int slot = decltype(slot_c)::value;
+        const int st = t / G, g = t % G;
+        if (g == G - 1 && st + 1 < steps) {
+            // own loads of stage st + 1 landed (the stages after it may stay in flight), own reads of
+            // stage st done (they are the operands of this group, needed below in any case)
+            const int younger = min(NS - 2, steps - 2 - st);
+            gd_wait_younger<LPW, NS - 2>(younger);
+            gd_wait_lds();
+            gd_barrier();
+            if (st + NS < steps) fetch(st % NS, (st + NS) * BK);
+        }
+        // (always, also after the last group, whose "next" is read from memory nobody needs: a read
+        // under a condition makes the compiler wait for every read in flight before the MFMAs,
+        // the ones just asked for included)
+        operands(std::integral_constant<int, slot ^ 1>{}, (t + 1) / G, (t + 1) % G);
+#pragma unroll
+        for (int i = 0; i < SL; ++i)
 #pragma unroll
             for (int a = 0; a < WN; ++a)
 #pragma unroll
                 for (int b = 0; b < WM; ++b)
-                    acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wa[ks & 1][a], xb[ks & 1][b], acc[a][b], 0, 0, 0);
-        }
+                    acc[a][b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wa[slot][i][a], xb[slot][i][b], acc[a][b], 0, 0, 0);
+        // The reads of the next group go out behind this group's second MFMA, into registers of
+        // their own, and have the rest of the group's MFMAs to arrive. (Left to itself the compiler
+        // gives both groups the same registers and asks for the next operands only after the
+        // MFMAs that use the present ones, three MFMAs before they are needed. Asked for ahead of
+        // the group's first MFMA they would be waited for at once: the compiler waits for every
+        // read in flight where this loop needs the older ones only.)
+        constexpr int FIRST = SL * WN * WM > 2 ? 2 : 1;
+        __builtin_amdgcn_sched_group_barrier(0x008, FIRST, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, SL * (WN + WM), 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, SL * WN * WM - FIRST, 0);
+    };
+    // (Nothing but LDS reads may be in flight on the counter they share with scalar loads when the
+    // loop is entered: with a scalar load among them the compiler can no longer count on arrival
+    // in order and waits, in every round, for all reads, the ones just asked for included.)
+    // (The arguments that only the epilogue uses are asked for here for the same reason: the
+    // compiler otherwise fetches them, with scalar loads, as late as it can.)
+    asm volatile("" ::"s"(bias), "s"(out), "s"(ldo), "s"(act), "s"(accumulate), "s"(out_dtype), "s"(M), "s"(N));
+    gd_wait_lds();
+    operands(std::integral_constant<int, 0>{}, 0, 0);
+    int t = 0;
+    for (; t + 1 < groups; t += 2) {
+        group(std::integral_constant<int, 0>{}, t);
+        group(std::integral_constant<int, 1>{}, t + 1);
     }
+    if (t < groups) group(std::integral_constant<int, 0>{}, t);
 
-    // epilogue: acc[a][b][v] is out[m][n] with n = n0 + wn*32*WN + a*32 + (v/4)*8 + lg*4 + v%4,
-    // m = m0 + wm*32*WM + b*32 + li
-    const bool vec_ok = (N % 4 == 0) && (ldo % 4 == 0);
+    // Epilogue. acc[a][b][v] is out[m][n] with n = n0 + wn*32*WN + a*32 + (v/4)*8 + lg*4 + v%4 and
+    // m = m0 + wm*32*WM + b*32 + li: a lane holds four neighbouring outputs of one row, and one
+    // store instruction of the wave would touch 32 rows with 16 (bf16) or 32 bytes each, which the
+    // memory system takes at a fraction of its rate (measured: 15 us of 79 for the 33 MB of the
+    // first feed-forward linear of a 2,048-token prompt). So a wave passes its outputs through its
+    // share of the stages' LDS, 32 rows at a time or more, and stores whole rows of its tile: 128
+    // or 256 contiguous bytes per row, 16 bytes per lane. Bias and activation are applied on the
+    // way in; an fp32 output that accumulates is read and added on the way out.
+    gd_barrier();                                        // the last stage has been read by everybody
     const bool bias_vec = (N % 4 == 0) && (reinterpret_cast<uintptr_t>(bias) % 16 == 0);
-    gd_static_for<0, WM>([&](auto bc) {
-        constexpr int b = decltype(bc)::value;
-        const int m = m0 + wm * 32 * WM + b * 32 + li;
-        gd_static_for<0, WN>([&](auto ac) {
-            constexpr int a = decltype(ac)::value;
-            gd_static_for<0, 4>([&](auto qc) {
-                constexpr int q = decltype(qc)::value;
-                const int n = n0 + wn * 32 * WN + a * 32 + q * 8 + lg * 4;
-                if (m >= M || n >= N) return;
-                floatx4 bv = {0.f, 0.f, 0.f, 0.f};
-                if (bias) {
-                    if (bias_vec) bv = *reinterpret_cast<const floatx4*>(bias + n);       // n + 3 < N: N % 4 == 0
-                    else
-                        for (int i = 0; i < 4 && n + i < N; ++i) bv[i] = bias[n + i];
-                }
-                float v[4];
+    auto staged = [&](auto* typed_out) {
+        using T = std::remove_pointer_t<decltype(typed_out)>;
+        constexpr int ES = sizeof(T);                    // 2 or 4
+        constexpr int PER = 16 / ES;                     // outputs per 16-byte store
+        constexpr int RB = 32 * WN * ES;                 // bytes of a row of the wave's tile
+        constexpr int RS = RB + (ES == 2 ? 8 : 16);      // its place in LDS: padded so that the lanes' writes spread over the banks
+        constexpr int SHARE = gd_smem(BN, BM, BK, NS) / WAVES;
+        constexpr int BP = SHARE / (32 * RS) < WM ? SHARE / (32 * RS) : WM;      // blocks of 32 rows per pass
+        static_assert(BP >= 1, "a wave's share of LDS does not hold 32 rows of its tile");
+        constexpr int CH = RB / 16;                      // 16-byte chunks of a row
+        constexpr int RPI = KA_WAVE / CH;                // rows one store instruction covers
+        unsigned char* mine = gb_lds + wave * SHARE;
+        const int n_wave = n0 + wn * 32 * WN, m_wave = m0 + wm * 32 * WM;
+        const bool wide = (ldo * ES) % 16 == 0 && reinterpret_cast<uintptr_t>(typed_out) % 16 == 0 && n0 % PER == 0;
+        gd_static_for<0, (WM + BP - 1) / BP>([&](auto pc) {
+            constexpr int b0 = decltype(pc)::value * BP;
+            constexpr int nb = b0 + BP <= WM ? BP : WM - b0;
+            gd_static_for<0, nb>([&](auto bc) {
+                constexpr int b = b0 + decltype(bc)::value;
+                gd_static_for<0, WN>([&](auto ac) {
+                    constexpr int a = decltype(ac)::value;
+                    gd_static_for<0, 4>([&](auto qc) {
+                        constexpr int q = decltype(qc)::value;
+                        const int nl = a * 32 + q * 8 + lg * 4;
+                        const int n = n_wave + nl;
+                        floatx4 bv = {0.f, 0.f, 0.f, 0.f};
+                        if (bias && n < N) {
+                            if (bias_vec) bv = *reinterpret_cast<const floatx4*>(bias + n);       // n + 3 < N: N % 4 == 0
+                            else
+                                for (int i = 0; i < 4 && n + i < N; ++i) bv[i] = bias[n + i];
+                        }
+                        float v[4];
 #pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    float x = acc[a][b][q * 4 + i] + bv[i];
-                    if (act) x = ka_activate_fast(act, x);
-                    v[i] = x;
-                }
-                size_t o = (size_t)m * ldo + n;
-                if (out_dtype == KA_F32) {
-                    float* op = reinterpret_cast<float*>(out) + o;
-                    if (vec_ok) {
-                        floatx4 cur = accumulate ? *reinterpret_cast<floatx4*>(op) : floatx4{0.f, 0.f, 0.f, 0.f};
-                        floatx4 res = {cur[0] + v[0], cur[1] + v[1], cur[2] + v[2], cur[3] + v[3]};
-                        *reinterpret_cast<floatx4*>(op) = res;
-                    } else {
-                        for (int i = 0; i < 4 && n + i < N; ++i) op[i] = accumulate ? op[i] + v[i] : v[i];
-                    }
-                } else {
-                    bf16_t* op = reinterpret_cast<bf16_t*>(out) + o;
-                    if (vec_ok) {
-                        bf16x4 res = {(bf16_t)v[0], (bf16_t)v[1], (bf16_t)v[2], (bf16_t)v[3]};
-                        *reinterpret_cast<bf16x4*>(op) = res;
-                    } else {
-                        for (int i = 0; i < 4 && n + i < N; ++i) op[i] = (bf16_t)v[i];
-                    }
-                }
+                        for (int i = 0; i < 4; ++i) {
+                            float x = acc[a][b][q * 4 + i] + bv[i];
+                            if (act) x = ka_activate_fast(act, x);
+                            v[i] = x;
+                        }
+                        unsigned char* at = mine + ((b - b0) * 32 + li) * RS + nl * ES;
+                        if constexpr (ES == 2) *reinterpret_cast<bf16x4*>(at) = bf16x4{(bf16_t)v[0], (bf16_t)v[1], (bf16_t)v[2], (bf16_t)v[3]};
+                        else *reinterpret_cast<floatx4*>(at) = floatx4{v[0], v[1], v[2], v[3]};
+                    });
+                });
             });
+            at_epilogue_wave_sync();
+#pragma unroll
+            for (int r0 = 0; r0 < nb * 32; r0 += RPI) {
+                const int rl = r0 + lane / CH, c = lane % CH;
+                const int m = m_wave + b0 * 32 + rl, n = n_wave + c * PER;
+                if (lane < RPI * CH && rl < nb * 32 && m < M && n < N) {      // (a row's chunks need not divide 64 lanes)
+                    const unsigned char* from = mine + rl * RS + c * 16;
+                    T* op = typed_out + (size_t)m * ldo + n;
+                    if (wide && n + PER <= N) {
+                        if constexpr (ES == 2) {
+                            *reinterpret_cast<bf16x8*>(op) = *reinterpret_cast<const bf16x8*>(from);
+                        } else {
+                            floatx4 x = *reinterpret_cast<const floatx4*>(from);
+                            if (accumulate) {
+                                const floatx4 cur = *reinterpret_cast<const floatx4*>(op);
+                                x = floatx4{cur[0] + x[0], cur[1] + x[1], cur[2] + x[2], cur[3] + x[3]};
+                            }
+                            *reinterpret_cast<floatx4*>(op) = x;
+                        }
+                    } else {
+                        const T* src = reinterpret_cast<const T*>(from);
+                        for (int i = 0; i < PER && n + i < N; ++i) {
+                            if constexpr (ES == 2) op[i] = src[i];
+                            else op[i] = accumulate ? op[i] + src[i] : src[i];
+                        }
+                    }
+                }
+            }
+            at_epilogue_wave_sync();                     // the next pass writes over what was just read
         });
-    });
+    };
+    if (out_dtype == KA_F32) staged(reinterpret_cast<float*>(out));
+    else staged(reinterpret_cast<bf16_t*>(out));
 }
 
-template <int WN, int WM, int GN, int GM, int BK, int NS>
+template <int WN, int WM, int GN, int GM, int BK, int NS, int SL = 1>
 static int launch_dma(const bf16_t* A, long lda, const bf16_t* W, long ldw, const float* bias, void* out,
                       int out_dtype, long ldo, int M, int N, int K, int act, int accumulate, hipStream_t stream,
                       int parts = 1, int k_per = 0) {
@@ -389,7 +500,7 @@ static int launch_dma(const bf16_t* A, long lda, const bf16_t* W, long ldw, cons
     constexpr int smem = gd_smem(BN, BM, BK, NS);
     static_assert(smem <= 160 * 1024, "the stages do not fit in LDS");
     if (!configured) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_dma_kernel<WN, WM, GN, GM, BK, NS>),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_dma_kernel<WN, WM, GN, GM, BK, NS, SL>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, smem);
         KA_CHECK(e == hipSuccess, "ka_linear_tiled_bf16: cannot reserve %d bytes of LDS: %s", smem, hipGetErrorString(e));
         configured = true;
@@ -398,7 +509,7 @@ static int launch_dma(const bf16_t* A, long lda, const bf16_t* W, long ldw, cons
     long total = (long)tiles_n * tiles_m;
     long launched = ((total + 7) / 8) * 8;
     KA_CHECK(launched < (1L << 31), "ka_linear_tiled_bf16: too many tiles");
-    hipLaunchKernelGGL((gemm_dma_kernel<WN, WM, GN, GM, BK, NS>), dim3((unsigned)launched, parts), dim3(KA_WAVE * GN * GM), smem,
+    hipLaunchKernelGGL((gemm_dma_kernel<WN, WM, GN, GM, BK, NS, SL>), dim3((unsigned)launched, parts), dim3(KA_WAVE * GN * GM), smem,
                        stream, A, lda, W, ldw, bias, out, out_dtype, ldo, M, N, K, act, accumulate, tiles_n, tiles_m, k_per);
     return 0;
 }
@@ -449,7 +560,7 @@ KA_API int ka_linear_tiled_bf16(const void* A, long lda, const void* W, long ldw
             // model at 2048 rows: N = 6144 and 8192). Where 128 x 128 tiles leave a CU with one
             // workgroup only, eight waves and three stages hide the trip to HBM that two
             // workgroups would otherwise hide for each other (N = 2048: 35 us of 120 at K = 8192).
-            const int cus = 256;
+            const int cus = ka_compute_units();
             long t256 = (long)ka_cdiv(N, 256) * ka_cdiv(M, 256);
             long t128 = (long)ka_cdiv(N, 128) * ka_cdiv(M, 128);
             long rounds = (t256 + cus - 1) / cus;
@@ -481,7 +592,7 @@ KA_API int ka_linear_tiled_bf16(const void* A, long lda, const void* W, long ldw
         int k_per = ka_cdiv(ka_cdiv(K, parts), 64) * 64;
         parts = ka_cdiv(K, k_per);
         if (parts >= 2 && partials && (long)parts * M * N <= partial_floats) {
-            rc = launch_dma<1, 2, 4, 2, 64, 3>(a, lda, w, ldw, nullptr, partials, KA_F32, N, M, N, K, 0, 0, stream, parts, k_per);
+            rc = launch_dma<1, 2, 4, 2, 64, 3, 4>(a, lda, w, ldw, nullptr, partials, KA_F32, N, M, N, K, 0, 0, stream, parts, k_per);
             if (rc) return rc;
             KA_LAUNCH_CHECK();
             const int quads = M * ka_cdiv(N, 4);
@@ -494,17 +605,17 @@ KA_API int ka_linear_tiled_bf16(const void* A, long lda, const void* W, long ldw
     switch (config) {
         case 221: rc = launch_config<2, 2, 64>(a, lda, w, ldw, bias, out, out_dtype, ldo, M, N, K, act, accumulate, stream); break;
         case 211: rc = launch_config<2, 1, 64>(a, lda, w, ldw, bias, out, out_dtype, ldo, M, N, K, act, accumulate, stream); break;
-#define KA_DMA(CODE, WNV, WMV, GNV, GMV, BKV, NSV)                                                               \
+#define KA_DMA(CODE, WNV, WMV, GNV, GMV, BKV, NSV, SLV)                                                               \
         case CODE:                                                                                                \
             KA_CHECK(K % BKV == 0, "ka_linear_tiled_bf16: this tile needs K to be a multiple of %d", BKV);        \
-            rc = launch_dma<WNV, WMV, GNV, GMV, BKV, NSV>(a, lda, w, ldw, bias, out, out_dtype, ldo, M, N, K, act, accumulate, stream); \
+            rc = launch_dma<WNV, WMV, GNV, GMV, BKV, NSV, SLV>(a, lda, w, ldw, bias, out, out_dtype, ldo, M, N, K, act, accumulate, stream); \
             break;
         // 10000 (four waves, 2 x 2) or 20000 (eight waves, 4 x 2) + stages * 1000 + (K-step / 32) * 100 + wave tile
-        KA_DMA(12222, 2, 2, 2, 2, 64, 2)      // 128 x 128, two workgroups per CU
-        KA_DMA(23212, 1, 2, 4, 2, 64, 3)      // 128 x 128 by eight waves, three stages: for one workgroup per CU
-        KA_DMA(22224, 2, 4, 4, 2, 64, 2)      // 256 x 256, one workgroup of eight waves per CU
-        KA_DMA(22232, 3, 2, 2, 4, 64, 2)      // 192 x 256 (N x M), eight waves: for an N that 256 leaves CUs idle with
-        KA_DMA(13122, 2, 2, 2, 2, 32, 3)      // (slower everywhere; kept as the test of K-steps of 32)
+        KA_DMA(12222, 2, 2, 2, 2, 64, 2, 2)      // 128 x 128, two workgroups per CU
+        KA_DMA(23212, 1, 2, 4, 2, 64, 3, 4)      // 128 x 128 by eight waves, three stages: for one workgroup per CU
+        KA_DMA(22224, 2, 4, 4, 2, 64, 2, 1)      // 256 x 256, one workgroup of eight waves per CU
+        KA_DMA(22232, 3, 2, 2, 4, 64, 2, 1)      // 192 x 256 (N x M), eight waves: for an N that 256 leaves CUs idle with
+        KA_DMA(13122, 2, 2, 2, 2, 32, 3, 2)      // (slower everywhere; kept as the test of K-steps of 32)
 #undef KA_DMA
         default: KA_CHECK(false, "ka_linear_tiled_bf16: unknown tile configuration %d", config);
     }

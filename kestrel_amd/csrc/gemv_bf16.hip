@@ -733,18 +733,7 @@ skinny_wide_kernel(WideArgs p) {
 // ----------------------------------------------------------------------------
 // Host side
 // ----------------------------------------------------------------------------
-static int sk_compute_units() {
-    static int cus = 0;
-    if (cus == 0) {
-        int dev = 0, n = 0;
-        if (hipGetDevice(&dev) == hipSuccess &&
-            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
-            cus = n;
-        else
-            cus = 256;
-    }
-    return cus;
-}
+static int sk_compute_units() { return ka_compute_units(); }
 
 // The persistent kernel is used wherever it fits; switching it off is for measurements and for
 // tests of the split kernel on sizes that it otherwise never sees.
