@@ -36,6 +36,20 @@ constexpr float AT_LOG2E = 1.4426950408889634f;
 
 __device__ __forceinline__ bf16x8 at_load8(const bf16_t* p) { return *reinterpret_cast<const bf16x8*>(p); }
 
+// A lane's value combined with that of the lane 32 away (the two hold the halves of one query's
+// scores): v_permlane32_swap exchanges the halves of two registers inside the vector unit, where a
+// shuffle would make a trip through LDS.
+__device__ __forceinline__ float at_max_with_other_half(float x) {
+    typedef __attribute__((ext_vector_type(2))) unsigned at_u2;
+    const at_u2 r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float at_sum_with_other_half(float x) {
+    typedef __attribute__((ext_vector_type(2))) unsigned at_u2;
+    const at_u2 r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+
 // Orders the LDS traffic of one wave: what its lanes wrote before is seen by its lanes after.
 __device__ __forceinline__ void at_wave_sync() {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
@@ -48,6 +62,7 @@ __device__ __forceinline__ void at_wave_sync() {
 // ----------------------------------------------------------------------------------------------
 constexpr int AP_WAVES = 4;                 // waves of a workgroup: all on the same 32 queries, keys interleaved
 constexpr int AP_QBLOCK = 32;               // queries per workgroup
+constexpr float AP_MAX_SLACK = 8.0f;        // powers of two the running maximum may grow before the outputs are rescaled
 constexpr int AP_MAX_TABLE = 24576;         // most block table entries of one row kept in LDS (393k keys)
 constexpr int ap_merge_floats(int hd) { return (hd + 31) / 32 * 16 + 2; }
 // block table entries of one row that fit in LDS beside the merge at head size hd
@@ -56,11 +71,18 @@ constexpr int ap_max_table(int hd) {
     return left < AP_MAX_TABLE ? left : AP_MAX_TABLE;
 }
 
-// (At least two waves per SIMD, except at head size 128, which needs more registers: with 256 registers a lane the compiler lets the MFMAs write
-// ordinary registers. Left to itself it puts their results in accumulator registers and then
-// spends a third of the loop's instructions moving them to where the softmax can read them.)
-template <int HD>
-__global__ void __launch_bounds__(KA_WAVE * AP_WAVES) __attribute__((amdgpu_waves_per_eu(HD <= 96 ? 2 : 1)))
+// Registers: with 256 a lane (two waves per SIMD) the compiler lets the MFMAs write ordinary
+// registers; left to itself it puts their results in accumulator registers and then spends a third
+// of the loop's instructions moving them to where the softmax can read them. Two blocks of queries
+// fit in 256 registers up to head size 64 (the prompt attention of 2,048 tokens: 63 to 48 us a
+// layer); beyond that they would take a SIMD's registers for one wave, which was measured far
+// slower than one block and two waves (head size 80: 98 against 63 us, 128: 267 against 139 us).
+constexpr int ap_waves_per_simd(int hd, int qb) { return qb == 1 ? (hd <= 96 ? 2 : 1) : (hd <= 64 ? 2 : 1); }
+
+// QB blocks of 32 queries per workgroup: every tile of keys and values that a wave fetches serves
+// QB tiles of scores (the fetches, their addresses and the block table look-ups are shared).
+template <int HD, int QB>
+__global__ void __launch_bounds__(KA_WAVE * AP_WAVES) __attribute__((amdgpu_waves_per_eu(ap_waves_per_simd(HD, QB))))
 attn_prefill_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t* __restrict__ k_cache,
                     const bf16_t* __restrict__ v_cache, const int* __restrict__ block_table, int max_pages,
                     const int* __restrict__ qblk_row, const int* __restrict__ qblk_tok,
@@ -68,6 +90,7 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_
                     const int* __restrict__ kv_lo, const int* __restrict__ kv_hi, bf16_t* __restrict__ out,
                     long out_row_stride, float scale, int H, int Hkv, int table_entries) {
     static_assert(HD % 16 == 0 && HD >= 16 && HD <= 256, "head sizes in steps of 16 up to 256");
+    static_assert(QB == 1 || QB == 2, "one or two blocks of queries");
     constexpr int QC = HD / 16;          // 16-byte chunks of half a head row = MFMA steps of the score product
     constexpr int DB = (HD + 31) / 32;   // 32-channel blocks of the output
     // A head size that is no multiple of 32 leaves the last block half used: its lanes 16..31
@@ -86,22 +109,40 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_
     const int kvh = h / (H / Hkv);
     const int row = qblk_row[blk];
     const int tok_end = cu_q[row + 1];
-    const int t = qblk_tok[blk] + li;
-    const bool q_valid = t < tok_end;
-    const int tq = q_valid ? t : tok_end - 1;
-    const int hi = q_valid ? kv_hi[tq] : 0;
-    const int lo = kv_lo ? kv_lo[tq] : 0;
-    int wave_hi = hi, wave_lo = q_valid ? lo : 0x7fffffff;
+    int t[QB], tq[QB], hi[QB], lo[QB];
+    bool q_valid[QB];
+    int wave_hi = 0, wave_lo = 0x7fffffff;
+    // lowest end and highest start of the visible ranges of the wave's queries: a tile inside
+    // [max_lo, min_hi) is seen whole by every query and needs no mask
+    int min_hi = 0x7fffffff, max_lo = 0;
+#pragma unroll
+    for (int b = 0; b < QB; ++b) {
+        t[b] = qblk_tok[blk] + b * 32 + li;
+        q_valid[b] = t[b] < tok_end;
+        tq[b] = q_valid[b] ? t[b] : tok_end - 1;
+        hi[b] = q_valid[b] ? kv_hi[tq[b]] : 0;
+        lo[b] = kv_lo ? kv_lo[tq[b]] : 0;
+        wave_hi = max(wave_hi, hi[b]);
+        if (q_valid[b]) {
+            wave_lo = min(wave_lo, lo[b]);
+            min_hi = min(min_hi, hi[b]);
+            max_lo = max(max_lo, lo[b]);
+        }
+    }
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) {
         wave_hi = max(wave_hi, __shfl_xor(wave_hi, off, KA_WAVE));
         wave_lo = min(wave_lo, __shfl_xor(wave_lo, off, KA_WAVE));
+        min_hi = min(min_hi, __shfl_xor(min_hi, off, KA_WAVE));
+        max_lo = max(max_lo, __shfl_xor(max_lo, off, KA_WAVE));
     }
     const int limit = kv_len[row];       // keys of this row that hold data
     // (the same in every lane: told to the compiler, which then counts tiles and looks up whole
     // pages in scalar registers)
     wave_hi = __builtin_amdgcn_readfirstlane(min(wave_hi, limit));
     wave_lo = __builtin_amdgcn_readfirstlane(wave_lo);
+    min_hi = __builtin_amdgcn_readfirstlane(min_hi);
+    max_lo = __builtin_amdgcn_readfirstlane(max_lo);
     // The row's block table goes to LDS once: a look-up per tile in global memory would put a
     // second trip to memory in front of every load of keys and values. (The host sees to it that
     // the table is long enough for every row of the launch.)
@@ -111,20 +152,40 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_
         for (int i = threadIdx.x; i < n_pages; i += KA_WAVE * AP_WAVES) pages[i] = bt[i];
         __syncthreads();
     }
+    // A block whose queries see no key at all (the rows that pad a captured batch): zeros, and no
+    // load is made from a table that has no entry.
+    if (wave_hi <= wave_lo || n_pages <= 0) {
+        if (wave == 0) {
+#pragma unroll
+            for (int b = 0; b < QB; ++b) {
+                if (!q_valid[b]) continue;
+                bf16_t* op = out + (size_t)t[b] * out_row_stride + (size_t)h * HD + lg * (HD / 2);
+#pragma unroll
+                for (int c = 0; c < QC; ++c) *reinterpret_cast<bf16x8*>(op + c * 8) = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+            }
+        }
+        return;
+    }
 
     // queries: lane (q = li, g = lg) holds channels [g * HD/2, (g + 1) * HD/2)
-    bf16x8 qreg[QC];
-    {
-        const bf16_t* qp = q + (size_t)tq * q_row_stride + (size_t)h * HD + lg * (HD / 2);
+    bf16x8 qreg[QB][QC];
 #pragma unroll
-        for (int c = 0; c < QC; ++c) qreg[c] = at_load8(qp + c * 8);
+    for (int b = 0; b < QB; ++b) {
+        const bf16_t* qp = q + (size_t)tq[b] * q_row_stride + (size_t)h * HD + lg * (HD / 2);
+#pragma unroll
+        for (int c = 0; c < QC; ++c) qreg[b][c] = at_load8(qp + c * 8);
     }
-    floatx16 o[DB];
+    floatx16 o[QB][DB];
+    float m_i[QB], l_i[QB];
 #pragma unroll
-    for (int db = 0; db < DB; ++db)
+    for (int b = 0; b < QB; ++b) {
+        m_i[b] = -INFINITY;
+        l_i[b] = 0.f;
 #pragma unroll
-        for (int v = 0; v < 16; ++v) o[db][v] = 0.f;
-    float m_i = -INFINITY, l_i = 0.f;
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) o[b][db][v] = 0.f;
+    }
     const float sl2 = scale * AT_LOG2E;
     const int kperm = (li & 16) | ((li & 4) << 1) | ((li & 8) >> 1) | (li & 3);
 
@@ -181,17 +242,6 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_
         }
     };
 
-    // lowest end and highest start of the visible ranges of the wave's queries: a tile inside
-    // [max_lo, min_hi) is seen whole by every query and needs no mask
-    int min_hi = q_valid ? hi : 0x7fffffff, max_lo = q_valid ? lo : 0;
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) {
-        min_hi = min(min_hi, __shfl_xor(min_hi, off, KA_WAVE));
-        max_lo = max(max_lo, __shfl_xor(max_lo, off, KA_WAVE));
-    }
-    min_hi = __builtin_amdgcn_readfirstlane(min_hi);
-    max_lo = __builtin_amdgcn_readfirstlane(max_lo);
-
     constexpr int STRIDE = 32 * AP_WAVES;
     // one tile of 32 keys whose key rows are in `kr`; the next tile's go to `kr_next`
     auto process = [&](int key0, const bf16x8* kr, bf16x8* kr_next) {
@@ -199,42 +249,66 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_
         load_values(key0, vr);                             // in flight during the scores and the softmax
         load_keys(key0 + STRIDE, kr_next);                 // in flight until the next tile
         __builtin_amdgcn_sched_barrier(0);
-        floatx16 s;
+        const bool whole = key0 >= max_lo && key0 + 32 <= min_hi;
+        // the scores of all blocks of queries first: the matrix pipes work on the later ones while
+        // the softmax of the first is computed, and the blocks' chains of dependent instructions
+        // (maximum, exchange with the other half of the wave, exponentials, sum) interleave
+        floatx16 s[QB];
 #pragma unroll
-        for (int v = 0; v < 16; ++v) s[v] = 0.f;
+        for (int b = 0; b < QB; ++b)
 #pragma unroll
-        for (int c = 0; c < QC; ++c) s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kr[c], qreg[c], s, 0, 0, 0);
+            for (int v = 0; v < 16; ++v) s[b][v] = 0.f;
+#pragma unroll
+        for (int c = 0; c < QC; ++c)               // (the blocks take turns: an MFMA that adds to the one before it waits for it)
+#pragma unroll
+            for (int b = 0; b < QB; ++b) s[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kr[c], qreg[b][c], s[b], 0, 0, 0);
         // lane holds, for its query, the keys key0 + (v / 8) * 16 + lg * 8 + v % 8
-        if (!(key0 >= max_lo && key0 + 32 <= min_hi)) {
+        if (!whole) {
+#pragma unroll
+            for (int b = 0; b < QB; ++b)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    int key = key0 + (v / 8) * 16 + lg * 8 + (v % 8);
+                    if (!(key >= lo[b] && key < hi[b])) s[b][v] = -INFINITY;
+                }
+        }
+        bf16x8 pb[QB][2];
+        float alpha[QB];
+        bool moved = false;
+#pragma unroll
+        for (int b = 0; b < QB; ++b) {
+            float mx = s[b][0];
+#pragma unroll
+            for (int v = 1; v < 16; ++v) mx = fmaxf(mx, s[b][v]);
+            mx = at_max_with_other_half(mx) * sl2;              // the scale is positive: max and scale commute
+            // The reference point of the exponentials follows the maximum only when that has grown by
+            // more than AP_MAX_SLACK (in powers of two): softmax does not care which point is taken, an
+            // exponential of up to 2^AP_MAX_SLACK is as exact in fp32 and bf16 as one below 1, and the
+            // outputs so far need no rescaling, which would otherwise be due in almost every tile
+            // (some query of the 64 finds a slightly larger score nearly every time).
+            const bool grow = mx > m_i[b] + AP_MAX_SLACK;       // (also from -inf to the first finite maximum)
+            const float m_new = grow ? mx : m_i[b];
+            const float m_use = m_new == -INFINITY ? 0.f : m_new;     // nothing visible yet: keep everything at zero
+            alpha[b] = grow ? __builtin_amdgcn_exp2f(m_i[b] - m_use) : 1.0f;
+            float rowsum = 0.f;
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
-                int key = key0 + (v / 8) * 16 + lg * 8 + (v % 8);
-                if (!(key >= lo && key < hi)) s[v] = -INFINITY;
+                float p = __builtin_amdgcn_exp2f(fmaf(s[b][v], sl2, -m_use));
+                rowsum += p;
+                pb[b][v / 8][v % 8] = (bf16_t)p;
             }
+            rowsum = at_sum_with_other_half(rowsum);
+            l_i[b] = l_i[b] * alpha[b] + rowsum;
+            m_i[b] = m_new;
+            moved = moved || alpha[b] != 1.0f;
         }
-        float mx = s[0];
+        if (__any(moved)) {
 #pragma unroll
-        for (int v = 1; v < 16; ++v) mx = fmaxf(mx, s[v]);
-        mx = fmaxf(mx, __shfl_xor(mx, 32, KA_WAVE)) * sl2;   // the scale is positive: max and scale commute
-        float m_new = fmaxf(m_i, mx);
-        float m_use = m_new == -INFINITY ? 0.f : m_new;     // nothing visible yet: keep everything at zero
-        float alpha = __builtin_amdgcn_exp2f(m_i - m_use);
-        float rowsum = 0.f;
-        bf16x8 pb[2];
+            for (int b = 0; b < QB; ++b)
 #pragma unroll
-        for (int v = 0; v < 16; ++v) {
-            float p = __builtin_amdgcn_exp2f(fmaf(s[v], sl2, -m_use));
-            rowsum += p;
-            pb[v / 8][v % 8] = (bf16_t)p;
-        }
-        rowsum += __shfl_xor(rowsum, 32, KA_WAVE);
-        l_i = l_i * alpha + rowsum;
-        m_i = m_new;
-        if (__any(alpha != 1.0f)) {
+                for (int db = 0; db < DB; ++db)
 #pragma unroll
-            for (int db = 0; db < DB; ++db)
-#pragma unroll
-                for (int v = 0; v < 16; ++v) o[db][v] *= alpha;
+                    for (int v = 0; v < 16; ++v) o[b][db][v] *= alpha[b];
         }
         // O^T[d][query] += V^T[d][key] P^T[key][query], one page per MFMA
         if (key0 + 32 > min(wave_hi, limit) || key0 < wave_lo) mask_values(key0, vr);
@@ -242,7 +316,9 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_
         for (int pg = 0; pg < 2; ++pg)
 #pragma unroll
             for (int db = 0; db < DB; ++db)
-                o[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vr[pg][db], pb[pg], o[db], 0, 0, 0);
+#pragma unroll
+                for (int b = 0; b < QB; ++b)
+                    o[b][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vr[pg][db], pb[b][pg], o[b][db], 0, 0, 0);
     };
 
     // two tiles per round, their key rows in two sets of registers: the next tile's keys are
@@ -257,48 +333,52 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_
         process(key0, kb, ka);
         key0 += STRIDE;
     }
-    // the waves took different keys of the same queries: merge in wave order
-    if (wave > 0) {
+    // the waves took different keys of the same queries: merge in wave order, a block of queries at a time
 #pragma unroll
-        for (int db = 0; db < DB; ++db)
+    for (int b = 0; b < QB; ++b) {
+        if (b > 0) __syncthreads();                        // the first block's sums have been read
+        if (wave > 0) {
 #pragma unroll
-            for (int v = 0; v < 16; ++v) mrg[wave - 1][db * 16 + v][lane] = o[db][v];
-        mrg[wave - 1][DB * 16][lane] = m_i;
-        mrg[wave - 1][DB * 16 + 1][lane] = l_i;
-    }
-    __syncthreads();
-    if (wave > 0 || !q_valid) return;
-    float M = m_i;
+            for (int db = 0; db < DB; ++db)
 #pragma unroll
-    for (int w = 0; w < AP_WAVES - 1; ++w) M = fmaxf(M, mrg[w][DB * 16][lane]);
-    float f0 = m_i == -INFINITY ? 0.f : exp2f(m_i - M);
-    float L = l_i * f0;
-#pragma unroll
-    for (int db = 0; db < DB; ++db)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) o[db][v] *= f0;
-#pragma unroll
-    for (int w = 0; w < AP_WAVES - 1; ++w) {
-        float mw = mrg[w][DB * 16][lane];
-        float f = mw == -INFINITY ? 0.f : exp2f(mw - M);
-        L += mrg[w][DB * 16 + 1][lane] * f;
-#pragma unroll
-        for (int db = 0; db < DB; ++db)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) o[db][v] += mrg[w][db * 16 + v][lane] * f;
-    }
-    float inv = L > 0.f ? 1.0f / L : 0.f;
-    bf16_t* op = out + (size_t)t * out_row_stride + (size_t)h * HD;
-#pragma unroll
-    for (int db = 0; db < DB; ++db)
-#pragma unroll
-        for (int qd = 0; qd < 4; ++qd) {
-            if (db * 32 + qd * 8 >= HD) continue;          // the unused half of the last block
-            int d = db * 32 + qd * 8 + lg * 4;
-            bf16x4 r = {(bf16_t)(o[db][qd * 4 + 0] * inv), (bf16_t)(o[db][qd * 4 + 1] * inv),
-                        (bf16_t)(o[db][qd * 4 + 2] * inv), (bf16_t)(o[db][qd * 4 + 3] * inv)};
-            *reinterpret_cast<bf16x4*>(op + d) = r;
+                for (int v = 0; v < 16; ++v) mrg[wave - 1][db * 16 + v][lane] = o[b][db][v];
+            mrg[wave - 1][DB * 16][lane] = m_i[b];
+            mrg[wave - 1][DB * 16 + 1][lane] = l_i[b];
         }
+        __syncthreads();
+        if (wave > 0 || !q_valid[b]) continue;
+        float M = m_i[b];
+#pragma unroll
+        for (int w = 0; w < AP_WAVES - 1; ++w) M = fmaxf(M, mrg[w][DB * 16][lane]);
+        float f0 = m_i[b] == -INFINITY ? 0.f : exp2f(m_i[b] - M);
+        float L = l_i[b] * f0;
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) o[b][db][v] *= f0;
+#pragma unroll
+        for (int w = 0; w < AP_WAVES - 1; ++w) {
+            float mw = mrg[w][DB * 16][lane];
+            float f = mw == -INFINITY ? 0.f : exp2f(mw - M);
+            L += mrg[w][DB * 16 + 1][lane] * f;
+#pragma unroll
+            for (int db = 0; db < DB; ++db)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) o[b][db][v] += mrg[w][db * 16 + v][lane] * f;
+        }
+        float inv = L > 0.f ? 1.0f / L : 0.f;
+        bf16_t* op = out + (size_t)t[b] * out_row_stride + (size_t)h * HD;
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int qd = 0; qd < 4; ++qd) {
+                if (db * 32 + qd * 8 >= HD) continue;          // the unused half of the last block
+                int d = db * 32 + qd * 8 + lg * 4;
+                bf16x4 r = {(bf16_t)(o[b][db][qd * 4 + 0] * inv), (bf16_t)(o[b][db][qd * 4 + 1] * inv),
+                            (bf16_t)(o[b][db][qd * 4 + 2] * inv), (bf16_t)(o[b][db][qd * 4 + 3] * inv)};
+                *reinterpret_cast<bf16x4*>(op + d) = r;
+            }
+    }
 }
 
 // ----------------------------------------------------------------------------------------------
@@ -809,16 +889,25 @@ KA_API int ka_attention_decode_supported(int hd, int page_size) {
     return page_size == AT_PAGE && at_head_size_covered(hd);
 }
 
+// Queries of one row that a workgroup of the prompt kernel takes at this head size: the blocks the
+// host lists (`qblk_row`, `qblk_tok`) must be cut to this size, or to 32, which every head size takes.
+KA_API int ka_attention_prefill_query_block(int hd) {
+    return at_head_size_covered(hd) && hd <= 64 ? 64 : 32;
+}
+
 KA_API int ka_attention_prefill_bf16(const void* q, long q_row_stride, const void* k_cache, const void* v_cache,
                                      const int* block_table, int max_pages, const int* qblk_row,
                                      const int* qblk_tok, int n_qblocks, const int* cu_q, const int* kv_len,
                                      const int* kv_lo, const int* kv_hi, void* out, long out_row_stride,
                                      float scale, int H, int Hkv, int hd, int page_size, int longest_row,
-                                     hipStream_t stream) {
+                                     int query_block, hipStream_t stream) {
     if (check_common("ka_attention_prefill_bf16", q, q_row_stride, out, out_row_stride, n_qblocks, H, Hkv, hd,
                      page_size, max_pages))
         return -1;
     KA_CHECK(ka_attention_prefill_supported(hd, page_size), "ka_attention_prefill_bf16: head size %d not covered", hd);
+    KA_CHECK(query_block == 32 || (query_block == 64 && ka_attention_prefill_query_block(hd) == 64),
+             "ka_attention_prefill_bf16: blocks of %d queries at head size %d (32%s)", query_block, hd,
+             ka_attention_prefill_query_block(hd) == 64 ? " or 64" : " only");
     // `longest_row`: no row of the launch holds more keys than this (0: not known, the whole
     // width of the block table is kept in LDS)
     int table_entries = max_pages;
@@ -828,34 +917,33 @@ KA_API int ka_attention_prefill_bf16(const void* q, long q_row_stride, const voi
     const size_t table_bytes = (size_t)table_entries * sizeof(int);
     KA_CHECK(n_qblocks <= 65535, "ka_attention_prefill_bf16: more than 65535 blocks of queries in one launch");
     dim3 grid(H, n_qblocks), block(KA_WAVE * AP_WAVES);
-#define KA_AP(HDV)                                                                                                  \
+#define KA_AP_LAUNCH(HDV, QBV)                                                                                      \
     {                                                                                                               \
         static bool configured = false;                                                                             \
         if (!configured) {                                                                                          \
-            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(attn_prefill_kernel<HDV>),             \
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(attn_prefill_kernel<HDV, QBV>),        \
                                                hipFuncAttributeMaxDynamicSharedMemorySize, ap_max_table(HDV) * sizeof(int)); \
             KA_CHECK(e == hipSuccess, "ka_attention_prefill_bf16: cannot reserve LDS: %s", hipGetErrorString(e));   \
             configured = true;                                                                                      \
         }                                                                                                           \
-    }                                                                                                               \
-    hipLaunchKernelGGL(attn_prefill_kernel<HDV>, grid, block, table_bytes, stream, (const bf16_t*)q, q_row_stride,  \
-                       (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, max_pages, qblk_row, qblk_tok,  \
-                       cu_q, kv_len, kv_lo, kv_hi, (bf16_t*)out, out_row_stride, scale, H, Hkv, table_entries)
+        hipLaunchKernelGGL((attn_prefill_kernel<HDV, QBV>), grid, block, table_bytes, stream, (const bf16_t*)q,     \
+                           q_row_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, max_pages,    \
+                           qblk_row, qblk_tok, cu_q, kv_len, kv_lo, kv_hi, (bf16_t*)out, out_row_stride, scale, H,  \
+                           Hkv, table_entries);                                                                     \
+    }
+#define KA_AP(HDV)                                                                                                  \
+    case HDV:                                                                                                       \
+        if (query_block == 64) KA_AP_LAUNCH(HDV, 2) else KA_AP_LAUNCH(HDV, 1)                                       \
+        break;
+#define KA_AP1(HDV) \
+    case HDV: KA_AP_LAUNCH(HDV, 1) break;
     switch (hd) {
-        case 16: KA_AP(16); break;
-        case 32: KA_AP(32); break;
-        case 48: KA_AP(48); break;
-        case 64: KA_AP(64); break;
-        case 80: KA_AP(80); break;
-        case 96: KA_AP(96); break;
-        case 112: KA_AP(112); break;
-        case 128: KA_AP(128); break;
-        case 160: KA_AP(160); break;
-        case 192: KA_AP(192); break;
-        case 224: KA_AP(224); break;
-        default: KA_AP(256); break;
+        KA_AP(16) KA_AP(32) KA_AP(48) KA_AP(64)
+        KA_AP1(80) KA_AP1(96) KA_AP1(112) KA_AP1(128) KA_AP1(160) KA_AP1(192) KA_AP1(224) KA_AP1(256)
     }
 #undef KA_AP
+#undef KA_AP1
+#undef KA_AP_LAUNCH
     KA_LAUNCH_CHECK();
     return 0;
 }

@@ -72,8 +72,9 @@ class StepBatch:
     logit_rows: torch.Tensor            # int32 [wanted]
     groups: Dict[int, GroupBatch]
     workspace: Workspace
-    qblk_row: Optional[torch.Tensor] = None       # int32 [blocks]: row of each block of 32 queries
-    qblk_tok: Optional[torch.Tensor] = None       # int32 [blocks]: its first token
+    # per size of block that a mixer's kernel asked for: (int32 [blocks] row of each block of that
+    # many queries of one row, int32 [blocks] its first token), the blocks that see the most keys first
+    query_blocks: Dict[int, Tuple[torch.Tensor, torch.Tensor]] = field(default_factory=dict)
     pending: Optional[torch.Tensor] = None        # int32 device table: an id <= -2 stands for pending[-2 - id]
     given_embeds: Optional[torch.Tensor] = None   # [m, dim]
     given_rows: Optional[torch.Tensor] = None     # int32 [m] token indices they go to

@@ -125,7 +125,6 @@ class ModelRunner:
 
     STAGING_RING = 4
     SCALAR_ROW = 16          # rows of at most this many tokens are laid out token by token, longer ones as arrays
-    QUERY_BLOCK = 32         # queries of one row a workgroup of the prompt attention kernel takes
 
     def __init__(self, model: DecoderModel, cache: CacheManager, device: torch.device,
                  max_tokens_per_step: int = 4096, enable_graphs: bool = False,
@@ -146,6 +145,10 @@ class ModelRunner:
         self.graph_replays = 0
         # the latest sampled token of every request slot, written by the sampling kernels
         self.pending = torch.zeros(max(1, cache.max_requests), dtype=torch.int32, device=device)
+        # Sizes of the blocks of queries that the mixers' kernels want a row cut into (a mixer says
+        # so through ``query_tile()``): the step lists the blocks of each size, most keys first.
+        tiles = getattr(model, "query_tiles", None)
+        self.query_tiles: List[int] = sorted(tiles()) if callable(tiles) else []
 
     # ------------------------------------------------------------------ requests
     def admit(self, reserve_length: int = 0, portion: int = 1) -> int:
@@ -247,7 +250,8 @@ class ModelRunner:
 
         n_groups = len(cache.groups)
         ids, positions, token_row, kv_hi = _Column(), _Column(), _Column(), _Column()
-        blocks: List[Tuple[int, int, int]] = []      # of queries: row, first token, most keys any of them sees
+        # blocks of queries, per size: row, first token, most keys any of them sees
+        blocks: Dict[int, List[Tuple[int, int, int]]] = {tile: [] for tile in self.query_tiles}
         logit_rows: List[int] = []
         given_rows: List[int] = []
         given: List[torch.Tensor] = []
@@ -301,14 +305,14 @@ class ModelRunner:
                 positions.extend(np.arange(start, start + q, dtype=np.int64))
                 token_row.extend(np.full(q, r, dtype=np.int64))
             kv_hi.extend(hi)
-            if isinstance(hi, np.ndarray):
-                # most keys any query of a block sees: the blocks' maxima in one go
-                pad = (-q) % self.QUERY_BLOCK
-                tops = np.pad(hi, (0, pad)).reshape(-1, self.QUERY_BLOCK).max(axis=1).tolist()
-                blocks.extend((r, base + i * self.QUERY_BLOCK, top) for i, top in enumerate(tops))
-            else:
-                for first in range(0, q, self.QUERY_BLOCK):
-                    blocks.append((r, base + first, max(hi[first:first + self.QUERY_BLOCK])))
+            for tile, listed in blocks.items():
+                if isinstance(hi, np.ndarray):
+                    # most keys any query of a block sees: the blocks' maxima in one go
+                    tops = np.pad(hi, (0, (-q) % tile)).reshape(-1, tile).max(axis=1).tolist()
+                    listed.extend((r, base + i * tile, top) for i, top in enumerate(tops))
+                else:
+                    for first in range(0, q, tile):
+                        listed.append((r, base + first, max(hi[first:first + tile])))
             logit_rows.extend(base + int(w) for w in e.want)
             cu_q.append(base + q)
             kv_len.append(start + q)
@@ -332,7 +336,8 @@ class ModelRunner:
             positions.append(0)
             token_row.append(r)
             kv_hi.append(0)
-            blocks.append((r, len(ids) - 1, 0))
+            for listed in blocks.values():
+                listed.append((r, len(ids) - 1, 0))
             logit_rows.append(len(ids) - 1)
             cu_q.append(len(ids))
             kv_len.append(0)
@@ -344,19 +349,18 @@ class ModelRunner:
         n_rows = max(n_real, pad_rows)
         n_tokens = len(ids)
 
-        qblk_row: List[int] = []
-        qblk_tok: List[int] = []
         # the blocks that see the most keys first: a launch then ends with short ones
-        blocks.sort(key=lambda b: -b[2])
-        for r, first, _ in blocks:
-            qblk_row.append(r)
-            qblk_tok.append(first)
+        for listed in blocks.values():
+            listed.sort(key=lambda b: -b[2])
         # one packed int32 buffer, every section starting on a 16-byte boundary
         sections: List[Tuple[str, object]] = [
             ("ids", ids), ("positions", positions), ("token_row", token_row), ("kv_hi", kv_hi),
             ("row_slot", row_slot), ("cu_q", cu_q), ("kv_len", kv_len), ("logit_rows", logit_rows),
-            ("given_rows", given_rows), ("qblk_row", qblk_row), ("qblk_tok", qblk_tok),
+            ("given_rows", given_rows),
         ]
+        for tile, listed in blocks.items():
+            sections.append((f"qblk_row{tile}", [b[0] for b in listed]))
+            sections.append((f"qblk_tok{tile}", [b[1] for b in listed]))
         for g in range(n_groups):
             sections.append((f"slots{g}", slots[g]))
             if kv_lo[g] is not None:
@@ -409,7 +413,8 @@ class ModelRunner:
             n_tokens=n_tokens, n_rows=n_rows, token_ids=view("ids"), positions=view("positions"),
             token_row=view("token_row"), kv_hi=view("kv_hi"), row_slot=view("row_slot"), cu_q=view("cu_q"),
             kv_len=view("kv_len"), logit_rows=view("logit_rows"), groups=groups,
-            workspace=workspace or self.workspace, qblk_row=view("qblk_row"), qblk_tok=view("qblk_tok"),
+            workspace=workspace or self.workspace,
+            query_blocks={tile: (view(f"qblk_row{tile}"), view(f"qblk_tok{tile}")) for tile in blocks},
             pending=self.pending, given_embeds=given_embeds, given_rows=view("given_rows") if given else None, max_q=max_q, max_kv=max_kv,
             decode_only=max_q == 1, causal_only=causal_only,
             host={"starts": starts, "q_lens": [len(e.tokens) for e in entries], "kv_len": kv_len, "meta_ints": total},

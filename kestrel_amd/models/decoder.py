@@ -74,6 +74,10 @@ class DecoderModel:
             needs.append((mixer.cache_spec(), mixer.state_spec(), entry.reads_cache_of))
         return needs
 
+    def query_tiles(self):
+        """Sizes of blocks of queries that the mixers' kernels want listed with a step."""
+        return {tile for tile in (block.mixer.query_tile() for block in self.blocks) if tile}
+
     # ------------------------------------------------------------------ forward
     def forward(self, batch, caches: List[LayerCache]) -> torch.Tensor:
         """Run the packed tokens of ``batch``; returns fp32 logits ``[wanted, vocab]``."""

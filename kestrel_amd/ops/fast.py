@@ -30,7 +30,7 @@ _SIGNATURES = {
                              _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_long, _c_void_p],
     "ka_attention_prefill_bf16": [_c_void_p, _c_long, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p,
                                   _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_long, _c_float,
-                                  _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
+                                  _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
     "ka_rope_cache_pages_bf16": [_c_void_p, _c_long, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p,
                                  _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
     "ka_attention_decode_bf16": [_c_void_p, _c_long, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p,
@@ -84,8 +84,9 @@ def lib():
         for name in ("ka_attention_prefill_supported", "ka_attention_decode_supported"):
             getattr(handle, name).argtypes = [_c_int, _c_int]
             getattr(handle, name).restype = _c_int
-        handle.ka_attention_prefill_max_keys.argtypes = [_c_int]
-        handle.ka_attention_prefill_max_keys.restype = _c_int
+        for name in ("ka_attention_prefill_max_keys", "ka_attention_prefill_query_block"):
+            getattr(handle, name).argtypes = [_c_int]
+            getattr(handle, name).restype = _c_int
         _lib = handle
     return _lib
 
@@ -315,6 +316,26 @@ def attention_decode_bf16(q, k_cache, v_cache, block_table, token_row, kv_lo, kv
     return True
 
 
+def prefill_query_block(head_dim: int) -> int:
+    """Queries of one row that a workgroup of the prompt attention kernel takes at this head size:
+    the size the step's lists of blocks of queries must be cut to for it."""
+    return int(lib().ka_attention_prefill_query_block(head_dim))
+
+
+def _query_blocks(batch, head_dim: int):
+    """``(rows, first tokens, size)`` of the blocks of queries of a step, at the size the kernel likes
+    best among those the step lists (``batch.query_blocks``: size -> lists), else at 32."""
+    listed = getattr(batch, "query_blocks", None) or {}
+    best = prefill_query_block(head_dim)
+    if best in listed:
+        return (*listed[best], best)
+    if 32 in listed:
+        return (*listed[32], 32)
+    if getattr(batch, "qblk_row", None) is not None:
+        return batch.qblk_row, batch.qblk_tok, 32
+    return None
+
+
 def attention_bf16(q, k_cache, v_cache, block_table, token_row, kv_lo, kv_hi, out, scale, n_heads, n_kv_heads,
                    head_dim, batch) -> bool:
     n = q.shape[0]
@@ -329,13 +350,14 @@ def attention_bf16(q, k_cache, v_cache, block_table, token_row, kv_lo, kv_hi, ou
     handle = lib()
     # the longest row's block table must fit in LDS (the whole table's width where the length is not known)
     longest = int(batch.max_kv) if batch.max_kv > 1 else block_table.shape[1] * page_size
-    if handle.ka_attention_prefill_supported(head_dim, page_size) and batch.qblk_row is not None \
-            and longest <= handle.ka_attention_prefill_max_keys(head_dim):
+    blocks = _query_blocks(batch, head_dim) if handle.ka_attention_prefill_supported(head_dim, page_size) else None
+    if blocks is not None and longest <= handle.ka_attention_prefill_max_keys(head_dim):
+        rows, first_tokens, size = blocks
         _check(handle.ka_attention_prefill_bf16(
             q.data_ptr(), q.stride(0), k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(),
-            block_table.shape[1], batch.qblk_row.data_ptr(), batch.qblk_tok.data_ptr(), int(batch.qblk_row.numel()),
+            block_table.shape[1], rows.data_ptr(), first_tokens.data_ptr(), int(rows.numel()),
             batch.cu_q.data_ptr(), batch.kv_len.data_ptr(), _ptr(kv_lo), kv_hi.data_ptr(), out.data_ptr(),
             out.stride(0), float(scale), n_heads, n_kv_heads, head_dim, page_size,
-            int(batch.max_kv) if batch.max_kv > 1 else 0, stream_ptr()))
+            int(batch.max_kv) if batch.max_kv > 1 else 0, size, stream_ptr()))
         return True
     return False

@@ -79,6 +79,12 @@ class PagedAttention(Mixer):
         else:
             self._table, self._pairing = None, "halves"
 
+    def query_tile(self) -> Optional[int]:
+        if self.dtype != torch.bfloat16:
+            return None                     # the generic kernel takes tokens one by one
+        from ..ops import fast
+        return fast.prefill_query_block(self.spec.head_dim)
+
     # The three stages are also offered one by one, so that a block may fuse the first with its
     # norm and the last with its feed-forward (see ``Mixer.input_projection``).
     def input_projection(self):

@@ -99,6 +99,12 @@ class Mixer(Part):
         """Fixed-size state kept per request, or ``None``."""
         return None
 
+    def query_tile(self) -> Optional[int]:
+        """If the mixer's kernel wants the queries of a row in blocks of a size of its own: that
+        size. The step then lists the blocks of that size in ``StepBatch.query_blocks[size]``
+        (called after ``bind``: the size may depend on the precision)."""
+        return None
+
     def forward(self, h: torch.Tensor, batch, cache: LayerCache, residual: torch.Tensor) -> None:
         """Add the mixer's output for the normalised input ``h`` into fp32 ``residual``."""
         raise NotImplementedError

@@ -378,17 +378,16 @@ class PagedCase:
             cu_q.append(len(token_row))
         n = len(token_row)
         self.q = torch.randn(n, h * hd, generator=gen).to(dtype)
-        qblk_row, qblk_tok = [], []
-        for r in range(n_rows):
-            for first in range(cu_q[r], cu_q[r + 1], 32):
-                qblk_row.append(r)
-                qblk_tok.append(first)
         i32 = lambda xs: torch.tensor(xs, dtype=torch.int32, device=DEV)
+        query_blocks = {}                            # blocks of 32 and of 64 queries of a row: (rows, first tokens)
+        for size in (32, 64):
+            listed = [(r, first) for r in range(n_rows) for first in range(cu_q[r], cu_q[r + 1], size)]
+            query_blocks[size] = (i32([r for r, _ in listed]), i32([first for _, first in listed]))
         self.token_row, self.kv_hi = i32(token_row), i32(kv_hi)
         self.kv_lo = i32(kv_lo) if window else None
         self.table, self.k_cache, self.v_cache = table.to(DEV), k_cache.to(DEV), v_cache.to(DEV)
         self.batch = SimpleNamespace(decode_only=all(ql == 1 for ql in q_lens), max_kv=max(kv_lens), cu_q=i32(cu_q),
-                                     kv_len=i32(kv_lens), qblk_row=i32(qblk_row), qblk_tok=i32(qblk_tok))
+                                     kv_len=i32(kv_lens), query_blocks=query_blocks)
         self.lists = (token_row, kv_lo if window else [0] * n, kv_hi)
 
     def reference(self, scale):
@@ -416,6 +415,13 @@ def _run_attention(case, fn_name, scale):
     else:
         assert fast.attention_bf16(q, case.k_cache, case.v_cache, case.table, case.token_row, case.kv_lo, case.kv_hi,
                                    out, scale, case.h, case.hkv, case.hd, case.batch)
+        if not case.batch.decode_only and fast.prefill_query_block(case.hd) != 32:
+            # the prompt kernel took blocks of 64 queries: the same through its form for blocks of 32
+            narrow = SimpleNamespace(**{**vars(case.batch), "query_blocks": {32: case.batch.query_blocks[32]}})
+            again = torch.full_like(out, float("nan"))
+            assert fast.attention_bf16(q, case.k_cache, case.v_cache, case.table, case.token_row, case.kv_lo, case.kv_hi,
+                                       again, scale, case.h, case.hkv, case.hd, narrow)
+            _close(again, out, case.dtype, scale=0.5)
     return out
 
 
