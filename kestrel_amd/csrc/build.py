@@ -30,9 +30,9 @@ ARCH = "gfx950"
 # bf16 MFMA kernels of serving.
 LIBRARIES: Dict[str, List[str]] = {
     "core": ["ka_error.hip", "elementwise.hip", "gemm_generic.hip", "attention_generic.hip", "sampling.hip", "peaks.hip"],
-    "fast": ["ka_error.hip", "gemm_bf16.hip", "gemv_bf16.hip", "attention_bf16.hip"],
+    "fast": ["ka_error.hip", "gemm_bf16.hip", "gemv_bf16.hip", "attention_bf16.hip", "decode_beside.hip"],
 }
-HEADERS = ["ka_common.h", "ka_partials.h", "ka_no_alloc.h"]
+HEADERS = ["ka_common.h", "ka_partials.h", "ka_no_alloc.h", "ka_attention_decode.h", "ka_skinny.h"]
 
 HIPCC_FLAGS = [
     f"--offload-arch={ARCH}", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",

@@ -38,6 +38,12 @@ _SIGNATURES = {
                                  _c_int, _c_int, _c_void_p, _c_long,
                                  _c_void_p, _c_void_p, _c_long, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p,
                                  _c_void_p],
+    "ka_attention_decode_beside_bf16": [
+        _c_void_p, _c_long, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_long,
+        _c_float, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_long,                # ..., splits, partial sums
+        _c_void_p, _c_void_p, _c_long, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p,          # the tokens' own keys and values
+        _c_void_p, _c_void_p, _c_void_p, _c_float, _c_int,                                          # ln_x, gamma, beta, eps, K
+        _c_void_p, _c_long, _c_void_p, _c_void_p, _c_int, _c_long, _c_int, _c_int, _c_void_p],      # W, ldw, bias, out, ..., stream
 }
 
 # Rows up to which the weight-streaming kernel is used instead of the tiled one.
@@ -49,6 +55,11 @@ SKINNY_LN_MAX_WIDTH = 4096
 # the persistent kernel then repeats the LayerNorm of all rows once; with a few hundred workgroups
 # that is cheaper than a launch of its own (measured on MI355X: 3 % of a decode step at batch 8).
 FUSE_LAYERNORM_PROLOGUE = True
+# Whether the decode attention of a few rows (whose workgroups fill at most a quarter of the chip)
+# takes the feed-forward's first linear into its own launch instead of leaving it to the launch of
+# the q|k|v projection before it (measured on MI355X at Moondream 2's sizes: 3 to 5 % of a decode
+# step at batch 1 to 4).
+ATTENTION_TAKES_LINEAR = True
 # Tile of the tiled kernels: 0 lets them choose by size; 221, 211 (any K), 12222, 23212, 22224, 22232, 13122
 # (K in steps of 64 or 32, loads straight into LDS) force one, and 1000000 * parts + 23212 forces K to be cut into
 # that many parts as well (for measurements and tests).
@@ -84,6 +95,8 @@ def lib():
         for name in ("ka_attention_prefill_supported", "ka_attention_decode_supported"):
             getattr(handle, name).argtypes = [_c_int, _c_int]
             getattr(handle, name).restype = _c_int
+        handle.ka_attention_decode_beside_supported.argtypes = [_c_int] * 6
+        handle.ka_attention_decode_beside_supported.restype = _c_int
         for name in ("ka_attention_prefill_max_keys", "ka_attention_prefill_query_block"):
             getattr(handle, name).argtypes = [_c_int]
             getattr(handle, name).restype = _c_int
@@ -282,17 +295,47 @@ def _attention_operands_ok(q, out) -> bool:
     return not (q.data_ptr() % 16 or q.stride(0) % 8 or out.data_ptr() % 16 or out.stride(0) % 4)
 
 
+def _norm_linear_ok(job) -> bool:
+    """Operands of a ``parts.NormLinear`` that the persistent kernel's LayerNorm prologue takes."""
+    x, w, out = job.x, job.linear_weight, job.out
+    m, k = x.shape
+    if x.dtype != torch.float32 or not x.is_contiguous() or x.data_ptr() % 16 or k % 8:
+        return False
+    for vec in (job.norm_weight, job.norm_bias):
+        if vec is not None and (vec.dtype != torch.float32 or vec.numel() != k or vec.data_ptr() % 16):
+            return False
+    if job.norm_weight is None:
+        return False
+    n = w.shape[0]
+    if not (_operand_ok(w, k) and _out_ok(out, m, n) and _bias_ok(job.linear_bias, n)):
+        return False
+    return job.linear_bias is None or (n % 4 == 0 and job.linear_bias.data_ptr() % 16 == 0)
+
+
+def attention_decode_takes(job, n: int, n_heads: int, head_dim: int, page_size: int, max_kv: int) -> bool:
+    """Whether ``attention_decode_bf16`` runs ``job`` (a ``parts.NormLinear``) in its own launch: a few
+    rows whose attention leaves most of the chip idle."""
+    if not ATTENTION_TAKES_LINEAR or n == 0 or not _norm_linear_ok(job):
+        return False
+    splits = decode_shape(max_kv, n * n_heads)[0]
+    return bool(lib().ka_attention_decode_beside_supported(n, n_heads, splits, head_dim, page_size, job.x.shape[1]))
+
+
 def attention_decode_bf16(q, k_cache, v_cache, block_table, token_row, kv_lo, kv_hi, out, scale, n_heads,
-                          n_kv_heads, head_dim, batch, fuse=None) -> bool:
+                          n_kv_heads, head_dim, batch, fuse=None, beside=None) -> bool:
     """One token per row. ``fuse = (k_new, v_new, table, slots)``: the kernel also rotates q and the
-    token's key and stores key and value in the cache (the rotary kernel is then not run)."""
+    token's key and stores key and value in the cache (the rotary kernel is then not run).
+    ``beside``: a ``parts.NormLinear`` for which ``attention_decode_takes`` said yes; the launch
+    computes it on the side (False: it does not after all, and nothing was run)."""
     n = q.shape[0]
     page_size = k_cache.shape[2]
     if n == 0:
-        return True
+        return beside is None
     handle = lib()
     if batch is None or not batch.decode_only or not _attention_operands_ok(q, out) \
             or not handle.ka_attention_decode_supported(head_dim, page_size):
+        return False
+    if beside is not None and not attention_decode_takes(beside, n, n_heads, head_dim, page_size, batch.max_kv):
         return False
     splits, waves = decode_shape(batch.max_kv, n * n_heads)
     partial = scratch(q.device)
@@ -307,6 +350,17 @@ def attention_decode_bf16(q, k_cache, v_cache, block_table, token_row, kv_lo, kv
         if rot % 16 or rot > head_dim or k_new.data_ptr() % 16 or v_new.data_ptr() % 16 \
                 or new_stride % 8 or v_new.stride(0) != new_stride:
             return False
+    if beside is not None:
+        w, lin_out = beside.linear_weight, beside.out
+        _check(handle.ka_attention_decode_beside_bf16(
+            q.data_ptr(), q.stride(0), k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(),
+            block_table.shape[1], token_row.data_ptr(), _ptr(kv_lo), kv_hi.data_ptr(), out.data_ptr(), out.stride(0),
+            float(scale), n, n_heads, n_kv_heads, head_dim, page_size, splits, partial.data_ptr(), partial.numel(),
+            _ptr(k_new), _ptr(v_new), new_stride, _ptr(table), rot, _ptr(slots), k_cache.data_ptr(), v_cache.data_ptr(),
+            beside.x.data_ptr(), beside.norm_weight.data_ptr(), _ptr(beside.norm_bias), float(beside.eps),
+            beside.x.shape[1], w.data_ptr(), w.stride(0), _ptr(beside.linear_bias), lin_out.data_ptr(),
+            _OUT_CODE[lin_out.dtype], lin_out.stride(0), w.shape[0], int(beside.act), stream_ptr()))
+        return True
     _check(handle.ka_attention_decode_bf16(
         q.data_ptr(), q.stride(0), k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(),
         block_table.shape[1], token_row.data_ptr(), _ptr(kv_lo), kv_hi.data_ptr(), out.data_ptr(), out.stride(0),

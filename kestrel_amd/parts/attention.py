@@ -93,22 +93,42 @@ class PagedAttention(Mixer):
     def output_projection(self):
         return self.proj_weight, self.proj_bias
 
-    def attend(self, qkv, batch, cache: LayerCache):
+    def _decodes_fused(self, batch, cache: LayerCache) -> bool:
+        """One token per row in bf16 with a rotation by halves: the decode kernel then rotates q and
+        k and stores k and v itself."""
+        return self.dtype == torch.bfloat16 and batch.decode_only and cache.writes and self._table is not None \
+            and self._pairing == "halves"          # the MFMA-path kernels turn halves; the generic one any pairing
+
+    def takes_beside(self, job, batch, cache: LayerCache) -> bool:
+        if not self._decodes_fused(batch, cache):
+            return False
+        from ..ops import fast
+        return fast.attention_decode_takes(job, job.x.shape[0], self.spec.n_heads, self.spec.head_dim, cache.k.shape[2],
+                                           batch.max_kv)
+
+    def attend(self, qkv, batch, cache: LayerCache, beside=None):
         """Position encoding, cache write and attention on the projected input ``[n, q|k|v]``."""
         spec = self.spec
         n = qkv.shape[0]
         group = batch.groups[cache.group]
         out = batch.workspace.get("attn.out", (n, self.q_dim), self.dtype)
-        halves = self._pairing == "halves"          # the MFMA-path kernels turn halves; the generic one any pairing
-        if qkv.dtype == torch.bfloat16 and batch.decode_only and cache.writes and self._table is not None and halves:
-            # one token per row: the decode kernel rotates q and k and stores k and v itself
+        halves = self._pairing == "halves"
+        if qkv.dtype == torch.bfloat16 and self._decodes_fused(batch, cache):
             from ..ops import fast
             k_new = qkv[:, self.q_dim:self.q_dim + self.kv_dim]
             v_new = qkv[:, self.q_dim + self.kv_dim:]
-            if fast.attention_decode_bf16(qkv, cache.k, cache.v, group.block_table, batch.token_row, group.kv_lo,
-                                          batch.kv_hi, out, self.scale, spec.n_heads, spec.n_kv_heads, spec.head_dim,
-                                          batch, fuse=(k_new, v_new, self._table, group.slots)):
+            operands = (qkv, cache.k, cache.v, group.block_table, batch.token_row, group.kv_lo, batch.kv_hi, out,
+                        self.scale, spec.n_heads, spec.n_kv_heads, spec.head_dim, batch)
+            fuse = (k_new, v_new, self._table, group.slots)
+            if beside is not None and fast.attention_decode_bf16(*operands, fuse=fuse, beside=beside):
                 return out
+            if beside is not None:
+                self._alone(beside)
+                beside = None
+            if fast.attention_decode_bf16(*operands, fuse=fuse):
+                return out
+        if beside is not None:
+            self._alone(beside)
         slots = group.slots if cache.writes else None
         done = False
         if qkv.dtype == torch.bfloat16 and halves:
@@ -121,6 +141,14 @@ class PagedAttention(Mixer):
         paged_attention(qkv, cache.k, cache.v, group.block_table, batch.token_row, group.kv_lo, batch.kv_hi, out,
                         self.scale, spec.n_heads, spec.n_kv_heads, spec.head_dim, batch)
         return out
+
+    @staticmethod
+    def _alone(job) -> None:
+        """A job that was promised a place in the attention launch and did not get one after all."""
+        from ..ops import fast
+        if not fast.layernorm_linear(job.x, job.norm_weight, job.norm_bias, job.eps, job.linear_weight,
+                                     job.linear_bias, job.out, job.act):
+            raise RuntimeError("a linear layer accepted for the attention launch is taken by no kernel")
 
     def forward(self, h, batch, cache: LayerCache, residual) -> None:
         qkv = batch.workspace.get("attn.qkv", (h.shape[0], self.qkv_dim), self.dtype)

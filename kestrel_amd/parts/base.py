@@ -90,6 +90,23 @@ class LayerCache:
         return self.tensors.get("v")
 
 
+@dataclass
+class NormLinear:
+    """``out = act(LayerNorm(x; weight, bias, eps) @ linear_weight.T + linear_bias)``: a piece of a
+    block's work that depends on nothing the mixer computes (the first linear of a feed-forward that
+    reads the same normalised input). A mixer that says so (``Mixer.takes_beside``) is handed it with
+    ``attend`` and runs it in its own launch, on the compute units that its core leaves idle."""
+
+    x: torch.Tensor                       # fp32 [n, dim]: the residual
+    norm_weight: torch.Tensor
+    norm_bias: Optional[torch.Tensor]
+    eps: float
+    linear_weight: torch.Tensor           # [out, dim]
+    linear_bias: Optional[torch.Tensor]
+    out: torch.Tensor                     # [n, out]
+    act: int                              # activation code of ``ops.linear``
+
+
 class Mixer(Part):
     def cache_spec(self) -> Optional[CacheSpec]:
         """Keys and values kept per token, or ``None``."""
@@ -117,9 +134,14 @@ class Mixer(Part):
         """``(weight [out, in], bias or None, out)`` of the first linear, or ``None``."""
         return None
 
-    def attend(self, projected: torch.Tensor, batch, cache: LayerCache) -> torch.Tensor:
-        """The core on the projected input; returns the input of the output projection."""
+    def attend(self, projected: torch.Tensor, batch, cache: LayerCache, beside: Optional[NormLinear] = None) -> torch.Tensor:
+        """The core on the projected input; returns the input of the output projection. ``beside``
+        is only ever given after ``takes_beside`` said yes, and is done when this returns."""
         raise NotImplementedError
+
+    def takes_beside(self, job: NormLinear, batch, cache: LayerCache) -> bool:
+        """Whether ``attend`` would run ``job`` inside its own launch for this batch."""
+        return False
 
     def output_projection(self):
         """``(weight, bias or None)`` of the last linear, whose result is added to the residual."""

@@ -6,7 +6,7 @@ from typing import Callable, Dict, Optional
 
 import torch
 
-from .base import LayerCache, Part, build_part
+from .base import LayerCache, NormLinear, Part, build_part
 from .specs import LayerSpec, ParamSpec
 
 
@@ -29,16 +29,25 @@ def _parallel_few_rows(block: "Block", x, batch, cache) -> bool:
     hidden = ws.get("block.ff_hidden", (n, f_in[2]), block.dtype)
     norm = block.norm
     fused = False
+    beside = None
     if fast.FUSE_LAYERNORM_PROLOGUE and getattr(norm.spec, "kind", None) == "layernorm":
-        fused = fast.layernorm_linear_pair(x, norm.weight, norm.bias, norm.spec.eps, m_in[0], m_in[1], projected, 0,
-                                           f_in[0], f_in[1], hidden, f_in[3])
+        # the feed-forward's first linear goes into the mixer's launch where the mixer takes it,
+        # else into the launch of the mixer's first linear
+        job = NormLinear(x, norm.weight, norm.bias, norm.spec.eps, f_in[0], f_in[1], hidden, f_in[3])
+        if block.mixer.takes_beside(job, batch, cache) and \
+                fast.layernorm_linear(x, norm.weight, norm.bias, norm.spec.eps, m_in[0], m_in[1], projected, 0):
+            fused, beside = True, job
+        else:
+            fused = fast.layernorm_linear_pair(x, norm.weight, norm.bias, norm.spec.eps, m_in[0], m_in[1], projected, 0,
+                                               f_in[0], f_in[1], hidden, f_in[3])
     if not fused:
         h = ws.get("block.h", tuple(x.shape), block.dtype)
         norm.forward(x, h)
         if not fast.linear_two_outputs(h, m_in[0], m_in[1], projected, 0, f_in[0], f_in[1], hidden, f_in[3]):
             linear(h, m_in[0], m_in[1], projected)
             linear(h, f_in[0], f_in[1], hidden, act=f_in[3])
-    mixed = block.mixer.attend(projected, batch, cache)
+    mixed = block.mixer.attend(projected, batch, cache, beside) if beside is not None \
+        else block.mixer.attend(projected, batch, cache)
     if not fast.linear_pair_accumulate(mixed, m_out[0], m_out[1], hidden, f_out[0], f_out[1], x):
         linear(mixed, m_out[0], m_out[1], x, accumulate=True)
         linear(hidden, f_out[0], f_out[1], x, accumulate=True)

@@ -767,6 +767,81 @@ def test_decode_attention_that_rotates_and_stores(shape):
         assert torch.equal(v_f[page, :, :, off], v_ref[page, :, :, off])
 
 
+@pytest.mark.parametrize("keys_per_workgroup", [4096, 256])
+@pytest.mark.parametrize("shape", [(4, 4, 64, 32, 2048, 8192, 1), (6, 2, 48, 16, 200, 100, 0), (16, 16, 64, 32, 2048, 1000, 3),
+                                   (2, 1, 16, 16, 1032, 24, 2), (3, 3, 32, 32, 64, 4100, 1)])
+def test_decode_attention_with_a_linear_layer_beside_it(shape, keys_per_workgroup, monkeypatch):
+    """One launch computes the decode attention (rotating and storing the tokens' own keys) and, in
+    other workgroups, a LayerNorm + linear of the same rows. Both results are, bit for bit, what the
+    two kernels give alone (attention with the same 8 waves a workgroup), and so is the cache."""
+    from kestrel_amd.ops import fast
+    from kestrel_amd.parts import NormLinear
+
+    h, hkv, hd, rot, k, n_out, act = shape
+    bf = torch.bfloat16
+    monkeypatch.setattr(fast, "DECODE_KEYS_PER_WORKGROUP", keys_per_workgroup)
+    shape_of = fast.decode_shape
+    monkeypatch.setattr(fast, "decode_shape", lambda max_kv, workgroups=1: (shape_of(max_kv, workgroups)[0], 8))
+    for kv_lens in ([1024, 16, 17, 300, 1], [700], [1000, 64, 65, 129, 2, 5, 33, 48]):
+        # (as many rows as leave attention within the quarter of a 256-CU chip's places that the launch takes)
+        kv_lens = kv_lens[:max(1, 128 // (h * shape_of(max(kv_lens))[0]))]
+        case = PagedCase(kv_lens, [1] * len(kv_lens), h, hkv, hd, 16, bf, seed=31)
+        n = len(kv_lens)
+        torch.manual_seed(32)
+        qkv = torch.randn(n, (h + 2 * hkv) * hd).to(bf).to(DEV)
+        slots = torch.tensor([int(case.table[r, (kv - 1) // 16]) * 16 + (kv - 1) % 16 for r, kv in enumerate(kv_lens)],
+                             dtype=torch.int32, device=DEV)
+        table = plain.rotary_table(rot, 2048, 10000.0, torch.float32).to(DEV)
+        x = (torch.randn(n, k) * 2 + 0.3).to(DEV)
+        gamma, beta = (1 + 0.1 * torch.randn(k)).to(DEV), (0.1 * torch.randn(k)).to(DEV)
+        w = (torch.randn(n_out, k) / k ** 0.5).bfloat16().to(DEV)
+        bias = torch.randn(n_out).to(DEV)
+        q_dim, kv_dim = h * hd, hkv * hd
+
+        def run(beside):
+            rows, k_c, v_c = qkv.clone(), case.k_cache.clone(), case.v_cache.clone()
+            out = torch.empty(n, q_dim, dtype=bf, device=DEV)
+            assert fast.attention_decode_bf16(rows, k_c, v_c, case.table, case.token_row, None, case.kv_hi, out,
+                                              hd ** -0.5, h, hkv, hd, case.batch,
+                                              fuse=(rows[:, q_dim:q_dim + kv_dim], rows[:, q_dim + kv_dim:], table, slots),
+                                              beside=beside)
+            return out, k_c, v_c
+
+        alone = torch.empty(n, n_out, dtype=bf, device=DEV)
+        assert fast.layernorm_linear(x, gamma, beta, 1e-5, w, bias, alone, act)
+        out_ref, k_ref, v_ref = run(None)
+        together = torch.full((n, n_out), float("nan"), dtype=bf, device=DEV)
+        job = NormLinear(x, gamma, beta, 1e-5, w, bias, together, act)
+        assert fast.attention_decode_takes(job, n, h, hd, 16, case.batch.max_kv)
+        out, k_c, v_c = run(job)
+        assert torch.equal(out, out_ref)
+        # (places of the cache that no row holds are filled with NaN: compared as bit patterns)
+        assert torch.equal(k_c.view(torch.int16), k_ref.view(torch.int16))
+        assert torch.equal(v_c.view(torch.int16), v_ref.view(torch.int16))
+        assert torch.equal(together, alone)
+        hidden = F.layer_norm(x.double(), (k,), gamma.double(), beta.double(), 1e-5).to(bf).double()
+        _close(together, _ACTIVATE[act](hidden @ w.double().T + bias.double()), bf, scale=2)
+
+
+def test_decode_attention_declines_a_linear_layer_it_cannot_carry():
+    from kestrel_amd.ops import fast
+    from kestrel_amd.parts import NormLinear
+
+    def job(rows, k, n_out=64, x_dtype=torch.float32):
+        return NormLinear(torch.zeros(rows, k, dtype=x_dtype, device=DEV), torch.ones(k, device=DEV), None, 1e-5,
+                          torch.zeros(n_out, k, dtype=torch.bfloat16, device=DEV), None,
+                          torch.empty(rows, n_out, dtype=torch.bfloat16, device=DEV), 0)
+
+    assert fast.attention_decode_takes(job(8, 2048), 8, 4, 64, 16, 1024)
+    assert not fast.attention_decode_takes(job(9, 2048), 9, 4, 64, 16, 1024)          # more rows than its prologue normalises
+    assert not fast.attention_decode_takes(job(8, 2056), 8, 4, 64, 16, 1024)          # a row too long for its registers
+    assert not fast.attention_decode_takes(job(8, 2048), 8, 4, 80, 16, 1024)          # a head size that needs a SIMD's registers
+    assert not fast.attention_decode_takes(job(8, 2048, x_dtype=torch.bfloat16), 8, 4, 64, 16, 1024)
+    assert fast.attention_decode_takes(job(4, 2048), 4, 32, 64, 16, 1024)
+    assert not fast.attention_decode_takes(job(5, 2048), 5, 32, 64, 16, 1024)         # attention that fills the chip by itself
+    assert not fast.attention_decode_takes(job(2, 2048), 2, 32, 64, 16, 3 * fast.DECODE_KEYS_PER_WORKGROUP)
+
+
 def test_decode_attention_splits_long_rows(monkeypatch):
     """Rows longer than a workgroup's share are cut into parts that a second kernel merges."""
     from kestrel_amd.ops import fast
