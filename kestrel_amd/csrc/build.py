@@ -30,9 +30,12 @@ ARCH = "gfx950"
 # bf16 MFMA kernels of serving.
 LIBRARIES: Dict[str, List[str]] = {
     "core": ["ka_error.hip", "elementwise.hip", "gemm_generic.hip", "attention_generic.hip", "sampling.hip", "peaks.hip"],
-    "fast": ["ka_error.hip", "gemm_bf16.hip", "gemv_bf16.hip", "attention_bf16.hip", "decode_beside.hip"],
+    "fast": ["ka_error.hip", "gemm_bf16.hip", "gemv_bf16.hip", "attention_bf16.hip", "decode_beside.hip", "gemm_library.hip"],
 }
 HEADERS = ["ka_common.h", "ka_partials.h", "ka_no_alloc.h", "ka_attention_decode.h", "ka_skinny.h"]
+
+# Libraries of the ROCm installation that a library of ours is linked against.
+LINK_LIBRARIES: Dict[str, List[str]] = {"fast": ["hipblaslt"]}
 
 HIPCC_FLAGS = [
     f"--offload-arch={ARCH}", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",
@@ -59,7 +62,7 @@ def _sources(name: str) -> List[Path]:
 def source_stamp(name: str) -> str:
     """Hash of the sources, headers and flags a library is built from."""
     digest = hashlib.sha256()
-    digest.update(" ".join(HIPCC_FLAGS).encode())
+    digest.update(" ".join(HIPCC_FLAGS + LINK_LIBRARIES.get(name, [])).encode())
     for path in [SOURCE_DIR / h for h in HEADERS] + _sources(name):
         digest.update(path.name.encode())
         digest.update(path.read_bytes())
@@ -159,7 +162,9 @@ def build(name: str, verbose: bool = True) -> Path:
                 last_note = time.time()
     target = library_path(name, folder)
     partial = target.with_suffix(f".tmp{os.getpid()}")
-    cmd = [hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", str(partial), *map(str, sorted(objects))]
+    rocm_lib = Path(hipcc).resolve().parent.parent / "lib"
+    links = [f"-L{rocm_lib}", f"-Wl,-rpath,{rocm_lib}"] + [f"-l{lib}" for lib in LINK_LIBRARIES.get(name, [])]
+    cmd = [hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", str(partial), *map(str, sorted(objects)), *links]
     done = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, env=env)
     if done.returncode != 0:
         raise KernelBuildError(f"linking {target.name} failed:\n{done.stdout.decode(errors='replace')}")

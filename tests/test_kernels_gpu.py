@@ -141,8 +141,13 @@ def test_every_activation_in_every_linear_kernel(name, code):
     def through_dispatch(a, w, bias, out, act, accumulate):
         linear(a, w, bias, out, act=act, accumulate=accumulate)
 
-    for m, n, k in ((8, 2048, 2048), (40, 4100, 2048), (200, 333, 520), (520, 2048, 8192), (2048, 512, 1024)):
-        _linear_case(through_dispatch, m, n, k, bf, bf, bf, code, False)
+    for library in (True, False):                            # many rows: the vendor library's epilogues, then this package's tiles
+        fast.LIBRARY_LINEAR, was = library, fast.LIBRARY_LINEAR
+        try:
+            for m, n, k in ((8, 2048, 2048), (40, 4100, 2048), (200, 333, 520), (520, 2048, 8192), (2048, 512, 1024)):
+                _linear_case(through_dispatch, m, n, k, bf, bf, bf, code, False)
+        finally:
+            fast.LIBRARY_LINEAR = was
     for mode in (0, 2):                                      # the split kernel, then the wide one wherever it can run
         fast.set_skinny_persistent(0 if mode == 0 else 1)
         fast.set_skinny_wide(mode)
@@ -206,12 +211,16 @@ def test_linear_skinny_is_the_same_on_every_run():
 
 @pytest.mark.parametrize("shape", [(65, 128, 64), (200, 2048, 2048), (129, 100, 200), (300, 333, 520),
                                    (2048, 512, 1024), (128, 6144, 2048), (70, 8, 8), (520, 2048, 8192), (300, 200, 1088)])
-def test_linear_tiled_bf16(shape):
-    """The tiled MFMA kernel with ragged edges in M, N and K (K cut into parts where there are few tiles)."""
+@pytest.mark.parametrize("library", [False, True])
+def test_linear_tiled_bf16(shape, library, monkeypatch):
+    """Linears of many rows with ragged edges in M, N and K: through the tiled MFMA kernel (K cut into
+    parts where there are few tiles), and through the vendor library with its epilogues, which
+    ``linear_bf16`` asks first."""
     from kestrel_amd.ops import fast
 
     m, n, k = shape
     bf, f32 = torch.bfloat16, torch.float32
+    monkeypatch.setattr(fast, "LIBRARY_LINEAR", library)
 
     def fn(a, w, bias, out, act, accumulate):
         assert fast.linear_bf16(a, w, bias, out, act, accumulate)
@@ -242,6 +251,39 @@ def test_linear_large_tile_bf16(shape, config, monkeypatch):
     for out_dtype, act, accumulate in [(bf, 0, False), (bf, 1, False), (f32, 0, True), (f32, 0, False)]:
         _linear_case(fn, m, n, k, bf, bf, out_dtype, act, accumulate)
     _linear_case(fn, m, n, k, bf, bf, bf, 0, False, lda=k + 8)
+
+
+def test_the_vendor_library_takes_the_linears_of_a_prompt():
+    """What ``linear_bf16`` hands to hipBLASLt is really run there (status 0, not "no kernel for the
+    case") for the cases a model brings: bias + activation into bf16, bias + sum into the fp32
+    residual, rows that are not packed; and it computes the tanh form of GELU, as the kernels here do."""
+    from kestrel_amd.ops import fast
+    from kestrel_amd.ops.core import stream_ptr
+
+    bf, f32 = torch.bfloat16, torch.float32
+    torch.manual_seed(9)
+    m, n, k = 300, 520, 264
+    a = torch.randn(m, k + 8).to(bf).to(DEV)[:, :k]
+    w = (torch.randn(n, k) / k ** 0.5).to(bf).to(DEV)
+    bias = torch.randn(n).to(DEV)
+    space = fast._library_workspace(a.device)
+    ref = a.double() @ w.double().T + bias.double()
+    for out_dtype, act, accumulate in [(bf, 1, False), (f32, 1, False), (f32, 0, True), (bf, 0, False), (f32, 3, False), (f32, 2, False)]:
+        start = torch.randn(m, n).to(out_dtype).to(DEV)
+        out = start.clone()
+        status = fast.lib().ka_linear_library_bf16(a.data_ptr(), a.stride(0), w.data_ptr(), w.stride(0), bias.data_ptr(),
+                                                   out.data_ptr(), 0 if out_dtype == f32 else 1, out.stride(0), m, n, k, act,
+                                                   int(accumulate), space.data_ptr(), space.numel(), stream_ptr())
+        assert status == 0, (out_dtype, act, accumulate, status)
+        expected = _ACTIVATE[act](ref) + (start.double() if accumulate else 0)
+        if out_dtype == f32:        # tight enough to tell the tanh form of GELU from the erf form (they differ by 5e-4)
+            assert (out.double() - expected).abs().max().item() < 2e-5
+        else:
+            _close(out, expected, bf, scale=2)
+    with pytest.raises(fast.KernelError, match="accumulate needs an fp32 output"):
+        fast._check(fast.lib().ka_linear_library_bf16(a.data_ptr(), a.stride(0), w.data_ptr(), w.stride(0), None,
+                                                      out.data_ptr(), 1, n, m, n, k, 0, 1, space.data_ptr(), space.numel(),
+                                                      stream_ptr()))
 
 
 def test_fast_linear_declines_what_it_does_not_cover():
