@@ -308,6 +308,9 @@ def main() -> int:
     parser.add_argument("--workload", default="decode", choices=["decode", "waves256", "mixed48"],
                         help="decode: the benchmark's decode step (default); the others run requests through InferenceEngine")
     parser.add_argument("--max-batch-size", type=int, default=None, help="for the workloads through the entry point")
+    parser.add_argument("--linears", default="library", choices=["library", "own"],
+                        help="linears of more than 64 rows (a prompt's): through hipBLASLt (the engine's default) or "
+                             "through this package's tiled kernels only")
     args = parser.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -319,6 +322,9 @@ def main() -> int:
         return 1
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
+    from kestrel_amd.ops import fast
+
+    fast.LIBRARY_LINEAR = args.linears == "library"
     dtype = torch.bfloat16 if args.dtype == "bf16" else torch.float32
     size = 2 if dtype == torch.bfloat16 else 4
     sizes = dict(SIZES[args.sizes])
@@ -351,7 +357,8 @@ def main() -> int:
                    "dim": typed.dim, "ff_dim": typed.ff_dim, "n_heads": typed.n_heads, "n_kv_heads": typed.n_kv_heads,
                    "head_dim": typed.head_dim, "rotary_dim": typed.rotary_dim, "vocab_size": typed.vocab_size,
                    "global_batch": args.batch, "seq_len": args.context, "prefix_attn": typed.prefix_attn,
-                   "page_size": PAGE_SIZE, "parallelism": "single-gpu"},
+                   "page_size": PAGE_SIZE, "parallelism": "single-gpu",
+                   "prompt_linears": "hipblaslt" if args.linears == "library" else "own"},
         "roofline": {"bound": "hbm", "achieved": round(achieved / 1e9, 1), "peak": PEAK_HBM / 1e9, "unit": "GB/s",
                      "frac": round(achieved / PEAK_HBM, 4)},
     }

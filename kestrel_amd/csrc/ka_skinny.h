@@ -4,6 +4,9 @@
 #pragma once
 #include "ka_common.h"
 
+#include <type_traits>
+#include <utility>
+
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
 typedef __attribute__((ext_vector_type(4))) __bf16 bf16x4;
 typedef __attribute__((ext_vector_type(4))) float floatx4;
@@ -36,6 +39,17 @@ template <typename T>
 __device__ __forceinline__ T sk_pinned(T v) {
     asm volatile("" : "+s"(v));
     return v;
+}
+
+// f(integral_constant<int, 0>), ..., f(integral_constant<int, N - 1>): a loop whose index is a
+// constant inside the body (register arrays are indexed by it).
+template <int N, typename F, int... I>
+__device__ __forceinline__ void sk_static_for_impl(F&& f, std::integer_sequence<int, I...>) {
+    (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, typename F>
+__device__ __forceinline__ void sk_static_for(F&& f) {
+    sk_static_for_impl<N>(f, std::make_integer_sequence<int, N>{});
 }
 
 struct SkinnyTarget {       // one weight matrix and where its product goes
@@ -258,7 +272,9 @@ __device__ __forceinline__ void skinny_persistent_body(const SkinnyArgs& p, cons
         __builtin_amdgcn_sched_barrier(0);
     }
     issue(0, 0);
-    if (DEPTH == 3 && mine > 1) issue(1, 1);
+    sk_static_for<DEPTH - 2>([&](auto d) {
+        if (d.value + 1 < mine) issue(d.value + 1, d.value + 1);
+    });
 
     // activations of this wave's k-blocks wave, wave + 8, ...: fetched (or normalised) once
     constexpr int XH = HALF ? 1 : 2;
@@ -341,55 +357,26 @@ __device__ __forceinline__ void skinny_persistent_body(const SkinnyArgs& p, cons
     };
 
     // Strip i + DEPTH - 1 is asked for before strip i is multiplied. No load of the loop stands
-    // under a condition, and the last strips are written out case by case without any: the
-    // compiler can then wait for exactly the strip it needs and leave the others in flight.
+    // under a condition, and the last strips are written out case by case (one case per number of
+    // strips left) without any: the compiler can then wait for exactly the strip it needs and leave
+    // the others in flight. Strip s lives in slot s % DEPTH.
     int i = 0;
-    if constexpr (DEPTH == 2) {
-        for (; i + 2 < mine; i += 2) {
-            issue(1, i + 1);
-            compute(0, i);
-            issue(0, i + 2);
-            compute(1, i + 1);
-        }
-        if (mine - i == 2) {
-            issue(1, i + 1);
-            compute(0, i);
-            compute(1, i + 1);
-        } else {
-            compute(0, i);
-        }
-    } else {
-        static_assert(DEPTH == 3, "one or two strips ahead");
-        if (mine == 1) {
-            compute(0, 0);
-            return;
-        }
-        for (; i + 5 <= mine; i += 3) {
-            issue(2, i + 2);
-            compute(0, i);
-            issue(0, i + 3);
-            compute(1, i + 1);
-            issue(1, i + 4);
-            compute(2, i + 2);
-        }
-        const int left = mine - i;          // 2, 3 or 4
-        if (left == 2) {
-            compute(0, i);
-            compute(1, i + 1);
-        } else if (left == 3) {
-            issue(2, i + 2);
-            compute(0, i);
-            compute(1, i + 1);
-            compute(2, i + 2);
-        } else {
-            issue(2, i + 2);
-            compute(0, i);
-            issue(0, i + 3);
-            compute(1, i + 1);
-            compute(2, i + 2);
-            compute(0, i + 3);
-        }
+    for (; i + 2 * DEPTH - 1 <= mine; i += DEPTH) {
+        sk_static_for<DEPTH>([&](auto j) {
+            issue((j.value + DEPTH - 1) % DEPTH, i + j.value + DEPTH - 1);
+            compute(j.value, i + j.value);
+        });
     }
+    // strips i .. mine - 1 are left, of which the first min(left, DEPTH - 1) are on their way
+    const int left = mine - i;
+    sk_static_for<2 * DEPTH - 2>([&](auto c) {
+        constexpr int LEFT = c.value + 1;
+        if (left != LEFT) return;
+        sk_static_for<LEFT>([&](auto j) {
+            if constexpr (j.value + DEPTH - 1 < LEFT) issue((j.value + DEPTH - 1) % DEPTH, i + j.value + DEPTH - 1);
+            compute(j.value % DEPTH, i + j.value);
+        });
+    });
 }
 
 // ----------------------------------------------------------------------------
