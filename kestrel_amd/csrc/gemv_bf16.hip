@@ -440,7 +440,7 @@ static int launch_split(int waves, int strips, hipStream_t stream, const SkinnyA
 // The general entry point. Segments: A1 [M, K1] with W (target a) and optionally A2 [M, K2] with
 // W2 (same rows as target a; not with a second target). ln_x non-null: A1 is replaced by
 // LayerNorm(ln_x) (M <= 16, K1 <= 2048). Target b (Wb non-null) shares the input.
-KA_API int ka_linear_skinny_fused(const void* A1, long lda1, int K1, const void* A2, long lda2, int K2,
+static int skinny_fused(const KaThenNorm* then, const void* A1, long lda1, int K1, const void* A2, long lda2, int K2,
                                   const void* W2, long ldw2, const float* bias2, const float* ln_x,
                                   const float* ln_gamma, const float* ln_beta, float ln_eps, const void* Wa,
                                   long ldwa, const float* biasa, void* outa, int out_dtype_a, long ldoa, int Na,
@@ -450,6 +450,15 @@ KA_API int ka_linear_skinny_fused(const void* A1, long lda1, int K1, const void*
     const char* who = "ka_linear_skinny_fused";
     KA_CHECK(M > 0 && M <= 64, "%s: M=%d outside 1..64", who, M);
     KA_CHECK(K1 > 0 && K1 % 8 == 0, "%s: K=%d must be a positive multiple of 8", who, K1);
+    if (then) {
+        KA_CHECK(out_dtype_a == KA_F32 && acta == KA_ACT_NONE && Wb == nullptr, "%s: a norm can follow one fp32 output without activation only", who);
+        KA_CHECK(ka_then_norm_fits(Na), "%s: a norm cannot follow rows of %d (multiples of 4 up to %d)", who, Na, KA_ROW_THREADS * 4 * KA_ROW_QUADS);
+        KA_CHECK(then->gamma && then->out && then->ld >= Na && ldoa % 4 == 0 && then->ld % 4 == 0 && (uintptr_t)outa % 16 == 0 &&
+                     (uintptr_t)then->gamma % 16 == 0 && (uintptr_t)then->beta % 16 == 0 && (uintptr_t)then->out % 8 == 0 &&
+                     (uintptr_t)biasa % 16 == 0 && (uintptr_t)bias2 % 16 == 0,
+                 "%s: the operands of the norm that follows must be aligned to four elements", who);
+        KA_CHECK(then->out_dtype == KA_F32 || then->out_dtype == KA_BF16, "%s: bad type of the normalised rows", who);
+    }
     SkinnyArgs args = {};
     args.M = M;
     args.K[0] = K1;
@@ -496,26 +505,33 @@ KA_API int ka_linear_skinny_fused(const void* A1, long lda1, int K1, const void*
     // the wide kernel shares them through LDS). Two targets go one after the other.
     const bool persistent_ok = !A2 && !accumulate_a && sk_persistent_enabled && persistent_fits(M, kblocks, args);
     if (M > 16 && Wb && partials && sk_wide_enabled && !persistent_ok) {
-        int rc = ka_linear_skinny_fused(A1, lda1, K1, nullptr, 0, 0, nullptr, 0, nullptr, nullptr, nullptr, nullptr, 0.f,
+        int rc = skinny_fused(nullptr, A1, lda1, K1, nullptr, 0, 0, nullptr, 0, nullptr, nullptr, nullptr, nullptr, 0.f,
                                         Wa, ldwa, biasa, outa, out_dtype_a, ldoa, Na, acta, accumulate_a, nullptr, 0,
                                         nullptr, nullptr, 0, 0, 0, 0, M, target_waves, partials, partial_floats, stream);
         if (rc) return rc;
-        return ka_linear_skinny_fused(A1, lda1, K1, nullptr, 0, 0, nullptr, 0, nullptr, nullptr, nullptr, nullptr, 0.f,
+        return skinny_fused(nullptr, A1, lda1, K1, nullptr, 0, 0, nullptr, 0, nullptr, nullptr, nullptr, nullptr, 0.f,
                                       Wb, ldwb, biasb, outb, out_dtype_b, ldob, Nb, actb, 0, nullptr, 0, nullptr,
                                       nullptr, 0, 0, 0, 0, M, target_waves, partials, partial_floats, stream);
     }
     // Up to 16 rows of two segments: where there are more strips than CUs the split kernel,
     // which gives a strip to a workgroup, takes about twice the time that it takes with one
     // strip a CU (N = 2560, K = 2560 + 10240, 16 rows: 40 us; 25 us here).
-    const bool crowded = A2 && strips > sk_compute_units() && M > 4;      // (a single row: 19 us against 24)
+    // With more than 8 rows of two segments the split kernel reads twice the weights' bytes in
+    // activations (it multiplies 16 rows with strips of 8): 16.4 us here against 17.7 at 12 rows and
+    // 18.3 at 16 (N = 2048, K = 2048 + 8192).
+    const bool crowded = A2 && ((strips > sk_compute_units() && M > 4) || M > 8);      // (a single row: 19 us against 24)
     if (!Wb && partials && ((sk_wide_enabled && (M > 16 ? (A2 || !persistent_ok) : crowded)) || sk_wide_enabled >= 2)) {
         WideArgs wide = {};
         wide.A[0] = args.A[0]; wide.lda[0] = args.lda[0]; wide.W[0] = args.a.W; wide.ldw[0] = args.a.ldw; wide.K[0] = K1;
         if (A2) { wide.A[1] = args.A[1]; wide.lda[1] = args.lda[1]; wide.W[1] = args.W2; wide.ldw[1] = args.ldw2; wide.K[1] = K2; }
         wide.M = M; wide.N = Na; wide.partial = partials;
-        // parts of K: two workgroups per CU where K is long enough for that, every part at least two chunks
+        // parts of K: as many as give every CU one workgroup and none a second (measured at N = 2048,
+        // K = 2048 + 8192, 32 groups of strips: 8 parts 18.1 us at 32 rows and 19.6 at 64, finishing
+        // kernel included; 6 parts 21.4 and 22.3, 10 parts 22.6 and 27.4, 16 parts 21.1 and 25.1),
+        // every part at least two chunks
         const int groups = ka_cdiv(Na, WD_WAVES * SK_STRIP);
-        int splits = ka_cdiv(2 * sk_compute_units(), groups);
+        int splits = sk_compute_units() / groups;
+        if (splits < 1) splits = 1;
         if (splits > ka_cdiv(kblocks, 2 * WD_CB)) splits = ka_cdiv(kblocks, 2 * WD_CB);
         while (splits > 1 && (long)splits * M * Na > partial_floats) --splits;
         if ((long)splits * M * Na <= partial_floats) {
@@ -528,15 +544,29 @@ KA_API int ka_linear_skinny_fused(const void* A1, long lda1, int K1, const void*
                 default: hipLaunchKernelGGL(skinny_wide_kernel<4>, grid, dim3(WD_WAVES * KA_WAVE), 0, stream, wide); break;
             }
             KA_LAUNCH_CHECK();
-            const int quads = M * ka_cdiv(Na, 4);
-            hipLaunchKernelGGL(ka_partials_finish_kernel, dim3(ka_cdiv(quads, 256)), dim3(256), 0, stream, partials, splits,
-                               biasa, A2 ? bias2 : nullptr, outa, out_dtype_a, ldoa, M, Na, acta, accumulate_a);
+            if (then) {
+                // the finishing kernel takes whole rows and normalises them as well
+                hipLaunchKernelGGL(ka_partials_finish_norm_kernel, dim3(M), dim3(KA_ROW_THREADS), 0, stream, partials, splits, biasa,
+                                   A2 ? bias2 : nullptr, (float*)outa, ldoa, M, Na, accumulate_a, *then);
+            } else {
+                const int quads = M * ka_cdiv(Na, 4);
+                hipLaunchKernelGGL(ka_partials_finish_kernel, dim3(ka_cdiv(quads, 256)), dim3(256), 0, stream, partials, splits,
+                                   biasa, A2 ? bias2 : nullptr, outa, out_dtype_a, ldoa, M, Na, acta, accumulate_a);
+            }
             KA_LAUNCH_CHECK();
             return 0;
         }
     }
+    // (where K was not cut into parts, a norm that follows is a launch of its own: the same kernel, no parts)
+    auto norm_after = [&]() {
+        if (then)
+            hipLaunchKernelGGL(ka_partials_finish_norm_kernel, dim3(M), dim3(KA_ROW_THREADS), 0, stream, (const float*)nullptr, 0,
+                               (const float*)nullptr, (const float*)nullptr, (float*)outa, ldoa, M, Na, 0, *then);
+    };
     if (persistent_ok) {
         if (launch_persistent(strips, M, kblocks, false, 0, stream, args)) return -1;
+        KA_LAUNCH_CHECK();
+        norm_after();
         KA_LAUNCH_CHECK();
         return 0;
     }
@@ -554,7 +584,37 @@ KA_API int ka_linear_skinny_fused(const void* A1, long lda1, int K1, const void*
     }
     if (rc) return rc;
     KA_LAUNCH_CHECK();
+    norm_after();
+    KA_LAUNCH_CHECK();
     return 0;
+}
+
+KA_API int ka_linear_skinny_fused(const void* A1, long lda1, int K1, const void* A2, long lda2, int K2,
+                                  const void* W2, long ldw2, const float* bias2, const float* ln_x,
+                                  const float* ln_gamma, const float* ln_beta, float ln_eps, const void* Wa,
+                                  long ldwa, const float* biasa, void* outa, int out_dtype_a, long ldoa, int Na,
+                                  int acta, int accumulate_a, const void* Wb, long ldwb, const float* biasb,
+                                  void* outb, int out_dtype_b, long ldob, int Nb, int actb, int M,
+                                  int target_waves, float* partials, long partial_floats, hipStream_t stream) {
+    return skinny_fused(nullptr, A1, lda1, K1, A2, lda2, K2, W2, ldw2, bias2, ln_x, ln_gamma, ln_beta, ln_eps, Wa, ldwa, biasa,
+                        outa, out_dtype_a, ldoa, Na, acta, accumulate_a, Wb, ldwb, biasb, outb, out_dtype_b, ldob, Nb, actb, M,
+                        target_waves, partials, partial_floats, stream);
+}
+
+// out (+)= A1 W1^T + b1 + A2 W2^T + b2 into fp32 rows, then normed = LayerNorm(out; gamma, beta, eps):
+// the last linears of one block and the first norm of the next. Where K is cut into parts (more than
+// 8 rows) the kernel that adds the parts up normalises the rows it has just finished; else the
+// norm is a launch of its own behind the linear's.
+KA_API int ka_linear_skinny_pair_norm(const void* A1, long lda1, int K1, const void* A2, long lda2, int K2,
+                                      const void* W1, long ldw1, const float* bias1, const void* W2, long ldw2,
+                                      const float* bias2, float* out, long ldo, int N, int accumulate, int M,
+                                      int target_waves, float* partials, long partial_floats, const float* gamma,
+                                      const float* beta, float eps, void* normed, int normed_dtype, long ldn,
+                                      hipStream_t stream) {
+    const KaThenNorm then = {gamma, beta, eps, normed, normed_dtype, ldn};
+    return skinny_fused(&then, A1, lda1, K1, A2, lda2, K2, W2, ldw2, bias2, nullptr, nullptr, nullptr, 0.f, W1, ldw1, bias1, out,
+                        KA_F32, ldo, N, KA_ACT_NONE, accumulate, nullptr, 0, nullptr, nullptr, 0, 0, 0, 0, M, target_waves,
+                        partials, partial_floats, stream);
 }
 
 // One input, one weight matrix, one output.

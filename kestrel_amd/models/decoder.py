@@ -87,8 +87,11 @@ class DecoderModel:
         core.embed(self.embedding, batch.token_ids, x, batch.pending)
         if batch.given_embeds is not None:
             core.scatter_rows(batch.given_embeds, batch.given_rows, x)
+        handed = None      # the next block's first norm of x, where a block's last launch has computed it
         for index, entry in enumerate(plan.schedule):
-            self.blocks[entry.layer].forward(x, batch, caches[index])
+            after = plan.schedule[index + 1] if index + 1 < len(plan.schedule) else None
+            then = self.blocks[after.layer].norm if after is not None else None
+            handed = self.blocks[entry.layer].forward(x, batch, caches[index], normed=handed, then=then)
         wanted = int(batch.logit_rows.numel())
         logits = ws.get("model.logits", (wanted, plan.vocab_size), torch.float32)
         if wanted:

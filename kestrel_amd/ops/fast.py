@@ -26,6 +26,11 @@ _SIGNATURES = {
         _c_void_p, _c_long, _c_void_p, _c_void_p, _c_int, _c_long, _c_int, _c_int, _c_int,   # target a
         _c_void_p, _c_long, _c_void_p, _c_void_p, _c_int, _c_long, _c_int, _c_int,           # target b
         _c_int, _c_int, _c_void_p, _c_long, _c_void_p],               # M, target_waves, partial sums and how many, stream
+    "ka_linear_skinny_pair_norm": [
+        _c_void_p, _c_long, _c_int, _c_void_p, _c_long, _c_int,                  # A1, lda1, K1, A2, lda2, K2
+        _c_void_p, _c_long, _c_void_p, _c_void_p, _c_long, _c_void_p,            # W1, ldw1, bias1, W2, ldw2, bias2
+        _c_void_p, _c_long, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_long,  # out, ldo, N, accumulate, M, target_waves, partial sums
+        _c_void_p, _c_void_p, _c_float, _c_void_p, _c_int, _c_long, _c_void_p],  # gamma, beta, eps, normed, its type and stride, stream
     "ka_linear_library_bf16": [_c_void_p, _c_long, _c_void_p, _c_long, _c_void_p, _c_void_p, _c_int, _c_long, _c_int,
                                _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_long, _c_void_p],
     "ka_linear_tiled_bf16": [_c_void_p, _c_long, _c_void_p, _c_long, _c_void_p, _c_void_p, _c_int, _c_long, _c_int,
@@ -53,6 +58,8 @@ SKINNY_MAX_ROWS = 64
 # Rows (and their width) up to which the weight-streaming kernel can normalise its input itself.
 SKINNY_LN_MAX_ROWS = 16
 SKINNY_LN_MAX_WIDTH = 4096
+# Width of rows up to which a norm can follow a pair of skinny linears in their own launches.
+NORM_AFTER_MAX_WIDTH = 8192
 # Whether blocks let the weight-streaming kernel normalise its input itself. Every workgroup of
 # the persistent kernel then repeats the LayerNorm of all rows once; with a few hundred workgroups
 # that is cheaper than a launch of its own (measured on MI355X: 3 % of a decode step at batch 8).
@@ -211,8 +218,11 @@ def linear_bf16(a, weight, bias, out, act, accumulate) -> bool:
     return True
 
 
-def linear_pair_accumulate(a1, w1, b1, a2, w2, b2, out) -> bool:
-    """``out += a1 @ w1.T + b1 + a2 @ w2.T + b2`` in one launch (few rows, fp32 ``out``)."""
+def linear_pair_accumulate(a1, w1, b1, a2, w2, b2, out, then_norm=None) -> bool:
+    """``out += a1 @ w1.T + b1 + a2 @ w2.T + b2`` in one launch (few rows, fp32 ``out``).
+    ``then_norm = (gamma, beta or None, eps, normed)``: also ``normed = LayerNorm(out)``, in the kernel
+    that finishes the rows where there is one (more than 8 rows), else in a launch behind it. False:
+    not covered, nothing was run (with ``then_norm``: try without)."""
     m, k1 = a1.shape
     k2 = a2.shape[1]
     n = w1.shape[0]
@@ -222,6 +232,21 @@ def linear_pair_accumulate(a1, w1, b1, a2, w2, b2, out) -> bool:
         return False
     if out.dtype != torch.float32 or not _out_ok(out, m, n) or not _bias_ok(b1, n) or not _bias_ok(b2, n):
         return False
+    if then_norm is not None:
+        gamma, beta, eps, normed = then_norm
+        if n % 4 or n > NORM_AFTER_MAX_WIDTH or out.stride(0) % 4 or normed.dtype not in _OUT_CODE or not _out_ok(normed, m, n) \
+                or normed.stride(0) % 4 or gamma.dtype != torch.float32 or gamma.numel() != n or gamma.data_ptr() % 16:
+            return False
+        if beta is not None and (beta.dtype != torch.float32 or beta.numel() != n or beta.data_ptr() % 16):
+            return False
+        if any(b is not None and b.data_ptr() % 16 for b in (b1, b2)):
+            return False
+        _check(lib().ka_linear_skinny_pair_norm(
+            a1.data_ptr(), a1.stride(0), k1, a2.data_ptr(), a2.stride(0), k2, w1.data_ptr(), w1.stride(0), _ptr(b1),
+            w2.data_ptr(), w2.stride(0), _ptr(b2), out.data_ptr(), out.stride(0), n, 1, m, SKINNY_TARGET_WAVES,
+            *_wide_args(a1.device, m), gamma.data_ptr(), _ptr(beta), float(eps), normed.data_ptr(), _OUT_CODE[normed.dtype],
+            normed.stride(0), stream_ptr()))
+        return True
     _check(lib().ka_linear_skinny_fused(
         a1.data_ptr(), a1.stride(0), k1, a2.data_ptr(), a2.stride(0), k2, w2.data_ptr(), w2.stride(0), _ptr(b2),
         None, None, None, 0.0,

@@ -10,10 +10,13 @@ from .base import LayerCache, NormLinear, Part, build_part
 from .specs import LayerSpec, ParamSpec
 
 
-def _parallel_few_rows(block: "Block", x, batch, cache) -> bool:
+def _parallel_few_rows(block: "Block", x, batch, cache, normed, then, handed) -> bool:
     """The parallel block for a few bf16 rows in three launches: norm + both first linears, the
     mixer's core, both last linears + residual. Needs a mixer and a feed-forward that offer their
-    stages (``input_projection`` / ``output_projection``); returns ``False`` otherwise."""
+    stages (``input_projection`` / ``output_projection``); returns ``False`` otherwise.
+    ``normed``: the block's norm of ``x``, where the block before has computed it; ``then``: the norm
+    the next block starts with, which the last launch computes as well where it pays (``handed``, a
+    list, then gets the normalised rows)."""
     from ..ops import fast
     from ..ops.linear import linear
 
@@ -30,7 +33,9 @@ def _parallel_few_rows(block: "Block", x, batch, cache) -> bool:
     norm = block.norm
     fused = False
     beside = None
-    if fast.FUSE_LAYERNORM_PROLOGUE and getattr(norm.spec, "kind", None) == "layernorm":
+    if normed is not None:
+        fused = fast.linear_two_outputs(normed, m_in[0], m_in[1], projected, 0, f_in[0], f_in[1], hidden, f_in[3])
+    if not fused and fast.FUSE_LAYERNORM_PROLOGUE and getattr(norm.spec, "kind", None) == "layernorm":
         # the feed-forward's first linear goes into the mixer's launch where the mixer takes it,
         # else into the launch of the mixer's first linear
         job = NormLinear(x, norm.weight, norm.bias, norm.spec.eps, f_in[0], f_in[1], hidden, f_in[3])
@@ -48,23 +53,38 @@ def _parallel_few_rows(block: "Block", x, batch, cache) -> bool:
             linear(h, f_in[0], f_in[1], hidden, act=f_in[3])
     mixed = block.mixer.attend(projected, batch, cache, beside) if beside is not None \
         else block.mixer.attend(projected, batch, cache)
+    # More rows than the next block's first launch normalises by itself: its norm is computed here,
+    # by the kernel that finishes this block's rows, instead of in a launch of its own.
+    if then is not None and n > fast.SKINNY_LN_MAX_ROWS and getattr(then.spec, "kind", None) == "layernorm":
+        rows = ws.get("block.handed", tuple(x.shape), block.dtype)
+        if fast.linear_pair_accumulate(mixed, m_out[0], m_out[1], hidden, f_out[0], f_out[1], x,
+                                       then_norm=(then.weight, then.bias, then.spec.eps, rows)):
+            handed.append(rows)
+            return True
     if not fast.linear_pair_accumulate(mixed, m_out[0], m_out[1], hidden, f_out[0], f_out[1], x):
         linear(mixed, m_out[0], m_out[1], x, accumulate=True)
         linear(hidden, f_out[0], f_out[1], x, accumulate=True)
     return True
 
 
-def _parallel(block: "Block", x, batch, cache) -> None:
+def _parallel(block: "Block", x, batch, cache, normed=None, then=None):
     """``x + mixer(norm(x)) + ff(norm(x))``: both branches read the same normalised input.
 
     Reference: ``kestrel/models/moondream/text.py:222-275``.
     """
-    if _parallel_few_rows(block, x, batch, cache):
-        return
-    h = batch.workspace.get("block.h", tuple(x.shape), block.dtype)
-    block.norm.forward(x, h)
+    handed = []
+    if _parallel_few_rows(block, x, batch, cache, normed, then, handed):
+        return handed[0] if handed else None
+    h = normed
+    if h is None:
+        h = batch.workspace.get("block.h", tuple(x.shape), block.dtype)
+        block.norm.forward(x, h)
     block.mixer.forward(h, batch, cache, x)
     block.feed_forward.forward(h, batch, x)
+    return None
+
+
+_parallel.hands_over = True
 
 
 def _sequential(block: "Block", x, batch, cache) -> None:
@@ -80,7 +100,11 @@ ARRANGEMENTS: Dict[str, Callable] = {"parallel": _parallel, "sequential": _seque
 
 
 def register_arrangement(name: str, fn: Callable) -> None:
-    """``fn(block, x, batch, cache)`` updates the fp32 residual ``x`` in place."""
+    """``fn(block, x, batch, cache)`` updates the fp32 residual ``x`` in place. A function with the
+    attribute ``hands_over = True`` is called as ``fn(block, x, batch, cache, normed=, then=)``:
+    ``normed`` is ``block.norm`` of ``x`` if the block before has computed it (else ``None``), ``then``
+    the first norm of the block that follows (or ``None``); it may return that norm of its result, or
+    ``None``."""
     ARRANGEMENTS[name] = fn
 
 
@@ -123,5 +147,12 @@ class Block:
             local = {name: tensors[self.spec.names[f"{part_name}.{name}"]] for name in part.params()}
             part.bind(local, dtype, device)
 
-    def forward(self, x: torch.Tensor, batch, cache: LayerCache) -> None:
+    def forward(self, x: torch.Tensor, batch, cache: LayerCache, normed: Optional[torch.Tensor] = None,
+                then: Optional[Part] = None) -> Optional[torch.Tensor]:
+        """Updates the fp32 residual ``x`` in place. ``normed``: this block's first norm of ``x``, if the
+        block before has computed it; ``then``: the first norm of the block that follows. Returns that
+        norm of the result where the block's last launch computed it, else ``None``."""
+        if getattr(self._run, "hands_over", False):
+            return self._run(self, x, batch, cache, normed=normed, then=then)
         self._run(self, x, batch, cache)
+        return None

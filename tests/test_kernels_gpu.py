@@ -725,6 +725,18 @@ def test_two_segment_skinny_linear(shape, wide):
     out3 = start.clone()
     assert fast.linear_pair_accumulate(a1, w1, None, a2, w2, None, out3)
     assert torch.equal(out2, out3)                      # the same bits on every run
+    # with the norm that follows: the same sums bit for bit, and their LayerNorm (computed by the
+    # kernel that adds up the parts of K where there is one, else by a launch behind the linear's)
+    gamma, beta = (1 + 0.1 * torch.randn(n)).to(DEV), (0.1 * torch.randn(n)).to(DEV)
+    for dtype, shift in ((torch.bfloat16, beta), (torch.float32, None)):
+        out4 = start.clone()
+        normed = torch.full((m, n), float("nan"), dtype=dtype, device=DEV)
+        taken = fast.linear_pair_accumulate(a1, w1, b1, a2, w2, b2, out4, then_norm=(gamma, shift, 1e-5, normed))
+        assert taken == (n % 4 == 0)
+        if taken:
+            assert torch.equal(out4, out)
+            expected = F.layer_norm(out4.double(), (n,), gamma.double(), None if shift is None else shift.double(), 1e-5)
+            _close(normed, expected, dtype, scale=4)
     fast.set_skinny_wide(1)
 
 
