@@ -126,7 +126,9 @@ attn_decode_body(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t* 
     const bool chunk_live = dg_lane < CPK;             // this lane holds a chunk of the key row
     const int dg = chunk_live ? dg_lane : 0;
     const float sl2 = scale * AT_LOG2E;
-    const bool takes_new = fused && wave == 0 && split == 0;     // this wave adds the token's own key and value
+    // this wave adds the token's own key and value: the last one, which has the fewest tiles where
+    // they do not divide over the waves
+    const bool takes_new = fused && wave == WAVES - 1 && split == 0;
 
     // The operands of q (and, for the wave that takes them, of the token's own key and value) are
     // asked for first and used after the first tile's keys and values have been asked for.
