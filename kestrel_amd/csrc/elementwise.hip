@@ -15,7 +15,7 @@ KA_API int ka_version() { return 1; }
 template <typename T>
 __global__ void embed_kernel(const T* __restrict__ table, const int* __restrict__ ids,
                              const int* __restrict__ pending, int n_pending, int vocab,
-                             float* __restrict__ out, int dim) {
+                             float* __restrict__ out, int dim, float scale) {
     int t = blockIdx.x;
     int id = ids[t];
     if (id == -1) return;
@@ -27,22 +27,43 @@ __global__ void embed_kernel(const T* __restrict__ table, const int* __restrict_
     }
     const T* src = table + (size_t)id * dim;
     float* dst = out + (size_t)t * dim;
-    for (int d = threadIdx.x; d < dim; d += blockDim.x) dst[d] = ka_to_float(src[d]);
+    for (int d = threadIdx.x; d < dim; d += blockDim.x) dst[d] = ka_to_float(src[d]) * scale;
 }
 
+// `scale`: a factor on the looked-up rows (1 for none; rows with id -1, which are given from
+// outside, are not touched).
 KA_API int ka_embed(const void* table, int table_dtype, const int* ids, const int* pending, int n_pending,
-                    int vocab, float* out, int n, int dim, hipStream_t stream) {
+                    int vocab, float* out, int n, int dim, float scale, hipStream_t stream) {
     KA_CHECK(n >= 0 && dim > 0 && vocab > 0 && n_pending >= 0, "ka_embed: bad sizes n=%d dim=%d vocab=%d", n, dim, vocab);
     if (n == 0) return 0;
     dim3 grid(n), block(256);
     if (table_dtype == KA_F32)
         hipLaunchKernelGGL(embed_kernel<float>, grid, block, 0, stream, (const float*)table, ids, pending, n_pending,
-                           vocab, out, dim);
+                           vocab, out, dim, scale);
     else if (table_dtype == KA_BF16)
         hipLaunchKernelGGL(embed_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)table, ids, pending,
-                           n_pending, vocab, out, dim);
+                           n_pending, vocab, out, dim, scale);
     else
         KA_CHECK(false, "ka_embed: unsupported table dtype %d", table_dtype);
+    KA_LAUNCH_CHECK();
+    return 0;
+}
+
+// logits *= scale; then, with cap > 0, logits = cap * tanh(logits / cap): what some architectures do
+// to their logits before sampling.
+__global__ void adjust_logits_kernel(float* __restrict__ logits, long count, float scale, float cap) {
+    const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= count) return;
+    float x = logits[i] * scale;
+    if (cap > 0.f) x = cap * tanhf(x / cap);
+    logits[i] = x;
+}
+
+KA_API int ka_adjust_logits(float* logits, long count, float scale, float cap, hipStream_t stream) {
+    KA_CHECK(count >= 0 && cap >= 0.f, "ka_adjust_logits: bad count %ld or cap %g", count, cap);
+    if (count == 0) return 0;
+    KA_CHECK((count + 255) / 256 < (1L << 31), "ka_adjust_logits: too many values");
+    hipLaunchKernelGGL(adjust_logits_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, stream, logits, count, scale, cap);
     KA_LAUNCH_CHECK();
     return 0;
 }

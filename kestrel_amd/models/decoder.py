@@ -84,7 +84,7 @@ class DecoderModel:
         plan = self.plan
         ws = batch.workspace
         x = ws.get("model.x", (batch.n_tokens, plan.dim), torch.float32)
-        core.embed(self.embedding, batch.token_ids, x, batch.pending)
+        core.embed(self.embedding, batch.token_ids, x, batch.pending, plan.embedding_scale)
         if batch.given_embeds is not None:
             core.scatter_rows(batch.given_embeds, batch.given_rows, x)
         handed = None      # the next block's first norm of x, where a block's last launch has computed it
@@ -98,4 +98,6 @@ class DecoderModel:
             normed = ws.get("model.head_in", (wanted, plan.dim), self.dtype)
             self.final_norm.forward(x, normed, rows=batch.logit_rows)
             linear(normed, self.head_weight, self.head_bias, logits)
+            if plan.logit_scale != 1.0 or plan.logit_softcap is not None:
+                core.adjust_logits(logits, plan.logit_scale, plan.logit_softcap)
         return logits

@@ -20,7 +20,8 @@ _DTYPE_CODE = {torch.float32: KA_F32, torch.bfloat16: KA_BF16}
 _c_void_p, _c_int, _c_long, _c_float = ctypes.c_void_p, ctypes.c_int, ctypes.c_long, ctypes.c_float
 
 _SIGNATURES = {
-    "ka_embed": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_void_p, _c_int, _c_int, _c_void_p],
+    "ka_embed": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_void_p, _c_int, _c_int, _c_float, _c_void_p],
+    "ka_adjust_logits": [_c_void_p, _c_long, _c_float, _c_float, _c_void_p],
     "ka_scatter_rows": [_c_void_p, _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_void_p],
     "ka_layernorm": [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_float, _c_void_p, _c_int, _c_int, _c_int,
                      _c_void_p],
@@ -144,8 +145,9 @@ def uniform(key: int, counter: int) -> float:
     return float(lib().ka_uniform_host(key & (2 ** 64 - 1), counter))
 
 
-def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor, pending: Optional[torch.Tensor] = None) -> None:
-    """``out[t] = table[ids[t]]`` in fp32. A row with id -1 is left untouched; an id ``<= -2`` is
+def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor, pending: Optional[torch.Tensor] = None,
+          scale: float = 1.0) -> None:
+    """``out[t] = scale * table[ids[t]]`` in fp32. A row with id -1 is left untouched; an id ``<= -2`` is
     replaced by ``pending[-2 - id]`` (int32 token ids kept on the device by earlier sampling)."""
     _dev(table, ids, out, pending)
     _need(pending is None or (pending.dtype == torch.int32 and pending.is_contiguous()), "embed: pending must be int32")
@@ -155,7 +157,15 @@ def embed(table: torch.Tensor, ids: torch.Tensor, out: torch.Tensor, pending: Op
     _need(out.dtype == torch.float32 and out.is_contiguous(), "embed: out must be contiguous fp32")
     _check(lib().ka_embed(table.data_ptr(), code_of(table.dtype), ids.data_ptr(), _ptr(pending),
                           0 if pending is None else pending.numel(), table.shape[0], out.data_ptr(), n, dim,
-                          stream_ptr()))
+                          float(scale), stream_ptr()))
+
+
+def adjust_logits(logits: torch.Tensor, scale: float = 1.0, softcap: Optional[float] = None) -> None:
+    """In place: ``logits *= scale``, then ``softcap * tanh(logits / softcap)`` if a cap is given."""
+    _dev(logits)
+    _need(logits.dtype == torch.float32 and logits.is_contiguous(), "adjust_logits: logits must be contiguous fp32")
+    _need(softcap is None or softcap > 0, "adjust_logits: the cap must be positive")
+    _check(lib().ka_adjust_logits(logits.data_ptr(), logits.numel(), float(scale), float(softcap or 0.0), stream_ptr()))
 
 
 def scatter_rows(src: torch.Tensor, rows: torch.Tensor, out: torch.Tensor) -> None:

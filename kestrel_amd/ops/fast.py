@@ -308,10 +308,6 @@ def layernorm_linear(x, gamma, beta, eps, wa, ba, out_a, act_a, wb=None, bb=None
     return True
 
 
-def layernorm_linear_pair(x, gamma, beta, eps, wa, ba, out_a, act_a, wb, bb, out_b, act_b) -> bool:
-    return layernorm_linear(x, gamma, beta, eps, wa, ba, out_a, act_a, wb, bb, out_b, act_b)
-
-
 def rope_cache_bf16(qkv, positions, slots, table, k_cache, v_cache, n_heads, n_kv_heads, head_dim, page_size) -> bool:
     """Rotary encoding of q (in place) and k, and the cache write of k and v, a page's worth of
     tokens per workgroup (``ops.core.rope_cache`` says what the operands are). False: not covered

@@ -43,8 +43,8 @@ def _parallel_few_rows(block: "Block", x, batch, cache, normed, then, handed) ->
                 fast.layernorm_linear(x, norm.weight, norm.bias, norm.spec.eps, m_in[0], m_in[1], projected, 0):
             fused, beside = True, job
         else:
-            fused = fast.layernorm_linear_pair(x, norm.weight, norm.bias, norm.spec.eps, m_in[0], m_in[1], projected, 0,
-                                               f_in[0], f_in[1], hidden, f_in[3])
+            fused = fast.layernorm_linear(x, norm.weight, norm.bias, norm.spec.eps, m_in[0], m_in[1], projected, 0,
+                                          f_in[0], f_in[1], hidden, f_in[3])
     if not fused:
         h = ws.get("block.h", tuple(x.shape), block.dtype)
         norm.forward(x, h)

@@ -149,6 +149,11 @@ class ModelPlan:
     names: Mapping[str, str]  # "embedding", "final_norm.weight", "head.weight", ... -> tensor name
     eos_token_ids: Tuple[int, ...] = ()
     bos_token_id: Optional[int] = None
+    # constants some architectures put around the stack (all neutral by default): a factor on the
+    # looked-up embeddings, a factor on the logits, and a cap ``c`` that turns logits into c * tanh(logits / c)
+    embedding_scale: float = 1.0
+    logit_scale: float = 1.0
+    logit_softcap: Optional[float] = None
 
     def describe(self) -> Dict[str, object]:
         return {"architecture": self.architecture, "layers": len(self.layers), "schedule": len(self.schedule),

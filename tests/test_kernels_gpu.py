@@ -756,11 +756,11 @@ def test_layernorm_prologue_skinny_linear(shape):
     ba, bb = torch.randn(na).to(DEV), torch.randn(nb).to(DEV)
     out_a = torch.empty(m, na, dtype=torch.bfloat16, device=DEV)
     out_b = torch.empty(m, nb, dtype=torch.bfloat16, device=DEV)
-    assert fast.layernorm_linear_pair(x, gamma, beta, 1e-5, wa, ba, out_a, 0, wb, bb, out_b, 1)
+    assert fast.layernorm_linear(x, gamma, beta, 1e-5, wa, ba, out_a, 0, wb, bb, out_b, 1)
     h = F.layer_norm(x.double(), (k,), gamma.double(), beta.double(), 1e-5).to(torch.bfloat16).double()
     _close(out_a, h @ wa.double().T + ba.double(), torch.bfloat16, scale=2)
     _close(out_b, plain.gelu_tanh(h @ wb.double().T + bb.double()), torch.bfloat16, scale=2)
-    assert not fast.layernorm_linear_pair(torch.randn(17, k, device=DEV), gamma, beta, 1e-5, wa, ba,
+    assert not fast.layernorm_linear(torch.randn(17, k, device=DEV), gamma, beta, 1e-5, wa, ba,
                                           torch.empty(17, na, dtype=torch.bfloat16, device=DEV), 0, wb, bb,
                                           torch.empty(17, nb, dtype=torch.bfloat16, device=DEV), 1)
 

@@ -568,6 +568,40 @@ def test_a_layer_may_read_another_layers_cache():
     helpers.assert_close(whole, plain.head(x, w, cfg), torch.float32, "shared cache against plain")
 
 
+def test_constants_around_the_stack():
+    """A plan may scale the looked-up embeddings (not the given ones), scale the logits and cap them
+    with a tanh: a tiny Moondream plan with all three against the plain model with the embedding
+    table scaled by hand and the logits adjusted by formula; eagerly and as a replayed graph."""
+    from kestrel_amd.config import get_spec
+    from kestrel_amd.engine.loading import make_runner
+    from kestrel_amd.engine.step import StepEntry
+    from kestrel_amd.models import DecoderModel
+    from dataclasses import replace
+
+    spec = get_spec("moondream2")
+    base = spec.build_plan(spec.read_config(helpers.TINY_A))
+    plan = replace(base, embedding_scale=3.0, logit_scale=0.5, logit_softcap=2.0)
+    model = DecoderModel(plan)
+    weights = {k: v.float() for k, v in helpers.stored_weights(helpers.model_dir("A")).items()}
+    model.bind(weights, torch.float32, DEV)
+    cfg = helpers.flat_config("A")
+    ids = helpers.random_ids(41, 24, cfg["vocab_size"])
+    given = torch.randn(5, cfg["dim"], generator=torch.Generator().manual_seed(42))
+    w = {k: v.double() for k, v in weights.items()}
+    w[plan.names["embedding"]] = w[plan.names["embedding"]] * 3.0
+    expected = plain.forward(cfg, w, ids, prefix_embeds=given.double())
+    expected = 2.0 * torch.tanh(expected * 0.5 / 2.0)
+    for graphs in (False, True):
+        runner = make_runner(model, 16, 8, 2, enable_graphs=graphs)
+        slot = runner.admit()
+        n = 5 + len(ids)
+        first = runner.step([StepEntry(slot, [-1] * 5 + ids[:10], want=list(range(15)), embeds=given.to(DEV),
+                                       bidirectional=[(0, 5)])]).clone()
+        rest = [runner.step([StepEntry(slot, [t], want=[0])]).clone() for t in ids[10:]]
+        helpers.assert_close(torch.cat([first] + rest), expected[:n], torch.float32, f"constants around the stack, graphs={graphs}")
+        runner.release(slot)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
 def test_a_windowed_layer_beside_a_full_one(dtype):
     """The second layer of a tiny Moondream plan is given a window of 24 keys: its keys and values
