@@ -49,7 +49,7 @@ attn_decode_beside_kernel(BesideAttention a, SkinnyArgs p, int strips, int atten
         return;
     }
     const int t = index % a.n, h = index / a.n % a.H, split = index / (a.n * a.H);
-    attn_decode_body<HD, BS_WAVES>(a.q, a.q_row_stride, a.k_cache, a.v_cache, a.block_table, a.max_pages, a.token_row,
+    attn_decode_body<HD, BS_WAVES, true>(a.q, a.q_row_stride, a.k_cache, a.v_cache, a.block_table, a.max_pages, a.token_row,
                                    a.kv_lo, a.kv_hi, a.out, a.out_row_stride, a.scale, a.H, a.Hkv, a.partial, a.fz, t, h,
                                    split, a.splits);
 }

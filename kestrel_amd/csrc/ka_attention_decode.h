@@ -91,7 +91,10 @@ __device__ __forceinline__ void at_rotated(const RotaryOperands& r, const Rotary
     }
 }
 
-template <int HD, int WAVES>
+// AHEAD: the keys of a wave's next tile are asked for before its current tile is worked on (32
+// registers more at head size 64): one trip to memory less per tile where a wave has more than one
+// tile and the kernel is a chain of trips (few rows), no gain where it streams (many rows).
+template <int HD, int WAVES, bool AHEAD = false>
 __device__ __forceinline__ void
 attn_decode_body(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t* __restrict__ k_cache,
                  const bf16_t* __restrict__ v_cache, const int* __restrict__ block_table, int max_pages,
@@ -205,18 +208,25 @@ attn_decode_body(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t* 
         for (int u = 0; u < VU; ++u) acc[u] = (lane & 1) == 0 ? (float)vnew[u] : 0.f;
     }
 
-    for (int tile0 = s_lo + wave * AD_TILE; tile0 < s_hi; tile0 += WAVES * AD_TILE) {
-        // All key loads of the tile go out before any arithmetic, and none stands under a
-        // condition: a place outside [lo, s_hi) is moved to one inside and masked afterwards. The
-        // compiler can then wait for exactly the register it needs instead of for everything.
-        bf16x8 kreg[KL];
+    // All key loads of a tile go out before any arithmetic, and none stands under a
+    // condition: a place outside [lo, s_hi) is moved to one inside and masked afterwards. The
+    // compiler can then wait for exactly the register it needs instead of for everything.
+    auto load_keys = [&](int tile0, bf16x8 (&dst)[KL]) {
 #pragma unroll
         for (int i = 0; i < KL; ++i) {
             int key = tile0 + i * KPI + ks;
             int kc = max(min(key, s_hi - 1), lo);   // a place that holds data (pages below lo may be gone)
             int page = bt[kc / AT_PAGE];
-            kreg[i] = at_load8(k_cache + (((size_t)page * Hkv + kvh) * AT_PAGE + kc % AT_PAGE) * HD + dg * 8);
+            dst[i] = at_load8(k_cache + (((size_t)page * Hkv + kvh) * AT_PAGE + kc % AT_PAGE) * HD + dg * 8);
         }
+    };
+    bf16x8 kreg[KL], knext[AHEAD ? KL : 1];
+    if constexpr (AHEAD) {
+        if (s_hi > lo) load_keys(s_lo + wave * AD_TILE, kreg);      // (a row without keys: nothing to clamp to)
+    }
+    for (int tile0 = s_lo + wave * AD_TILE; tile0 < s_hi; tile0 += WAVES * AD_TILE) {
+        if constexpr (AHEAD) load_keys(tile0 + WAVES * AD_TILE, knext);
+        else load_keys(tile0, kreg);
         __builtin_amdgcn_sched_barrier(0);     // all of them, before the first is used
         float sc[KL];
         float mx = -INFINITY;
@@ -235,7 +245,13 @@ attn_decode_body(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t* 
 #pragma unroll
         for (int off = LPK; off < KA_WAVE; off <<= 1) mx = fmaxf(mx, __shfl_xor(mx, off, KA_WAVE));
         float m_new = fmaxf(m_i, mx);
-        if (m_new == -INFINITY) continue;      // a tile wholly below lo (wave-uniform)
+        if (m_new == -INFINITY) {              // a tile wholly below lo (wave-uniform)
+            if constexpr (AHEAD) {
+#pragma unroll
+                for (int i = 0; i < KL; ++i) kreg[i] = knext[i];
+            }
+            continue;
+        }
         // the values: asked for as soon as the keys' registers are free, all at once and, like
         // the keys, without a condition; the softmax below runs while they are on their way
         bf16x8 vreg[TP][VU];
@@ -285,6 +301,10 @@ attn_decode_body(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t* 
                 }
                 acc[u] += sum;
             }
+        }
+        if constexpr (AHEAD) {
+#pragma unroll
+            for (int i = 0; i < KL; ++i) kreg[i] = knext[i];
         }
     }
     // the two halves of a channel row
