@@ -9,15 +9,19 @@
 // fills the gaps in the other. Nothing passes between the two kinds: a workgroup is of one kind
 // from start to end, chosen by its index (the kinds alternate while both last).
 //
-// The linear part is the persistent skinny kernel with its LayerNorm prologue (ka_skinny.h): at
-// most 8 rows, K up to 2048. The attention part is the decode kernel (ka_attention_decode.h) with
-// 8 waves a workgroup, head sizes up to 64 (larger heads need more registers than half a SIMD's).
+// The linear part is the persistent skinny kernel (ka_skinny.h) on bf16 rows that an earlier launch
+// has left (the block's normalised input): at most 8 rows, K up to 2048. Normalising the rows here,
+// in every workgroup's prologue, was measured and dropped: within half a CU's registers that
+// prologue makes the linear part the longer of the two (13.8 against 11.3 us alone at one row).
+// The attention part is the decode kernel (ka_attention_decode.h) with 8 waves a workgroup, head
+// sizes up to 64 (larger heads need more registers than half a SIMD's).
 #include "ka_attention_decode.h"
 #include "ka_skinny.h"
 
 constexpr int BS_WAVES = SP_WAVES;       // waves of a workgroup, of either kind
 constexpr int BS_ROWS = 8;               // most rows (tokens) of a launch
 constexpr int BS_MAX_PER = 4;            // k-blocks per wave that the linear part keeps activations for: K <= 2048
+constexpr int BS_DEPTH = 3;              // strips of weights in flight per linear workgroup, the one at work included
 
 struct BesideAttention {
     const bf16_t* q;
@@ -45,7 +49,7 @@ attn_decode_beside_kernel(BesideAttention a, SkinnyArgs p, int strips, int atten
     const bool linear = b < 2 * pairs ? (b & 1) != 0 : linear_groups > attention_groups;
     const int index = b < 2 * pairs ? b >> 1 : b - pairs;
     if (linear) {
-        skinny_persistent_body<PER, 1, true, true, 2, false>(p, strips, index, linear_groups);
+        skinny_persistent_body<PER, 1, true, false, BS_DEPTH, false>(p, strips, index, linear_groups);
         return;
     }
     const int t = index % a.n, h = index / a.n % a.H, split = index / (a.n * a.H);
@@ -66,17 +70,16 @@ KA_API int ka_attention_decode_beside_supported(int n, int H, int splits, int hd
 }
 
 // Attention as ka_attention_decode_bf16 computes it (same operands, 8 waves a workgroup), and beside it
-// ln_out = act(LayerNorm(ln_x; gamma, beta, eps) @ W^T + bias) for the same n rows: ln_x fp32 [n, K].
+// lin_out = act(A @ W^T + bias) for the same n rows: A bf16 [n, K], rows lda apart.
 KA_API int ka_attention_decode_beside_bf16(const void* q, long q_row_stride, const void* k_cache, const void* v_cache,
                                            const int* block_table, int max_pages, const int* token_row,
                                            const int* kv_lo, const int* kv_hi, void* out, long out_row_stride,
                                            float scale, int n, int H, int Hkv, int hd, int page_size, int splits,
                                            float* partial, long partial_floats, const void* k_new, const void* v_new,
                                            long new_stride, const float* table, int rot, const int* slots,
-                                           void* k_cache_w, void* v_cache_w, const float* ln_x, const float* ln_gamma,
-                                           const float* ln_beta, float ln_eps, int K, const void* W, long ldw,
-                                           const float* bias, void* ln_out, int ln_out_dtype, long ldo, int N, int act,
-                                           hipStream_t stream) {
+                                           void* k_cache_w, void* v_cache_w, const void* A, long lda, int K,
+                                           const void* W, long ldw, const float* bias, void* lin_out, int lin_out_dtype,
+                                           long ldo, int N, int act, hipStream_t stream) {
     const char* who = "ka_attention_decode_beside_bf16";
     BesideAttention a = {};
     if (decode_check(who, q, q_row_stride, out, out_row_stride, n, H, Hkv, hd, page_size, max_pages, splits, partial,
@@ -95,26 +98,23 @@ KA_API int ka_attention_decode_beside_bf16(const void* q, long q_row_stride, con
     SkinnyArgs p = {};
     p.M = n;
     p.K[0] = K;
-    p.a = SkinnyTarget{(const bf16_t*)W, ldw, bias, ln_out, ldo, ln_out_dtype, N, act, 0};
+    p.a = SkinnyTarget{(const bf16_t*)W, ldw, bias, lin_out, ldo, lin_out_dtype, N, act, 0};
     if (check_target(who, p.a, K)) return -1;
     KA_CHECK(persistent_bias_ok(p.a), "%s: the bias must be 16-byte aligned and N a multiple of 4", who);
-    KA_CHECK(ln_x && ln_gamma && ln_eps >= 0.f && (uintptr_t)ln_x % 16 == 0 && (uintptr_t)ln_gamma % 16 == 0 &&
-                 (uintptr_t)ln_beta % 16 == 0, "%s: LayerNorm operands must be 16-byte aligned", who);
-    p.ln_x = ln_x; p.ln_gamma = ln_gamma; p.ln_beta = ln_beta; p.ln_eps = ln_eps;
+    KA_CHECK(A && lda % 8 == 0 && lda >= K && (uintptr_t)A % 16 == 0, "%s: the linear layer's input rows must be 16-byte aligned and >= K", who);
+    p.A[0] = (const bf16_t*)A; p.lda[0] = lda;
     const int strips = ka_cdiv(N, SK_STRIP);
     p.strips_a = strips;
-    const size_t dyn = (size_t)n * (K + SK_PAD) * sizeof(bf16_t);
+    const size_t dyn = 0;
 
-    // linear workgroups: the chip holds two workgroups of this launch per compute unit; as many
-    // as leave the attention workgroups their places (an eighth more was measured harmless, more
-    // than that costly), cut so that every one walks over the same number of strips
+    // linear workgroups: the chip holds two workgroups of this launch per compute unit; as many as
+    // fill the places that attention leaves, and no more: a workgroup that has to wait for a place
+    // starts when the first ones end, and the launch takes twice as long. Strips go round the
+    // workgroups, so some walk over one strip more than others.
     const long attention_groups = (long)n * H * splits;
     const int cus = ka_compute_units();
-    int linear_groups = strips;
-    for (int rounds = 1; rounds <= strips; ++rounds) {
-        linear_groups = ka_cdiv(strips, rounds);
-        if (linear_groups <= cus || attention_groups + linear_groups <= 2 * cus + cus / 4) break;
-    }
+    int linear_groups = (int)(2 * cus - attention_groups);
+    if (linear_groups > strips) linear_groups = strips;
     KA_CHECK(attention_groups + linear_groups < (1L << 31), "%s: too many workgroups", who);
     const int per = ka_cdiv(ka_cdiv(K, SK_KBLOCK), SP_WAVES);
     dim3 grid((unsigned)(attention_groups + linear_groups)), block(BS_WAVES * KA_WAVE);

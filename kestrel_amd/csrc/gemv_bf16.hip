@@ -440,7 +440,13 @@ static int launch_split(int waves, int strips, hipStream_t stream, const SkinnyA
 // The general entry point. Segments: A1 [M, K1] with W (target a) and optionally A2 [M, K2] with
 // W2 (same rows as target a; not with a second target). ln_x non-null: A1 is replaced by
 // LayerNorm(ln_x) (M <= 16, K1 <= 2048). Target b (Wb non-null) shares the input.
-static int skinny_fused(const KaThenNorm* then, const void* A1, long lda1, int K1, const void* A2, long lda2, int K2,
+struct SkinnyExtras {                 // what only some callers of skinny_fused bring
+    const KaThenNorm* then = nullptr; // a norm of the finished rows
+    void* ln_store = nullptr;         // where the LayerNorm prologue also leaves its normalised rows (bf16)
+    long ln_store_ld = 0;
+};
+
+static int skinny_fused(const SkinnyExtras& extras, const void* A1, long lda1, int K1, const void* A2, long lda2, int K2,
                                   const void* W2, long ldw2, const float* bias2, const float* ln_x,
                                   const float* ln_gamma, const float* ln_beta, float ln_eps, const void* Wa,
                                   long ldwa, const float* biasa, void* outa, int out_dtype_a, long ldoa, int Na,
@@ -448,6 +454,7 @@ static int skinny_fused(const KaThenNorm* then, const void* A1, long lda1, int K
                                   void* outb, int out_dtype_b, long ldob, int Nb, int actb, int M,
                                   int target_waves, float* partials, long partial_floats, hipStream_t stream) {
     const char* who = "ka_linear_skinny_fused";
+    const KaThenNorm* then = extras.then;
     KA_CHECK(M > 0 && M <= 64, "%s: M=%d outside 1..64", who, M);
     KA_CHECK(K1 > 0 && K1 % 8 == 0, "%s: K=%d must be a positive multiple of 8", who, K1);
     if (then) {
@@ -472,6 +479,11 @@ static int skinny_fused(const KaThenNorm* then, const void* A1, long lda1, int K
                      (uintptr_t)ln_beta % 16 == 0, "%s: LayerNorm operands must be 16-byte aligned", who);
         KA_CHECK(A2 == nullptr && !accumulate_a, "%s: no second segment and no accumulation with a LayerNorm prologue", who);
         args.ln_x = ln_x; args.ln_gamma = ln_gamma; args.ln_beta = ln_beta; args.ln_eps = ln_eps;
+        if (extras.ln_store) {
+            KA_CHECK(extras.ln_store_ld >= K1 && extras.ln_store_ld % 8 == 0 && (uintptr_t)extras.ln_store % 16 == 0,
+                     "%s: the stored normalised rows must be 16-byte aligned and >= K apart", who);
+            args.ln_store = (bf16_t*)extras.ln_store; args.ln_store_ld = extras.ln_store_ld;
+        }
     } else {
         KA_CHECK(A1 && lda1 % 8 == 0 && lda1 >= K1 && (uintptr_t)A1 % 16 == 0, "%s: input rows must be 16-byte aligned and >= K", who);
         args.A[0] = (const bf16_t*)A1; args.lda[0] = lda1;
@@ -505,11 +517,11 @@ static int skinny_fused(const KaThenNorm* then, const void* A1, long lda1, int K
     // the wide kernel shares them through LDS). Two targets go one after the other.
     const bool persistent_ok = !A2 && !accumulate_a && sk_persistent_enabled && persistent_fits(M, kblocks, args);
     if (M > 16 && Wb && partials && sk_wide_enabled && !persistent_ok) {
-        int rc = skinny_fused(nullptr, A1, lda1, K1, nullptr, 0, 0, nullptr, 0, nullptr, nullptr, nullptr, nullptr, 0.f,
+        int rc = skinny_fused(SkinnyExtras{}, A1, lda1, K1, nullptr, 0, 0, nullptr, 0, nullptr, nullptr, nullptr, nullptr, 0.f,
                                         Wa, ldwa, biasa, outa, out_dtype_a, ldoa, Na, acta, accumulate_a, nullptr, 0,
                                         nullptr, nullptr, 0, 0, 0, 0, M, target_waves, partials, partial_floats, stream);
         if (rc) return rc;
-        return skinny_fused(nullptr, A1, lda1, K1, nullptr, 0, 0, nullptr, 0, nullptr, nullptr, nullptr, nullptr, 0.f,
+        return skinny_fused(SkinnyExtras{}, A1, lda1, K1, nullptr, 0, 0, nullptr, 0, nullptr, nullptr, nullptr, nullptr, 0.f,
                                       Wb, ldwb, biasb, outb, out_dtype_b, ldob, Nb, actb, 0, nullptr, 0, nullptr,
                                       nullptr, 0, 0, 0, 0, M, target_waves, partials, partial_floats, stream);
     }
@@ -596,7 +608,7 @@ KA_API int ka_linear_skinny_fused(const void* A1, long lda1, int K1, const void*
                                   int acta, int accumulate_a, const void* Wb, long ldwb, const float* biasb,
                                   void* outb, int out_dtype_b, long ldob, int Nb, int actb, int M,
                                   int target_waves, float* partials, long partial_floats, hipStream_t stream) {
-    return skinny_fused(nullptr, A1, lda1, K1, A2, lda2, K2, W2, ldw2, bias2, ln_x, ln_gamma, ln_beta, ln_eps, Wa, ldwa, biasa,
+    return skinny_fused(SkinnyExtras{}, A1, lda1, K1, A2, lda2, K2, W2, ldw2, bias2, ln_x, ln_gamma, ln_beta, ln_eps, Wa, ldwa, biasa,
                         outa, out_dtype_a, ldoa, Na, acta, accumulate_a, Wb, ldwb, biasb, outb, out_dtype_b, ldob, Nb, actb, M,
                         target_waves, partials, partial_floats, stream);
 }
@@ -612,9 +624,25 @@ KA_API int ka_linear_skinny_pair_norm(const void* A1, long lda1, int K1, const v
                                       const float* beta, float eps, void* normed, int normed_dtype, long ldn,
                                       hipStream_t stream) {
     const KaThenNorm then = {gamma, beta, eps, normed, normed_dtype, ldn};
-    return skinny_fused(&then, A1, lda1, K1, A2, lda2, K2, W2, ldw2, bias2, nullptr, nullptr, nullptr, 0.f, W1, ldw1, bias1, out,
+    SkinnyExtras extras;
+    extras.then = &then;
+    return skinny_fused(extras, A1, lda1, K1, A2, lda2, K2, W2, ldw2, bias2, nullptr, nullptr, nullptr, 0.f, W1, ldw1, bias1, out,
                         KA_F32, ldo, N, KA_ACT_NONE, accumulate, nullptr, 0, nullptr, nullptr, 0, 0, 0, 0, M, target_waves,
                         partials, partial_floats, stream);
+}
+
+// out = act(LayerNorm(x; gamma, beta, eps) W^T + bias) as ka_linear_skinny_fused computes it with its
+// LayerNorm prologue (at most 16 rows), and the normalised rows themselves in `normed` (bf16 [M, K],
+// rows ldn apart), for launches that follow and read the same normalised input.
+KA_API int ka_linear_skinny_norm_store(const float* x, const float* gamma, const float* beta, float eps, int K,
+                                       const void* W, long ldw, const float* bias, void* out, int out_dtype, long ldo,
+                                       int N, int act, int M, void* normed, long ldn, hipStream_t stream) {
+    KA_CHECK(normed, "ka_linear_skinny_norm_store: nowhere to store the normalised rows");
+    SkinnyExtras extras;
+    extras.ln_store = normed;
+    extras.ln_store_ld = ldn;
+    return skinny_fused(extras, nullptr, 0, K, nullptr, 0, 0, nullptr, 0, nullptr, x, gamma, beta, eps, W, ldw, bias, out, out_dtype,
+                        ldo, N, act, 0, nullptr, 0, nullptr, nullptr, 0, 0, 0, 0, M, 0, nullptr, 0, stream);
 }
 
 // One input, one weight matrix, one output.

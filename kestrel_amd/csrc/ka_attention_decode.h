@@ -94,6 +94,8 @@ __device__ __forceinline__ void at_rotated(const RotaryOperands& r, const Rotary
 // AHEAD: the keys of a wave's next tile are asked for before its current tile is worked on (32
 // registers more at head size 64): one trip to memory less per tile where a wave has more than one
 // tile and the kernel is a chain of trips (few rows), no gain where it streams (many rows).
+// (A tile's values asked for together with its keys instead: slower, 11.8 against 11.2 us for the
+// attention of one row with eight waves.)
 template <int HD, int WAVES, bool AHEAD = false>
 __device__ __forceinline__ void
 attn_decode_body(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t* __restrict__ k_cache,

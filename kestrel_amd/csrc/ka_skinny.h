@@ -76,6 +76,8 @@ struct SkinnyArgs {
     const float* ln_gamma;
     const float* ln_beta;
     float ln_eps;
+    bf16_t* ln_store;       // non-null: workgroup 0 also stores the normalised rows here, [M, K[0]] rows ln_store_ld apart
+    long ln_store_ld;
     SkinnyTarget a, b;      // b.W null: one target
     int strips_a;
     int M;
@@ -289,6 +291,13 @@ __device__ __forceinline__ void skinny_persistent_body(const SkinnyArgs& p, cons
         }
         __syncthreads();
         const int ld = K + SK_PAD;
+        if (p.ln_store != nullptr && block == 0) {
+            // (every workgroup has normalised the same rows; one of them leaves them for later launches)
+            for (int c = threadIdx.x; c < M * (K / 8); c += SP_WAVES * KA_WAVE) {
+                const int m = c / (K / 8), k = (c % (K / 8)) * 8;
+                *reinterpret_cast<bf16x8*>(p.ln_store + (size_t)m * p.ln_store_ld + k) = *reinterpret_cast<const bf16x8*>(xs + m * ld + k);
+            }
+        }
 #pragma unroll
         for (int u = 0; u < PER; ++u) {
             const int k = (wave + u * SP_WAVES) * SK_KBLOCK;

@@ -49,8 +49,10 @@ _SIGNATURES = {
         _c_void_p, _c_long, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_long,
         _c_float, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_long,                # ..., splits, partial sums
         _c_void_p, _c_void_p, _c_long, _c_void_p, _c_int, _c_void_p, _c_void_p, _c_void_p,          # the tokens' own keys and values
-        _c_void_p, _c_void_p, _c_void_p, _c_float, _c_int,                                          # ln_x, gamma, beta, eps, K
+        _c_void_p, _c_long, _c_int,                                                                  # A, lda, K
         _c_void_p, _c_long, _c_void_p, _c_void_p, _c_int, _c_long, _c_int, _c_int, _c_void_p],      # W, ldw, bias, out, ..., stream
+    "ka_linear_skinny_norm_store": [_c_void_p, _c_void_p, _c_void_p, _c_float, _c_int, _c_void_p, _c_long, _c_void_p, _c_void_p,
+                                    _c_int, _c_long, _c_int, _c_int, _c_int, _c_void_p, _c_long, _c_void_p],
 }
 
 # Rows up to which the weight-streaming kernel is used instead of the tiled one.
@@ -274,10 +276,11 @@ def linear_two_outputs(a, wa, ba, out_a, act_a, wb, bb, out_b, act_b) -> bool:
     return True
 
 
-def layernorm_linear(x, gamma, beta, eps, wa, ba, out_a, act_a, wb=None, bb=None, out_b=None, act_b=0) -> bool:
+def layernorm_linear(x, gamma, beta, eps, wa, ba, out_a, act_a, wb=None, bb=None, out_b=None, act_b=0, store=None) -> bool:
     """``h = LayerNorm(x)``; ``out_a = act_a(h @ wa.T + ba)`` and, if a second target is given,
     ``out_b = act_b(h @ wb.T + bb)`` in one launch: the kernel normalises the fp32 rows itself
-    (at most 16 of them, at most 4096 wide, and no more than fit in 96 KB of LDS as bf16)."""
+    (at most 16 of them, at most 4096 wide, and no more than fit in 96 KB of LDS as bf16).
+    ``store`` (one target only): bf16 ``[m, k]`` that also receives ``h``, for launches that follow."""
     m, k = x.shape
     if not (0 < m <= SKINNY_LN_MAX_ROWS) or k % 8 or k > SKINNY_LN_MAX_WIDTH or x.dtype != torch.float32 \
             or not x.is_contiguous():
@@ -298,6 +301,14 @@ def layernorm_linear(x, gamma, beta, eps, wa, ba, out_a, act_a, wb=None, bb=None
     for bias, n in ((ba, na), (bb, nb)):
         if bias is not None and (n % 4 or bias.data_ptr() % 16):
             return False
+    if store is not None:
+        if two or store.dtype != torch.bfloat16 or not _out_ok(store, m, k) or store.stride(0) % 8:
+            return False
+        _check(lib().ka_linear_skinny_norm_store(
+            x.data_ptr(), gamma.data_ptr(), _ptr(beta), float(eps), k, wa.data_ptr(), wa.stride(0), _ptr(ba),
+            out_a.data_ptr(), _OUT_CODE[out_a.dtype], out_a.stride(0), na, act_a, m, store.data_ptr(), store.stride(0),
+            stream_ptr()))
+        return True
     _check(lib().ka_linear_skinny_fused(
         None, 0, k, None, 0, 0, None, 0, None,
         x.data_ptr(), gamma.data_ptr(), _ptr(beta), float(eps),
@@ -353,37 +364,32 @@ def _attention_operands_ok(q, out) -> bool:
     return not (q.data_ptr() % 16 or q.stride(0) % 8 or out.data_ptr() % 16 or out.stride(0) % 4)
 
 
-def _norm_linear_ok(job) -> bool:
-    """Operands of a ``parts.NormLinear`` that the persistent kernel's LayerNorm prologue takes."""
-    x, w, out = job.x, job.linear_weight, job.out
-    m, k = x.shape
-    if x.dtype != torch.float32 or not x.is_contiguous() or x.data_ptr() % 16 or k % 8:
+def _side_linear_ok(job) -> bool:
+    """Operands of a ``parts.SideLinear`` that the persistent skinny kernel takes."""
+    a, w, out = job.a, job.weight, job.out
+    if a.dim() != 2 or a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
         return False
-    for vec in (job.norm_weight, job.norm_bias):
-        if vec is not None and (vec.dtype != torch.float32 or vec.numel() != k or vec.data_ptr() % 16):
-            return False
-    if job.norm_weight is None:
-        return False
+    m, k = a.shape
     n = w.shape[0]
-    if not (_operand_ok(w, k) and _out_ok(out, m, n) and _bias_ok(job.linear_bias, n)):
+    if k % 8 or not (_operand_ok(a, k) and _operand_ok(w, k) and _out_ok(out, m, n) and _bias_ok(job.bias, n)):
         return False
-    return job.linear_bias is None or (n % 4 == 0 and job.linear_bias.data_ptr() % 16 == 0)
+    return job.bias is None or (n % 4 == 0 and job.bias.data_ptr() % 16 == 0)
 
 
 def attention_decode_takes(job, n: int, n_heads: int, head_dim: int, page_size: int, max_kv: int) -> bool:
-    """Whether ``attention_decode_bf16`` runs ``job`` (a ``parts.NormLinear``) in its own launch: a few
+    """Whether ``attention_decode_bf16`` runs ``job`` (a ``parts.SideLinear``) in its own launch: a few
     rows whose attention leaves most of the chip idle."""
-    if not ATTENTION_TAKES_LINEAR or n == 0 or not _norm_linear_ok(job):
+    if not ATTENTION_TAKES_LINEAR or n == 0 or not _side_linear_ok(job) or job.a.shape[0] != n:
         return False
     splits = decode_shape(max_kv, n * n_heads)[0]
-    return bool(lib().ka_attention_decode_beside_supported(n, n_heads, splits, head_dim, page_size, job.x.shape[1]))
+    return bool(lib().ka_attention_decode_beside_supported(n, n_heads, splits, head_dim, page_size, job.a.shape[1]))
 
 
 def attention_decode_bf16(q, k_cache, v_cache, block_table, token_row, kv_lo, kv_hi, out, scale, n_heads,
                           n_kv_heads, head_dim, batch, fuse=None, beside=None) -> bool:
     """One token per row. ``fuse = (k_new, v_new, table, slots)``: the kernel also rotates q and the
     token's key and stores key and value in the cache (the rotary kernel is then not run).
-    ``beside``: a ``parts.NormLinear`` for which ``attention_decode_takes`` said yes; the launch
+    ``beside``: a ``parts.SideLinear`` for which ``attention_decode_takes`` said yes; the launch
     computes it on the side (False: it does not after all, and nothing was run)."""
     n = q.shape[0]
     page_size = k_cache.shape[2]
@@ -409,15 +415,14 @@ def attention_decode_bf16(q, k_cache, v_cache, block_table, token_row, kv_lo, kv
                 or new_stride % 8 or v_new.stride(0) != new_stride:
             return False
     if beside is not None:
-        w, lin_out = beside.linear_weight, beside.out
+        w, lin_out = beside.weight, beside.out
         _check(handle.ka_attention_decode_beside_bf16(
             q.data_ptr(), q.stride(0), k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(),
             block_table.shape[1], token_row.data_ptr(), _ptr(kv_lo), kv_hi.data_ptr(), out.data_ptr(), out.stride(0),
             float(scale), n, n_heads, n_kv_heads, head_dim, page_size, splits, partial.data_ptr(), partial.numel(),
             _ptr(k_new), _ptr(v_new), new_stride, _ptr(table), rot, _ptr(slots), k_cache.data_ptr(), v_cache.data_ptr(),
-            beside.x.data_ptr(), beside.norm_weight.data_ptr(), _ptr(beside.norm_bias), float(beside.eps),
-            beside.x.shape[1], w.data_ptr(), w.stride(0), _ptr(beside.linear_bias), lin_out.data_ptr(),
-            _OUT_CODE[lin_out.dtype], lin_out.stride(0), w.shape[0], int(beside.act), stream_ptr()))
+            beside.a.data_ptr(), beside.a.stride(0), beside.a.shape[1], w.data_ptr(), w.stride(0), _ptr(beside.bias),
+            lin_out.data_ptr(), _OUT_CODE[lin_out.dtype], lin_out.stride(0), w.shape[0], int(beside.act), stream_ptr()))
         return True
     _check(handle.ka_attention_decode_bf16(
         q.data_ptr(), q.stride(0), k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(),

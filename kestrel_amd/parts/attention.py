@@ -103,7 +103,7 @@ class PagedAttention(Mixer):
         if not self._decodes_fused(batch, cache):
             return False
         from ..ops import fast
-        return fast.attention_decode_takes(job, job.x.shape[0], self.spec.n_heads, self.spec.head_dim, cache.k.shape[2],
+        return fast.attention_decode_takes(job, job.a.shape[0], self.spec.n_heads, self.spec.head_dim, cache.k.shape[2],
                                            batch.max_kv)
 
     def attend(self, qkv, batch, cache: LayerCache, beside=None):
@@ -145,10 +145,7 @@ class PagedAttention(Mixer):
     @staticmethod
     def _alone(job) -> None:
         """A job that was promised a place in the attention launch and did not get one after all."""
-        from ..ops import fast
-        if not fast.layernorm_linear(job.x, job.norm_weight, job.norm_bias, job.eps, job.linear_weight,
-                                     job.linear_bias, job.out, job.act):
-            raise RuntimeError("a linear layer accepted for the attention launch is taken by no kernel")
+        linear(job.a, job.weight, job.bias, job.out, act=job.act)
 
     def forward(self, h, batch, cache: LayerCache, residual) -> None:
         qkv = batch.workspace.get("attn.qkv", (h.shape[0], self.qkv_dim), self.dtype)

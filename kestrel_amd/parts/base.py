@@ -91,18 +91,15 @@ class LayerCache:
 
 
 @dataclass
-class NormLinear:
-    """``out = act(LayerNorm(x; weight, bias, eps) @ linear_weight.T + linear_bias)``: a piece of a
-    block's work that depends on nothing the mixer computes (the first linear of a feed-forward that
-    reads the same normalised input). A mixer that says so (``Mixer.takes_beside``) is handed it with
-    ``attend`` and runs it in its own launch, on the compute units that its core leaves idle."""
+class SideLinear:
+    """``out = act(a @ weight.T + bias)``: a piece of a block's work that depends on nothing the mixer
+    computes (the first linear of a feed-forward that reads the same normalised input ``a``). A mixer
+    that says so (``Mixer.takes_beside``) is handed it with ``attend`` and runs it in its own launch,
+    on the compute units that its core leaves idle."""
 
-    x: torch.Tensor                       # fp32 [n, dim]: the residual
-    norm_weight: torch.Tensor
-    norm_bias: Optional[torch.Tensor]
-    eps: float
-    linear_weight: torch.Tensor           # [out, dim]
-    linear_bias: Optional[torch.Tensor]
+    a: torch.Tensor                       # [n, in], the block's normalised input
+    weight: torch.Tensor                  # [out, in]
+    bias: Optional[torch.Tensor]
     out: torch.Tensor                     # [n, out]
     act: int                              # activation code of ``ops.linear``
 
@@ -134,12 +131,12 @@ class Mixer(Part):
         """``(weight [out, in], bias or None, out)`` of the first linear, or ``None``."""
         return None
 
-    def attend(self, projected: torch.Tensor, batch, cache: LayerCache, beside: Optional[NormLinear] = None) -> torch.Tensor:
+    def attend(self, projected: torch.Tensor, batch, cache: LayerCache, beside: Optional[SideLinear] = None) -> torch.Tensor:
         """The core on the projected input; returns the input of the output projection. ``beside``
         is only ever given after ``takes_beside`` said yes, and is done when this returns."""
         raise NotImplementedError
 
-    def takes_beside(self, job: NormLinear, batch, cache: LayerCache) -> bool:
+    def takes_beside(self, job: SideLinear, batch, cache: LayerCache) -> bool:
         """Whether ``attend`` would run ``job`` inside its own launch for this batch."""
         return False
 

@@ -6,7 +6,7 @@ from typing import Callable, Dict, Optional
 
 import torch
 
-from .base import LayerCache, NormLinear, Part, build_part
+from .base import LayerCache, Part, SideLinear, build_part
 from .specs import LayerSpec, ParamSpec
 
 
@@ -36,11 +36,13 @@ def _parallel_few_rows(block: "Block", x, batch, cache, normed, then, handed) ->
     if normed is not None:
         fused = fast.linear_two_outputs(normed, m_in[0], m_in[1], projected, 0, f_in[0], f_in[1], hidden, f_in[3])
     if not fused and fast.FUSE_LAYERNORM_PROLOGUE and getattr(norm.spec, "kind", None) == "layernorm":
-        # the feed-forward's first linear goes into the mixer's launch where the mixer takes it,
-        # else into the launch of the mixer's first linear
-        job = NormLinear(x, norm.weight, norm.bias, norm.spec.eps, f_in[0], f_in[1], hidden, f_in[3])
+        # the feed-forward's first linear goes into the mixer's launch where the mixer takes it (the
+        # launch of the mixer's first linear then leaves the normalised rows for it), else into the
+        # launch of the mixer's first linear
+        h = ws.get("block.h", tuple(x.shape), block.dtype)
+        job = SideLinear(h, f_in[0], f_in[1], hidden, f_in[3])
         if block.mixer.takes_beside(job, batch, cache) and \
-                fast.layernorm_linear(x, norm.weight, norm.bias, norm.spec.eps, m_in[0], m_in[1], projected, 0):
+                fast.layernorm_linear(x, norm.weight, norm.bias, norm.spec.eps, m_in[0], m_in[1], projected, 0, store=h):
             fused, beside = True, job
         else:
             fused = fast.layernorm_linear(x, norm.weight, norm.bias, norm.spec.eps, m_in[0], m_in[1], projected, 0,

@@ -826,10 +826,11 @@ def test_decode_attention_that_rotates_and_stores(shape):
                                    (2, 1, 16, 16, 1032, 24, 2), (3, 3, 32, 32, 64, 4100, 1)])
 def test_decode_attention_with_a_linear_layer_beside_it(shape, keys_per_workgroup, monkeypatch):
     """One launch computes the decode attention (rotating and storing the tokens' own keys) and, in
-    other workgroups, a LayerNorm + linear of the same rows. Both results are, bit for bit, what the
-    two kernels give alone (attention with the same 8 waves a workgroup), and so is the cache."""
+    other workgroups, a linear layer on bf16 rows that an earlier launch normalised and left behind.
+    Both results are, bit for bit, what the kernels give alone (attention with the same 8 waves a
+    workgroup), and so is the cache; the rows left behind are the LayerNorm of the input."""
     from kestrel_amd.ops import fast
-    from kestrel_amd.parts import NormLinear
+    from kestrel_amd.parts import SideLinear
 
     h, hkv, hd, rot, k, n_out, act = shape
     bf = torch.bfloat16
@@ -861,11 +862,21 @@ def test_decode_attention_with_a_linear_layer_beside_it(shape, keys_per_workgrou
                                               beside=beside)
             return out, k_c, v_c
 
+        # the launch before: LayerNorm + some linear, which leaves the normalised rows
+        first = torch.empty(n, 24, dtype=bf, device=DEV)
+        normed = torch.full((n, k), float("nan"), dtype=bf, device=DEV)
+        w_first = (torch.randn(24, k) / k ** 0.5).bfloat16().to(DEV)
+        assert fast.layernorm_linear(x, gamma, beta, 1e-5, w_first, None, first, 0, store=normed)
+        hidden = F.layer_norm(x.double(), (k,), gamma.double(), beta.double(), 1e-5)
+        _close(normed, hidden, bf, scale=2)
+        without = torch.empty(n, 24, dtype=bf, device=DEV)
+        assert fast.layernorm_linear(x, gamma, beta, 1e-5, w_first, None, without, 0)
+        assert torch.equal(first, without)
         alone = torch.empty(n, n_out, dtype=bf, device=DEV)
-        assert fast.layernorm_linear(x, gamma, beta, 1e-5, w, bias, alone, act)
+        assert fast.linear_bf16(normed, w, bias, alone, act, False)
         out_ref, k_ref, v_ref = run(None)
         together = torch.full((n, n_out), float("nan"), dtype=bf, device=DEV)
-        job = NormLinear(x, gamma, beta, 1e-5, w, bias, together, act)
+        job = SideLinear(normed, w, bias, together, act)
         assert fast.attention_decode_takes(job, n, h, hd, 16, case.batch.max_kv)
         out, k_c, v_c = run(job)
         assert torch.equal(out, out_ref)
@@ -873,24 +884,22 @@ def test_decode_attention_with_a_linear_layer_beside_it(shape, keys_per_workgrou
         assert torch.equal(k_c.view(torch.int16), k_ref.view(torch.int16))
         assert torch.equal(v_c.view(torch.int16), v_ref.view(torch.int16))
         assert torch.equal(together, alone)
-        hidden = F.layer_norm(x.double(), (k,), gamma.double(), beta.double(), 1e-5).to(bf).double()
-        _close(together, _ACTIVATE[act](hidden @ w.double().T + bias.double()), bf, scale=2)
+        _close(together, _ACTIVATE[act](normed.double() @ w.double().T + bias.double()), bf, scale=2)
 
 
 def test_decode_attention_declines_a_linear_layer_it_cannot_carry():
     from kestrel_amd.ops import fast
-    from kestrel_amd.parts import NormLinear
+    from kestrel_amd.parts import SideLinear
 
-    def job(rows, k, n_out=64, x_dtype=torch.float32):
-        return NormLinear(torch.zeros(rows, k, dtype=x_dtype, device=DEV), torch.ones(k, device=DEV), None, 1e-5,
-                          torch.zeros(n_out, k, dtype=torch.bfloat16, device=DEV), None,
-                          torch.empty(rows, n_out, dtype=torch.bfloat16, device=DEV), 0)
+    def job(rows, k, n_out=64, a_dtype=torch.bfloat16):
+        return SideLinear(torch.zeros(rows, k, dtype=a_dtype, device=DEV), torch.zeros(n_out, k, dtype=torch.bfloat16, device=DEV),
+                          None, torch.empty(rows, n_out, dtype=torch.bfloat16, device=DEV), 0)
 
     assert fast.attention_decode_takes(job(8, 2048), 8, 4, 64, 16, 1024)
-    assert not fast.attention_decode_takes(job(9, 2048), 9, 4, 64, 16, 1024)          # more rows than its prologue normalises
+    assert not fast.attention_decode_takes(job(9, 2048), 9, 4, 64, 16, 1024)          # more rows than it takes
     assert not fast.attention_decode_takes(job(8, 2056), 8, 4, 64, 16, 1024)          # a row too long for its registers
     assert not fast.attention_decode_takes(job(8, 2048), 8, 4, 80, 16, 1024)          # a head size that needs a SIMD's registers
-    assert not fast.attention_decode_takes(job(8, 2048, x_dtype=torch.bfloat16), 8, 4, 64, 16, 1024)
+    assert not fast.attention_decode_takes(job(8, 2048, a_dtype=torch.float32), 8, 4, 64, 16, 1024)
     assert fast.attention_decode_takes(job(4, 2048), 4, 32, 64, 16, 1024)
     assert not fast.attention_decode_takes(job(5, 2048), 5, 32, 64, 16, 1024)         # attention that fills the chip by itself
     assert not fast.attention_decode_takes(job(2, 2048), 2, 32, 64, 16, 3 * fast.DECODE_KEYS_PER_WORKGROUP)
