@@ -226,11 +226,10 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_
     };
 
     constexpr int STRIDE = 32 * AP_WAVES;
-    // one tile of 32 keys whose key rows are in `kr`; the next tile's go to `kr_next`
-    auto process = [&](int key0, const bf16x8* kr, bf16x8* kr_next) {
+    // one tile of 32 keys whose key rows are in `kr`, which the next tile's then take
+    auto process = [&](int key0, bf16x8* kr) {
         bf16x8 vr[2][DB];
         load_values(key0, vr);                             // in flight during the scores and the softmax
-        load_keys(key0 + STRIDE, kr_next);                 // in flight until the next tile
         __builtin_amdgcn_sched_barrier(0);
         const bool whole = key0 >= max_lo && key0 + 32 <= min_hi;
         // the scores of all blocks of queries first: the matrix pipes work on the later ones while
@@ -245,6 +244,12 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_
         for (int c = 0; c < QC; ++c)               // (the blocks take turns: an MFMA that adds to the one before it waits for it)
 #pragma unroll
             for (int b = 0; b < QB; ++b) s[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kr[c], qreg[b][c], s[b], 0, 0, 0);
+        // The next tile's key rows go into the registers that the products above have read: in flight
+        // until the next tile. (Two sets of registers taken in turn made the compiler keep the
+        // outputs in two places as well and copy all 64 registers of them over in every tile.)
+        __builtin_amdgcn_sched_barrier(0);
+        load_keys(key0 + STRIDE, kr);
+        __builtin_amdgcn_sched_barrier(0);
         // lane holds, for its query, the keys key0 + (v / 8) * 16 + lg * 8 + v % 8
         if (!whole) {
 #pragma unroll
@@ -304,18 +309,11 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_
                     o[b][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vr[pg][db], pb[b][pg], o[b][db], 0, 0, 0);
     };
 
-    // two tiles per round, their key rows in two sets of registers: the next tile's keys are
-    // always in flight while a tile is processed
-    bf16x8 ka[QC], kb[QC];
+    // the next tile's keys are always in flight while a tile is processed
+    bf16x8 kr[QC];
     int key0 = (wave_lo & ~31) + wave * 32;
-    load_keys(key0, ka);
-    while (key0 < wave_hi) {
-        process(key0, ka, kb);
-        key0 += STRIDE;
-        if (key0 >= wave_hi) break;
-        process(key0, kb, ka);
-        key0 += STRIDE;
-    }
+    load_keys(key0, kr);
+    for (; key0 < wave_hi; key0 += STRIDE) process(key0, kr);
     // the waves took different keys of the same queries: merge in wave order, a block of queries at a time
 #pragma unroll
     for (int b = 0; b < QB; ++b) {
