@@ -3,7 +3,8 @@
 // Every entry point is `extern "C"`, takes raw device pointers, plain integers and
 // a hipStream_t, validates its sizes on the host and returns 0 on success or a
 // negative code; `ka_last_error()` then gives the reason as text. Entry points
-// never allocate and never synchronise.
+// never allocate device memory and never synchronise (ka_linear_library_bf16 makes the
+// vendor library's handle and its plan for a set of sizes at the first call with them).
 #pragma once
 
 #include <hip/hip_runtime.h>
