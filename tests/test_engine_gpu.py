@@ -111,11 +111,14 @@ def test_mixed_batches_with_page_reuse(name, dtype):
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=DTYPE_IDS)
 @pytest.mark.parametrize("name", ["D", "F"])
-def test_many_requests_decoded_together(name, dtype):
-    """More rows than the weight-streaming kernels take (70 and 130): short prompts fed together in
-    one step, then decoded side by side, one token each a step."""
-    for count in (70, 130):
-        runner = _runner(name, dtype, n_pages=2 * count + 8, max_requests=count)
+@pytest.mark.parametrize("graphs", [False, True], ids=["eager", "graphs"])
+def test_many_requests_decoded_together(name, dtype, graphs):
+    """Short prompts fed together in one step, then decoded side by side, one token each a step: 12
+    rows (the kernel that cuts K into parts takes the last linears from 9 rows on), 24 and 48 (a
+    block's last launch also computes the next block's norm from 17 rows on; replayed in the buckets
+    of 32 and 48 rows, with padding rows), 70 and 130 (more rows than the weight-streaming kernels take)."""
+    for count in (12, 24, 48, 70, 130):
+        runner = _runner(name, dtype, n_pages=2 * count + 8, max_requests=count, graphs=graphs)
         reqs = {f"r{i}": _request(name, f"r{i}", 900 + i, 6 + i % 9) for i in range(count)}
         steps = [[(tag, 3 + int(tag[1:]) % 4) for tag in reqs]]
         while True:
