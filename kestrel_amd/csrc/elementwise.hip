@@ -208,10 +208,16 @@ KA_API int ka_layernorm(const float* x, const int* rows, const float* gamma, con
     KA_CHECK(out_dtype == KA_F32 || out_dtype == KA_BF16, "ka_layernorm: unsupported out dtype %d", out_dtype);
     const bool aligned = dim % 4 == 0 && (uintptr_t)x % 16 == 0 && (uintptr_t)gamma % 16 == 0;
     if (aligned && dim <= LN_THREADS * 4 * 4) {
-        if (out_dtype == KA_F32)
-            hipLaunchKernelGGL((layernorm_regs_kernel<float, 4>), grid, block, 0, stream, x, rows, gamma, beta, eps, (float*)out, dim);
-        else
-            hipLaunchKernelGGL((layernorm_regs_kernel<bf16_t, 4>), grid, block, 0, stream, x, rows, gamma, beta, eps, (bf16_t*)out, dim);
+        // (as many loads per thread as the row needs: 1, 2 or 4 of 16 bytes)
+#define KA_LN_REGS(ITEMS)                                                                                                     \
+    if (out_dtype == KA_F32)                                                                                                  \
+        hipLaunchKernelGGL((layernorm_regs_kernel<float, ITEMS>), grid, block, 0, stream, x, rows, gamma, beta, eps, (float*)out, dim); \
+    else                                                                                                                      \
+        hipLaunchKernelGGL((layernorm_regs_kernel<bf16_t, ITEMS>), grid, block, 0, stream, x, rows, gamma, beta, eps, (bf16_t*)out, dim)
+        if (dim <= LN_THREADS * 4) { KA_LN_REGS(1); }
+        else if (dim <= LN_THREADS * 4 * 2) { KA_LN_REGS(2); }
+        else { KA_LN_REGS(4); }
+#undef KA_LN_REGS
     } else if (out_dtype == KA_F32) {
         hipLaunchKernelGGL(layernorm_kernel<float>, grid, block, 0, stream, x, rows, gamma, beta, eps, (float*)out, dim);
     } else {
