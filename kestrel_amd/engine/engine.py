@@ -139,6 +139,9 @@ class InferenceEngine:
         self._startup_error: Optional[BaseException] = None
         self._fatal: Optional[BaseException] = None
         self._stop = False
+        self._run_gate = threading.Event()          # set: the scheduler thread may launch steps
+        self._run_gate.set()
+        self._paused = threading.Event()            # set by the scheduler thread once a pause has drained
         self._next_id = 0
         self._id_lock = threading.Lock()
         self.runner = None
@@ -216,6 +219,16 @@ class InferenceEngine:
                         self._deliver_error(item, exc)
                 if self._stop and not scheduler.has_pending_work():
                     break
+                if not self._run_gate.is_set():
+                    # paused: what is in flight is read, the device is left idle, and nothing is
+                    # launched until resume(); requests that arrive meanwhile wait in the scheduler
+                    scheduler.drain()
+                    for result in scheduler.pop_completed():
+                        self._deliver(pending.pop(result.request_id), result)
+                    torch.cuda.synchronize(self.runner.device)
+                    self._paused.set()
+                    self._run_gate.wait(timeout=0.1)
+                    continue
                 if scheduler.has_pending_work():
                     scheduler.advance()
                     for result in scheduler.pop_completed():
@@ -250,9 +263,25 @@ class InferenceEngine:
         if not item.future.done():
             item.future.set_exception(exc)
 
+    def pause(self, *, timeout: Optional[float] = None) -> bool:
+        """Stop launching steps and wait until the device is idle (``kestrel/engine/core.py:810-825``).
+        Requests in flight keep their pages and go on after ``resume``; requests submitted meanwhile
+        wait. Returns whether the scheduler thread has acknowledged within ``timeout`` seconds."""
+        if self._thread is None or self._fatal is not None:
+            return True
+        self._paused.clear()
+        self._run_gate.clear()
+        return self._paused.wait(timeout)
+
+    def resume(self) -> None:
+        """Let the scheduler thread launch steps again (``kestrel/engine/core.py:827-836``)."""
+        self._paused.clear()
+        self._run_gate.set()
+
     def shutdown_sync(self) -> None:
         if self._thread is None:
             return
+        self._run_gate.set()
         self._inbox.put(None)
         self._thread.join()
         self._thread = None

@@ -261,6 +261,12 @@ class GenerationScheduler:
             did = True
         return did or self._fail_unfittable()
 
+    def drain(self) -> None:
+        """Read every step that is still in flight (``kestrel/engine/core.py:1556-1569``: what a pause
+        does before it reports). Nothing is launched; requests keep their pages."""
+        while self._inflight:
+            self._commit_step(self._inflight.popleft())
+
     def _sample(self, plan: StepPlan, logits: torch.Tensor):
         """Queue the sampling of the rows that end a prompt or decode, and the copy of their
         tokens to the host. Returns ``(ids, event, logprobs)``."""

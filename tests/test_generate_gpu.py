@@ -313,6 +313,39 @@ def test_a_request_too_large_for_the_cache_fails_alone():
         engine.shutdown_sync()
 
 
+def test_pause_leaves_nothing_in_flight_and_resume_goes_on():
+    """``pause`` / ``resume`` (``kestrel/engine/core.py:810-836``): after ``pause`` returns no step is in
+    flight and no token arrives, requests keep what they hold, a request submitted meanwhile waits; after
+    ``resume`` all of them end with the tokens an undisturbed run gives."""
+    import queue
+    import time
+
+    cfg = helpers.flat_config("B")
+    prompts = [helpers.random_ids(1240 + i, n, cfg["vocab_size"]) for i, n in enumerate([21, 9])]
+    late = helpers.random_ids(1243, 12, cfg["vocab_size"])
+    options = dict(max_new_tokens=200, temperature=0.8, top_p=0.9, seed=11, stop_ids=())
+    engine = _engine("B", "float32", pipeline_depth=2, kv_cache_pages=60)
+    try:
+        undisturbed = [r.tokens for r in engine.generate_batch_sync(prompts + [late], **options)]
+        stream: "queue.Queue" = queue.Queue()
+        futures = [engine.submit_sync(prompts[0], _stream=stream, **options), engine.submit_sync(prompts[1], **options)]
+        stream.get(timeout=60)                                    # decoding is under way
+        assert engine.pause(timeout=60)
+        assert len(engine.scheduler._inflight) == 0
+        while not stream.empty():
+            stream.get_nowait()
+        futures.append(engine.submit_sync(late, **options))
+        time.sleep(0.3)
+        assert stream.empty() and not any(f.done() for f in futures)
+        held = [g.pool.n_pages - g.pool.free_count for g in engine.runner.cache.groups]
+        assert all(n > 0 for n in held)
+        engine.resume()
+        assert [f.result(timeout=120).tokens for f in futures] == undisturbed
+        assert engine.pause(timeout=60)                           # an idle engine pauses too, and shuts down paused
+    finally:
+        engine.shutdown_sync()
+
+
 def test_async_entry_point_and_streaming():
     from kestrel_amd import InferenceEngine, RuntimeConfig
 
