@@ -24,6 +24,7 @@
 #include "ka_no_alloc.h"
 
 #include <mutex>
+#include <type_traits>
 
 // A lane's value combined with that of the lane 32 away (the two hold the halves of one query's
 // scores): v_permlane32_swap exchanges the halves of two registers inside the vector unit, where a
@@ -46,6 +47,7 @@ __device__ __forceinline__ float at_sum_with_other_half(float x) {
 constexpr int AP_WAVES = 4;                 // waves of a workgroup: all on the same 32 queries, keys interleaved
 constexpr int AP_QBLOCK = 32;               // queries per workgroup
 constexpr float AP_MAX_SLACK = 8.0f;        // powers of two the running maximum may grow before the outputs are rescaled
+constexpr float AP_SUM_LIMIT = 4096.0f;     // a query's exponentials of one tile may add up to this before the tile is run again with a new reference point
 constexpr int AP_MAX_TABLE = 24576;         // most block table entries of one row kept in LDS (393k keys)
 constexpr int ap_merge_floats(int hd) { return (hd + 31) / 32 * 16 + 2; }
 // block table entries of one row that fit in LDS beside the merge at head size hd
@@ -159,10 +161,12 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_
         for (int c = 0; c < QC; ++c) qreg[b][c] = at_load8(qp + c * 8);
     }
     floatx16 o[QB][DB];
-    float m_i[QB], l_i[QB];
+    float m_i[QB], m_ref[QB], l_i[QB];
+    bool settled = false;                // every live query of the wave has a reference point (the same in all lanes)
 #pragma unroll
     for (int b = 0; b < QB; ++b) {
         m_i[b] = -INFINITY;
+        m_ref[b] = 0.f;                  // m_i, or 0 while that is -inf
         l_i[b] = 0.f;
 #pragma unroll
         for (int db = 0; db < DB; ++db)
@@ -226,15 +230,21 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_
     };
 
     constexpr int STRIDE = 32 * AP_WAVES;
-    // one tile of 32 keys whose key rows are in `kr`, which the next tile's then take
-    auto process = [&](int key0, bf16x8* kr) {
+    // One tile of 32 keys whose key rows are in `kr`, which the next tile's then take, in two forms.
+    // Careful: the softmax looks for the tile's maximum and moves the queries' reference point where
+    // it has to. Plain (most tiles): the exponentials are taken straight from the reference point the
+    // queries have and no maximum is looked for; a tile whose scores lie far above that point shows
+    // in the sum of its exponentials (an overflow as infinity): the tile then adds zeros and `false`
+    // is returned, for the tile to be run again carefully.
+    auto process = [&](auto careful_tag, int key0, bf16x8* kr) -> bool {
+        constexpr bool CAREFUL = decltype(careful_tag)::value;
         bf16x8 vr[2][DB];
         load_values(key0, vr);                             // in flight during the scores and the softmax
         __builtin_amdgcn_sched_barrier(0);
         const bool whole = key0 >= max_lo && key0 + 32 <= min_hi;
         // the scores of all blocks of queries first: the matrix pipes work on the later ones while
         // the softmax of the first is computed, and the blocks' chains of dependent instructions
-        // (maximum, exchange with the other half of the wave, exponentials, sum) interleave
+        // (exchange with the other half of the wave, exponentials, sum) interleave
         floatx16 s[QB];
 #pragma unroll
         for (int b = 0; b < QB; ++b)
@@ -261,42 +271,72 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_
                 }
         }
         bf16x8 pb[QB][2];
-        float alpha[QB];
-        bool moved = false;
+        bool again = false;
+        if constexpr (!CAREFUL) {
+            float total[QB];
+            bool over = false;
 #pragma unroll
-        for (int b = 0; b < QB; ++b) {
-            float mx = s[b][0];
+            for (int b = 0; b < QB; ++b) {
+                float rowsum = 0.f;
 #pragma unroll
-            for (int v = 1; v < 16; ++v) mx = fmaxf(mx, s[b][v]);
-            mx = at_max_with_other_half(mx) * sl2;              // the scale is positive: max and scale commute
-            // The reference point of the exponentials follows the maximum only when that has grown by
-            // more than AP_MAX_SLACK (in powers of two): softmax does not care which point is taken, an
-            // exponential of up to 2^AP_MAX_SLACK is as exact in fp32 and bf16 as one below 1, and the
-            // outputs so far need no rescaling, which would otherwise be due in almost every tile
-            // (some query of the 64 finds a slightly larger score nearly every time).
-            const bool grow = mx > m_i[b] + AP_MAX_SLACK;       // (also from -inf to the first finite maximum)
-            const float m_new = grow ? mx : m_i[b];
-            const float m_use = m_new == -INFINITY ? 0.f : m_new;     // nothing visible yet: keep everything at zero
-            alpha[b] = grow ? __builtin_amdgcn_exp2f(m_i[b] - m_use) : 1.0f;
-            float rowsum = 0.f;
-#pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                float p = __builtin_amdgcn_exp2f(fmaf(s[b][v], sl2, -m_use));
-                rowsum += p;
-                pb[b][v / 8][v % 8] = (bf16_t)p;
+                for (int v = 0; v < 16; ++v) {
+                    float p = __builtin_amdgcn_exp2f(fmaf(s[b][v], sl2, -m_ref[b]));
+                    rowsum += p;
+                    pb[b][v / 8][v % 8] = (bf16_t)p;
+                }
+                total[b] = at_sum_with_other_half(rowsum);
+                over = over || !(total[b] <= AP_SUM_LIMIT);
             }
-            rowsum = at_sum_with_other_half(rowsum);
-            l_i[b] = l_i[b] * alpha[b] + rowsum;
-            m_i[b] = m_new;
-            moved = moved || alpha[b] != 1.0f;
-        }
-        if (__any(moved)) {
+            if (__any(over)) {                  // (a side path that only clears what the tile would add)
+                again = true;
 #pragma unroll
-            for (int b = 0; b < QB; ++b)
+                for (int b = 0; b < QB; ++b) {
+                    total[b] = 0.f;
+                    pb[b][0] = pb[b][1] = bf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+                }
+            }
 #pragma unroll
-                for (int db = 0; db < DB; ++db)
+            for (int b = 0; b < QB; ++b) l_i[b] += total[b];
+        } else {
+            float alpha[QB];
+            bool moved = false, unset = false;
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) o[b][db][v] *= alpha[b];
+            for (int b = 0; b < QB; ++b) {
+                float mx = s[b][0];
+#pragma unroll
+                for (int v = 1; v < 16; ++v) mx = fmaxf(mx, s[b][v]);
+                mx = at_max_with_other_half(mx) * sl2;              // the scale is positive: max and scale commute
+                // The reference point follows the maximum only when that has grown by more than
+                // AP_MAX_SLACK (in powers of two): softmax does not care which point is taken, an
+                // exponential of up to 2^AP_MAX_SLACK is as exact in fp32 and bf16 as one below 1, and the
+                // outputs so far need no rescaling.
+                const bool grow = mx > m_i[b] + AP_MAX_SLACK;       // (also from -inf to the first finite maximum)
+                const float m_new = grow ? mx : m_i[b];
+                const float m_use = m_new == -INFINITY ? 0.f : m_new;     // nothing visible yet: keep everything at zero
+                alpha[b] = grow ? __builtin_amdgcn_exp2f(m_i[b] - m_use) : 1.0f;
+                float rowsum = 0.f;
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    float p = __builtin_amdgcn_exp2f(fmaf(s[b][v], sl2, -m_use));
+                    rowsum += p;
+                    pb[b][v / 8][v % 8] = (bf16_t)p;
+                }
+                rowsum = at_sum_with_other_half(rowsum);
+                l_i[b] = l_i[b] * alpha[b] + rowsum;
+                m_i[b] = m_new;
+                m_ref[b] = m_use;
+                moved = moved || alpha[b] != 1.0f;
+                unset = unset || (q_valid[b] && m_new == -INFINITY);
+            }
+            settled = !__any(unset);
+            if (__any(moved)) {
+#pragma unroll
+                for (int b = 0; b < QB; ++b)
+#pragma unroll
+                    for (int db = 0; db < DB; ++db)
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) o[b][db][v] *= alpha[b];
+            }
         }
         // O^T[d][query] += V^T[d][key] P^T[key][query], one page per MFMA
         if (key0 + 32 > min(wave_hi, limit) || key0 < wave_lo) mask_values(key0, vr);
@@ -307,13 +347,22 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_
 #pragma unroll
                 for (int b = 0; b < QB; ++b)
                     o[b][db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vr[pg][db], pb[b][pg], o[b][db], 0, 0, 0);
+        return !again;
     };
 
     // the next tile's keys are always in flight while a tile is processed
     bf16x8 kr[QC];
     int key0 = (wave_lo & ~31) + wave * 32;
-    load_keys(key0, kr);
-    for (; key0 < wave_hi; key0 += STRIDE) process(key0, kr);
+    // Careful tiles until every live query has a reference point (a wave's first tile at the least),
+    // plain ones from there on, and back whenever a plain one has found scores too far above it.
+    while (key0 < wave_hi) {
+        load_keys(key0, kr);
+        do {
+            process(std::true_type{}, key0, kr);
+            key0 += STRIDE;
+        } while (key0 < wave_hi && !settled);
+        while (key0 < wave_hi && process(std::false_type{}, key0, kr)) key0 += STRIDE;
+    }
     // the waves took different keys of the same queries: merge in wave order, a block of queries at a time
 #pragma unroll
     for (int b = 0; b < QB; ++b) {

@@ -542,6 +542,28 @@ def test_a_far_key_among_hundreds_is_found(heads):
 
 
 @pytest.mark.parametrize("heads", EDGE_HEADS)
+def test_scores_that_climb_along_the_keys(heads):
+    """Every key lines up with the queries a little better than the one before it, so that each
+    tile of keys lies far above everything a query has seen so far: the prompt kernel, which takes
+    its exponentials from the reference point a query already has and looks for a new maximum only
+    when their sum says so, has to move that point again and again (by more than an exponential
+    can hold between some tiles, by little between others). And the other way round: scores that
+    fall, where the first tile's reference point serves to the end."""
+    h, hkv, hd = heads
+    bf = torch.bfloat16
+    for step, q_len in ((0.05, 300), (0.004, 300), (-0.05, 300), (0.3, 70), (0.05, 1)):
+        case = PagedCase([700], [q_len], h, hkv, hd, 16, bf, seed=31)
+        ramp = (torch.arange(700, dtype=torch.float32) * step).to(bf)
+        case.q[:, :hd] = 1.0
+        case.k[0][:, 0, :] = ramp[:, None]
+        for key in range(700):
+            case.k_cache[int(case.table[0, key // 16]), 0, key % 16, :] = ramp[key]
+        want = case.reference(hd ** -0.5)
+        for name in ("generic", "fast"):
+            _close(_run_attention(case, name, hd ** -0.5), want, bf)
+
+
+@pytest.mark.parametrize("heads", EDGE_HEADS)
 def test_a_windows_edge_is_kept(heads):
     """The key just outside a window lines up with the query far better than any other, the
     first key inside it second best: a kernel that lets the edge slip by one returns the wrong
