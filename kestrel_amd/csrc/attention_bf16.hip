@@ -187,22 +187,31 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_
     const unsigned v_lane_half = (unsigned)((kvh * HD + (DB - 1) * 32 + (li & 15)) * AT_PAGE + lg * 8);
 
     // half a key row of tile `key0` for this lane's (permuted) key
-    auto load_keys = [&](int key0, bf16x8* dst) {
+    auto key_address = [&](int key0) -> const bf16_t* {
         unsigned key = (unsigned)min(max(key0 + kperm, first_live), last_live);
         unsigned page = (unsigned)pages[key / AT_PAGE];
-        const bf16_t* kp = k_cache + ((size_t)page * page_stride + (k_lane + (key % AT_PAGE) * HD));
+        return k_cache + ((size_t)page * page_stride + (k_lane + (key % AT_PAGE) * HD));
+    };
+    auto load_keys_at = [&](const bf16_t* kp, bf16x8* dst) {
 #pragma unroll
         for (int c = 0; c < QC; ++c) dst[c] = at_load8(kp + c * 8);
     };
+    auto load_keys = [&](int key0, bf16x8* dst) { load_keys_at(key_address(key0), dst); };
 
     // the two value pages of tile `key0`: lane (d = li, g) loads 8 consecutive keys of channel d.
     // The page is the same for all lanes: its address is made in scalar registers.
-    auto load_values = [&](int key0, bf16x8 (*dst)[DB]) {
+    // (the pages are looked up a tile ahead, `value_pages`: the loads of a tile then start at once)
+    auto value_pages = [&](int key0, unsigned* page) {
 #pragma unroll
         for (int pg = 0; pg < 2; ++pg) {
             unsigned kbase = (unsigned)min(max(key0 + pg * AT_PAGE, first_live), last_live);
-            unsigned page = (unsigned)__builtin_amdgcn_readfirstlane(pages[kbase / AT_PAGE]);
-            const bf16_t* vp = v_cache + (size_t)page * page_stride;
+            page[pg] = (unsigned)__builtin_amdgcn_readfirstlane(pages[kbase / AT_PAGE]);
+        }
+    };
+    auto load_values = [&](const unsigned* page, bf16x8 (*dst)[DB]) {
+#pragma unroll
+        for (int pg = 0; pg < 2; ++pg) {
+            const bf16_t* vp = v_cache + (size_t)page[pg] * page_stride;
 #pragma unroll
             for (int db = 0; db < DB; ++db)
                 dst[pg][db] = at_load8(vp + (HALF_BLOCK && db == DB - 1 ? v_lane_half : v_lane + db * 32 * AT_PAGE));
@@ -236,11 +245,14 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_
     // queries have and no maximum is looked for; a tile whose scores lie far above that point shows
     // in the sum of its exponentials (an overflow as infinity): the tile then adds zeros and `false`
     // is returned, for the tile to be run again carefully.
-    auto process = [&](auto careful_tag, int key0, bf16x8* kr) -> bool {
+    auto process = [&](auto careful_tag, int key0, bf16x8* kr, unsigned* vpage) -> bool {
         constexpr bool CAREFUL = decltype(careful_tag)::value;
         bf16x8 vr[2][DB];
-        load_values(key0, vr);                             // in flight during the scores and the softmax
+        load_values(vpage, vr);                            // in flight during the scores and the softmax
         __builtin_amdgcn_sched_barrier(0);
+        // where the next tile's keys and values are: worked out beside the matrix products
+        const bf16_t* next_keys = key_address(key0 + STRIDE);
+        value_pages(key0 + STRIDE, vpage);
         const bool whole = key0 >= max_lo && key0 + 32 <= min_hi;
         // the scores of all blocks of queries first: the matrix pipes work on the later ones while
         // the softmax of the first is computed, and the blocks' chains of dependent instructions
@@ -258,7 +270,7 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_
         // until the next tile. (Two sets of registers taken in turn made the compiler keep the
         // outputs in two places as well and copy all 64 registers of them over in every tile.)
         __builtin_amdgcn_sched_barrier(0);
-        load_keys(key0 + STRIDE, kr);
+        load_keys_at(next_keys, kr);
         __builtin_amdgcn_sched_barrier(0);
         // lane holds, for its query, the keys key0 + (v / 8) * 16 + lg * 8 + v % 8
         if (!whole) {
@@ -355,13 +367,15 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_
     int key0 = (wave_lo & ~31) + wave * 32;
     // Careful tiles until every live query has a reference point (a wave's first tile at the least),
     // plain ones from there on, and back whenever a plain one has found scores too far above it.
+    unsigned vpage[2];
     while (key0 < wave_hi) {
         load_keys(key0, kr);
+        value_pages(key0, vpage);
         do {
-            process(std::true_type{}, key0, kr);
+            process(std::true_type{}, key0, kr, vpage);
             key0 += STRIDE;
         } while (key0 < wave_hi && !settled);
-        while (key0 < wave_hi && process(std::false_type{}, key0, kr)) key0 += STRIDE;
+        while (key0 < wave_hi && process(std::false_type{}, key0, kr, vpage)) key0 += STRIDE;
     }
     // the waves took different keys of the same queries: merge in wave order, a block of queries at a time
 #pragma unroll
