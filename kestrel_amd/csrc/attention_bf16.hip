@@ -446,66 +446,92 @@ attn_decode_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t
 // ----------------------------------------------------------------------------------------------
 // rotary encoding + cache write, a page's worth of tokens per workgroup
 // ----------------------------------------------------------------------------------------------
-// A workgroup takes 16 consecutive tokens of the packed batch. Queries are rotated in place and
-// keys rotated into the cache with 16-byte loads and stores (8 channels of a head and their 8
-// partners in the other half of the rotated part per thread). Values: the cache keeps a page
-// transposed, [channel][16 tokens]; when the 16 tokens fill one page in order (which they do
-// inside a prompt that starts on a page boundary) a thread gathers 8 channels of all 16 tokens
-// and stores 8 rows of 32 bytes, 256 contiguous bytes; other tokens are stored one by one.
+// A group of workgroups (grid y) takes 16 consecutive tokens of the packed batch. Queries are
+// rotated in place and keys rotated into the cache with 16-byte loads and stores (8 channels of a
+// head and their 8 partners in the other half of the rotated part per thread; the channels of a
+// key that are not rotated are copied, those of a query left alone). Values: the cache keeps a
+// page transposed, [channel][16 tokens]; when the 16 tokens fill one page in order (which they do
+// inside a prompt that starts on a page boundary) they are turned through LDS, 256 channels at a
+// time; other tokens are stored one by one. The first `light_parts`
+// workgroups of a group share the queries and keys, one piece of work per thread and round, the
+// others the values. (One workgroup of sixteen turning all the values in registers, its stores 256
+// bytes apart, and threads that met a query's plain channels with nothing to do: 18.7 us for 2,048
+// tokens of 32 heads of 64 launched back to back, against 13.1 us now.)
 constexpr int RC_TOKENS = AT_PAGE;
 constexpr int RC_THREADS = 256;
+constexpr int RC_VCHANNELS = 256;           // channels of the values that a workgroup turns at a time
 
 __global__ void __launch_bounds__(RC_THREADS)
 rope_cache_pages_kernel(bf16_t* __restrict__ qkv, long row_stride, const int* __restrict__ positions,
                         const int* __restrict__ slots, const float* __restrict__ table,
                         bf16_t* __restrict__ k_cache, bf16_t* __restrict__ v_cache, int n, int H, int Hkv,
-                        int hd, int rot) {
+                        int hd, int rot, int light_parts) {
     const int t0 = blockIdx.x * RC_TOKENS;
     const int n_here = min(RC_TOKENS, n - t0);
     const int half = rot / 2;
     const int pair_units = half / 8;                  // per head: 8 channels + their 8 partners
     const int plain_units = (hd - rot) / 8;           // per head: 8 channels that are not rotated
     const size_t page_elems = (size_t)Hkv * AT_PAGE * hd;
+    // (rows padded by 8 bytes: the two halves of the tokens, which neighbouring lanes read, then lie 16 banks apart)
+    __shared__ __attribute__((aligned(8))) bf16_t vtile[RC_TOKENS][RC_VCHANNELS + 4];
 
-    // queries and keys: (token, head, unit); heads 0..H-1 are queries, H..H+Hkv-1 keys
-    const int units = pair_units + plain_units;
-    const int per_token = (H + Hkv) * units;
-    // (the work of a group of tokens is dealt out over gridDim.y workgroups: there are few groups)
-    const int lane_id = blockIdx.y * RC_THREADS + threadIdx.x, lanes = gridDim.y * RC_THREADS;
-    for (int idx = lane_id; idx < n_here * per_token; idx += lanes) {
-        const int i = idx / per_token, rest = idx % per_token;
-        const int head = rest / units, u = rest % units;
-        const int t = t0 + i;
-        const bool is_key = head >= H;
-        const int slot = is_key && slots ? slots[t] : -1;
-        if (is_key && slot < 0) continue;                       // nothing is cached for this token
-        bf16_t* src = qkv + (size_t)t * row_stride + (size_t)head * hd;     // the keys follow the queries
-        bf16_t* kdst = nullptr;
-        if (is_key) kdst = k_cache + (size_t)(slot / AT_PAGE) * page_elems + ((size_t)(head - H) * AT_PAGE + slot % AT_PAGE) * hd;
-        if (u < pair_units) {
-            const int c0 = u * 8;
-            bf16x8 a = at_load8(src + c0), b = at_load8(src + half + c0);
-            const float* cs = table + (size_t)positions[t] * rot;
-            floatx4 c[2] = {*reinterpret_cast<const floatx4*>(cs + c0), *reinterpret_cast<const floatx4*>(cs + c0 + 4)};
-            floatx4 sn[2] = {*reinterpret_cast<const floatx4*>(cs + half + c0), *reinterpret_cast<const floatx4*>(cs + half + c0 + 4)};
-            bf16x8 ra, rb;
+    if ((int)blockIdx.y < light_parts) {
+        // Rotated pairs of the queries: (token, head, unit), the order of the rows of `qkv`; of the keys:
+        // (kv head, token, unit), the order of the page; then the plain channels of the keys, likewise:
+        // neighbouring lanes write neighbouring addresses
+        const int q_items = n_here * H * pair_units, k_items = slots ? n_here * Hkv * pair_units : 0;
+        const int pair_items = q_items + k_items;
+        const int items = pair_items + (slots ? n_here * Hkv * plain_units : 0);
+        const int lanes = light_parts * RC_THREADS;
+        for (int idx = blockIdx.y * RC_THREADS + threadIdx.x; idx < items; idx += lanes) {
+            if (idx < pair_items) {
+                const bool is_key = idx >= q_items;
+                int i, head, c0;
+                if (!is_key) {
+                    i = idx / (H * pair_units);
+                    head = idx % (H * pair_units) / pair_units;
+                } else {
+                    const int j = idx - q_items;
+                    head = H + j / (n_here * pair_units);
+                    i = j % (n_here * pair_units) / pair_units;
+                }
+                c0 = idx % pair_units * 8;                               // (q_items is a multiple of pair_units)
+                const int t = t0 + i;
+                const int slot = is_key ? slots[t] : -1;
+                if (is_key && slot < 0) continue;                       // nothing is cached for this token
+                bf16_t* src = qkv + (size_t)t * row_stride + (size_t)head * hd;     // the keys follow the queries
+                bf16_t* dst = src;
+                if (is_key) dst = k_cache + (size_t)(slot / AT_PAGE) * page_elems + ((size_t)(head - H) * AT_PAGE + slot % AT_PAGE) * hd;
+                bf16x8 a = at_load8(src + c0), b = at_load8(src + half + c0);
+                const float* cs = table + (size_t)positions[t] * rot;
+                floatx4 c[2] = {*reinterpret_cast<const floatx4*>(cs + c0), *reinterpret_cast<const floatx4*>(cs + c0 + 4)};
+                floatx4 sn[2] = {*reinterpret_cast<const floatx4*>(cs + half + c0), *reinterpret_cast<const floatx4*>(cs + half + c0 + 4)};
+                bf16x8 ra, rb;
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                float x = (float)a[j], y = (float)b[j], cc = c[j / 4][j % 4], ss = sn[j / 4][j % 4];
-                ra[j] = (bf16_t)(x * cc - y * ss);
-                rb[j] = (bf16_t)(y * cc + x * ss);
+                for (int j = 0; j < 8; ++j) {
+                    float x = (float)a[j], y = (float)b[j], cc = c[j / 4][j % 4], ss = sn[j / 4][j % 4];
+                    ra[j] = (bf16_t)(x * cc - y * ss);
+                    rb[j] = (bf16_t)(y * cc + x * ss);
+                }
+                *reinterpret_cast<bf16x8*>(dst + c0) = ra;
+                *reinterpret_cast<bf16x8*>(dst + half + c0) = rb;
+            } else {
+                const int j = idx - pair_items;                          // (kv head, token, unit): neighbouring lanes, neighbouring addresses in the page
+                const int kvh = j / (n_here * plain_units), rest = j % (n_here * plain_units);
+                const int i = rest / plain_units, c0 = rot + (rest % plain_units) * 8;
+                const int t = t0 + i, slot = slots[t];
+                if (slot < 0) continue;
+                const bf16_t* src = qkv + (size_t)t * row_stride + (size_t)(H + kvh) * hd;
+                bf16_t* dst = k_cache + (size_t)(slot / AT_PAGE) * page_elems + ((size_t)kvh * AT_PAGE + slot % AT_PAGE) * hd;
+                *reinterpret_cast<bf16x8*>(dst + c0) = at_load8(src + c0);
             }
-            bf16_t* dst = is_key ? kdst : src;
-            *reinterpret_cast<bf16x8*>(dst + c0) = ra;
-            *reinterpret_cast<bf16x8*>(dst + half + c0) = rb;
-        } else if (is_key) {
-            const int c0 = rot + (u - pair_units) * 8;
-            *reinterpret_cast<bf16x8*>(kdst + c0) = at_load8(src + c0);
         }
+        return;
     }
     if (!slots) return;
 
     // values
+    const int lane_id = (blockIdx.y - light_parts) * RC_THREADS + threadIdx.x, lanes = (gridDim.y - light_parts) * RC_THREADS;
     const int first = slots[t0];
     bool whole_page = n_here == RC_TOKENS && first >= 0 && first % AT_PAGE == 0;
     if (whole_page) {
@@ -514,23 +540,34 @@ rope_cache_pages_kernel(bf16_t* __restrict__ qkv, long row_stride, const int* __
     const int vwidth = Hkv * hd;
     const bf16_t* vsrc = qkv + (size_t)t0 * row_stride + (size_t)(H + Hkv) * hd;
     if (whole_page) {
+        // 256 channels of the 16 tokens at a time through LDS: read as 16-byte pieces of a token's row,
+        // written as 16-byte pieces of a channel's row of the page (8 tokens), neighbouring lanes
+        // neighbouring addresses both times
         bf16_t* vpage = v_cache + (size_t)(first / AT_PAGE) * page_elems;
-        for (int c0 = lane_id * 8; c0 < vwidth; c0 += lanes * 8) {
-            bf16x8 v[RC_TOKENS];
+        for (int cs = (blockIdx.y - light_parts) * RC_VCHANNELS; cs < vwidth; cs += (gridDim.y - light_parts) * RC_VCHANNELS) {
+            if (cs != (int)(blockIdx.y - light_parts) * RC_VCHANNELS) __syncthreads();      // the slice before has been read
 #pragma unroll
-            for (int i = 0; i < RC_TOKENS; ++i) v[i] = at_load8(vsrc + (size_t)i * row_stride + c0);
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                bf16x8 lo, hi;
-#pragma unroll
-                for (int i = 0; i < 8; ++i) {
-                    lo[i] = v[i][j];
-                    hi[i] = v[8 + i][j];
+            for (int r = 0; r < RC_TOKENS * RC_VCHANNELS / 8 / RC_THREADS; ++r) {
+                const int idx = threadIdx.x + r * RC_THREADS;
+                const int i = idx / (RC_VCHANNELS / 8), c0 = idx % (RC_VCHANNELS / 8) * 8;
+                if (cs + c0 < vwidth) {
+                    const bf16x8 piece = at_load8(vsrc + (size_t)i * row_stride + cs + c0);
+                    bf16x4* to = reinterpret_cast<bf16x4*>(&vtile[i][c0]);
+                    to[0] = bf16x4{piece[0], piece[1], piece[2], piece[3]};
+                    to[1] = bf16x4{piece[4], piece[5], piece[6], piece[7]};
                 }
-                // channel c0 + j = (head, d): its 16 tokens are one row of the page
-                bf16_t* dst = vpage + (size_t)(c0 + j) * AT_PAGE;
-                *reinterpret_cast<bf16x8*>(dst) = lo;
-                *reinterpret_cast<bf16x8*>(dst + 8) = hi;
+            }
+            __syncthreads();
+#pragma unroll
+            for (int r = 0; r < RC_VCHANNELS * 2 / RC_THREADS; ++r) {
+                const int c = threadIdx.x / 2 + r * (RC_THREADS / 2), part = threadIdx.x % 2;
+                if (cs + c < vwidth) {
+                    bf16x8 piece;
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) piece[i] = vtile[part * 8 + i][c];
+                    // channel cs + c = (head, d): its 16 tokens are one row of the page
+                    *reinterpret_cast<bf16x8*>(vpage + (size_t)(cs + c) * AT_PAGE + part * 8) = piece;
+                }
             }
         }
     } else {
@@ -561,10 +598,17 @@ KA_API int ka_rope_cache_pages_bf16(void* qkv, long row_stride, const int* posit
     KA_CHECK(!slots || (k_cache && v_cache && (uintptr_t)k_cache % 16 == 0 && (uintptr_t)v_cache % 16 == 0), "%s: cache tensors missing or not 16-byte aligned", who);
     if (n == 0) return 0;
     const int groups = ka_cdiv(n, RC_TOKENS);
-    int parts = ka_cdiv(2048, groups);           // enough workgroups for the chip, whatever the number of tokens
-    if (parts > 16) parts = 16;
-    hipLaunchKernelGGL(rope_cache_pages_kernel, dim3(groups, parts), dim3(RC_THREADS), 0, stream, (bf16_t*)qkv,
-                       row_stride, positions, slots, table, (bf16_t*)k_cache, (bf16_t*)v_cache, n, H, Hkv, hd, rot);
+    // workgroups per group of tokens: a piece of work per thread for queries and keys, as many for
+    // the values as have a piece each, and no more than fill the chip a few times over
+    const int pair_units = rot / 16, plain_units = (hd - rot) / 8;
+    const long light_items = (long)RC_TOKENS * ((H + Hkv) * pair_units + (slots ? Hkv * plain_units : 0));
+    int light_parts = ka_cdiv(light_items, RC_THREADS), value_parts = slots ? ka_cdiv((long)Hkv * hd, RC_VCHANNELS) : 0;
+    const int most = groups >= 256 ? 16 : 64;
+    if (light_parts > most) light_parts = most;
+    if (value_parts > most / 4) value_parts = most / 4;
+    hipLaunchKernelGGL(rope_cache_pages_kernel, dim3(groups, light_parts + value_parts), dim3(RC_THREADS), 0, stream,
+                       (bf16_t*)qkv, row_stride, positions, slots, table, (bf16_t*)k_cache, (bf16_t*)v_cache, n, H, Hkv, hd,
+                       rot, light_parts);
     KA_LAUNCH_CHECK();
     return 0;
 }
