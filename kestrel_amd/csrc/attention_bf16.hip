@@ -647,6 +647,8 @@ KA_API int ka_attention_prefill_bf16(const void* q, long q_row_stride, const voi
                      page_size, max_pages))
         return -1;
     KA_CHECK(ka_attention_prefill_supported(hd, page_size), "ka_attention_prefill_bf16: head size %d not covered", hd);
+    // (the kernel takes maxima of unscaled scores and turns masked scores into -inf before it scales them)
+    KA_CHECK(scale > 0.f && scale < INFINITY, "ka_attention_prefill_bf16: the scale must be positive and finite, got %g", (double)scale);
     KA_CHECK(query_block == 32 || (query_block == 64 && ka_attention_prefill_query_block(hd) == 64),
              "ka_attention_prefill_bf16: blocks of %d queries at head size %d (32%s)", query_block, hd,
              ka_attention_prefill_query_block(hd) == 64 ? " or 64" : " only");

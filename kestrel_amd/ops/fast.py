@@ -468,7 +468,8 @@ def attention_bf16(q, k_cache, v_cache, block_table, token_row, kv_lo, kv_hi, ou
     # the longest row's block table must fit in LDS (the whole table's width where the length is not known)
     longest = int(batch.max_kv) if batch.max_kv > 1 else block_table.shape[1] * page_size
     blocks = _query_blocks(batch, head_dim) if handle.ka_attention_prefill_supported(head_dim, page_size) else None
-    if blocks is not None and longest <= handle.ka_attention_prefill_max_keys(head_dim):
+    # (the prompt kernel is written for a positive scale; any other goes to the generic kernel)
+    if blocks is not None and longest <= handle.ka_attention_prefill_max_keys(head_dim) and 0.0 < scale < float("inf"):
         rows, first_tokens, size = blocks
         _check(handle.ka_attention_prefill_bf16(
             q.data_ptr(), q.stride(0), k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(),

@@ -541,6 +541,32 @@ def test_a_far_key_among_hundreds_is_found(heads):
         _close(out[-1, :hd], prompt.v[0][target, 0].double(), bf)
 
 
+def test_a_scale_that_is_not_positive_goes_to_the_generic_kernel():
+    """The prompt kernel assumes a positive scale (it scales a tile's maximum, not every score): a
+    negative or zero scale is declined by the fast path and refused by the library's entry point, and
+    the dispatcher's result is that of the generic kernel, which takes any scale."""
+    from kestrel_amd.ops import fast
+    from kestrel_amd.ops.attention import paged_attention
+
+    bf = torch.bfloat16
+    case = PagedCase([70, 40], [70, 9], 4, 2, 64, 16, bf, seed=41)
+    q = case.q.to(DEV)
+    for scale in (-0.2, 0.0):
+        out = torch.full((q.shape[0], case.h * case.hd), float("nan"), dtype=bf, device=DEV)
+        assert not fast.attention_bf16(q, case.k_cache, case.v_cache, case.table, case.token_row, case.kv_lo, case.kv_hi,
+                                       out, scale, case.h, case.hkv, case.hd, case.batch)
+        paged_attention(q, case.k_cache, case.v_cache, case.table, case.token_row, case.kv_lo, case.kv_hi, out, scale,
+                        case.h, case.hkv, case.hd, case.batch)
+        _close(out, case.reference(scale), bf)
+    rows, firsts = case.batch.query_blocks[64]
+    out = torch.empty((q.shape[0], case.h * case.hd), dtype=bf, device=DEV)
+    status = fast.lib().ka_attention_prefill_bf16(
+        q.data_ptr(), q.stride(0), case.k_cache.data_ptr(), case.v_cache.data_ptr(), case.table.data_ptr(), case.table.shape[1],
+        rows.data_ptr(), firsts.data_ptr(), int(rows.numel()), case.batch.cu_q.data_ptr(), case.batch.kv_len.data_ptr(), None,
+        case.kv_hi.data_ptr(), out.data_ptr(), out.stride(0), -0.2, case.h, case.hkv, case.hd, 16, 70, 64, None)
+    assert status != 0 and "positive" in fast.lib().ka_last_error().decode()
+
+
 @pytest.mark.parametrize("heads", EDGE_HEADS)
 def test_scores_that_climb_along_the_keys(heads):
     """Every key lines up with the queries a little better than the one before it, so that each
