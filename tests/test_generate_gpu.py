@@ -334,11 +334,13 @@ def test_pause_leaves_nothing_in_flight_and_resume_goes_on():
         assert len(engine.scheduler._inflight) == 0
         while not stream.empty():
             stream.get_nowait()
+        done_before = [f.done() for f in futures]          # (a slow host may let them end before the pause is asked for)
         futures.append(engine.submit_sync(late, **options))
         time.sleep(0.3)
-        assert stream.empty() and not any(f.done() for f in futures)
-        held = [g.pool.n_pages - g.pool.free_count for g in engine.runner.cache.groups]
-        assert all(n > 0 for n in held)
+        assert stream.empty() and [f.done() for f in futures[:2]] == done_before and not futures[2].done()
+        if not all(done_before):
+            held = [g.pool.n_pages - g.pool.free_count for g in engine.runner.cache.groups]
+            assert all(n > 0 for n in held)
         engine.resume()
         assert [f.result(timeout=120).tokens for f in futures] == undisturbed
         assert engine.pause(timeout=60)                           # an idle engine pauses too, and shuts down paused
