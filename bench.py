@@ -172,7 +172,7 @@ def time_decode(net, typed, batch, context, steps, warmup):
     return elapsed, 0.5 * (kv_start + kv_end)
 
 
-def time_prefill(net, typed, tokens, repeats=3):
+def time_prefill(net, typed, tokens, repeats=8):
     import torch
 
     from kestrel_amd.engine.loading import make_runner
