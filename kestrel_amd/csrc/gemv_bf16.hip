@@ -365,6 +365,7 @@ KA_API void ka_skinny_set_persistent(int enabled) { sk_persistent_enabled = enab
 // registers: 30 against 48 us for Moondream 2's output projection + fc2 at 64 rows; one segment
 // of 2048: 21 against 15 us), 2 wherever it can run (for tests), 0 nowhere.
 static int sk_wide_enabled = 1;
+KA_API int ka_linear_skinny_pair_in_parts(int M, int N);
 KA_API void ka_skinny_set_wide(int enabled) { sk_wide_enabled = enabled; }
 
 template <int PER, int MB, bool HALF, bool LN>
@@ -531,7 +532,7 @@ static int skinny_fused(const SkinnyExtras& extras, const void* A1, long lda1, i
     // With more than 8 rows of two segments the split kernel reads twice the weights' bytes in
     // activations (it multiplies 16 rows with strips of 8): 16.4 us here against 17.7 at 12 rows and
     // 18.3 at 16 (N = 2048, K = 2048 + 8192).
-    const bool crowded = A2 && ((strips > sk_compute_units() && M > 4) || M > 8);      // (a single row: 19 us against 24)
+    const bool crowded = A2 && M <= 16 && ka_linear_skinny_pair_in_parts(M, Na);      // (a single row: 19 us against 24)
     if (!Wb && partials && ((sk_wide_enabled && (M > 16 ? (A2 || !persistent_ok) : crowded)) || sk_wide_enabled >= 2)) {
         WideArgs wide = {};
         wide.A[0] = args.A[0]; wide.lda[0] = args.lda[0]; wide.W[0] = args.a.W; wide.ldw[0] = args.a.ldw; wide.K[0] = K1;
@@ -617,6 +618,14 @@ KA_API int ka_linear_skinny_fused(const void* A1, long lda1, int K1, const void*
 // the last linears of one block and the first norm of the next. Where K is cut into parts (more than
 // 8 rows) the kernel that adds the parts up normalises the rows it has just finished; else the
 // norm is a launch of its own behind the linear's.
+// Whether `out += A1 W1^T + A2 W2^T` of M rows and N outputs goes through the kernel that cuts K into
+// parts (a second kernel then finishes the rows, and can normalise them as well at no launch of its own).
+KA_API int ka_linear_skinny_pair_in_parts(int M, int N) {
+    if (!sk_wide_enabled || M < 1 || M > 64) return 0;
+    const int strips = ka_cdiv(N, SK_STRIP);
+    return M > 16 || (strips > sk_compute_units() && M > 4) || M > 8;
+}
+
 KA_API int ka_linear_skinny_pair_norm(const void* A1, long lda1, int K1, const void* A2, long lda2, int K2,
                                       const void* W1, long ldw1, const float* bias1, const void* W2, long ldw2,
                                       const float* bias2, float* out, long ldo, int N, int accumulate, int M,

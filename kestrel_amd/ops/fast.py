@@ -31,6 +31,7 @@ _SIGNATURES = {
         _c_void_p, _c_long, _c_void_p, _c_void_p, _c_long, _c_void_p,            # W1, ldw1, bias1, W2, ldw2, bias2
         _c_void_p, _c_long, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_long,  # out, ldo, N, accumulate, M, target_waves, partial sums
         _c_void_p, _c_void_p, _c_float, _c_void_p, _c_int, _c_long, _c_void_p],  # gamma, beta, eps, normed, its type and stride, stream
+    "ka_linear_skinny_pair_in_parts": [_c_int, _c_int],
     "ka_linear_library_bf16": [_c_void_p, _c_long, _c_void_p, _c_long, _c_void_p, _c_void_p, _c_int, _c_long, _c_int,
                                _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_long, _c_void_p],
     "ka_linear_tiled_bf16": [_c_void_p, _c_long, _c_void_p, _c_long, _c_void_p, _c_void_p, _c_int, _c_long, _c_int,
@@ -256,6 +257,12 @@ def linear_pair_accumulate(a1, w1, b1, a2, w2, b2, out, then_norm=None) -> bool:
         w1.data_ptr(), w1.stride(0), _ptr(b1), out.data_ptr(), KA_F32, out.stride(0), n, 0, 1,
         None, 0, None, None, 0, 0, 0, 0, m, SKINNY_TARGET_WAVES, *_wide_args(a1.device, m), stream_ptr()))
     return True
+
+
+def pair_finishes_rows(m: int, n: int) -> bool:
+    """Whether ``linear_pair_accumulate`` of ``m`` rows and ``n`` outputs ends in a kernel that finishes
+    whole rows (K cut into parts): that kernel normalises them as well at no launch of its own."""
+    return bool(lib().ka_linear_skinny_pair_in_parts(int(m), int(n)))
 
 
 def linear_two_outputs(a, wa, ba, out_a, act_a, wb, bb, out_b, act_b) -> bool:

@@ -55,9 +55,13 @@ def _parallel_few_rows(block: "Block", x, batch, cache, normed, then, handed) ->
             linear(h, f_in[0], f_in[1], hidden, act=f_in[3])
     mixed = block.mixer.attend(projected, batch, cache, beside) if beside is not None \
         else block.mixer.attend(projected, batch, cache)
-    # More rows than the next block's first launch normalises by itself: its norm is computed here,
-    # by the kernel that finishes this block's rows, instead of in a launch of its own.
-    if then is not None and n > fast.SKINNY_LN_MAX_ROWS and getattr(then.spec, "kind", None) == "layernorm":
+    # More rows than the next block's first launch normalises by itself, or a last launch of this block that
+    # ends in a kernel that finishes whole rows anyway: the next block's norm is computed here, by that
+    # kernel, instead of in a launch or a prologue of its own (9 to 16 rows of 2048: 1 to 2 % of a step;
+    # rows of 2560, which leave the prologue's kernel no registers for a third strip of weights in flight, from
+    # 5 rows on: 3 to 4 %).
+    handing = n > fast.SKINNY_LN_MAX_ROWS or fast.pair_finishes_rows(n, x.shape[1])
+    if then is not None and handing and getattr(then.spec, "kind", None) == "layernorm":
         rows = ws.get("block.handed", tuple(x.shape), block.dtype)
         if fast.linear_pair_accumulate(mixed, m_out[0], m_out[1], hidden, f_out[0], f_out[1], x,
                                        then_norm=(then.weight, then.bias, then.spec.eps, rows)):
