@@ -559,8 +559,7 @@ static int skinny_fused(const SkinnyExtras& extras, const void* A1, long lda1, i
             KA_LAUNCH_CHECK();
             if (then) {
                 // the finishing kernel takes whole rows and normalises them as well
-                hipLaunchKernelGGL(ka_partials_finish_norm_kernel, dim3(M), dim3(KA_ROW_THREADS), 0, stream, partials, splits, biasa,
-                                   A2 ? bias2 : nullptr, (float*)outa, ldoa, M, Na, accumulate_a, *then);
+                ka_launch_finish_norm(M, Na, stream, partials, splits, biasa, A2 ? bias2 : nullptr, (float*)outa, ldoa, accumulate_a, *then);
             } else {
                 const int quads = M * ka_cdiv(Na, 4);
                 hipLaunchKernelGGL(ka_partials_finish_kernel, dim3(ka_cdiv(quads, 256)), dim3(256), 0, stream, partials, splits,
@@ -573,8 +572,7 @@ static int skinny_fused(const SkinnyExtras& extras, const void* A1, long lda1, i
     // (where K was not cut into parts, a norm that follows is a launch of its own: the same kernel, no parts)
     auto norm_after = [&]() {
         if (then)
-            hipLaunchKernelGGL(ka_partials_finish_norm_kernel, dim3(M), dim3(KA_ROW_THREADS), 0, stream, (const float*)nullptr, 0,
-                               (const float*)nullptr, (const float*)nullptr, (float*)outa, ldoa, M, Na, 0, *then);
+            ka_launch_finish_norm(M, Na, stream, nullptr, 0, nullptr, nullptr, (float*)outa, ldoa, 0, *then);
     };
     if (persistent_ok) {
         if (launch_persistent(strips, M, kblocks, false, 0, stream, args)) return -1;
