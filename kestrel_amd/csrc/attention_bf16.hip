@@ -4,17 +4,19 @@
 // page), page size 16. Every token t of the packed batch reads the keys [kv_lo[t], kv_hi[t]) of
 // its row through the row's block table; the step's own keys are already in the cache.
 //
-// Prompt kernel. A workgroup owns 32 consecutive queries of one row and one head; its four waves
-// take every fourth tile of 32 keys (two pages) each and merge at the end, which gives the
-// chip eight waves per SIMD to hide the latency of the cache reads behind; the next tile's keys
-// and the current tile's values are in flight while the current scores are computed. Scores are computed transposed, S^T = K Q^T, with
-// v_mfma_f32_32x32x16_bf16: the keys are the row operand (a lane loads half a key row straight
-// from the cache), the queries the column operand (held in registers for the whole loop). A
-// lane then holds, for ONE query, 16 scores: softmax needs only in-lane work and one exchange
-// with the lane 32 apart. The key rows are fed to the MFMA in a permuted order (bits 2 and 3 of
-// the row index swapped) so that the 8 probabilities a lane holds for a page are those of 8
-// consecutive keys: they are, as they stand, the column operand of O^T += V^T P^T, whose row
-// operand is one 16-byte load from the transposed value page. LDS is used for the merge only.
+// Prompt kernel. A workgroup owns one or two blocks of 32 consecutive queries of one row and one
+// head; its four waves take every fourth tile of 32 keys (two pages) each and merge at the end; the
+// next tile's keys and the current tile's values are in flight while the current scores are
+// computed. Scores are computed transposed, S^T = K Q^T, with v_mfma_f32_32x32x16_bf16: the keys are
+// the row operand (a lane loads half a key row straight from the cache), the queries the column
+// operand (held in registers for the whole loop). A lane then holds, for ONE query, 16 scores:
+// softmax needs only in-lane work and one exchange with the lane 32 apart, and most tiles take
+// their exponentials from the reference point the query already has (the sum of a tile's
+// exponentials tells when that point has to move). The key rows are fed to the MFMA in a permuted
+// order (bits 2 and 3 of the row index swapped) so that the 8 probabilities a lane holds for a
+// page are those of 8 consecutive keys: they are, as they stand, the column operand of
+// O^T += V^T P^T, whose row operand is one 16-byte load from the transposed value page. LDS holds
+// the row's block table and is used for the merge.
 //
 // Decode kernel. One query per row: a bandwidth problem. The keys of a row are cut into splits
 // (grid z) and 64-key tiles (waves); 16-byte loads are fully coalesced for keys (8 lanes per key
