@@ -448,7 +448,9 @@ attn_decode_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t
 // ----------------------------------------------------------------------------------------------
 // rotary encoding + cache write, a page's worth of tokens per workgroup
 // ----------------------------------------------------------------------------------------------
-// A group of workgroups (grid y) takes 16 consecutive tokens of the packed batch. Queries are
+// A group of workgroups (grid y) takes a run of up to 16 consecutive tokens of the packed batch: the
+// runs the host lists (`run_first`, `run_count`: the tokens that fill a page of their row in order
+// are a run of their own, whatever their place in the batch), else every 16 tokens. Queries are
 // rotated in place and keys rotated into the cache with 16-byte loads and stores (8 channels of a
 // head and their 8 partners in the other half of the rotated part per thread; the channels of a
 // key that are not rotated are copied, those of a query left alone). Values: the cache keeps a
@@ -467,9 +469,11 @@ __global__ void __launch_bounds__(RC_THREADS)
 rope_cache_pages_kernel(bf16_t* __restrict__ qkv, long row_stride, const int* __restrict__ positions,
                         const int* __restrict__ slots, const float* __restrict__ table,
                         bf16_t* __restrict__ k_cache, bf16_t* __restrict__ v_cache, int n, int H, int Hkv,
-                        int hd, int rot, int light_parts) {
-    const int t0 = blockIdx.x * RC_TOKENS;
-    const int n_here = min(RC_TOKENS, n - t0);
+                        int hd, int rot, int light_parts, const int* __restrict__ run_first,
+                        const int* __restrict__ run_count) {
+    const int t0 = run_first ? run_first[blockIdx.x] : blockIdx.x * RC_TOKENS;
+    const int n_here = run_first ? min(run_count[blockIdx.x], min(RC_TOKENS, n - t0)) : min(RC_TOKENS, n - t0);
+    if (t0 < 0 || n_here <= 0) return;
     const int half = rot / 2;
     const int pair_units = half / 8;                  // per head: 8 channels + their 8 partners
     const int plain_units = (hd - rot) / 8;           // per head: 8 channels that are not rotated
@@ -573,11 +577,17 @@ rope_cache_pages_kernel(bf16_t* __restrict__ qkv, long row_stride, const int* __
             }
         }
     } else {
-        for (int idx = lane_id; idx < n_here * vwidth; idx += lanes) {
-            const int i = idx / vwidth, c = idx % vwidth;
+        // tokens of different rows, or of a page's middle: eight channels of a token per thread, one load
+        // of 16 bytes and eight stores of one value into the token's column of its page
+        const int chunks = vwidth / 8;
+        for (int idx = lane_id; idx < n_here * chunks; idx += lanes) {
+            const int i = idx / chunks, c0 = idx % chunks * 8;
             const int slot = slots[t0 + i];
             if (slot < 0) continue;
-            v_cache[(size_t)(slot / AT_PAGE) * page_elems + (size_t)c * AT_PAGE + slot % AT_PAGE] = vsrc[(size_t)i * row_stride + c];
+            const bf16x8 piece = at_load8(vsrc + (size_t)i * row_stride + c0);
+            bf16_t* col = v_cache + (size_t)(slot / AT_PAGE) * page_elems + (size_t)c0 * AT_PAGE + slot % AT_PAGE;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) col[j * AT_PAGE] = piece[j];
         }
     }
 }
@@ -591,15 +601,18 @@ KA_API int ka_rope_cache_pages_supported(int hd, int rot, int page_size) {
 
 KA_API int ka_rope_cache_pages_bf16(void* qkv, long row_stride, const int* positions, const int* slots,
                                     const float* table, int table_rows, void* k_cache, void* v_cache, int n, int H,
-                                    int Hkv, int hd, int rot, int page_size, hipStream_t stream) {
+                                    int Hkv, int hd, int rot, int page_size, const int* run_first,
+                                    const int* run_count, int n_runs, hipStream_t stream) {
     const char* who = "ka_rope_cache_pages_bf16";
     KA_CHECK(n >= 0 && H > 0 && Hkv > 0, "%s: bad sizes", who);
     KA_CHECK(ka_rope_cache_pages_supported(hd, rot, page_size), "%s: head size %d, rotary size %d, page size %d not covered", who, hd, rot, page_size);
     KA_CHECK(row_stride >= (long)(H + 2 * Hkv) * hd && row_stride % 8 == 0 && (uintptr_t)qkv % 16 == 0, "%s: rows must be 16-byte aligned and hold q, k and v", who);
     KA_CHECK(table && table_rows > 0 && (uintptr_t)table % 16 == 0, "%s: rotary table missing or not 16-byte aligned", who);
     KA_CHECK(!slots || (k_cache && v_cache && (uintptr_t)k_cache % 16 == 0 && (uintptr_t)v_cache % 16 == 0), "%s: cache tensors missing or not 16-byte aligned", who);
-    if (n == 0) return 0;
-    const int groups = ka_cdiv(n, RC_TOKENS);
+    KA_CHECK((run_first == nullptr) == (run_count == nullptr) && n_runs >= 0, "%s: the runs of tokens come as two lists", who);
+    if (n == 0 || (run_first && n_runs == 0)) return 0;
+    // (runs: every token in exactly one, none longer than 16: the host's promise)
+    const int groups = run_first ? n_runs : ka_cdiv(n, RC_TOKENS);
     // workgroups per group of tokens: a piece of work per thread for queries and keys, as many for
     // the values as have a piece each, and no more than fill the chip a few times over
     const int pair_units = rot / 16, plain_units = (hd - rot) / 8;
@@ -610,7 +623,7 @@ KA_API int ka_rope_cache_pages_bf16(void* qkv, long row_stride, const int* posit
     if (value_parts > most / 4) value_parts = most / 4;
     hipLaunchKernelGGL(rope_cache_pages_kernel, dim3(groups, light_parts + value_parts), dim3(RC_THREADS), 0, stream,
                        (bf16_t*)qkv, row_stride, positions, slots, table, (bf16_t*)k_cache, (bf16_t*)v_cache, n, H, Hkv, hd,
-                       rot, light_parts);
+                       rot, light_parts, run_first, run_count);
     KA_LAUNCH_CHECK();
     return 0;
 }

@@ -75,6 +75,9 @@ class StepBatch:
     # per size of block that a mixer's kernel asked for: (int32 [blocks] row of each block of that
     # many queries of one row, int32 [blocks] its first token), the blocks that see the most keys first
     query_blocks: Dict[int, Tuple[torch.Tensor, torch.Tensor]] = field(default_factory=dict)
+    # (int32 [runs] first token, int32 [runs] count): the tokens cut into runs that fill one page of their row in
+    # order, and runs of up to a page's worth of other tokens (for the kernels that write the cache by pages)
+    page_runs: Optional[Tuple[torch.Tensor, torch.Tensor]] = None
     pending: Optional[torch.Tensor] = None        # int32 device table: an id <= -2 stands for pending[-2 - id]
     given_embeds: Optional[torch.Tensor] = None   # [m, dim]
     given_rows: Optional[torch.Tensor] = None     # int32 [m] token indices they go to

@@ -120,6 +120,56 @@ class _GraphState:
         self.logits: Optional[torch.Tensor] = None
 
 
+class _PageRuns:
+    """The packed tokens of a step cut into runs for the kernels that write the cache: a run is
+    either the tokens that fill one page of their row in order (``page_size`` of them, the first at a
+    page's start), or up to ``page_size`` neighbouring tokens of any kind (a prompt's first or last few,
+    single decoded tokens of different rows)."""
+
+    def __init__(self, page_size: int) -> None:
+        self.ps = page_size
+        self._first: List[int] = []
+        self._count: List[int] = []
+        self._loose_first = 0
+        self._loose = 0
+
+    def _close(self) -> None:
+        if self._loose:
+            self._first.append(self._loose_first)
+            self._count.append(self._loose)
+            self._loose = 0
+
+    def _add_loose(self, at: int, n: int) -> None:
+        if self._loose and (self._loose_first + self._loose != at or self._loose + n > self.ps):
+            self._close()
+        if not self._loose:
+            self._loose_first = at
+        self._loose += n
+
+    def add(self, base: int, start: int, q: int) -> None:
+        """``q`` tokens of one row at positions ``start...``, the first of them token ``base`` of the step."""
+        ps = self.ps
+        lead = min(q, (-start) % ps)               # up to the next page's start
+        if lead:
+            self._add_loose(base, lead)
+        pages = (q - lead) // ps
+        if pages:
+            self._close()
+            self._first.extend(range(base + lead, base + lead + pages * ps, ps))
+            self._count.extend([ps] * pages)
+        tail = q - lead - pages * ps
+        if tail:
+            self._add_loose(base + lead + pages * ps, tail)
+
+    def first(self) -> List[int]:
+        self._close()
+        return self._first
+
+    def count(self) -> List[int]:
+        self._close()
+        return self._count
+
+
 class ModelRunner:
     """Owns the model, its cache and the scratch memory; ``step`` is the only way in."""
 
@@ -263,9 +313,11 @@ class ModelRunner:
         max_pages = max(1, fixed_pages)
         max_q = max_kv = 1
         causal_only = True
+        runs = _PageRuns(ps)
         for r, (e, start) in enumerate(zip(entries, starts)):
             q = len(e.tokens)
             base = len(ids)
+            runs.add(base, start, q)
             if e.bidirectional:
                 causal_only = False
             if q <= self.SCALAR_ROW:
@@ -332,6 +384,7 @@ class ModelRunner:
                     kv_lo[g].extend(cache.window_start(g, p) for p in range(start, start + q))
         n_real = len(entries)
         for r in range(n_real, pad_rows):          # rows that only fill the bucket
+            runs.add(len(ids), 0, 1)
             ids.append(0)
             positions.append(0)
             token_row.append(r)
@@ -356,7 +409,7 @@ class ModelRunner:
         sections: List[Tuple[str, object]] = [
             ("ids", ids), ("positions", positions), ("token_row", token_row), ("kv_hi", kv_hi),
             ("row_slot", row_slot), ("cu_q", cu_q), ("kv_len", kv_len), ("logit_rows", logit_rows),
-            ("given_rows", given_rows),
+            ("given_rows", given_rows), ("run_first", runs.first()), ("run_count", runs.count()),
         ]
         for tile, listed in blocks.items():
             sections.append((f"qblk_row{tile}", [b[0] for b in listed]))
@@ -416,7 +469,7 @@ class ModelRunner:
             workspace=workspace or self.workspace,
             query_blocks={tile: (view(f"qblk_row{tile}"), view(f"qblk_tok{tile}")) for tile in blocks},
             pending=self.pending, given_embeds=given_embeds, given_rows=view("given_rows") if given else None, max_q=max_q, max_kv=max_kv,
-            decode_only=max_q == 1, causal_only=causal_only,
+            decode_only=max_q == 1, causal_only=causal_only, page_runs=(view("run_first"), view("run_count")),
             host={"starts": starts, "q_lens": [len(e.tokens) for e in entries], "kv_len": kv_len, "meta_ints": total},
         )
 

@@ -40,7 +40,7 @@ _SIGNATURES = {
                                   _c_int, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_long, _c_float,
                                   _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
     "ka_rope_cache_pages_bf16": [_c_void_p, _c_long, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p,
-                                 _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p],
+                                 _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p, _c_void_p, _c_int, _c_void_p],
     "ka_attention_decode_bf16": [_c_void_p, _c_long, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_void_p, _c_void_p,
                                  _c_void_p, _c_void_p, _c_long, _c_float, _c_int, _c_int, _c_int, _c_int, _c_int,
                                  _c_int, _c_int, _c_void_p, _c_long,
@@ -326,9 +326,12 @@ def layernorm_linear(x, gamma, beta, eps, wa, ba, out_a, act_a, wb=None, bb=None
     return True
 
 
-def rope_cache_bf16(qkv, positions, slots, table, k_cache, v_cache, n_heads, n_kv_heads, head_dim, page_size) -> bool:
+def rope_cache_bf16(qkv, positions, slots, table, k_cache, v_cache, n_heads, n_kv_heads, head_dim, page_size,
+                    runs=None) -> bool:
     """Rotary encoding of q (in place) and k, and the cache write of k and v, a page's worth of
-    tokens per workgroup (``ops.core.rope_cache`` says what the operands are). False: not covered
+    tokens per workgroup (``ops.core.rope_cache`` says what the operands are). ``runs``: (int32 first
+    token, int32 count) of the runs the tokens are cut into, every token in exactly one and none longer
+    than a page (``StepBatch.page_runs``); without them every 16 tokens are a run. False: not covered
     (another page size, a rotary size that is no multiple of 16, rows that are not 16-byte aligned)."""
     if table is None or qkv.dtype != torch.bfloat16 or qkv.stride(1) != 1 or qkv.stride(0) % 8 or qkv.data_ptr() % 16:
         return False
@@ -338,9 +341,11 @@ def rope_cache_bf16(qkv, positions, slots, table, k_cache, v_cache, n_heads, n_k
         return False
     if slots is not None and (k_cache.data_ptr() % 16 or v_cache.data_ptr() % 16):
         return False
+    first, count = runs if runs is not None else (None, None)
     _check(handle.ka_rope_cache_pages_bf16(qkv.data_ptr(), qkv.stride(0), positions.data_ptr(), _ptr(slots), table.data_ptr(),
                                            int(table.shape[0]), _ptr(k_cache), _ptr(v_cache), qkv.shape[0], n_heads,
-                                           n_kv_heads, head_dim, rot, page_size, stream_ptr()))
+                                           n_kv_heads, head_dim, rot, page_size, _ptr(first), _ptr(count),
+                                           int(first.numel()) if first is not None else 0, stream_ptr()))
     return True
 
 

@@ -134,7 +134,8 @@ class PagedAttention(Mixer):
         if qkv.dtype == torch.bfloat16 and halves:
             from ..ops import fast
             done = fast.rope_cache_bf16(qkv, batch.positions, slots, self._table, cache.k, cache.v, spec.n_heads,
-                                        spec.n_kv_heads, spec.head_dim, group.page_size)
+                                        spec.n_kv_heads, spec.head_dim, group.page_size,
+                                        runs=getattr(batch, "page_runs", None))
         if not done:
             core.rope_cache(qkv, batch.positions, slots, self._table, cache.k, cache.v, spec.n_heads, spec.n_kv_heads,
                             spec.head_dim, group.page_size, self._pairing)

@@ -382,6 +382,66 @@ def test_rope_and_cache_write_by_pages(heads):
                                     h, hkv, hd, ps)               # a rotary size that is no multiple of 16
 
 
+@pytest.mark.parametrize("heads", [(4, 4, 64, 32), (6, 2, 48, 16), (2, 2, 80, 32)])
+def test_rope_and_cache_write_by_listed_runs(heads):
+    """The same kernel with the runs of tokens that the step function lists: a second prompt whose
+    pages start at odd places of the packed batch (its whole pages are runs of their own and take the
+    fast way), the loose ends of both prompts and single tokens of other rows in runs of their own."""
+    from kestrel_amd.engine.step import _PageRuns
+    from kestrel_amd.ops import fast
+
+    h, hkv, hd, rot = heads
+    bf = torch.bfloat16
+    torch.manual_seed(15)
+    ps, pages = 16, 16
+    order = torch.randperm(pages).tolist()
+    runs = _PageRuns(ps)
+    slots, positions = [], []
+    at = 0
+    # a prompt of 37 tokens from position 0 (pages order[0..2]), one of 50 from position 16 (its first page
+    # is held already: pages order[4..7]), five single tokens of other rows
+    for first_page, start, q in ((0, 0, 37), (3, 16, 50)):
+        runs.add(at, start, q)
+        for p in range(start, start + q):
+            slots.append(order[first_page + p // ps] * ps + p % ps)
+            positions.append(p)
+        at += q
+    for i in range(5):
+        runs.add(at, 100 + i, 1)
+        slots.append(order[8 + i] * ps + (100 + i) % ps if i != 2 else -1)
+        positions.append(100 + i)
+        at += 1
+    n = at
+    first, count = runs.first(), runs.count()
+    assert sum(count) == n and max(count) <= ps and count.count(ps) == 2 + 3        # whole pages: 2 of the first prompt, 3 of the second
+    assert 37 in first and 53 in first                   # (whole pages that start at odd places of the batch)
+    qkv = torch.randn(n, (h + 2 * hkv) * hd).to(bf)
+    table = plain.rotary_table(rot, 256, 777.0, torch.float32)
+    k_cache = torch.zeros(pages, hkv, ps, hd, dtype=bf, device=DEV)
+    v_cache = torch.zeros(pages, hkv, hd, ps, dtype=bf, device=DEV)
+    dev = qkv.to(DEV)
+    i32 = lambda xs: torch.tensor(xs, dtype=torch.int32, device=DEV)
+    assert fast.rope_cache_bf16(dev, i32(positions), i32(slots), table.to(DEV), k_cache, v_cache, h, hkv, hd, ps,
+                                runs=(i32(first), i32(count)))
+    t64 = plain.rotary_table(rot, 256, 777.0)
+    pos_t = torch.tensor(positions, dtype=torch.int32)
+    q = plain.apply_rotary(qkv[:, :h * hd].double().view(n, h, hd), pos_t, t64)
+    k = plain.apply_rotary(qkv[:, h * hd:(h + hkv) * hd].double().view(n, hkv, hd), pos_t, t64)
+    v = qkv[:, (h + hkv) * hd:].view(n, hkv, hd)
+    _close(dev[:, :h * hd].view(n, h, hd), q, bf)
+    for t in range(n):
+        if slots[t] < 0:
+            continue
+        page, off = slots[t] // ps, slots[t] % ps
+        _close(k_cache[page, :, off, :], k[t], bf)
+        assert torch.equal(v_cache[page, :, :, off].cpu(), v[t])
+    written = {s for s in slots if s >= 0}
+    for slot in range(pages * ps):
+        if slot not in written:
+            assert float(k_cache[slot // ps, :, slot % ps, :].abs().max()) == 0.0
+            assert float(v_cache[slot // ps, :, :, slot % ps].abs().max()) == 0.0
+
+
 class PagedCase:
     """Rows of cached keys and values scattered over shuffled pages, and packed query tokens."""
 
