@@ -78,6 +78,16 @@ class DecoderModel:
         """Sizes of blocks of queries that the mixers' kernels want listed with a step."""
         return {tile for tile in (block.mixer.query_tile() for block in self.blocks) if tile}
 
+    def _head_with_norm(self, x, batch, logits) -> bool:
+        """A few decoded rows, every one of them wanted, in order: the head's launch normalises them itself
+        (one launch less a step)."""
+        if self.dtype != torch.bfloat16 or not batch.decode_only or logits.shape[0] != batch.n_tokens \
+                or getattr(self.final_norm.spec, "kind", None) != "layernorm":
+            return False
+        from ..ops import fast
+        norm = self.final_norm
+        return fast.layernorm_linear(x, norm.weight, norm.bias, norm.spec.eps, self.head_weight, self.head_bias, logits, 0)
+
     # ------------------------------------------------------------------ forward
     def forward(self, batch, caches: List[LayerCache]) -> torch.Tensor:
         """Run the packed tokens of ``batch``; returns fp32 logits ``[wanted, vocab]``."""
@@ -95,9 +105,10 @@ class DecoderModel:
         wanted = int(batch.logit_rows.numel())
         logits = ws.get("model.logits", (wanted, plan.vocab_size), torch.float32)
         if wanted:
-            normed = ws.get("model.head_in", (wanted, plan.dim), self.dtype)
-            self.final_norm.forward(x, normed, rows=batch.logit_rows)
-            linear(normed, self.head_weight, self.head_bias, logits)
+            if not self._head_with_norm(x, batch, logits):
+                normed = ws.get("model.head_in", (wanted, plan.dim), self.dtype)
+                self.final_norm.forward(x, normed, rows=batch.logit_rows)
+                linear(normed, self.head_weight, self.head_bias, logits)
             if plan.logit_scale != 1.0 or plan.logit_softcap is not None:
                 core.adjust_logits(logits, plan.logit_scale, plan.logit_softcap)
         return logits
