@@ -116,13 +116,10 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_
             max_lo = max(max_lo, lo[b]);
         }
     }
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) {
-        wave_hi = max(wave_hi, __shfl_xor(wave_hi, off, KA_WAVE));
-        wave_lo = min(wave_lo, __shfl_xor(wave_lo, off, KA_WAVE));
-        min_hi = min(min_hi, __shfl_xor(min_hi, off, KA_WAVE));
-        max_lo = max(max_lo, __shfl_xor(max_lo, off, KA_WAVE));
-    }
+    wave_hi = ka_lanes_reduce<1, KA_WAVE>(wave_hi, KaIntMax{});
+    wave_lo = ka_lanes_reduce<1, KA_WAVE>(wave_lo, KaIntMin{});
+    min_hi = ka_lanes_reduce<1, KA_WAVE>(min_hi, KaIntMin{});
+    max_lo = ka_lanes_reduce<1, KA_WAVE>(max_lo, KaIntMax{});
     const int limit = kv_len[row];       // keys of this row that hold data
     // (the same in every lane: told to the compiler, which then counts tiles and looks up whole
     // pages in scalar registers)

@@ -176,9 +176,7 @@ gemv_f32_kernel(const float* __restrict__ A, long lda, const float* __restrict__
 #pragma unroll
     for (int m = 0; m < GV_ROWS; ++m) {
         if (m >= M) break;
-        float v = acc[m];
-#pragma unroll
-        for (int off = KA_WAVE / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, KA_WAVE);
+        float v = ka_wave_sum(acc[m]);
         if (lane == 0) {
             v += bias ? bias[n] : 0.f;
             if (act) v = ka_activate(act, v);

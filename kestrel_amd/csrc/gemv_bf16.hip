@@ -337,12 +337,10 @@ skinny_wide_kernel(WideArgs p) {
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
         floatx4 v = g < 2 ? lo[mb] : hi[mb];
-        floatx4 o;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) o[i] = __shfl_xor(v[i], 32, KA_WAVE);
+        for (int i = 0; i < 4; ++i) v[i] = ka_lanes_reduce<32, KA_WAVE>(v[i], KaSum{});
         const int m = mb * 16 + r, n = n0 + g * 4;
         if (g < 2 && m < M) {
-            v += o;
             float* dst = mine + (size_t)m * N + n;
             if (n + 3 < N && (N % 4) == 0) *reinterpret_cast<floatx4*>(dst) = v;
             else

@@ -202,8 +202,7 @@ attn_decode_body(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t* 
         float dot = 0.f;
 #pragma unroll
         for (int j = 0; j < 8; ++j) dot = fmaf(qf[j], kn[j], dot);
-#pragma unroll
-        for (int off = 1; off < LPK; off <<= 1) dot += __shfl_xor(dot, off, KA_WAVE);
+        dot = ka_lanes_reduce<1, LPK>(dot, KaSum{});
         m_i = dot;                // the only key so far: its weight is 1
         l_i = 1.f;
 #pragma unroll
@@ -239,13 +238,11 @@ attn_decode_body(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t* 
             float dot = 0.f;
 #pragma unroll
             for (int j = 0; j < 8; ++j) dot = fmaf(qf[j], (float)kreg[i][j], dot);
-#pragma unroll
-            for (int off = 1; off < LPK; off <<= 1) dot += __shfl_xor(dot, off, KA_WAVE);
+            dot = ka_lanes_reduce<1, LPK>(dot, KaSum{});           // the LPK lanes of a key
             sc[i] = ok ? dot : -INFINITY;
             mx = fmaxf(mx, sc[i]);
         }
-#pragma unroll
-        for (int off = LPK; off < KA_WAVE; off <<= 1) mx = fmaxf(mx, __shfl_xor(mx, off, KA_WAVE));
+        mx = ka_lanes_reduce<LPK, KA_WAVE>(mx, KaMax{});            // (the lanes of a key hold one value)
         float m_new = fmaxf(m_i, mx);
         if (m_new == -INFINITY) {              // a tile wholly below lo (wave-uniform)
             if constexpr (AHEAD) {
@@ -277,8 +274,7 @@ attn_decode_body(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t* 
             rowsum += p;
             if (dg_lane == 0) ps[wave][i * KPI + ks] = p;
         }
-#pragma unroll
-        for (int off = LPK; off < KA_WAVE; off <<= 1) rowsum += __shfl_xor(rowsum, off, KA_WAVE);
+        rowsum = ka_lanes_reduce<LPK, KA_WAVE>(rowsum, KaSum{});
         l_i = l_i * alpha + rowsum;
         m_i = m_new;
 #pragma unroll
@@ -311,7 +307,7 @@ attn_decode_body(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t* 
     }
     // the two halves of a channel row
 #pragma unroll
-    for (int u = 0; u < VU; ++u) acc[u] += __shfl_xor(acc[u], 1, KA_WAVE);
+    for (int u = 0; u < VU; ++u) acc[u] = ka_lanes_reduce<1, 2>(acc[u], KaSum{});
     if (lane == 0) { merge[wave][0] = m_i; merge[wave][1] = l_i; }
     if ((lane & 1) == 0) {
 #pragma unroll

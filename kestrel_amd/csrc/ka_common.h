@@ -50,17 +50,84 @@ __device__ __forceinline__ float ka_from_float<float>(float v) { return v; }
 template <>
 __device__ __forceinline__ bf16_t ka_from_float<bf16_t>(float v) { return (bf16_t)v; }
 
-__device__ __forceinline__ float ka_wave_sum(float v) {
-#pragma unroll
-    for (int off = KA_WAVE / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, KA_WAVE);
+// Reductions over groups of neighbouring lanes inside the vector unit: lane moves that ride on the
+// arithmetic instruction (DPP) up to a row of 16 lanes and the row and half-wave swaps of gfx950
+// above that, where a shuffle (ds_bpermute) makes a trip through the LDS pipe for every step.
+//
+// ka_lanes_reduce<FROM, TO>(v, op): every lane gets op over its aligned group of TO lanes, given
+// that the lanes of each aligned group of FROM lanes already hold one value (FROM = 1: any values).
+// The steps of 4 and 8 lanes mirror a half row and a row, which pairs a lane with one of the other
+// group, not with lane ^ 4 or lane ^ 8: that is the same only because of that condition. `op` must
+// be commutative; every lane of a group ends with the same bits. All 64 lanes must be active.
+struct KaSum { __device__ __forceinline__ float operator()(float a, float b) const { return a + b; } };
+struct KaMax { __device__ __forceinline__ float operator()(float a, float b) const { return fmaxf(a, b); } };
+struct KaIntMax { __device__ __forceinline__ int operator()(int a, int b) const { return a > b ? a : b; } };
+struct KaIntMin { __device__ __forceinline__ int operator()(int a, int b) const { return a < b ? a : b; } };
+
+// `v` of the lane that the DPP control names, in the rows of 16 lanes that ROWS has a bit for; 0 in the
+// other rows and, if ZERO_OUTSIDE, in a lane whose source lies outside its row.
+template <int CTRL, typename T, int ROWS = 0xF, bool ZERO_OUTSIDE = true>
+__device__ __forceinline__ T ka_dpp_move(T v) {
+    static_assert(sizeof(T) == 4, "lane moves carry 32 bits");
+    return __builtin_bit_cast(T, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, ROWS, 0xF, ZERO_OUTSIDE));
+}
+
+// One step of such a reduction: `a` and `b` are the values of the two groups of STEP lanes that
+// meet in this lane (which of them is this lane's own differs from lane to lane).
+template <int STEP, typename T>
+__device__ __forceinline__ void ka_lanes_pair(T v, T& a, T& b) {
+    static_assert(sizeof(T) == 4 && STEP >= 1 && STEP < KA_WAVE && (STEP & (STEP - 1)) == 0, "a power of two within a wave");
+    typedef __attribute__((ext_vector_type(2))) unsigned ka_u2;
+    if constexpr (STEP <= 8) {
+        a = v;
+        if constexpr (STEP == 1) b = ka_dpp_move<0xB1>(v);            // quad_perm [1,0,3,2]
+        else if constexpr (STEP == 2) b = ka_dpp_move<0x4E>(v);       // quad_perm [2,3,0,1]
+        else if constexpr (STEP == 4) b = ka_dpp_move<0x141>(v);      // row_half_mirror
+        else b = ka_dpp_move<0x140>(v);                               // row_mirror
+    } else {
+        const unsigned bits = __builtin_bit_cast(unsigned, v);
+        ka_u2 s;
+        // 16: rows 1 and 3 of the first register change places with rows 0 and 2 of the second;
+        // 32: the upper half of the first with the lower half of the second
+        if constexpr (STEP == 16) s = __builtin_amdgcn_permlane16_swap(bits, bits, false, false);
+        else s = __builtin_amdgcn_permlane32_swap(bits, bits, false, false);
+        a = __builtin_bit_cast(T, (unsigned)s[0]);
+        b = __builtin_bit_cast(T, (unsigned)s[1]);
+    }
+}
+
+template <int FROM, int TO, typename T, typename Op>
+__device__ __forceinline__ T ka_lanes_reduce(T v, Op op) {
+    static_assert(TO <= KA_WAVE && (TO & (TO - 1)) == 0, "groups are powers of two within a wave");
+    if constexpr (FROM >= TO) {
+        return v;
+    } else {
+        T a, b;
+        ka_lanes_pair<FROM>(v, a, b);
+        return ka_lanes_reduce<FROM * 2, TO>(op(a, b), op);
+    }
+}
+
+// Running sums along the lanes of a wave (lane i gets the sum of lanes 0..i), by the same means:
+// four shifts inside each row of 16 (a lane that has no neighbour so far down gets 0), then the
+// last lane of a row handed to the rows after it. All 64 lanes must be active.
+__device__ __forceinline__ float ka_wave_running_sum(float v) {
+    v += ka_dpp_move<0x111>(v);                          // row_shr:1
+    v += ka_dpp_move<0x112>(v);                          // row_shr:2
+    v += ka_dpp_move<0x114>(v);                          // row_shr:4
+    v += ka_dpp_move<0x118>(v);                          // row_shr:8
+    v += ka_dpp_move<0x142, float, 0xA, false>(v);       // row_bcast:15, into rows 1 and 3
+    v += ka_dpp_move<0x143, float, 0xC, false>(v);       // row_bcast:31, into rows 2 and 3
     return v;
 }
 
-__device__ __forceinline__ float ka_wave_max(float v) {
-#pragma unroll
-    for (int off = KA_WAVE / 2; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, KA_WAVE));
-    return v;
+// The value of one lane (a number known at compile time or the same in every lane) in all lanes.
+__device__ __forceinline__ float ka_lane_value(float v, int lane) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
 }
+
+__device__ __forceinline__ float ka_wave_sum(float v) { return ka_lanes_reduce<1, KA_WAVE>(v, KaSum{}); }
+__device__ __forceinline__ float ka_wave_max(float v) { return ka_lanes_reduce<1, KA_WAVE>(v, KaMax{}); }
 
 // GELU with the tanh approximation: 0.5 x (1 + tanh(sqrt(2/pi) (x + 0.044715 x^3))).
 __device__ __forceinline__ float ka_gelu_tanh(float x) {

@@ -12,6 +12,7 @@
 constexpr int SM_THREADS = 1024;
 constexpr int SM_WAVES = SM_THREADS / KA_WAVE;
 constexpr float SM_GREEDY_EPS = 1e-6f;
+constexpr int SM_PICKED = 4 * SM_THREADS;       // probabilities that the search for the nucleus gathers once so few are left
 
 __device__ __forceinline__ float block_reduce_sum(float v, float* smem) {
     v = ka_wave_sum(v);
@@ -33,6 +34,21 @@ __device__ __forceinline__ float block_reduce_max(float v, float* smem) {
 #pragma unroll
     for (int w = 0; w < SM_WAVES; ++w) t = fmaxf(t, smem[w]);
     return t;
+}
+
+// The greatest value of the wave and the lowest index that has it, in every lane.
+template <int STEP = 1>
+__device__ __forceinline__ void wave_argmax(float& best, int& best_i) {
+    if constexpr (STEP < KA_WAVE) {
+        float va, vb;
+        int ia, ib;
+        ka_lanes_pair<STEP>(best, va, vb);
+        ka_lanes_pair<STEP>(best_i, ia, ib);
+        const bool second = vb > va || (vb == va && ib < ia);
+        best = second ? vb : va;
+        best_i = second ? ib : ia;
+        wave_argmax<STEP * 2>(best, best_i);
+    }
 }
 
 // splitmix64 of (key + counter * odd constant): uniform in [0, 1) with 24 bits.
@@ -79,12 +95,7 @@ __device__ int block_argmax(const float* __restrict__ row, int V, float* smem_f,
             if (i < V && (v[u] > best || (v[u] == best && i < best_i))) { best = v[u]; best_i = i; }
         }
     }
-#pragma unroll
-    for (int off = KA_WAVE / 2; off > 0; off >>= 1) {
-        float ov = __shfl_xor(best, off, KA_WAVE);
-        int oi = __shfl_xor(best_i, off, KA_WAVE);
-        if (ov > best || (ov == best && oi < best_i)) { best = ov; best_i = oi; }
-    }
+    wave_argmax(best, best_i);
     __syncthreads();
     if (threadIdx.x % KA_WAVE == 0) { smem_f[threadIdx.x / KA_WAVE] = best; smem_i[threadIdx.x / KA_WAVE] = best_i; }
     __syncthreads();
@@ -117,12 +128,7 @@ argmax_regs_kernel(const float* __restrict__ logits, long ld, int* __restrict__ 
         const int i = j * SM_THREADS + tid;
         if (i < V && x[j] > best) { best = x[j]; best_i = i; }      // j rises with i: the first of equals stays
     }
-#pragma unroll
-    for (int off = KA_WAVE / 2; off > 0; off >>= 1) {
-        float ov = __shfl_xor(best, off, KA_WAVE);
-        int oi = __shfl_xor(best_i, off, KA_WAVE);
-        if (ov > best || (ov == best && oi < best_i)) { best = ov; best_i = oi; }
-    }
+    wave_argmax(best, best_i);
     if (tid % KA_WAVE == 0) { sf[tid / KA_WAVE] = best; si[tid / KA_WAVE] = best_i; }
     __syncthreads();
     if (tid != 0) return;
@@ -205,12 +211,7 @@ sample_kernel(const float* __restrict__ logits, long ld, const float* __restrict
             if (p < thresh || p <= 0.f) p = 0.f;
         }
         // inclusive scan inside the wave
-        float scan = p;
-#pragma unroll
-        for (int off = 1; off < KA_WAVE; off <<= 1) {
-            float o = __shfl_up(scan, off, KA_WAVE);
-            if (lane >= off) scan += o;
-        }
+        const float scan = ka_wave_running_sum(p);
         __syncthreads();
         if (lane == KA_WAVE - 1) wave_tot[wave] = scan;
         __syncthreads();
@@ -231,7 +232,8 @@ sample_kernel(const float* __restrict__ logits, long ld, const float* __restrict
 // The same selection for rows of at most R * 1024 logits, each read once: a thread keeps its R
 // logits (then probabilities) in registers. The threshold of the nucleus is bisected between 0
 // and the largest probability and the search ends as soon as no probability lies between its
-// bounds (the set {p >= threshold} is then settled); the draw is located by wave sums of the
+// bounds (the set {p >= threshold} is then settled); a round looks only at the registers that
+// still hold a probability between the bounds. The draw is located by wave sums of the
 // groups of 64 neighbouring tokens, one scan of those, and one scan inside the group found.
 // sample_kernel above passes over the row about 35 times (300 us at a vocabulary of 51200: a
 // quarter of a decode step); this one takes about a tenth of that.
@@ -244,6 +246,8 @@ sample_regs_kernel(const float* __restrict__ logits, long ld, const float* __res
     __shared__ float sf[SM_WAVES];
     __shared__ int si[SM_WAVES];
     __shared__ float group_sum[R * SM_WAVES];       // of tokens (j * 1024 + wave * 64) .. + 64, in that order
+    __shared__ float round_sums[2][3][SM_WAVES];
+    __shared__ float picked_list[SM_PICKED];
     __shared__ int found_group;
     __shared__ float found_before;
     const int r = blockIdx.x, tid = threadIdx.x;
@@ -266,12 +270,7 @@ sample_regs_kernel(const float* __restrict__ logits, long ld, const float* __res
         const int i = j * SM_THREADS + tid;
         if (i < V && x[j] > best) { best = x[j]; best_i = i; }      // j rises with i: the first of equals stays
     }
-#pragma unroll
-    for (int off = KA_WAVE / 2; off > 0; off >>= 1) {
-        float ov = __shfl_xor(best, off, KA_WAVE);
-        int oi = __shfl_xor(best_i, off, KA_WAVE);
-        if (ov > best || (ov == best && oi < best_i)) { best = ov; best_i = oi; }
-    }
+    wave_argmax(best, best_i);
     if (lane == 0) { sf[wave] = best; si[wave] = best_i; }
     __syncthreads();
     best = sf[0]; best_i = si[0];
@@ -298,44 +297,91 @@ sample_regs_kernel(const float* __restrict__ logits, long ld, const float* __res
     const float top_p = top_ps ? top_ps[r] : 1.0f;
     float thresh = 0.f, mass = 1.0f;
     if (top_p < 1.0f) {
-        // f(t) = mass of {p >= t} falls with t; keep the largest t with f(t) >= top_p
-        float lo = 0.f, hi = inv_z * (1.0f + 1e-6f) + 1e-30f;      // just above the largest probability
-        for (int it = 0; it < 32; ++it) {
-            const float mid = 0.5f * (lo + hi);
-            // the mass at and above mid and, every fourth round (it costs more than the mass),
-            // how many probabilities lie in [lo, hi)
-            const bool count = it % 4 == 3;
-            float f = 0.f, between = 2.f;
-            if (count) {
-                between = 0.f;
+        // f(t) = mass of {p >= t} falls with t; keep the largest t with f(t) >= top_p. The lower
+        // bound starts at the smallest normal number: what lies below it holds less than 1e-33
+        // together and is never needed to reach top_p (at most 1 - 6e-8).
+        float lo = 1.17549435e-38f, hi = inv_z * (1.0f + 1e-6f) + 1e-30f;      // hi: just above the largest probability
+        float above = 0.f;                                                     // f(hi): the mass at and above hi
+        // Once at most SM_PICKED probabilities are left between the bounds they are gathered, a few
+        // per thread, and the rounds after that look at those alone (a round over all R registers
+        // costs 2.4 us at R = 52, one over the few 0.4 us).
+        bool picked = false;
+        float c[SM_PICKED / SM_THREADS];
+#pragma unroll
+        for (int k = 0; k < SM_PICKED / SM_THREADS; ++k) c[k] = 0.f;
+        for (int it = 0; it < 40; ++it) {
+            // The first threshold tried is 1 / SM_PICKED: no more than SM_PICKED probabilities can be
+            // that large, so if they reach top_p (a model that is sure of itself) the gathering
+            // follows at once. After that, the middle of the bounds.
+            const float first = 1.0f / (float)SM_PICKED;
+            const float mid = it == 0 && first < hi ? first : 0.5f * (lo + hi);
+            // the mass at and above mid (of the gathered ones: below hi), the number of probabilities
+            // in [lo, hi) and of those in [mid, hi)
+            float f = 0.f;
+            int n_in = 0, n_up = 0;
+            if (!picked) {
 #pragma unroll
                 for (int j = 0; j < R; ++j) {
-                    f += x[j] >= mid ? x[j] : 0.f;
-                    between += (x[j] >= lo && x[j] < hi && x[j] > 0.f) ? 1.f : 0.f;
+                    const bool up = x[j] >= mid, in = x[j] >= lo && x[j] < hi;
+                    f += up ? x[j] : 0.f;
+                    n_in += in ? 1 : 0;
+                    n_up += in && up ? 1 : 0;
                 }
             } else {
 #pragma unroll
-                for (int j = 0; j < R; ++j) f += x[j] >= mid ? x[j] : 0.f;
+                for (int k = 0; k < SM_PICKED / SM_THREADS; ++k) {
+                    const bool in = c[k] >= lo && c[k] < hi, up = in && c[k] >= mid;
+                    f += up ? c[k] : 0.f;
+                    n_in += in ? 1 : 0;
+                    n_up += up ? 1 : 0;
+                }
             }
-            // both sums at once: two values per wave through LDS, in one of two sets of places by
-            // turns, so that one barrier a round is enough (a wave that is a round ahead writes
-            // the other set)
+            // three sums over the workgroup: a value per wave through LDS, in one of two sets of
+            // places by turns, so that one barrier a round is enough (a wave that is a round ahead
+            // writes the other set); each row of 16 lanes then adds up the 16 waves' values, all
+            // in one order, so every lane decides alike
+            static_assert(SM_WAVES == 16, "the waves' sums meet in a row of 16 lanes");
             f = ka_wave_sum(f);
-            between = ka_wave_sum(between);
-            float* places = group_sum + (it & 1) * 2 * SM_WAVES;
-            if (lane == 0) { places[wave] = f; places[SM_WAVES + wave] = between; }
+            const float wave_in = ka_wave_sum((float)n_in), wave_up = ka_wave_sum((float)n_up);
+            float* places = &round_sums[it & 1][0][0];
+            if (lane == 0) { places[wave] = f; places[SM_WAVES + wave] = wave_in; places[2 * SM_WAVES + wave] = wave_up; }
             __syncthreads();
-            f = 0.f; between = 0.f;
-#pragma unroll
-            for (int w = 0; w < SM_WAVES; ++w) { f += places[w]; between += places[SM_WAVES + w]; }   // (a round that did not count: 2 a wave)
-            const bool exhausted = !(mid > lo && mid < hi);          // no float left between the bounds
-            if (f >= top_p) lo = mid; else hi = mid;
+            const float mass_up = ka_lanes_reduce<1, SM_WAVES>(places[lane % SM_WAVES], KaSum{});
+            const float all_in = ka_lanes_reduce<1, SM_WAVES>(places[SM_WAVES + lane % SM_WAVES], KaSum{});
+            const float all_up = ka_lanes_reduce<1, SM_WAVES>(places[2 * SM_WAVES + lane % SM_WAVES], KaSum{});
+            const float at_mid = picked ? above + mass_up : mass_up;           // f(mid)
+            const bool exhausted = !(mid > lo && mid < hi);                   // no float left between the bounds
+            const bool rises = at_mid >= top_p;
+            float between;                                                    // probabilities between the new bounds
+            if (rises) { lo = mid; between = all_up; }
+            else { hi = mid; above = at_mid; between = all_in - all_up; }
             // f(lo) >= top_p > f(hi) throughout. With at most one probability in [lo, hi) the
             // tokens above hi do not reach top_p, so that one is needed: {p >= lo} is the nucleus,
-            // the same set for the old and the new bounds. (Tracking the least and the greatest
-            // probability between the bounds instead, which also ends the search on equal
-            // probabilities, costs more per round than it saves: 172 against 115 us per step.)
+            // the same set for the old and the new bounds.
             if (between <= 1.f || exhausted) break;
+            if (!picked && between <= (float)SM_PICKED) {
+                // every wave knows how many each wave brings (the sums above, per wave): its own
+                // start in the list follows from those before it, and a lane's place from the
+                // lanes before it
+                int at = 0;
+                for (int w = 0; w < wave; ++w)
+                    at += (int)(rises ? places[2 * SM_WAVES + w] : places[SM_WAVES + w] - places[2 * SM_WAVES + w]);
+#pragma unroll
+                for (int j = 0; j < R; ++j) {
+                    const bool in = x[j] >= lo && x[j] < hi;
+                    const unsigned long long holds = __ballot(in);
+                    if (holds) {
+                        const int before = __builtin_amdgcn_mbcnt_hi((unsigned)(holds >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)holds, 0u));
+                        if (in) picked_list[min(at + before, SM_PICKED - 1)] = x[j];
+                        at += __popcll(holds);
+                    }
+                }
+                __syncthreads();
+                const int n = (int)between;
+#pragma unroll
+                for (int k = 0; k < SM_PICKED / SM_THREADS; ++k) c[k] = k * SM_THREADS + tid < n ? picked_list[k * SM_THREADS + tid] : 0.f;
+                picked = true;
+            }
         }
         thresh = lo;
         float f = 0.f;
@@ -363,12 +409,7 @@ sample_regs_kernel(const float* __restrict__ logits, long ld, const float* __res
         for (int base = 0; base < R * SM_WAVES; base += KA_WAVE) {
             const int gi = base + lane;
             const float v = gi < R * SM_WAVES ? group_sum[gi] : 0.f;
-            float scan = v;
-#pragma unroll
-            for (int off = 1; off < KA_WAVE; off <<= 1) {
-                float o = __shfl_up(scan, off, KA_WAVE);
-                if (lane >= off) scan += o;
-            }
+            const float scan = ka_wave_running_sum(v);
             // sums only grow along the lanes: the first one past the target is the group (its own
             // sum is then positive: the one before was not past it)
             const float incl = running + scan;
@@ -378,7 +419,7 @@ sample_regs_kernel(const float* __restrict__ logits, long ld, const float* __res
                 if (lane == first) { found_group = gi; found_before = incl - v; }
                 break;
             }
-            running += __shfl(scan, KA_WAVE - 1, KA_WAVE);
+            running += ka_lane_value(scan, KA_WAVE - 1);
         }
     }
     __syncthreads();
@@ -391,12 +432,7 @@ sample_regs_kernel(const float* __restrict__ logits, long ld, const float* __res
 #pragma unroll
             for (int jj = 0; jj < R; ++jj)
                 if (jj == j) p = x[jj];
-            float scan = p;
-#pragma unroll
-            for (int off = 1; off < KA_WAVE; off <<= 1) {
-                float o = __shfl_up(scan, off, KA_WAVE);
-                if (lane >= off) scan += o;
-            }
+            const float scan = ka_wave_running_sum(p);
             const float incl = found_before + scan;
             const unsigned long long past = __ballot(p > 0.f && incl > target);
             const unsigned long long any = __ballot(p > 0.f);

@@ -708,11 +708,11 @@ def test_argmax_and_sampling():
 
 
 @pytest.mark.parametrize("passes_only", [False, True])
-@pytest.mark.parametrize("vocab", [51200, 1003, 40000, 70000])
+@pytest.mark.parametrize("vocab", [51200, 1003, 40000, 60000, 70000])
 def test_every_draw_is_the_inversion_of_the_nucleus(vocab, passes_only):
     """The token drawn is the first, in index order, whose cumulative mass in the plain
-    implementation's nucleus distribution exceeds the request's uniform number: for peaked and
-    flat rows, masked tokens, equal logits; by the kernel that keeps a row in registers and by
+    implementation's nucleus distribution exceeds the request's uniform number: for peaked, very
+    peaked and flat rows, masked tokens, equal logits; by the kernel that keeps a row in registers and by
     the one that passes over it (which alone takes rows of more than 65536)."""
     from kestrel_amd.ops import core
     from kestrel_amd.sampling import Sampler, mix_key
@@ -725,6 +725,7 @@ def test_every_draw_is_the_inversion_of_the_nucleus(vocab, passes_only):
     logits[12, 100:200] = float("-inf")                # masked tokens
     logits[13, :] = 0.5                                # all equal
     logits[14, 7] = logits[14, 900] = 9.0              # two equal leaders
+    logits[16:20] *= 25.0                              # a token or two hold the whole nucleus
     temps = [0.7] * 8 + [1.0] * 8 + [1.3] * 8
     tops = ([0.9, 0.5, 0.99, 0.3] * 6)
     tops[13] = 1.0                                     # (equal probabilities at the nucleus's edge are all kept by the
