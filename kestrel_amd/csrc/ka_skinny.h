@@ -20,6 +20,17 @@ constexpr int SK_PAD = 8;          // bf16 of padding per LDS row (keeps 16-byte
 constexpr int SP_WAVES = 8;        // waves of a persistent workgroup
 constexpr int SP_MAX_PER = 8;      // most k-blocks per wave it keeps activations for
 
+// Orders the LDS traffic of one wave: what its lanes wrote before is seen by its lanes after.
+__device__ __forceinline__ void sk_wave_sync() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// bf16 of LDS in which a wave of the persistent kernel turns one k-block of MB * 16 rows around
+// (rows padded so that the lanes of a 16-byte read stay off each other's banks).
+__host__ __device__ constexpr int sk_stage_elements(int MB) { return MB * 16 * (SK_KBLOCK + SK_PAD); }
+
 // Every operand lives in global memory. Saying so at the load matters: a pointer that went
 // through sk_pinned() below is "generic" to the compiler, and generic (flat) loads count as LDS
 // traffic too, which forces a wait for everything in flight at each use.
@@ -308,6 +319,39 @@ __device__ __forceinline__ void skinny_persistent_body(const SkinnyArgs& p, cons
                 const bf16_t* xp = xs + min(r, M - 1) * ld + k + g * 8;
                 x[u][0][0] = r < M && k + g * 8 < K ? *reinterpret_cast<const bf16x8*>(xp) : zero;
                 x[u][0][1] = r < M && k + 32 + g * 8 < K ? *reinterpret_cast<const bf16x8*>(xp + 32) : zero;
+            }
+        }
+    } else if constexpr (MB >= 2) {
+        // More than 16 rows: an instruction that loaded a k-block for the multiplications directly
+        // would touch half a cache line of each of 16 rows, 4 KB apart, and every line twice
+        // (10 us for 64 rows of 2048, most of this kernel's time before its first strip). Here an
+        // instruction takes whole lines of 8 rows, and the wave turns what it has loaded into the
+        // multiplications' order through a piece of LDS of its own, k-block by k-block.
+        constexpr int LDR = SK_KBLOCK + SK_PAD;
+        bf16_t* stage = reinterpret_cast<bf16_t*>(sk_dyn) + (size_t)wave * sk_stage_elements(MB);
+        const int srow = lane / 8, schunk = lane % 8;
+#pragma unroll
+        for (int u = 0; u < PER; ++u) {
+            const int k = (wave + u * SP_WAVES) * SK_KBLOCK;
+#pragma unroll
+            for (int j = 0; j < 2 * MB; ++j)
+                x[u][j / 2][j % 2] = sk_load8(p.A[0] + (size_t)min(j * 8 + srow, M - 1) * p.lda[0] + min(k + schunk * 8, K - 8));
+        }
+#pragma unroll
+        for (int u = 0; u < PER; ++u) {
+            const int k = (wave + u * SP_WAVES) * SK_KBLOCK;
+            sk_wave_sync();                    // the k-block before has been read
+#pragma unroll
+            for (int j = 0; j < 2 * MB; ++j)
+                *reinterpret_cast<bf16x8*>(stage + (j * 8 + srow) * LDR + schunk * 8) = x[u][j / 2][j % 2];
+            sk_wave_sync();
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb) {
+                const int m = mb * 16 + r;
+                const bf16x8 va = *reinterpret_cast<const bf16x8*>(stage + m * LDR + g * 8);
+                const bf16x8 vb = *reinterpret_cast<const bf16x8*>(stage + m * LDR + 32 + g * 8);
+                x[u][mb][0] = m < M && k + g * 8 < K ? va : zero;
+                x[u][mb][1] = m < M && k + 32 + g * 8 < K ? vb : zero;
             }
         }
     } else {

@@ -169,7 +169,7 @@ def test_every_activation_in_every_linear_kernel(name, code):
 @pytest.mark.parametrize("persistent,wide", [(1, 0), (0, 0), (1, 2)])
 @pytest.mark.parametrize("shape", [(1, 48, 64), (8, 2048, 2048), (5, 100, 200), (16, 6144, 2048), (33, 77, 8192),
                                    (64, 51200, 512), (17, 2048, 8192), (3, 16, 8), (9, 20000, 1032), (40, 4100, 2048),
-                                   (8, 1000, 4096), (12, 515, 3000), (64, 9000, 1024)])
+                                   (8, 1000, 4096), (12, 515, 3000), (64, 9000, 1024), (50, 333, 1000), (20, 1000, 200)])
 def test_linear_skinny_bf16(shape, persistent, wide):
     """The weight-streaming MFMA kernels: the persistent one (activations in registers, workgroups
     walk over strips; a form of its own for at most 8 rows), the one with K-splits that takes
