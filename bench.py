@@ -131,7 +131,7 @@ class DecodeBench:
         torch = self.torch
         entries = [self.StepEntry(slot, [self.PENDING], want=[0]) for slot in self.slots]
         logits = self.runner.step(entries)
-        ids = self.sampler.greedy(logits, slots=self.slots)
+        ids = self.sampler.greedy(logits, slots=self.runner.logit_slots)
         host = self.host[self.n_steps % 2]
         host.copy_(ids, non_blocking=True)
         event = torch.cuda.Event()

@@ -145,7 +145,7 @@ def _profile_decode(args) -> int:
 
     def run_decode():
         logits = runner.step([StepEntry(slot, [PENDING_TOKEN], want=[0]) for slot in slots])
-        sampler.greedy(logits, slots=slots)
+        sampler.greedy(logits, slots=runner.logit_slots)
 
     print(f"Running {args.warmup} warmup decode iterations...")
     for _ in range(args.warmup):

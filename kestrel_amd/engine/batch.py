@@ -70,6 +70,7 @@ class StepBatch:
     cu_q: torch.Tensor                  # int32 [rows + 1]
     kv_len: torch.Tensor                # int32 [rows]: keys held after this step
     logit_rows: torch.Tensor            # int32 [wanted]
+    logit_slot: torch.Tensor            # int32 [wanted]: the slot of the request a row of logits belongs to (-1: a padding row)
     groups: Dict[int, GroupBatch]
     workspace: Workspace
     # per size of block that a mixer's kernel asked for: (int32 [blocks] row of each block of that

@@ -291,7 +291,12 @@ class GenerationScheduler:
             if any(r.return_logprobs for r in requests):
                 extras["logprobs"] = True
             if self.pipeline_depth > 1:
-                extras["slots"] = [row.seq.slot for row in sampled_rows]
+                # the step function has left every logits row's slot on the device
+                on_device = getattr(self.runner, "logit_slots", None)
+                if on_device is not None and on_device.numel() == len(sampled_rows) == logits.shape[0]:
+                    extras["slots"] = on_device
+                else:
+                    extras["slots"] = [row.seq.slot for row in sampled_rows]
             if extras.keys() - {"slots"}:
                 ids, logprobs = self.sampler.sample_step(logits, temps, tops, seeds, indices, **extras)
             else:

@@ -193,6 +193,7 @@ class ModelRunner:
         self._graphs: Dict[int, _GraphState] = {}
         self._pages_cap = -(-model.plan.max_positions // cache.page_size)
         self.graph_replays = 0
+        self.logit_slots: Optional[torch.Tensor] = None     # of the last step: the slot per row of logits, on the device
         # the latest sampled token of every request slot, written by the sampling kernels
         self.pending = torch.zeros(max(1, cache.max_requests), dtype=torch.int32, device=device)
         # Sizes of the blocks of queries that the mixers' kernels want a row cut into (a mixer says
@@ -303,6 +304,7 @@ class ModelRunner:
         # blocks of queries, per size: row, first token, most keys any of them sees
         blocks: Dict[int, List[Tuple[int, int, int]]] = {tile: [] for tile in self.query_tiles}
         logit_rows: List[int] = []
+        logit_slot: List[int] = []            # the request's slot, per row of logits
         given_rows: List[int] = []
         given: List[torch.Tensor] = []
         row_slot: List[int] = []
@@ -366,6 +368,7 @@ class ModelRunner:
                     for first in range(0, q, tile):
                         listed.append((r, base + first, max(hi[first:first + tile])))
             logit_rows.extend(base + int(w) for w in e.want)
+            logit_slot.extend(e.slot for _ in e.want)
             cu_q.append(base + q)
             kv_len.append(start + q)
             row_slot.append(e.slot)
@@ -392,6 +395,7 @@ class ModelRunner:
             for listed in blocks.values():
                 listed.append((r, len(ids) - 1, 0))
             logit_rows.append(len(ids) - 1)
+            logit_slot.append(-1)
             cu_q.append(len(ids))
             kv_len.append(0)
             row_slot.append(-1)                    # no request: a mixer with state must pass these rows over
@@ -409,6 +413,7 @@ class ModelRunner:
         sections: List[Tuple[str, object]] = [
             ("ids", ids), ("positions", positions), ("token_row", token_row), ("kv_hi", kv_hi),
             ("row_slot", row_slot), ("cu_q", cu_q), ("kv_len", kv_len), ("logit_rows", logit_rows),
+            ("logit_slot", logit_slot),
             ("given_rows", given_rows), ("run_first", runs.first()), ("run_count", runs.count()),
         ]
         for tile, listed in blocks.items():
@@ -465,7 +470,7 @@ class ModelRunner:
         return StepBatch(
             n_tokens=n_tokens, n_rows=n_rows, token_ids=view("ids"), positions=view("positions"),
             token_row=view("token_row"), kv_hi=view("kv_hi"), row_slot=view("row_slot"), cu_q=view("cu_q"),
-            kv_len=view("kv_len"), logit_rows=view("logit_rows"), groups=groups,
+            kv_len=view("kv_len"), logit_rows=view("logit_rows"), logit_slot=view("logit_slot"), groups=groups,
             workspace=workspace or self.workspace,
             query_blocks={tile: (view(f"qblk_row{tile}"), view(f"qblk_tok{tile}")) for tile in blocks},
             pending=self.pending, given_embeds=given_embeds, given_rows=view("given_rows") if given else None, max_q=max_q, max_kv=max_kv,
@@ -512,10 +517,11 @@ class ModelRunner:
             with torch.cuda.graph(graph):
                 state.logits = self.model.forward(blank, self.layer_caches)
             state.graph = graph
-        self.build_batch(entries, pad_rows=bucket, fixed_pages=self._pages_cap, meta=state.meta,
-                         workspace=state.workspace)
+        batch = self.build_batch(entries, pad_rows=bucket, fixed_pages=self._pages_cap, meta=state.meta,
+                                 workspace=state.workspace)
         state.graph.replay()
         self.graph_replays += 1
+        self.logit_slots = batch.logit_slot[:len(entries)]
         return state.logits[:len(entries)]
 
     # ------------------------------------------------------------------ the step
@@ -523,7 +529,8 @@ class ModelRunner:
     def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
         """Run the entries as one batch. Returns fp32 logits ``[wanted, vocab]`` in the order of
         the entries and of their ``want``; the tensor is scratch memory and is overwritten by
-        the next step."""
+        the next step. ``logit_slots`` then holds, on the device, the slot of the request that each
+        row of logits belongs to (until the next step, like the logits)."""
         if not entries:
             raise ValueError("a step needs at least one entry")
         bucket = self._graph_bucket(entries)
@@ -533,6 +540,7 @@ class ModelRunner:
         else:
             batch = self.build_batch(entries)
             logits = self.model.forward(batch, self.layer_caches)
+            self.logit_slots = batch.logit_slot
             starts = batch.host["starts"]
         for e, start in zip(entries, starts):
             self.held[e.slot] = start + len(e.tokens)

@@ -86,12 +86,15 @@ class Sampler:
 
     def sample_step(self, logits: torch.Tensor, temperatures: Sequence[float], top_ps: Sequence[float],
                     request_seeds: Sequence[int], token_indices: Sequence[int],
-                    slots: Optional[Sequence[int]] = None,
+                    slots=None,
                     suppress: Sequence[Tuple[int, int]] = (),
                     allowed: Optional[Sequence[Optional[Sequence[int]]]] = None,
                     logprobs: bool = False) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
         """Masks, then one token id per row, then (if asked) the chosen tokens' log-probabilities.
 
+        ``slots``: per row the place in the table of latest tokens (``pending``) that also receives
+        the row's token: a list, or an int32 tensor that is on the device already (the step
+        function leaves one there: ``ModelRunner.logit_slots``).
         ``suppress``: pairs (row, token) whose logit becomes -inf. ``allowed``: per row ``None`` or
         the only tokens the row may choose. Both change ``logits`` in place. Returns int32 ids and
         fp32 log-probabilities (or ``None``), both on the device.
@@ -99,6 +102,9 @@ class Sampler:
         rows = logits.shape[0]
         if not (len(temperatures) == len(top_ps) == len(request_seeds) == len(token_indices) == rows):
             raise ValueError("sampling parameters must have one entry per row of logits")
+        slots_on_device = None
+        if isinstance(slots, torch.Tensor):
+            slots_on_device, slots = self._device_slots(slots, rows), None
         if slots is not None and (self.pending is None or len(slots) != rows):
             raise ValueError("slots need a pending table and one entry per row of logits")
         if allowed is not None and len(allowed) != rows:
@@ -138,11 +144,12 @@ class Sampler:
             core.suppress_tokens(logits, arg["suppress_rows"], arg["suppress_tokens"])
         if restrict:
             core.allow_tokens(logits, arg["allow_starts"], arg["allow_tokens"])
-        pending = self.pending if slots is not None else None
+        places = slots_on_device if slots_on_device is not None else arg.get("slots")
+        pending = self.pending if places is not None else None
         if greedy:
-            core.argmax(logits, out, pending, arg.get("slots"))
+            core.argmax(logits, out, pending, places)
         else:
-            core.sample(logits, arg["temps"], arg["tops"], arg["keys"], arg["counters"], out, pending, arg.get("slots"))
+            core.sample(logits, arg["temps"], arg["tops"], arg["keys"], arg["counters"], out, pending, places)
         chosen = None
         if logprobs:
             chosen = torch.empty(rows, dtype=torch.float32, device=self.device)
@@ -155,7 +162,16 @@ class Sampler:
             out = torch.empty(logits.shape[0], dtype=torch.int32, device=self.device)
         if slots is None:
             core.argmax(logits, out)
+        elif isinstance(slots, torch.Tensor):
+            core.argmax(logits, out, self.pending, self._device_slots(slots, logits.shape[0]))
         else:
             (pending_at,) = self._upload([np.asarray(slots, dtype=np.int32)])
             core.argmax(logits, out, self.pending, pending_at)
         return out
+
+    def _device_slots(self, slots: torch.Tensor, rows: int) -> torch.Tensor:
+        if slots.dtype != torch.int32 or slots.device != self.device or slots.numel() != rows or not slots.is_contiguous():
+            raise ValueError("slots on the device must be contiguous int32, one per row of logits")
+        if self.pending is None:
+            raise ValueError("slots need a pending table")
+        return slots

@@ -707,6 +707,41 @@ def test_argmax_and_sampling():
     assert 0.0 <= core.uniform(mix_key(5, 42), 7) < 1.0
 
 
+def test_sampler_takes_the_rows_slots_from_the_device():
+    """The table of latest tokens gets a row's token at the row's slot, whether the slots come as a
+    list or as the int32 tensor that the step function has left on the device; a negative slot
+    (a padding row) is passed over."""
+    from kestrel_amd.sampling import Sampler
+
+    torch.manual_seed(5)
+    logits = torch.randn(5, 777, device=DEV)
+    slots = [3, 0, -1, 6, 2]
+    want = logits.argmax(dim=1).tolist()
+    for sampled in (False, True):
+        tables = []
+        for on_device in (False, True):
+            pending = torch.full((8,), -7, dtype=torch.int32, device=DEV)
+            sampler = Sampler(torch.device(DEV), seed=3, pending=pending)
+            given = torch.tensor(slots, dtype=torch.int32, device=DEV) if on_device else slots
+            if sampled:
+                ids = sampler.sample(logits.clone(), [0.0, 0.8, 0.8, 0.0, 0.8], [1.0, 0.9, 0.9, 1.0, 0.5], [1, 2, 3, 4, 5],
+                                     [0, 1, 2, 3, 4], slots=given).tolist()
+                assert ids[0] == want[0] and ids[3] == want[3]
+            else:
+                ids = sampler.greedy(logits, slots=given).tolist()
+                assert ids == want
+            table = pending.tolist()
+            for row, slot in enumerate(slots):
+                if slot >= 0:
+                    assert table[slot] == ids[row]
+            assert [table[i] for i in (1, 4, 5, 7)] == [-7] * 4
+            tables.append((ids, table))
+        assert tables[0] == tables[1]
+    with pytest.raises(ValueError):
+        Sampler(torch.device(DEV), seed=3, pending=torch.zeros(8, dtype=torch.int32, device=DEV)).greedy(
+            logits, slots=torch.zeros(4, dtype=torch.int32, device=DEV))
+
+
 @pytest.mark.parametrize("passes_only", [False, True])
 @pytest.mark.parametrize("vocab", [51200, 1003, 40000, 60000, 70000])
 def test_every_draw_is_the_inversion_of_the_nucleus(vocab, passes_only):
