@@ -297,14 +297,22 @@ class GenerationScheduler:
                     extras["slots"] = on_device
                 else:
                     extras["slots"] = [row.seq.slot for row in sampled_rows]
-            if extras.keys() - {"slots"}:
+            if logits.is_cuda and "logprobs" not in extras:
+                # the sampling kernel writes the ids into pinned host memory itself: no copy behind it
+                # (the kernel of the log-probabilities reads them on the device)
+                extras["out"] = self._host_buffer(len(sampled_rows), torch.int32)
+            if extras.keys() - {"slots", "out"}:
                 ids, logprobs = self.sampler.sample_step(logits, temps, tops, seeds, indices, **extras)
             else:
                 ids = self.sampler.sample(logits, temps, tops, seeds, indices, **extras)
-            if ids.is_cuda:
-                ids, event = self._to_host(ids)
+            if logits.is_cuda:
+                if ids.is_cuda:                       # (a sampler that brought its own output)
+                    ids, event = self._to_host(ids)
                 if logprobs is not None:
                     logprobs, event = self._to_host(logprobs)
+                else:
+                    event = torch.cuda.Event()
+                    event.record()
         return ids, event, logprobs
 
     def _launch(self, plan: StepPlan) -> None:
@@ -345,15 +353,20 @@ class GenerationScheduler:
                 self._finish(row.seq, "error", now, f"{type(exc).__name__}: {exc}")
         self.failed_steps += 1
 
+    def _host_buffer(self, n: int, dtype) -> torch.Tensor:
+        """Pinned memory for a step's tokens or log-probabilities, from a ring with more buffers than
+        steps in flight."""
+        index = self._host_next
+        self._host_next = (index + 1) % self.HOST_RING
+        buf = self._host_ids[index]
+        if buf is None or buf.numel() < n:
+            buf = self._host_ids[index] = torch.empty(max(n, 256), dtype=torch.int32, pin_memory=True)
+        return buf[:n].view(dtype)                            # int32 or float32: four bytes either way
+
     def _to_host(self, values: torch.Tensor):
         """Start the copy of a step's tokens (or their log-probabilities) into pinned memory; the
         event tells when it is done."""
-        index = self._host_next
-        self._host_next = (index + 1) % self.HOST_RING       # more buffers than copies in flight
-        buf = self._host_ids[index]
-        if buf is None or buf.numel() < values.numel():
-            buf = self._host_ids[index] = torch.empty(max(values.numel(), 256), dtype=torch.int32, pin_memory=True)
-        host = buf[:values.numel()].view(values.dtype)        # int32 or float32: four bytes either way
+        host = self._host_buffer(values.numel(), values.dtype)
         host.copy_(values, non_blocking=True)
         event = torch.cuda.Event()
         event.record()

@@ -92,6 +92,12 @@ def _dev(*tensors) -> None:
             _need(t.is_cuda, "kernel operand is not on the GPU")
 
 
+def _dev_or_pinned(t: torch.Tensor) -> None:
+    """A small output may lie in pinned host memory, which the GPU writes directly: the host then
+    needs no copy behind the kernel, only its end."""
+    _need(t.is_cuda or t.is_pinned(), "kernel output is neither on the GPU nor in pinned host memory")
+
+
 def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
     return None if t is None else t.data_ptr()
 
@@ -282,9 +288,11 @@ def _pending_args(who: str, rows: int, pending, pending_at):
 
 def argmax(logits: torch.Tensor, out: torch.Tensor, pending: Optional[torch.Tensor] = None,
            pending_at: Optional[torch.Tensor] = None) -> None:
-    """Index of the largest logit of every fp32 row into int32 ``out``, and into
-    ``pending[pending_at[row]]`` if a table of latest tokens is given (negative place: skipped)."""
-    _dev(logits, out, pending, pending_at)
+    """Index of the largest logit of every fp32 row into int32 ``out`` (on the device or in pinned
+    host memory), and into ``pending[pending_at[row]]`` if a table of latest tokens is given
+    (negative place: skipped)."""
+    _dev(logits, pending, pending_at)
+    _dev_or_pinned(out)
     rows, vocab = logits.shape
     _need(logits.dtype == torch.float32 and logits.stride(1) == 1, "argmax: logits must be fp32 rows")
     _need(out.dtype == torch.int32 and out.numel() == rows and out.is_contiguous(), "argmax: out int32 [rows]")
@@ -297,7 +305,8 @@ def sample(logits: torch.Tensor, temps: torch.Tensor, top_ps: Optional[torch.Ten
            pending_at: Optional[torch.Tensor] = None) -> None:
     """Temperature and top-p sampling of every row (greedy where temperature <= 1e-6); the
     token also goes to ``pending[pending_at[row]]`` if given."""
-    _dev(logits, temps, top_ps, rng_key, rng_counter, out, pending, pending_at)
+    _dev(logits, temps, top_ps, rng_key, rng_counter, pending, pending_at)
+    _dev_or_pinned(out)
     rows, vocab = logits.shape
     _need(logits.dtype == torch.float32 and logits.stride(1) == 1, "sample: logits must be fp32 rows")
     _need(temps.dtype == torch.float32 and temps.numel() == rows, "sample: temps fp32 [rows]")

@@ -80,21 +80,24 @@ class Sampler:
 
     def sample(self, logits: torch.Tensor, temperatures: Sequence[float], top_ps: Sequence[float],
                request_seeds: Sequence[int], token_indices: Sequence[int],
-               slots: Optional[Sequence[int]] = None) -> torch.Tensor:
-        """One token id per row of fp32 ``logits``; int32 on the device."""
-        return self.sample_step(logits, temperatures, top_ps, request_seeds, token_indices, slots=slots)[0]
+               slots=None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """One token id per row of fp32 ``logits``; int32 on the device (or in ``out``)."""
+        return self.sample_step(logits, temperatures, top_ps, request_seeds, token_indices, slots=slots, out=out)[0]
 
     def sample_step(self, logits: torch.Tensor, temperatures: Sequence[float], top_ps: Sequence[float],
                     request_seeds: Sequence[int], token_indices: Sequence[int],
                     slots=None,
                     suppress: Sequence[Tuple[int, int]] = (),
                     allowed: Optional[Sequence[Optional[Sequence[int]]]] = None,
-                    logprobs: bool = False) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+                    logprobs: bool = False,
+                    out: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
         """Masks, then one token id per row, then (if asked) the chosen tokens' log-probabilities.
 
         ``slots``: per row the place in the table of latest tokens (``pending``) that also receives
         the row's token: a list, or an int32 tensor that is on the device already (the step
         function leaves one there: ``ModelRunner.logit_slots``).
+        ``out``: where the ids go, int32 ``[rows]``, on the device or in pinned host memory (the
+        kernel then writes them there itself and the host only waits for its end).
         ``suppress``: pairs (row, token) whose logit becomes -inf. ``allowed``: per row ``None`` or
         the only tokens the row may choose. Both change ``logits`` in place. Returns int32 ids and
         fp32 log-probabilities (or ``None``), both on the device.
@@ -109,7 +112,10 @@ class Sampler:
             raise ValueError("slots need a pending table and one entry per row of logits")
         if allowed is not None and len(allowed) != rows:
             raise ValueError("allowed needs one entry per row of logits")
-        out = torch.empty(rows, dtype=torch.int32, device=self.device)
+        if out is None:
+            out = torch.empty(rows, dtype=torch.int32, device=self.device)
+        elif out.dtype != torch.int32 or out.numel() != rows or not out.is_contiguous():
+            raise ValueError("out must be contiguous int32, one entry per row of logits")
         if rows == 0:
             return out, (torch.empty(0, dtype=torch.float32, device=self.device) if logprobs else None)
         greedy = all(t <= GREEDY_EPS for t in temperatures)

@@ -707,7 +707,7 @@ def test_argmax_and_sampling():
     assert 0.0 <= core.uniform(mix_key(5, 42), 7) < 1.0
 
 
-def test_sampler_takes_the_rows_slots_from_the_device():
+def test_sampler_takes_slots_from_the_device_and_writes_ids_to_pinned_memory():
     """The table of latest tokens gets a row's token at the row's slot, whether the slots come as a
     list or as the int32 tensor that the step function has left on the device; a negative slot
     (a padding row) is passed over."""
@@ -740,6 +740,20 @@ def test_sampler_takes_the_rows_slots_from_the_device():
     with pytest.raises(ValueError):
         Sampler(torch.device(DEV), seed=3, pending=torch.zeros(8, dtype=torch.int32, device=DEV)).greedy(
             logits, slots=torch.zeros(4, dtype=torch.int32, device=DEV))
+    # the ids may go straight into pinned host memory: the same ids, there once the stream has got so far
+    sampler = Sampler(torch.device(DEV), seed=3)
+    args = ([0.0, 0.8, 0.8, 0.0, 0.8], [1.0, 0.9, 0.9, 1.0, 0.5], [1, 2, 3, 4, 5], [0, 1, 2, 3, 4])
+    on_device = sampler.sample(logits.clone(), *args).tolist()
+    host = torch.full((5,), -1, dtype=torch.int32).pin_memory()
+    assert sampler.sample(logits.clone(), *args, out=host) is host
+    torch.cuda.synchronize()
+    assert host.tolist() == on_device
+    host.fill_(-1)
+    sampler.greedy(logits, out=host)
+    torch.cuda.synchronize()
+    assert host.tolist() == want
+    with pytest.raises(Exception):
+        sampler.greedy(logits, out=torch.empty(5, dtype=torch.int32))          # pageable host memory: refused
 
 
 @pytest.mark.parametrize("passes_only", [False, True])
