@@ -415,8 +415,8 @@ static int launch_persistent(int strips, int M, int kblocks, bool ln, size_t dyn
     }
     if (M <= 8) return launch_persistent_per<1, true, false>(per, grid, 0, strips, stream, args);
     switch (MB) {
-        case 1: return launch_persistent_per<1, false, false>(per, grid, 0, strips, stream, args);
         // (LDS in which every wave turns the activations it loads into the multiplications' order)
+        case 1: return launch_persistent_per<1, false, false>(per, grid, SP_WAVES * sk_stage_elements(1) * sizeof(bf16_t), strips, stream, args);
         case 2: return launch_persistent_per<2, false, false>(per, grid, SP_WAVES * sk_stage_elements(2) * sizeof(bf16_t), strips, stream, args);
         case 3: return launch_persistent_per<3, false, false>(per, grid, SP_WAVES * sk_stage_elements(3) * sizeof(bf16_t), strips, stream, args);
         default: return launch_persistent_per<4, false, false>(per, grid, SP_WAVES * sk_stage_elements(4) * sizeof(bf16_t), strips, stream, args);

@@ -321,8 +321,8 @@ __device__ __forceinline__ void skinny_persistent_body(const SkinnyArgs& p, cons
                 x[u][0][1] = r < M && k + 32 + g * 8 < K ? *reinterpret_cast<const bf16x8*>(xp + 32) : zero;
             }
         }
-    } else if constexpr (MB >= 2) {
-        // More than 16 rows: an instruction that loaded a k-block for the multiplications directly
+    } else if constexpr (!HALF) {
+        // More than 8 rows: an instruction that loaded a k-block for the multiplications directly
         // would touch half a cache line of each of 16 rows, 4 KB apart, and every line twice
         // (10 us for 64 rows of 2048, most of this kernel's time before its first strip). Here an
         // instruction takes whole lines of 8 rows, and the wave turns what it has loaded into the
