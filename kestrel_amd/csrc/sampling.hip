@@ -232,8 +232,9 @@ sample_kernel(const float* __restrict__ logits, long ld, const float* __restrict
 // The same selection for rows of at most R * 1024 logits, each read once: a thread keeps its R
 // logits (then probabilities) in registers. The threshold of the nucleus is bisected between 0
 // and the largest probability and the search ends as soon as no probability lies between its
-// bounds (the set {p >= threshold} is then settled); a round looks only at the registers that
-// still hold a probability between the bounds. The draw is located by wave sums of the
+// bounds (the set {p >= threshold} is then settled); once few probabilities are left between
+// the bounds they are gathered, a few per thread, and the rounds after that look at those alone.
+// The draw is located by wave sums of the
 // groups of 64 neighbouring tokens, one scan of those, and one scan inside the group found.
 // sample_kernel above passes over the row about 35 times (300 us at a vocabulary of 51200: a
 // quarter of a decode step); this one takes about a tenth of that.
