@@ -176,7 +176,9 @@ class Sampler:
         return out
 
     def _device_slots(self, slots: torch.Tensor, rows: int) -> torch.Tensor:
-        if slots.dtype != torch.int32 or slots.device != self.device or slots.numel() != rows or not slots.is_contiguous():
+        here = torch.device(self.device)
+        same = slots.device.type == here.type and (here.index is None or slots.device.index == here.index)
+        if slots.dtype != torch.int32 or not same or slots.numel() != rows or not slots.is_contiguous():
             raise ValueError("slots on the device must be contiguous int32, one per row of logits")
         if self.pending is None:
             raise ValueError("slots need a pending table")
