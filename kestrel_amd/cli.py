@@ -30,6 +30,10 @@ def _add_runtime_options(parser: argparse.ArgumentParser) -> None:
     parser.add_argument("--disable-graphs", action="store_true", help="do not replay decode steps as HIP graphs")
     parser.add_argument("--pipeline-depth", type=int, default=2, choices=(1, 2),
                         help="2: launch a step before the previous step's tokens have reached the host")
+    parser.add_argument("--no-warmup", action="store_true",
+                        help="do not capture the decode graphs and make scratch memory and plans at start")
+    parser.add_argument("--log-level", default="WARNING", choices=["DEBUG", "INFO", "WARNING", "ERROR"],
+                        help="what the engine's logger reports on stderr (INFO: load, pool size, warm-up)")
 
 
 def _parse_ids(text: str) -> List[int]:
@@ -37,11 +41,14 @@ def _parse_ids(text: str) -> List[int]:
 
 
 def _generate(args) -> int:
+    import logging
+
     import torch
 
     from .config import RuntimeConfig
     from .engine import InferenceEngine
 
+    logging.basicConfig(level=getattr(logging, args.log_level), format="%(asctime)s %(name)s %(levelname)s %(message)s")
     prompts: List[List[int]] = []
     for text in args.prompt_ids or []:
         prompts.append(_parse_ids(text))
@@ -53,7 +60,8 @@ def _generate(args) -> int:
                         max_batch_size=args.max_batch_size, page_size=args.page_size,
                         kv_cache_pages=args.kv_cache_pages, kv_cache_bytes=args.kv_cache_bytes,
                         max_num_batched_tokens=args.max_num_batched_tokens,
-                        seed=args.seed, enable_graphs=not args.disable_graphs, pipeline_depth=args.pipeline_depth)
+                        seed=args.seed, enable_graphs=not args.disable_graphs, pipeline_depth=args.pipeline_depth,
+                        warmup=not args.no_warmup)
     engine = InferenceEngine.create_sync(cfg)
     try:
         if args.random_prompts:

@@ -43,6 +43,9 @@ class RuntimeConfig:
     ``pipeline_depth``: 2 launches a step before the tokens of the one before have reached
     the host (``kestrel/scheduler/pipeline.py:49-65``); 1 reads every step first.
     ``seed``: base of the sampling generator.
+    ``warmup``: make everything at start that steps would otherwise make when they first need it (the
+    graph of every bucket of decode rows, scratch buffers, the plans of the prompt's linears), as
+    the reference does before ``create`` returns (``kestrel/engine/core.py:458-484``).
     """
 
     model_path: Union[str, Path, None] = None
@@ -59,6 +62,7 @@ class RuntimeConfig:
     model: Optional[str] = None
     seed: int = 0
     max_seq_len: Optional[int] = None
+    warmup: bool = True
 
     def __post_init__(self) -> None:
         self.dtype = parse_dtype(self.dtype)

@@ -10,9 +10,15 @@
 // Row-major out [M, N] is the library's column-major D [N, M] = W (stored as column-major [K, N],
 // transposed) x A (column-major [K, M]); the bias runs along D's rows.
 //
-// A plan (descriptors and the algorithm the library's heuristic names first) is made at the first
-// call with a set of sizes and kept. The caller brings the workspace; nothing here allocates
-// device memory.
+// Plans. Asking the library's heuristic for an algorithm is the expensive part of a first call
+// (hundreds of microseconds to milliseconds on the host), and under continuous batching the number
+// of rows changes with almost every step. So the heuristic is asked once per bucket of rows (M
+// rounded up to a multiple of 64, of 256 beyond 4,096 rows) at the bucket's upper edge, and that
+// algorithm serves every row count of the bucket: a plan keeps the descriptors, whose row count is
+// set per call, and the algorithm. Should the library refuse the bucket's algorithm for a row
+// count, the heuristic is asked for exactly that count and the answer kept under its own key.
+// The plans live in a map bounded at LT_MAX_PLANS; the one used longest ago makes room.
+// The caller brings the workspace; nothing here allocates device memory.
 #include "ka_common.h"
 
 #include <hipblaslt/hipblaslt.h>
@@ -25,19 +31,26 @@ namespace {
 
 constexpr int LT_MAX_DEVICES = 64;
 constexpr int LT_CANDIDATES = 8;
+constexpr size_t LT_MAX_PLANS = 512;
 
 struct Plan {
     hipblasLtMatmulDesc_t desc = nullptr;
     hipblasLtMatrixLayout_t w = nullptr, a = nullptr, out = nullptr;
     hipblasLtMatmulAlgo_t algo;
     bool usable = false;
+    bool every_count = true;       // false once the library has refused the algorithm for a row count of the bucket
+    int rows_set = 0;              // the row count the layouts of a and out stand at
+    unsigned long used = 0;        // the call that used the plan last
 };
 
+// device, rows (a bucket's upper edge, or minus an exact count), N, K, lda, ldw, ldo, output type, activation,
+// bias, accumulate, workspace
 using Key = std::tuple<int, int, int, int, long, long, long, int, int, int, int, size_t>;
 
 std::mutex g_lock;
 hipblasLtHandle_t g_handle[LT_MAX_DEVICES];
 std::map<Key, Plan> g_plans;
+unsigned long g_calls = 0, g_heuristic_calls = 0, g_evicted = 0;
 
 bool epilogue_of(int act, bool bias, hipblasLtEpilogue_t* epilogue) {
     switch (act) {
@@ -49,12 +62,36 @@ bool epilogue_of(int act, bool bias, hipblasLtEpilogue_t* epilogue) {
     return false;
 }
 
-// The plan for these sizes on this device; made (and the library asked for an algorithm) at the
-// first call. `usable` false: the library has no kernel for the case.
-const Plan* plan_for(hipblasLtHandle_t handle, const Key& key, int M, int N, int K, long lda, long ldw, long ldo,
-                     int out_dtype, int act, bool bias, bool accumulate, size_t workspace_bytes) {
-    auto found = g_plans.find(key);
-    if (found != g_plans.end()) return &found->second;
+int rows_bucket(int M) {
+    const int step = M > 4096 ? 256 : 64;
+    return (M + step - 1) / step * step;
+}
+
+void destroy(Plan& plan) {
+    if (plan.w) hipblasLtMatrixLayoutDestroy(plan.w);
+    if (plan.a) hipblasLtMatrixLayoutDestroy(plan.a);
+    if (plan.out) hipblasLtMatrixLayoutDestroy(plan.out);
+    if (plan.desc) hipblasLtMatmulDescDestroy(plan.desc);
+    plan = Plan{};
+}
+
+// Room for one more plan: the one used longest ago goes (a linear scan over at most LT_MAX_PLANS
+// entries, once per new plan beyond the bound).
+void make_room() {
+    while (g_plans.size() >= LT_MAX_PLANS) {
+        auto oldest = g_plans.begin();
+        for (auto it = g_plans.begin(); it != g_plans.end(); ++it)
+            if (it->second.used < oldest->second.used) oldest = it;
+        destroy(oldest->second);
+        g_plans.erase(oldest);
+        ++g_evicted;
+    }
+}
+
+// Descriptors for `rows` rows and the algorithm the library's heuristic names first for them.
+// `usable` false: the library has no kernel for the case.
+Plan make_plan(hipblasLtHandle_t handle, int rows, int N, int K, long lda, long ldw, long ldo, int out_dtype, int act,
+               bool bias, size_t workspace_bytes) {
     Plan plan;
     hipblasLtEpilogue_t epilogue;
     const hipDataType out_type = out_dtype == KA_F32 ? HIP_R_32F : HIP_R_16BF;
@@ -70,8 +107,9 @@ const Plan* plan_for(hipblasLtHandle_t handle, const Key& key, int M, int N, int
             ok = hipblasLtMatmulDescSetAttribute(plan.desc, HIPBLASLT_MATMUL_DESC_BIAS_DATA_TYPE, &bias_type, sizeof(bias_type)) == HIPBLAS_STATUS_SUCCESS;
     }
     ok = ok && hipblasLtMatrixLayoutCreate(&plan.w, HIP_R_16BF, K, N, ldw) == HIPBLAS_STATUS_SUCCESS &&
-         hipblasLtMatrixLayoutCreate(&plan.a, HIP_R_16BF, K, M, lda) == HIPBLAS_STATUS_SUCCESS &&
-         hipblasLtMatrixLayoutCreate(&plan.out, out_type, N, M, ldo) == HIPBLAS_STATUS_SUCCESS;
+         hipblasLtMatrixLayoutCreate(&plan.a, HIP_R_16BF, K, rows, lda) == HIPBLAS_STATUS_SUCCESS &&
+         hipblasLtMatrixLayoutCreate(&plan.out, out_type, N, rows, ldo) == HIPBLAS_STATUS_SUCCESS;
+    plan.rows_set = rows;
     if (ok) {
         hipblasLtMatmulPreference_t preference = nullptr;
         ok = hipblasLtMatmulPreferenceCreate(&preference) == HIPBLAS_STATUS_SUCCESS;
@@ -79,6 +117,7 @@ const Plan* plan_for(hipblasLtHandle_t handle, const Key& key, int M, int N, int
             const uint64_t cap = workspace_bytes;
             hipblasLtMatmulHeuristicResult_t candidates[LT_CANDIDATES];
             int n = 0;
+            ++g_heuristic_calls;
             ok = hipblasLtMatmulPreferenceSetAttribute(preference, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &cap, sizeof(cap)) == HIPBLAS_STATUS_SUCCESS &&
                  hipblasLtMatmulAlgoGetHeuristic(handle, plan.desc, plan.w, plan.a, plan.out, plan.out, preference,
                                                  LT_CANDIDATES, candidates, &n) == HIPBLAS_STATUS_SUCCESS;
@@ -92,8 +131,29 @@ const Plan* plan_for(hipblasLtHandle_t handle, const Key& key, int M, int N, int
             hipblasLtMatmulPreferenceDestroy(preference);
         }
     }
-    (void)accumulate;
-    return &g_plans.emplace(key, plan).first->second;
+    return plan;
+}
+
+Plan* plan_for(hipblasLtHandle_t handle, const Key& key, int rows, int N, int K, long lda, long ldw, long ldo,
+               int out_dtype, int act, bool bias, size_t workspace_bytes) {
+    auto found = g_plans.find(key);
+    if (found == g_plans.end()) {
+        make_room();
+        found = g_plans.emplace(key, make_plan(handle, rows, N, K, lda, ldw, ldo, out_dtype, act, bias, workspace_bytes)).first;
+    }
+    found->second.used = ++g_calls;
+    return &found->second;
+}
+
+// The layouts of a plan's A and out at M rows (they are made at the bucket's edge).
+bool set_rows(Plan* plan, int M) {
+    if (plan->rows_set == M) return true;
+    const uint64_t cols = (uint64_t)M;
+    if (hipblasLtMatrixLayoutSetAttribute(plan->a, HIPBLASLT_MATRIX_LAYOUT_COLS, &cols, sizeof(cols)) != HIPBLAS_STATUS_SUCCESS ||
+        hipblasLtMatrixLayoutSetAttribute(plan->out, HIPBLASLT_MATRIX_LAYOUT_COLS, &cols, sizeof(cols)) != HIPBLAS_STATUS_SUCCESS)
+        return false;
+    plan->rows_set = M;
+    return true;
 }
 
 }  // namespace
@@ -121,17 +181,42 @@ KA_API int ka_linear_library_bf16(const void* A, long lda, const void* W, long l
         hipblasStatus_t s = hipblasLtCreate(&g_handle[device]);
         KA_CHECK(s == HIPBLAS_STATUS_SUCCESS, "%s: hipblasLtCreate failed with status %d", who, (int)s);
     }
-    const Key key{device, M, N, K, lda, ldw, ldo, out_dtype, act, bias != nullptr, accumulate != 0, (size_t)workspace_bytes};
-    const Plan* plan = plan_for(g_handle[device], key, M, N, K, lda, ldw, ldo, out_dtype, act, bias != nullptr, accumulate != 0,
-                                (size_t)workspace_bytes);
-    if (!plan->usable) return 1;
-    if (bias) {
-        hipblasStatus_t s = hipblasLtMatmulDescSetAttribute(plan->desc, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &bias, sizeof(bias));
-        KA_CHECK(s == HIPBLAS_STATUS_SUCCESS, "%s: cannot set the bias (status %d)", who, (int)s);
-    }
     const float alpha = 1.0f, beta = accumulate ? 1.0f : 0.0f;
-    hipblasStatus_t s = hipblasLtMatmul(g_handle[device], plan->desc, &alpha, W, plan->w, A, plan->a, &beta, out, plan->out, out,
-                                        plan->out, &plan->algo, workspace, (size_t)workspace_bytes, stream);
-    KA_CHECK(s == HIPBLAS_STATUS_SUCCESS, "%s: hipblasLtMatmul failed with status %d (M=%d N=%d K=%d)", who, (int)s, M, N, K);
-    return 0;
+    // first the plan of the bucket of rows, then (if the library refuses its algorithm for this row
+    // count) a plan for exactly these rows
+    for (int attempt = 0; attempt < 2; ++attempt) {
+        const int rows = attempt == 0 ? rows_bucket(M) : M;
+        const Key key{device, attempt == 0 ? rows : -M, N, K, lda, ldw, ldo, out_dtype, act, bias != nullptr, accumulate != 0,
+                      (size_t)workspace_bytes};
+        Plan* plan = plan_for(g_handle[device], key, rows, N, K, lda, ldw, ldo, out_dtype, act, bias != nullptr,
+                              (size_t)workspace_bytes);
+        if (!plan->usable) {
+            if (attempt == 0 && rows != M) continue;
+            return 1;
+        }
+        if (rows != M && !plan->every_count) continue;
+        if (!set_rows(plan, M)) continue;
+        if (bias) {
+            hipblasStatus_t s = hipblasLtMatmulDescSetAttribute(plan->desc, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &bias, sizeof(bias));
+            KA_CHECK(s == HIPBLAS_STATUS_SUCCESS, "%s: cannot set the bias (status %d)", who, (int)s);
+        }
+        hipblasStatus_t s = hipblasLtMatmul(g_handle[device], plan->desc, &alpha, W, plan->w, A, plan->a, &beta, out, plan->out,
+                                            out, plan->out, &plan->algo, workspace, (size_t)workspace_bytes, stream);
+        if (s == HIPBLAS_STATUS_SUCCESS) return 0;
+        if (attempt == 0 && rows != M) {
+            plan->every_count = false;
+            continue;
+        }
+        KA_CHECK(false, "%s: hipblasLtMatmul failed with status %d (M=%d N=%d K=%d)", who, (int)s, M, N, K);
+    }
+    return 1;
+}
+
+// For measurements and tests: how many plans are kept, how often the heuristic was asked, how many
+// plans had to make room.
+KA_API void ka_linear_library_stats(long* plans, long* heuristic_calls, long* evicted) {
+    std::lock_guard<std::mutex> hold(g_lock);
+    if (plans) *plans = (long)g_plans.size();
+    if (heuristic_calls) *heuristic_calls = (long)g_heuristic_calls;
+    if (evicted) *evicted = (long)g_evicted;
 }

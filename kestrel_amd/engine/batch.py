@@ -87,4 +87,5 @@ class StepBatch:
     max_kv: int = 1
     decode_only: bool = False
     causal_only: bool = True            # no token sees past its own position
+    wants_every_token: bool = False     # ``logit_rows`` is 0, 1, ..., n_tokens - 1: every token's logits, in order
     host: dict = field(default_factory=dict)

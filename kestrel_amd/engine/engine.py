@@ -12,6 +12,7 @@ this engine: prompts are token ids, an image is a block of given embeddings.
 from __future__ import annotations
 
 import asyncio
+import logging
 import queue
 import threading
 import time
@@ -27,6 +28,8 @@ from ..sampling.sampler import Sampler
 from .loading import load_model, make_runner
 from .scheduler import GenerationScheduler
 from .types import GeneratedPrefix, GenerationRequest, SchedulerResult
+
+_LOGGER = logging.getLogger(__name__)
 
 
 @dataclass
@@ -65,32 +68,32 @@ class _Pending:
 
 
 def _generated_prefix(raw) -> GeneratedPrefix:
-    """``None``, a ``GeneratedPrefix`` or a mapping with ``tokens`` and optionally ``logprobs``
-    (``kestrel/engine/core.py:1260-1294``)."""
+    """What a resumed request brings: ``None``, a ``GeneratedPrefix``, or a mapping with ``tokens`` and
+    optionally ``logprobs`` (the reference's private setting, ``kestrel/engine/core.py:1260-1294``)."""
     if raw is None:
         return GeneratedPrefix()
     if isinstance(raw, GeneratedPrefix):
         tokens, logprobs = raw.tokens, raw.logprobs
-    else:
-        if not isinstance(raw, Mapping):
-            raise TypeError("_generated_prefix must be a mapping or None")
-        extra = set(raw) - {"tokens", "logprobs"}
-        if extra:
-            raise TypeError(f"_generated_prefix has unsupported key(s): {', '.join(sorted(map(str, extra)))}")
+    elif isinstance(raw, Mapping):
+        unknown = sorted(str(key) for key in set(raw) - {"tokens", "logprobs"})
+        if unknown:
+            raise TypeError(f"generated_prefix takes the keys 'tokens' and 'logprobs', not {', '.join(unknown)}")
         if "tokens" not in raw:
-            raise ValueError("_generated_prefix.tokens is required")
+            raise ValueError("generated_prefix needs 'tokens': the ids the request generated before")
         tokens, logprobs = raw["tokens"], raw.get("logprobs")
-    if tokens is None:
-        tokens = ()
-    if isinstance(tokens, (str, bytes)) or not isinstance(tokens, (Sequence_abc, torch.Tensor)):
-        raise TypeError("_generated_prefix.tokens must be a sequence of token ids")
-    tokens = tuple(int(t) for t in tokens)
+    else:
+        raise TypeError(f"generated_prefix is a mapping with 'tokens' (and 'logprobs') or None, got {type(raw).__name__}")
+
+    def listed(values, what):
+        if isinstance(values, (str, bytes)) or not isinstance(values, (Sequence_abc, torch.Tensor)):
+            raise TypeError(f"generated_prefix: {what} must be a sequence, got {type(values).__name__}")
+        return values
+
+    tokens = tuple(int(t) for t in listed(() if tokens is None else tokens, "'tokens'"))
     if logprobs is not None:
-        if isinstance(logprobs, (str, bytes)) or not isinstance(logprobs, (Sequence_abc, torch.Tensor)):
-            raise TypeError("_generated_prefix.logprobs must be a sequence of floats or None")
-        logprobs = tuple(float(v) for v in logprobs)
+        logprobs = tuple(float(v) for v in listed(logprobs, "'logprobs'"))
         if len(logprobs) != len(tokens):
-            raise ValueError("_generated_prefix.logprobs must have the same length as generated prefix tokens")
+            raise ValueError(f"generated_prefix: {len(logprobs)} log-probabilities for {len(tokens)} tokens")
     return GeneratedPrefix(tokens, logprobs)
 
 
@@ -176,8 +179,12 @@ class InferenceEngine:
             raise ValueError("RuntimeConfig.model_path must name a folder with config.json and model.safetensors")
         device = cfg.resolved_device()
         torch.cuda.set_device(device)
+        started = time.perf_counter()
         net = load_model(cfg.model_path, cfg.dtype, device, cfg.model)
         self.plan = net.plan
+        _LOGGER.info("loaded %s from %s as %s on %s in %.2f s (%d layers, width %d, vocabulary %d)", net.plan.architecture,
+                     cfg.model_path, str(cfg.dtype).replace("torch.", ""), device, time.perf_counter() - started,
+                     len(net.plan.layers), net.plan.dim, net.plan.vocab_size)
         max_seq = min(cfg.max_seq_len or net.plan.max_positions, net.plan.max_positions)
         from ..cache.manager import CacheManager
 
@@ -186,14 +193,24 @@ class InferenceEngine:
         n_pages = pool_pages(cfg, sizing.bytes_per_page(), max_seq, free_bytes)
         self.runner = make_runner(net, cfg.page_size, n_pages, cfg.max_batch_size,
                                   max_tokens_per_step=cfg.max_num_batched_tokens, enable_graphs=cfg.enable_graphs)
-        self.scheduler = GenerationScheduler(self.runner, Sampler(device, cfg.seed, pending=self.runner.pending),
-                                             cfg.max_batch_size, cfg.max_num_batched_tokens, net.plan.eos_token_ids,
-                                             max_seq, pipeline_depth=cfg.pipeline_depth)
+        _LOGGER.info("cache pool: %d pages of %d tokens per group of layers (%.2f GiB), %d request slots, contexts up to %d",
+                     n_pages, cfg.page_size, n_pages * sizing.bytes_per_page() / float(1 << 30), cfg.max_batch_size, max_seq)
+        sampler = Sampler(device, cfg.seed, pending=self.runner.pending)
+        self.scheduler = GenerationScheduler(self.runner, sampler, cfg.max_batch_size, cfg.max_num_batched_tokens,
+                                             net.plan.eos_token_ids, max_seq, pipeline_depth=cfg.pipeline_depth)
+        if cfg.warmup:
+            # graphs, scratch memory and plans now, not in the middle of the first steps that need them
+            done = self.runner.prepare(cfg.max_num_batched_tokens, wanted_rows=cfg.max_batch_size)
+            sampler.reserve(cfg.max_batch_size)
+            _LOGGER.info("warm-up: %d decode graphs captured in %.2f s, %d prompt steps in %.2f s, %.0f MiB of kernel scratch",
+                         int(done.get("graphs", 0)), done.get("capture_s", 0.0), int(done.get("prompt_steps", 0)),
+                         done.get("prompt_s", 0.0), done.get("kernel_scratch_bytes", 0) / float(1 << 20))
 
     def _scheduler_loop(self) -> None:
         try:
             self._build()
         except BaseException as exc:  # surfaced to the caller of start()
+            _LOGGER.error("start-up failed: %s: %s", type(exc).__name__, exc)
             self._startup_error = exc
             self._started.set()
             return
@@ -216,6 +233,8 @@ class InferenceEngine:
                         scheduler.enqueue_request(item.request)
                         pending[item.request.request_id] = item
                     except Exception as exc:
+                        _LOGGER.warning("request %d refused at the door: %s: %s", item.request.request_id,
+                                        type(exc).__name__, exc)
                         self._deliver_error(item, exc)
                 if self._stop and not scheduler.has_pending_work():
                     break
@@ -235,6 +254,7 @@ class InferenceEngine:
                         self._deliver(pending.pop(result.request_id), result)
         except BaseException as exc:
             self._fatal = exc
+            _LOGGER.exception("the scheduler thread has stopped; %d requests fail with it", len(pending))
             for item in pending.values():
                 self._deliver_error(item, exc)
             while True:
@@ -292,7 +312,7 @@ class InferenceEngine:
     # ------------------------------------------------------------------ requests
     def _make_request(self, prompt_ids, max_new_tokens, temperature, top_p, prefix_embeds, prefix_ids, stop_ids, seed,
                       on_token, return_logprobs=False, suppress_next_token_ids=(), suppressed_token_ids=(),
-                      allowed_token_ids=None, generated_prefix=None) -> GenerationRequest:
+                      allowed_token_ids=None, generated_prefix=None, prompt_embeds=None, blocks=None) -> GenerationRequest:
         if self._fatal is not None:
             raise RuntimeError("the engine has stopped after an error") from self._fatal
         if self._thread is None:
@@ -310,7 +330,8 @@ class InferenceEngine:
                                  suppressed_token_ids=tuple(int(t) for t in suppressed_token_ids or ()),
                                  allowed_token_ids=None if allowed_token_ids is None
                                  else tuple(int(t) for t in allowed_token_ids),
-                                 generated_prefix=_generated_prefix(generated_prefix))
+                                 generated_prefix=_generated_prefix(generated_prefix), prompt_embeds=prompt_embeds,
+                                 blocks=None if blocks is None else tuple((int(lo), int(hi)) for lo, hi in blocks))
 
     def submit_sync(self, prompt_ids: Sequence[int], *, max_new_tokens: int, temperature: Optional[float] = None,
                     top_p: Optional[float] = None, prefix_embeds: Optional[torch.Tensor] = None,
@@ -320,9 +341,11 @@ class InferenceEngine:
         ``return_logprobs``, ``suppress_next_token_ids``, ``suppressed_token_ids``,
         ``allowed_token_ids`` and ``generated_prefix`` (tokens the request generated before: they are
         fed after the prompt, count against ``max_new_tokens`` and head the result)
-        (``kestrel/engine/core.py:556-597``)."""
+        (``kestrel/engine/core.py:556-597``); and, for prompts with more than one block of given
+        embeddings, ``prompt_embeds`` (rows for the places of ``prompt_ids`` that hold -1) and ``blocks``
+        (the position ranges that see each other both ways)."""
         unknown = set(sampling) - {"return_logprobs", "suppress_next_token_ids", "suppressed_token_ids",
-                                   "allowed_token_ids", "generated_prefix"}
+                                   "allowed_token_ids", "generated_prefix", "prompt_embeds", "blocks"}
         if unknown:
             raise TypeError(f"unknown options: {sorted(unknown)}")
         on_token = None

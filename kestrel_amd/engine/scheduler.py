@@ -34,6 +34,7 @@ are known without the token, so no step is launched beyond them.
 
 from __future__ import annotations
 
+import logging
 import time
 from collections import deque
 from dataclasses import dataclass, field
@@ -44,6 +45,8 @@ import torch
 
 from .step import PENDING_TOKEN, StepEntry, StepRefused
 from .types import GenerationRequest, RequestMetrics, RequestPhase, SchedulerResult, Sequence_
+
+_LOGGER = logging.getLogger(__name__)
 
 
 @dataclass
@@ -113,8 +116,8 @@ class GenerationScheduler:
         if request.prefill_length >= self.max_positions:
             raise ValueError(f"prompt of {request.prefill_length} tokens leaves no room in a context of {self.max_positions}")
         self._check_contents(request)
-        if request.block_length > self.max_num_batched_tokens:
-            raise ValueError(f"the bidirectional block of {request.block_length} positions does not fit in one step "
+        if request.longest_block > self.max_num_batched_tokens:
+            raise ValueError(f"the bidirectional block of {request.longest_block} positions does not fit in one step "
                              f"of {self.max_num_batched_tokens} tokens")
         self.waiting.append(Sequence_(request))
 
@@ -134,17 +137,28 @@ class GenerationScheduler:
             values = np.asarray(ids)
             if values.ndim != 1 or values.dtype.kind not in "iu":
                 raise ValueError(f"{name} must be a flat sequence of integer token ids")
+            if name == "prompt_ids" and request.prompt_embeds is not None:
+                values = values[values != -1]             # places whose embeddings are given
+                if values.size == 0:
+                    continue
             low, high = int(values.min()), int(values.max())
             if low < 0 or high >= vocab:
                 bad = low if low < 0 else high
                 raise ValueError(f"{name}: token id {bad} outside the vocabulary of {vocab}")
-        embeds = request.prefix_embeds
-        if embeds is not None:
-            dim = getattr(plan, "dim", None)
+        dim = getattr(plan, "dim", None)
+        for name, embeds in (("prefix_embeds", request.prefix_embeds), ("prompt_embeds", request.prompt_embeds)):
+            if embeds is None:
+                continue
             if not isinstance(embeds, torch.Tensor) or embeds.dim() != 2 or not embeds.is_floating_point() \
                     or (dim is not None and embeds.shape[1] != dim):
                 shape = tuple(embeds.shape) if isinstance(embeds, torch.Tensor) else type(embeds).__name__
-                raise ValueError(f"prefix_embeds must be a floating-point tensor [rows, {dim}], got {shape}")
+                raise ValueError(f"{name} must be a floating-point tensor [rows, {dim}], got {shape}")
+        if request.prompt_embeds is not None:
+            n_places = int((np.asarray(request.prompt_ids) == -1).sum()) if len(request.prompt_ids) else 0
+            if n_places != int(request.prompt_embeds.shape[0]):
+                raise ValueError(f"prompt_embeds has {int(request.prompt_embeds.shape[0])} rows for {n_places} places of "
+                                 f"prompt_ids that hold -1")
+        request.check_blocks()
 
     def has_pending_work(self) -> bool:
         return bool(self.waiting or self.prefilling or self.running or self._inflight)
@@ -158,41 +172,35 @@ class GenerationScheduler:
         return min(request.prompt_length + request.max_new_tokens, self.max_positions)
 
     def _portion(self, seq: Sequence_, budget: int) -> int:
-        """Places of the prompt to feed next within ``budget`` (0: does not fit now)."""
+        """Places of the prompt to feed next within ``budget`` (0: does not fit now). A portion that
+        does not end the prompt ends on a page boundary where it can, and never inside a
+        bidirectional block: it is cut back to the block's start, and a block that starts the
+        portion goes in whole or not at all."""
         request = seq.request
         left = request.prefill_length - seq.fed
-        take = min(left, budget)
-        block = request.block_length
-        if take < left:
+        end = seq.fed + min(left, budget)
+        blocks = request.block_ranges
+
+        def inside_a_block(place: int) -> Optional[Tuple[int, int]]:
+            return next(((lo, hi) for lo, hi in blocks if lo < place < hi), None)
+
+        split = inside_a_block(end)
+        if split is not None:
+            end = split[0]                # the block waits for a portion that holds all of it
+        if seq.fed < end < request.prefill_length:
             # cut on a page boundary where that is possible, so that the next portion starts on one
             page = self.runner.cache.page_size
-            aligned = (seq.fed + take) // page * page - seq.fed
-            if aligned > 0 and not (seq.fed < block and seq.fed + aligned < block):
-                take = aligned
-        if seq.fed < block and seq.fed + take < block:
-            return 0                      # the block must go in whole
-        return take
+            aligned = end // page * page
+            if aligned > seq.fed and inside_a_block(aligned) is None:
+                end = aligned
+        return max(0, end - seq.fed)
 
     def _prompt_slice(self, seq: Sequence_, take: int) -> StepEntry:
         request = seq.request
         lo, hi = seq.fed, seq.fed + take
-        n_ids = len(request.prefix_ids)
-        n_emb = 0 if request.prefix_embeds is None else int(request.prefix_embeds.shape[0])
-        tokens: List[int] = []
-        embeds = None
-        for p in range(lo, min(hi, n_ids)):
-            tokens.append(int(request.prefix_ids[p]))
-        if hi > n_ids and lo < n_ids + n_emb:
-            a, b = max(lo, n_ids) - n_ids, min(hi, n_ids + n_emb) - n_ids
-            tokens.extend([-1] * (b - a))
-            embeds = request.prefix_embeds[a:b]
-        n_prompt = request.prompt_length
-        for p in range(max(lo, n_ids + n_emb), min(hi, n_prompt)):
-            tokens.append(int(request.prompt_ids[p - n_ids - n_emb]))
-        for p in range(max(lo, n_prompt), hi):       # what it had generated before follows the prompt
-            tokens.append(int(request.generated_prefix.tokens[p - n_prompt]))
-        block = request.block_length
-        bidirectional = [(0, block)] if block and lo == 0 else []
+        ids, embeds = request.places(lo, hi)
+        tokens = ids.tolist() if take <= 64 else ids
+        bidirectional = [block for block in request.block_ranges if lo <= block[0] and block[1] <= hi]
         ends_prompt = hi == request.prefill_length
         return StepEntry(seq.slot, tokens, want=[take - 1] if ends_prompt else [], embeds=embeds,
                          bidirectional=bidirectional, start=lo)
@@ -348,6 +356,8 @@ class GenerationScheduler:
             rows = [plan.rows[exc.entry_index]]
         else:
             rows = list(plan.rows)
+        _LOGGER.error("step %d failed (%s: %s): %d of its %d requests fail: %s", self.steps, type(exc).__name__, exc,
+                      len(rows), len(plan.rows), [row.seq.request.request_id for row in rows])
         for row in rows:
             if row.seq.finish_reason is None:
                 self._finish(row.seq, "error", now, f"{type(exc).__name__}: {exc}")
@@ -442,6 +452,7 @@ class GenerationScheduler:
         seq = self.waiting.popleft()
         needed = self._target_length(seq.request)
         message = f"Insufficient KV cache capacity for request {seq.request.request_id} (needs {needed} tokens)."
+        _LOGGER.warning("%s", message)
         self._finish(seq, "error", time.perf_counter(), message)
         return True
 

@@ -17,6 +17,7 @@ anything but the replays, so a mixer that keeps state is advanced once a step.
 
 from __future__ import annotations
 
+import operator
 from dataclasses import dataclass
 from typing import Dict, List, Optional, Sequence, Tuple
 
@@ -251,7 +252,10 @@ class ModelRunner:
             if q <= self.SCALAR_ROW:
                 n_given = 0
                 for tok in e.tokens:
-                    tok = int(tok)
+                    try:
+                        tok = operator.index(tok)
+                    except TypeError:
+                        raise refuse("token ids must be a flat sequence of integers") from None
                     if tok >= plan.vocab_size or tok < PENDING_TOKEN:
                         raise refuse(f"token id {tok} outside the vocabulary of {plan.vocab_size}")
                     n_given += tok == GIVEN_TOKEN
@@ -474,7 +478,8 @@ class ModelRunner:
             workspace=workspace or self.workspace,
             query_blocks={tile: (view(f"qblk_row{tile}"), view(f"qblk_tok{tile}")) for tile in blocks},
             pending=self.pending, given_embeds=given_embeds, given_rows=view("given_rows") if given else None, max_q=max_q, max_kv=max_kv,
-            decode_only=max_q == 1, causal_only=causal_only, page_runs=(view("run_first"), view("run_count")),
+            decode_only=max_q == 1, causal_only=causal_only, wants_every_token=logit_rows == list(range(n_tokens)),
+            page_runs=(view("run_first"), view("run_count")),
             host={"starts": starts, "q_lens": [len(e.tokens) for e in entries], "kv_len": kv_len, "meta_ints": total},
         )
 
@@ -485,19 +490,27 @@ class ModelRunner:
         if not self.enable_graphs or len(entries) > self._buckets[-1]:
             return None
         for e in entries:
-            token = int(e.tokens[0])
-            if len(e.tokens) != 1 or (token < 0 and token != PENDING_TOKEN) or list(e.want) != [0] or e.embeds is not None:
+            # (anything odd about an entry is left to ``_check_entries``, which names it: the eager path)
+            if len(e.tokens) != 1 or list(e.want) != [0] or e.embeds is not None:
+                return None
+            try:
+                token = operator.index(e.tokens[0])
+            except TypeError:
+                return None
+            if token < 0 and token != PENDING_TOKEN:
                 return None
         return next(b for b in self._buckets if b >= len(entries))
 
-    def _step_graph(self, entries: Sequence[StepEntry], bucket: int) -> torch.Tensor:
+    def _capture(self, bucket: int) -> _GraphState:
+        """The graph of a decode step of ``bucket`` rows, made if it is not there yet.
+
+        Warm-up and capture run on padding rows alone (no slot, no keys, nothing written): the
+        layout of the metadata depends on the bucket only, and nothing of a live request,
+        per-request state included, is touched before the first replay."""
         state = self._graphs.get(bucket)
         if state is None:
             state = self._graphs[bucket] = _GraphState(self.device)
         if state.graph is None:
-            # Warm-up and capture on padding rows alone (no slot, no keys, nothing written): the
-            # layout of the metadata depends on the bucket only, and nothing of a live request,
-            # per-request state included, is touched before the first replay.
             probe = self.build_batch([], pad_rows=bucket, fixed_pages=self._pages_cap)
             state.meta = torch.empty(probe.host["meta_ints"], dtype=torch.int32, device=self.device)
             blank = self.build_batch([], pad_rows=bucket, fixed_pages=self._pages_cap, meta=state.meta,
@@ -517,12 +530,69 @@ class ModelRunner:
             with torch.cuda.graph(graph):
                 state.logits = self.model.forward(blank, self.layer_caches)
             state.graph = graph
+        return state
+
+    def _step_graph(self, entries: Sequence[StepEntry], bucket: int) -> torch.Tensor:
+        state = self._capture(bucket)
         batch = self.build_batch(entries, pad_rows=bucket, fixed_pages=self._pages_cap, meta=state.meta,
                                  workspace=state.workspace)
         state.graph.replay()
         self.graph_replays += 1
         self.logit_slots = batch.logit_slot[:len(entries)]
         return state.logits[:len(entries)]
+
+    # ------------------------------------------------------------------ everything made at start
+    @torch.inference_mode()
+    def prepare(self, prompt_tokens: Optional[int] = None, wanted_rows: int = 1) -> Dict[str, float]:
+        """Make now what steps would otherwise make when they first need it, with live requests
+        waiting (``kestrel/runtime/decode_graph.py:70-93``, ``kestrel/models/moondream/runtime.py:886-888``,
+        ``kestrel/engine/core.py:458-484``): the kernels' scratch buffers, the graph of every bucket of
+        decode rows (captured on padding rows), the metadata buffer at its largest, and the scratch
+        tensors and vendor-library plans of prompt steps, by running prompts of ids 0 of every
+        multiple of 64 tokens up to ``prompt_tokens`` (default: the step's token limit) through a slot
+        that is given back. No request may be live. Returns what was done and how long it took."""
+        if self.held:
+            raise RuntimeError("prepare() runs before the first request is admitted")
+        import time
+
+        done: Dict[str, float] = {}
+        started = time.perf_counter()
+        if self.model.dtype == torch.bfloat16:
+            from ..ops import fast
+            done["kernel_scratch_bytes"] = fast.prepare(self.device)
+        cache, plan = self.cache, self.model.plan
+        limit = self.max_tokens_per_step if prompt_tokens is None else min(prompt_tokens, self.max_tokens_per_step)
+        rows = max(cache.max_requests, 1)
+        per_token = 8 + 2 * len(cache.groups) + 2 * max(len(self.query_tiles), 1)
+        ints = per_token * (limit + rows) + rows * (8 + len(cache.groups) * (self._pages_cap + 4)) + 4096
+        if self._meta_device is None or self._meta_device.numel() < ints:
+            self._meta_device = torch.empty(ints, dtype=torch.int32, device=self.device)
+        if self.enable_graphs:
+            for bucket in self._buckets:
+                self._capture(bucket)
+            done["graphs"] = len(self._buckets)
+            done["capture_s"] = time.perf_counter() - started
+        # prompts: the largest first (every scratch tensor at its largest), then one per bucket of rows of
+        # the vendor library's plans, the smallest (64 tokens: the kernels of few rows) last
+        fits = min(limit, plan.max_positions - 1, min(g.pool.free_count for g in cache.groups) * cache.page_size
+                   if cache.groups else limit)
+        sizes = sorted({fits} | set(range(64, fits, 64)), reverse=True) if fits >= 1 else []
+        if self.model.dtype != torch.bfloat16:
+            sizes = sizes[:1] + ([64] if fits > 64 else [])      # no library plans on the 32-bit path
+        prompt_started = time.perf_counter()
+        for tokens in sizes:
+            if not cache.can_admit(tokens, tokens):
+                continue
+            slot = self.admit(tokens, tokens)
+            try:
+                self.step([StepEntry(slot, np.zeros(tokens, dtype=np.int64), want=list(range(min(tokens, wanted_rows, rows))))])
+            finally:
+                self.release(slot)
+        torch.cuda.synchronize(self.device)
+        done["prompt_steps"] = len(sizes)
+        done["prompt_s"] = time.perf_counter() - prompt_started
+        done["seconds"] = time.perf_counter() - started
+        return done
 
     # ------------------------------------------------------------------ the step
     @torch.inference_mode()

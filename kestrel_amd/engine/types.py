@@ -12,6 +12,7 @@ import time
 from dataclasses import dataclass, field
 from typing import Callable, List, Optional, Sequence, Tuple
 
+import numpy as np
 import torch
 
 
@@ -34,9 +35,15 @@ class RequestPhase(enum.Enum):
 @dataclass
 class GenerationRequest:
     """One generation. The sequence is ``prefix_ids`` then ``prefix_embeds`` (given
-    embeddings, e.g. an encoded image) then ``prompt_ids``. If embeddings are given,
-    ``prefix_ids`` and the embeddings form one block whose positions see each other both
-    ways (the reference's BOS + image block, ``kestrel/models/moondream/runtime.py:1733-1743``)."""
+    embeddings, e.g. an encoded image) then ``prompt_ids``. If ``prefix_embeds`` are given,
+    ``prefix_ids`` and those embeddings form one block whose positions see each other both
+    ways (the reference's BOS + image block, ``kestrel/models/moondream/runtime.py:1733-1743``).
+
+    More than one block (the reference's mask is "dynamic in the number and position of image
+    blocks", ``kestrel/models/moondream/text.py:146-157``, ``runtime.py:1711-1743``): ``prompt_ids`` may hold
+    ``-1`` at places whose embeddings are the rows of ``prompt_embeds``, in order, and ``blocks`` names the
+    position ranges ``[lo, hi)`` of the whole sequence whose tokens see each other both ways (``None``:
+    the one block described above, if there is one; ``()``: none at all)."""
 
     request_id: int
     prompt_ids: Sequence[int]
@@ -54,26 +61,74 @@ class GenerationRequest:
     suppressed_token_ids: Sequence[int] = ()        # never to be generated
     allowed_token_ids: Optional[Sequence[int]] = None   # if given, the only tokens that may be generated
     generated_prefix: GeneratedPrefix = field(default_factory=GeneratedPrefix)
+    prompt_embeds: Optional[torch.Tensor] = None    # rows for the places of ``prompt_ids`` that hold -1
+    blocks: Optional[Sequence[Tuple[int, int]]] = None
 
     def __post_init__(self) -> None:
-        # the checks of ``kestrel/scheduler/types.py:215-237``
+        # what a resumed request brings must be consistent (``kestrel/scheduler/types.py:215-237``)
         prefix = self.generated_prefix
         if prefix.logprobs is not None and len(prefix.logprobs) != len(prefix.tokens):
-            raise ValueError("generated_prefix.logprobs must have the same length as generated_prefix.tokens")
+            raise ValueError(f"a resumed request brings {len(prefix.tokens)} tokens but {len(prefix.logprobs)} "
+                             f"log-probabilities: one per token, or none")
         if prefix.tokens and len(prefix.tokens) >= self.max_new_tokens:
-            raise ValueError("generated_prefix.tokens must be shorter than max_new_tokens")
+            raise ValueError(f"a resumed request brings {len(prefix.tokens)} tokens, which leaves nothing to generate "
+                             f"within max_new_tokens={self.max_new_tokens}")
         if prefix.tokens and self.return_logprobs and prefix.logprobs is None:
-            raise ValueError("generated_prefix.logprobs is required when return_logprobs is true")
+            raise ValueError("a resumed request that wants log-probabilities back must bring those of the tokens "
+                             "it generated before")
+        self._ids: Optional[np.ndarray] = None
+        self._given_before: Optional[np.ndarray] = None
 
     @property
-    def block_length(self) -> int:
-        n = 0 if self.prefix_embeds is None else int(self.prefix_embeds.shape[0])
-        return n + len(self.prefix_ids) if n else 0
+    def _n_prefix_embeds(self) -> int:
+        return 0 if self.prefix_embeds is None else int(self.prefix_embeds.shape[0])
 
     @property
     def prompt_length(self) -> int:
-        n = 0 if self.prefix_embeds is None else int(self.prefix_embeds.shape[0])
-        return len(self.prefix_ids) + n + len(self.prompt_ids)
+        return len(self.prefix_ids) + self._n_prefix_embeds + len(self.prompt_ids)
+
+    @property
+    def block_ranges(self) -> Tuple[Tuple[int, int], ...]:
+        """The bidirectional blocks as sorted position ranges ``[lo, hi)``."""
+        if self.blocks is not None:
+            return tuple(sorted((int(lo), int(hi)) for lo, hi in self.blocks))
+        n = self._n_prefix_embeds
+        return ((0, n + len(self.prefix_ids)),) if n else ()
+
+    @property
+    def longest_block(self) -> int:
+        return max((hi - lo for lo, hi in self.block_ranges), default=0)
+
+    def check_blocks(self) -> None:
+        """Blocks lie inside the prompt, hold at least one position and do not overlap."""
+        at = 0
+        for lo, hi in self.block_ranges:
+            if not (at <= lo < hi <= self.prompt_length):
+                raise ValueError(f"the bidirectional block [{lo}, {hi}) must hold at least one position, lie inside the "
+                                 f"prompt of {self.prompt_length} positions and not overlap the block before it")
+            at = hi
+
+    def places(self, lo: int, hi: int):
+        """The places ``[lo, hi)`` of what is fed before the first token is sampled: ``(ids, embeds)``, ids with
+        -1 where an embedding is given, embeds the rows for those places (or ``None``)."""
+        if self._ids is None:
+            ids = np.concatenate([np.asarray(self.prefix_ids, dtype=np.int64).reshape(-1),
+                                  np.full(self._n_prefix_embeds, -1, dtype=np.int64),
+                                  np.asarray(self.prompt_ids, dtype=np.int64).reshape(-1),
+                                  np.asarray(self.generated_prefix.tokens, dtype=np.int64).reshape(-1)])
+            self._given_before = np.concatenate([[0], np.cumsum(ids == -1)])
+            self._ids = ids
+        ids = self._ids[lo:hi]
+        a, b = int(self._given_before[lo]), int(self._given_before[hi])
+        if a == b:
+            return ids, None
+        n_first = self._n_prefix_embeds                # rows come from the prefix first, then from prompt_embeds
+        rows = []
+        if a < n_first:
+            rows.append(self.prefix_embeds[a:min(b, n_first)])
+        if b > n_first:
+            rows.append(self.prompt_embeds[max(a, n_first) - n_first:b - n_first])
+        return ids, rows[0] if len(rows) == 1 else torch.cat([r.to(rows[0].device, rows[0].dtype) for r in rows])
 
     @property
     def generated_prefix_length(self) -> int:

@@ -81,7 +81,7 @@ class DecoderModel:
     def _head_with_norm(self, x, batch, logits) -> bool:
         """A few decoded rows, every one of them wanted, in order: the head's launch normalises them itself
         (one launch less a step)."""
-        if self.dtype != torch.bfloat16 or not batch.decode_only or logits.shape[0] != batch.n_tokens \
+        if self.dtype != torch.bfloat16 or not batch.decode_only or not getattr(batch, "wants_every_token", False) \
                 or getattr(self.final_norm.spec, "kind", None) != "layernorm":
             return False
         from ..ops import fast

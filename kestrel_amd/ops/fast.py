@@ -7,7 +7,7 @@ caller then takes the generic kernel) and raises when they do but the call fails
 from __future__ import annotations
 
 import ctypes
-from typing import Dict, Optional
+from typing import Dict, NamedTuple, Optional
 
 import torch
 
@@ -83,19 +83,42 @@ TILED_CONFIG = 0
 LIBRARY_LINEAR = True
 LIBRARY_WORKSPACE_BYTES = 128 << 20
 _library_space = {}
-# Waves the split weight-streaming kernel aims to have on the chip: 8 per workgroup at 256 strips
-# (measured best for the output projection + second feed-forward linear of Moondream 2).
-SKINNY_TARGET_WAVES = 2048
 SCRATCH_FLOATS = 8 << 20
 WIDE_FLOATS = 8 << 20              # 32 MB of partial sums for the wide skinny kernel
 _wide_scratch = {}
 # Keys of one row a workgroup of the decode attention kernel takes before the row is split.
 DECODE_KEYS_PER_WORKGROUP = 4096
-DECODE_WAVE_SLOTS = 4096            # waves of the decode attention kernel that the chip holds at once
-DECODE_FOUR_WAVE_PLACES = 1280      # ... and its workgroups of four waves (five to a CU)
+
+
+class ChipSizes(NamedTuple):
+    """What the choices between kernel forms need to know of the GPU at hand, all of it following
+    from its number of compute units (four SIMDs each)."""
+
+    compute_units: int
+    # waves the split weight-streaming kernel aims to have on the chip: 8 per compute unit (one workgroup
+    # of 8 waves per strip where there are as many strips as compute units; measured best on an MI355X
+    # for an output projection + second feed-forward linear of 2048 outputs)
+    skinny_target_waves: int
+    # waves of the decode attention kernel that the chip holds at once (16 per compute unit: four per
+    # SIMD at the registers the kernel needs), and its workgroups of four waves (five per compute unit)
+    decode_wave_slots: int
+    decode_four_wave_places: int
+
+
+_chips: Dict[int, ChipSizes] = {}
+
+
+def chip_sizes(device=None) -> ChipSizes:
+    """The sizes for ``device`` (default: the current one), asked from the driver once per device."""
+    index = torch.cuda.current_device() if device is None else _device_index(device)
+    if index not in _chips:
+        units = int(torch.cuda.get_device_properties(index).multi_processor_count)
+        _chips[index] = ChipSizes(units, 8 * units, 16 * units, 5 * units)
+    return _chips[index]
+
 
 _lib = None
-_scratch: Dict[torch.device, tuple] = {}
+_scratch: Dict[int, torch.Tensor] = {}
 _OUT_CODE = {torch.float32: KA_F32, torch.bfloat16: KA_BF16}
 
 
@@ -108,6 +131,8 @@ def lib():
             fn.argtypes = argtypes
             fn.restype = _c_int
         handle.ka_last_error.restype = ctypes.c_char_p
+        handle.ka_linear_library_stats.argtypes = [ctypes.POINTER(ctypes.c_long)] * 3
+        handle.ka_linear_library_stats.restype = None
         handle.ka_skinny_set_persistent.argtypes = [_c_int]
         handle.ka_skinny_set_persistent.restype = None
         handle.ka_rope_cache_pages_supported.argtypes = [_c_int, _c_int, _c_int]
@@ -144,10 +169,16 @@ def _check(status: int) -> None:
         raise KernelError(lib().ka_last_error().decode())
 
 
+def _device_index(device) -> int:
+    """One key per GPU, whether or not the device's name carries its index."""
+    device = torch.device(device)
+    return torch.cuda.current_device() if device.index is None else device.index
+
+
 def scratch(device: torch.device) -> torch.Tensor:
     """Partial results that the parts of a row's keys meet through in decode attention (one
     buffer per device). Calls on one device must not overlap."""
-    key = torch.device(device)
+    key = _device_index(device)
     if key not in _scratch:
         _scratch[key] = torch.zeros(SCRATCH_FLOATS, dtype=torch.float32, device=device)
     return _scratch[key]
@@ -157,21 +188,42 @@ def _wide_args(device: torch.device, rows: int):
     """Scratch memory for the parts of K of a skinny linear that goes to the wide kernel: fp32
     partial sums, one buffer per device, made at the first skinny call (a step's first run is
     never inside a graph capture). Calls on one device must not overlap."""
-    key = torch.device(device)
+    buf = _wide_scratch_buffer(device)
+    return buf.data_ptr(), buf.numel()
+
+
+def _wide_scratch_buffer(device: torch.device) -> torch.Tensor:
+    key = _device_index(device)
     if key not in _wide_scratch:
         _wide_scratch[key] = torch.empty(WIDE_FLOATS, dtype=torch.float32, device=device)
-    buf = _wide_scratch[key]
-    return buf.data_ptr(), buf.numel()
+    return _wide_scratch[key]
 
 
 def _library_workspace(device: torch.device) -> torch.Tensor:
     """Scratch memory the vendor library's kernels may use (parts of K that meet in it), one buffer
     per device, made at the first call (a step's first run is never inside a graph capture).
     Calls on one device must not overlap."""
-    key = torch.device(device)
+    key = _device_index(device)
     if key not in _library_space:
         _library_space[key] = torch.empty(LIBRARY_WORKSPACE_BYTES, dtype=torch.uint8, device=device)
     return _library_space[key]
+
+
+def prepare(device: torch.device) -> int:
+    """Everything these kernels keep per device, made now instead of at the first call that needs it
+    (which may be the first step of a live request): the partial results of decode attention, the
+    partial sums of the wide skinny kernel and the vendor library's workspace. Returns their bytes."""
+    buffers = (scratch(device), _library_workspace(device), _wide_scratch_buffer(device))
+    return sum(b.numel() * b.element_size() for b in buffers)
+
+
+def library_stats() -> Dict[str, int]:
+    """Plans the vendor-library linears keep, how often the library's heuristic was asked for an
+    algorithm, and how many plans had to make room (all since the process started)."""
+    handle = lib()
+    values = [ctypes.c_long(0) for _ in range(3)]
+    handle.ka_linear_library_stats(*[ctypes.byref(v) for v in values])
+    return dict(zip(("plans", "heuristic_calls", "evicted"), (int(v.value) for v in values)))
 
 
 def _operand_ok(t: torch.Tensor, k: int) -> bool:
@@ -205,7 +257,7 @@ def linear_bf16(a, weight, bias, out, act, accumulate) -> bool:
     if m <= SKINNY_MAX_ROWS:
         _check(handle.ka_linear_skinny_bf16(a.data_ptr(), a.stride(0), weight.data_ptr(), weight.stride(0), _ptr(bias),
                                             out.data_ptr(), _OUT_CODE[out.dtype], out.stride(0), m, n, k, act,
-                                            int(accumulate), SKINNY_TARGET_WAVES, *_wide_args(a.device, m), stream_ptr()))
+                                            int(accumulate), chip_sizes(a.device).skinny_target_waves, *_wide_args(a.device, m), stream_ptr()))
     else:
         if LIBRARY_LINEAR and TILED_CONFIG == 0:
             space = _library_workspace(a.device)
@@ -247,7 +299,7 @@ def linear_pair_accumulate(a1, w1, b1, a2, w2, b2, out, then_norm=None) -> bool:
             return False
         _check(lib().ka_linear_skinny_pair_norm(
             a1.data_ptr(), a1.stride(0), k1, a2.data_ptr(), a2.stride(0), k2, w1.data_ptr(), w1.stride(0), _ptr(b1),
-            w2.data_ptr(), w2.stride(0), _ptr(b2), out.data_ptr(), out.stride(0), n, 1, m, SKINNY_TARGET_WAVES,
+            w2.data_ptr(), w2.stride(0), _ptr(b2), out.data_ptr(), out.stride(0), n, 1, m, chip_sizes(a1.device).skinny_target_waves,
             *_wide_args(a1.device, m), gamma.data_ptr(), _ptr(beta), float(eps), normed.data_ptr(), _OUT_CODE[normed.dtype],
             normed.stride(0), stream_ptr()))
         return True
@@ -255,7 +307,7 @@ def linear_pair_accumulate(a1, w1, b1, a2, w2, b2, out, then_norm=None) -> bool:
         a1.data_ptr(), a1.stride(0), k1, a2.data_ptr(), a2.stride(0), k2, w2.data_ptr(), w2.stride(0), _ptr(b2),
         None, None, None, 0.0,
         w1.data_ptr(), w1.stride(0), _ptr(b1), out.data_ptr(), KA_F32, out.stride(0), n, 0, 1,
-        None, 0, None, None, 0, 0, 0, 0, m, SKINNY_TARGET_WAVES, *_wide_args(a1.device, m), stream_ptr()))
+        None, 0, None, None, 0, 0, 0, 0, m, chip_sizes(a1.device).skinny_target_waves, *_wide_args(a1.device, m), stream_ptr()))
     return True
 
 
@@ -279,7 +331,7 @@ def linear_two_outputs(a, wa, ba, out_a, act_a, wb, bb, out_b, act_b) -> bool:
         None, None, None, 0.0,
         wa.data_ptr(), wa.stride(0), _ptr(ba), out_a.data_ptr(), _OUT_CODE[out_a.dtype], out_a.stride(0), na, act_a, 0,
         wb.data_ptr(), wb.stride(0), _ptr(bb), out_b.data_ptr(), _OUT_CODE[out_b.dtype], out_b.stride(0), nb, act_b,
-        m, SKINNY_TARGET_WAVES, *_wide_args(a.device, m), stream_ptr()))
+        m, chip_sizes(a.device).skinny_target_waves, *_wide_args(a.device, m), stream_ptr()))
     return True
 
 
@@ -322,7 +374,7 @@ def layernorm_linear(x, gamma, beta, eps, wa, ba, out_a, act_a, wb=None, bb=None
         wa.data_ptr(), wa.stride(0), _ptr(ba), out_a.data_ptr(), _OUT_CODE[out_a.dtype], out_a.stride(0), na, act_a, 0,
         _ptr(wb), wb.stride(0) if two else 0, _ptr(bb) if two else None, _ptr(out_b),
         _OUT_CODE[out_b.dtype] if two else 0, out_b.stride(0) if two else 0, nb, act_b,
-        m, SKINNY_TARGET_WAVES, None, 0, stream_ptr()))
+        m, chip_sizes(x.device).skinny_target_waves, None, 0, stream_ptr()))
     return True
 
 
@@ -357,17 +409,18 @@ def decode_shape(max_kv: int, workgroups: int = 1):
     they all fit on the chip at once (measured at 1024 keys: 16 waves up to 256 workgroups, 8 up to
     512, 4 beyond: workgroups of four waves fit five to a CU; 8 again where those of four would end
     in a round that leaves much of the chip idle)."""
+    chip = chip_sizes()
     splits = max(1, -(-max_kv // DECODE_KEYS_PER_WORKGROUP))
     tiles = -(-max_kv // (64 * splits))
     waves = 4 if tiles <= 4 else 8 if tiles <= 8 else 16
     groups = workgroups * splits
-    fit = 16 if groups <= DECODE_WAVE_SLOTS // 16 else 8 if groups <= DECODE_WAVE_SLOTS // 8 else 4
+    fit = 16 if groups <= chip.decode_wave_slots // 16 else 8 if groups <= chip.decode_wave_slots // 8 else 4
     if fit == 4:
-        # workgroups of four waves run in rounds of DECODE_FOUR_WAVE_PLACES; where the last round would
-        # leave much of the chip idle, workgroups of eight waves come out better (48 rows x 32 heads are
+        # workgroups of four waves run in rounds of as many as the chip has places for; where the last round
+        # would leave much of the chip idle, workgroups of eight waves come out better (48 rows x 32 heads are
         # 1.2 rounds of the one, 3 rounds of the other: 14.9k against 15.2k tok/s)
-        rounds = -(-groups // DECODE_FOUR_WAVE_PLACES)
-        if groups < 0.7 * rounds * DECODE_FOUR_WAVE_PLACES:
+        rounds = -(-groups // chip.decode_four_wave_places)
+        if groups < 0.7 * rounds * chip.decode_four_wave_places:
             fit = 8
     return splits, min(waves, fit)
 

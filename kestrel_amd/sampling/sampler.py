@@ -49,6 +49,15 @@ class Sampler:
         self._device_args: List[Optional[torch.Tensor]] = [None] * self.STAGING_RING
         self._next = 0
 
+    def reserve(self, rows: int) -> None:
+        """Argument buffers for steps of up to ``rows`` rows, made now (all of the ring) instead of at
+        the first steps that fill them."""
+        words = max(1024, 32 * rows)
+        for index in range(self.STAGING_RING):
+            if self._staging[index] is None or self._staging[index].numel() < words:
+                self._staging[index] = torch.empty(words, dtype=torch.int32, pin_memory=True)
+                self._device_args[index] = torch.empty(words, dtype=torch.int32, device=self.device)
+
     def _upload(self, columns: Sequence[np.ndarray]) -> List[torch.Tensor]:
         """Small arguments (4- or 8-byte columns of any length) to the device with one copy out of
         pinned memory."""

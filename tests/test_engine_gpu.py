@@ -163,6 +163,49 @@ def test_split_bidirectional_block_is_refused():
         runner.step([StepEntry(slot, [-1] * 8, embeds=embeds, bidirectional=[(0, 17)])])
 
 
+@pytest.mark.parametrize("graphs", [False, True], ids=["eager", "graphs"])
+def test_an_odd_entry_is_refused_by_its_index_before_the_cache_is_touched(graphs):
+    """No tokens at all, a token that is no integer, wanted places that repeat a row: each is named by
+    ``StepRefused.entry_index`` (also where steps are replayed as graphs, whose bucket is looked for
+    first), and the request beside it holds what it held."""
+    from kestrel_amd.engine.step import StepEntry, StepRefused
+
+    runner = _runner("A", torch.float32, graphs=graphs)
+    good, odd = runner.admit(), runner.admit()
+    runner.step([StepEntry(good, [5, 6, 7], want=[2]), StepEntry(odd, [9, 10], want=[1])])
+    free = [g.pool.free_count for g in runner.cache.groups]
+    for tokens, message in (([], "at least one token"), (["x"], "integers"), ([1.5], "integers")):
+        with pytest.raises(StepRefused, match=message) as caught:
+            runner.step([StepEntry(good, [8], want=[0]), StepEntry(odd, tokens, want=[0] if tokens else [])])
+        assert caught.value.entry_index == 1
+        assert runner.held == {good: 3, odd: 2} and [g.pool.free_count for g in runner.cache.groups] == free
+    logits = runner.step([StepEntry(good, [8], want=[0]), StepEntry(odd, [11], want=[0])])
+    assert logits.shape[0] == 2 and bool(torch.isfinite(logits).all())
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=DTYPE_IDS)
+def test_wanted_places_that_number_the_tokens_but_are_not_them(dtype):
+    """A decode-only step of three rows that wants three rows of logits, but not one of each: the first
+    row's twice, the second's not at all. The head's launch that normalises 'every row, in order'
+    itself must not be taken for it."""
+    from kestrel_amd.engine.step import StepEntry
+
+    name = "D"
+    runner = _runner(name, dtype)
+    reqs = [_request(name, f"w{i}", 1700 + i, n) for i, n in enumerate((9, 21, 14))]
+    slots = [runner.admit() for _ in reqs]
+    runner.step([StepEntry(slot, req.ids[:-1]) for slot, req in zip(slots, reqs)])
+    logits = runner.step([StepEntry(slots[0], req_last(reqs[0]), want=[0, 0]), StepEntry(slots[1], req_last(reqs[1])),
+                          StepEntry(slots[2], req_last(reqs[2]), want=[0])]).clone()
+    expected = [_expected(name, req)[-1] for req in reqs]
+    for row, which in enumerate((0, 0, 2)):
+        helpers.assert_close(logits[row], expected[which], dtype, f"row {row} of logits is request {which}'s")
+
+
+def req_last(req: Request):
+    return req.ids[-1:]
+
+
 @pytest.mark.parametrize("dtype", DTYPES, ids=DTYPE_IDS)
 @pytest.mark.parametrize("name", ["B", "D", "F"])
 def test_long_decoding(name, dtype):

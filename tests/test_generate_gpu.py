@@ -288,9 +288,9 @@ def test_a_request_resumed_with_its_generated_tokens_goes_on_as_before(temperatu
                 "_generated_prefix": {"tokens": whole.tokens[:4], "logprobs": whole.logprobs[:4]}})
 
         resumed = asyncio.run(resume())
-        with pytest.raises(ValueError, match="shorter than max_new_tokens"):
+        with pytest.raises(ValueError, match="leaves nothing to generate"):
             engine.generate_sync(prompt, max_new_tokens=4, generated_prefix={"tokens": whole.tokens[:4]})
-        with pytest.raises(TypeError, match="unsupported key"):
+        with pytest.raises(TypeError, match="takes the keys"):
             engine.generate_sync(prompt, max_new_tokens=8, generated_prefix={"tokens": [1], "scores": [0.0]})
     finally:
         engine.shutdown_sync()
@@ -410,3 +410,103 @@ def test_profile_decode_command(tmp_path):
                                "--prompt-len", "250", "--decode-iters", "50"], capture_output=True, text=True, env=env,
                               cwd=ROOT, timeout=300)
     assert too_long.returncode == 2 and "exceed the model's context" in too_long.stderr
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_everything_is_made_at_start(dtype, caplog):
+    """With ``warmup`` (the default) the graph of every bucket of decode rows exists before the first
+    request, and a mixed run (prompts cut into portions beside decoded tokens, requests of many lengths,
+    sampling with and without temperature) allocates no device memory between its first request's
+    end and its last; the logger says what was made, and names a request that is refused."""
+    import logging
+
+    from kestrel_amd.engine.step import graph_buckets
+
+    name = "D"
+    cfg = helpers.flat_config(name)
+    with caplog.at_level(logging.INFO, logger="kestrel_amd"):
+        engine = _engine(name, dtype, max_batch_size=6, kv_cache_pages=60, max_num_batched_tokens=64)
+    try:
+        runner = engine.runner
+        assert sorted(runner._graphs) == graph_buckets(6) == [1, 2, 4, 6]
+        assert all(state.graph is not None for state in runner._graphs.values())
+        assert not runner.held and runner.cache.free_slots == runner.cache.max_requests
+        first = engine.generate_sync(helpers.random_ids(1800, 9, cfg["vocab_size"]), max_new_tokens=4, stop_ids=())
+        assert len(first.tokens) == 4
+        torch.cuda.synchronize()
+        before = torch.cuda.memory_allocated()
+        prompts = [helpers.random_ids(1801 + i, n, cfg["vocab_size"]) for i, n in enumerate((3, 70, 150, 31, 64, 5, 97, 200, 12))]
+        futures = [engine.submit_sync(p, max_new_tokens=5 + 3 * (i % 4), temperature=0.0 if i % 2 else 0.8, top_p=0.9,
+                                      seed=i, stop_ids=()) for i, p in enumerate(prompts)]
+        results = [f.result(timeout=120) for f in futures]
+        torch.cuda.synchronize()
+        assert torch.cuda.memory_allocated() == before, "a step of the mixed run allocated device memory"
+        assert all(r.finish_reason == "length" for r in results)
+        with caplog.at_level(logging.WARNING, logger="kestrel_amd"):
+            with pytest.raises(ValueError, match="outside the vocabulary"):
+                engine.generate_sync([1, cfg["vocab_size"] + 5], max_new_tokens=2)
+    finally:
+        engine.shutdown_sync()
+    text = caplog.text
+    assert "warm-up: 4 decode graphs captured" in text and "cache pool: 60 pages" in text and "loaded" in text
+    assert "refused at the door" in text and "outside the vocabulary" in text
+
+
+def test_without_warmup_nothing_is_captured_before_it_is_needed():
+    engine = _engine("A", "bfloat16", warmup=False)
+    try:
+        assert not engine.runner._graphs
+        engine.generate_sync([1, 2, 3], max_new_tokens=3, stop_ids=())
+        assert sorted(engine.runner._graphs) == [1]
+    finally:
+        engine.shutdown_sync()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_prompt_with_two_blocks_of_given_embeddings(dtype):
+    """Text, a block of given rows, text, another block, text: the positions of each block see each other
+    both ways and everything else is causal (``kestrel/models/moondream/text.py:146-157``). The step budget
+    of 16 tokens cuts the prompt of 31 into portions that keep each block whole; a second request decodes
+    beside them. Every generated token must be the plain implementation's choice."""
+    name = "B"
+    cfg = helpers.flat_config(name)
+    weights = helpers.stored_weights(helpers.model_dir(name))
+    gen = torch.Generator().manual_seed(77)
+    pieces = [helpers.random_ids(1900, 4, cfg["vocab_size"]), torch.randn(7, cfg["dim"], generator=gen),
+              helpers.random_ids(1901, 9, cfg["vocab_size"]), torch.randn(5, cfg["dim"], generator=gen),
+              helpers.random_ids(1902, 6, cfg["vocab_size"])]
+    ids, rows, blocks, block_of, embedded = [], [], [], [], []
+    table = weights["text.wte"].double()
+    for piece in pieces:
+        if isinstance(piece, torch.Tensor):
+            blocks.append((len(ids), len(ids) + piece.shape[0]))
+            block_of += [len(blocks) - 1] * piece.shape[0]
+            ids += [-1] * piece.shape[0]
+            rows.append(piece)
+            embedded.append(piece.double())
+        else:
+            block_of += [-1] * len(piece)
+            ids += piece
+            embedded.append(table[piece])
+    assert blocks == [(4, 11), (20, 25)]
+    other = helpers.random_ids(1903, 12, cfg["vocab_size"])
+    engine = _engine(name, dtype, max_num_batched_tokens=16)
+    try:
+        beside = engine.submit_sync(other, max_new_tokens=10, stop_ids=())
+        result = engine.generate_sync(ids, max_new_tokens=8, prompt_embeds=torch.cat(rows), blocks=blocks, stop_ids=())
+        beside = beside.result(timeout=60)
+    finally:
+        engine.shutdown_sync()
+    slack = 1e-4 if dtype == "float32" else 5e-2
+    tokens = result.tokens
+    assert len(tokens) == 8
+    logits = plain.forward(cfg, weights, tokens[:-1], prefix_embeds=torch.cat(embedded),
+                           block_ids=block_of + [-1] * (len(tokens) - 1))
+    for i, token in enumerate(tokens):
+        row = logits[len(ids) - 1 + i]
+        gap = float(row.max() - row[token])
+        assert gap <= slack, f"token {i} is {token}, the plain implementation gives {int(row.argmax())} ({gap:.3g} better)"
+    # the blocks matter: read causally, the same prompt leads elsewhere
+    causal = plain.forward(cfg, weights, [], prefix_embeds=torch.cat(embedded), block_ids=[-1] * len(ids))[-1]
+    assert float((causal - logits[len(ids) - 1]).abs().max()) > 1e-3
+    helpers.assert_greedy_follows(cfg, weights, other, beside.tokens, slack, f"beside the blocks, {dtype}")

@@ -93,3 +93,139 @@ def test_real_layer_sizes_against_the_plain_implementation(sizes, dtype):
     expected = _expected(sizes)
     for tag, req in reqs.items():
         helpers.assert_close(got[tag], expected[tag], dtype, f"{sizes} sizes, {N_LAYERS} layers, request {tag}")
+
+
+# ----------------------------------------------------------------------------------------------------
+# the decode path that serving and the benchmark run: steps replayed as HIP graphs
+# ----------------------------------------------------------------------------------------------------
+N_GRAPH = 64
+SAMPLED = ("g1", "g9")     # their tokens after the prompt are the engine's own greedy choices, fed as PENDING_TOKEN
+
+
+def _graph_workload(sizes: str):
+    """64 short requests and one long one (1,030 places: past 1,024 keys a row's tiles do not divide over
+    the waves of the decode attention kernel), their prompts in eager steps, then decode-only steps of
+    1, 2, 4, 5, 8 and 64 rows, a request that ends and another that takes its slot and pages over,
+    and returns to buckets captured earlier. Returns the requests, the prompt steps and the decode steps."""
+    cfg = SIZES[sizes]
+    vocab, n_prefix = cfg["vocab_size"], cfg["prefix_attn"]
+    prefix = torch.randn(n_prefix, cfg["dim"], generator=torch.Generator().manual_seed(78)) if n_prefix else None
+    tags = [f"g{i}" for i in range(N_GRAPH)]
+    every = ["g0", "g1", "g2", "g3", "n0"] + tags[5:]
+    decode = [["g0"], ["g0", "g1"], ["g0", "g1", "g2", "g3"], ["g0", "g1", "g2", "g3", "g4"],
+              "g4 ends, n0 joins",
+              ["g0", "g1", "g2", "g3", "n0", "g5", "g6", "g7"], every, ["g1"], every, ["g0", "g1"], ["g9", "g1", "g0", "g12"]]
+    counts = {}
+    for step in decode:
+        if isinstance(step, list):
+            for tag in step:
+                counts[tag] = counts.get(tag, 0) + 1
+    prompt_len = {tag: 6 + (11 * i) % 17 for i, tag in enumerate(tags)}
+    prompt_len["g0"] = 1030
+    prompt_len["n0"] = 21
+    reqs = {}
+    for i, tag in enumerate(tags + ["n0"]):
+        n_ids = prompt_len[tag] + (0 if tag in SAMPLED else counts[tag])
+        if tag == "g0":
+            reqs[tag] = Request(tag, helpers.random_ids(1500, n_ids - n_prefix, vocab), prefix)
+        else:
+            reqs[tag] = Request(tag, helpers.random_ids(1500 + i, n_ids, vocab))
+    prompts = [[("g0", prompt_len["g0"])], [(tag, prompt_len[tag]) for tag in tags[1:]]]
+    return reqs, prompt_len, prompts, decode
+
+
+def _step_graph_workload(runner, sampler, reqs, prompt_len, entries_of):
+    """One step: ``entries_of`` = [(tag, count)]. Only the last place of each entry is wanted; every row of
+    logits is sampled greedily into the device table of pending tokens (as the scheduler does), and the
+    requests in SAMPLED take their next token from there. Returns {tag: logits row}."""
+    from kestrel_amd.engine.step import PENDING_TOKEN, StepEntry
+
+    entries = []
+    for tag, count in entries_of:
+        req = reqs[tag]
+        if req.slot is None:
+            req.slot = runner.admit()
+        if tag in SAMPLED and req.done >= prompt_len[tag]:
+            assert count == 1 and req.done == len(req.ids) - 1
+            entries.append(StepEntry(req.slot, [PENDING_TOKEN], want=[0]))
+            req.done += 1
+        else:
+            tokens, embeds, bidir, _lo = req.take(count)
+            entries.append(StepEntry(req.slot, tokens, want=[len(tokens) - 1], embeds=embeds, bidirectional=bidir))
+    logits = runner.step(entries)
+    ids = sampler.greedy(logits, slots=runner.logit_slots).tolist()
+    rows = logits.clone()
+    out = {}
+    for row, (tag, _count) in enumerate(entries_of):
+        out[tag] = rows[row]
+        if tag in SAMPLED:
+            reqs[tag].ids.append(int(ids[row]))          # what the next step's PENDING_TOKEN stands for
+            reqs[tag].length += 1
+    return out
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+@pytest.mark.parametrize("sizes", ["moondream2", "phi2"])
+def test_replayed_decode_graphs_at_real_layer_sizes(sizes, dtype, monkeypatch):
+    """What serving runs when it decodes: graphs on, buckets of 1, 2, 4, 8 and 64 rows captured on padding rows
+    and replayed (with padding rows at 5 of 8), ids taken from the device table that sampling filled, a
+    slot and its pages taken over between replays, the head's launch that normalises the rows itself; at
+    Moondream 2's widths in bf16 the steps of 1, 2 and 4 rows run the feed-forward's first linear inside the
+    attention launch. Every row of logits against the plain implementation."""
+    from kestrel_amd.engine.loading import load_model, make_runner
+    from kestrel_amd.ops import fast
+    from kestrel_amd.sampling import Sampler
+
+    reqs, prompt_len, prompts, decode = _graph_workload(sizes)
+    net = load_model(_folder(sizes), dtype, torch.device("cuda:0"))
+    pages = sum(-(-(req.length + 12) // 16) for tag, req in reqs.items() if tag != "n0") + 1
+    runner = make_runner(net, 16, pages, N_GRAPH, max_tokens_per_step=2048, enable_graphs=True)
+    helpers.poison_cache(runner)
+    sampler = Sampler(net.device, pending=runner.pending)
+    launches = []
+    plain_decode = fast.attention_decode_bf16
+
+    def watched(*args, **kwargs):
+        done = plain_decode(*args, **kwargs)
+        if done:
+            launches.append((args[0].shape[0], kwargs.get("beside") is not None))
+        return done
+
+    monkeypatch.setattr(fast, "attention_decode_bf16", watched)
+    got = {tag: {} for tag in reqs}            # request -> {position: logits row}
+    n_replays = 0
+    for step in prompts:
+        for tag, row in _step_graph_workload(runner, sampler, reqs, prompt_len, step).items():
+            got[tag][reqs[tag].done - 1] = row
+    assert runner.graph_replays == 0
+    for step in decode:
+        if not isinstance(step, list):
+            gone = reqs["g4"]
+            assert gone.done == gone.length
+            slot = gone.slot
+            runner.release(slot)
+            gone.slot = None
+            for tag, row in _step_graph_workload(runner, sampler, reqs, prompt_len, [("n0", prompt_len["n0"])]).items():
+                got[tag][reqs[tag].done - 1] = row
+            assert reqs["n0"].slot == slot, "the request that joins takes the slot that was given back"
+            continue
+        for tag, row in _step_graph_workload(runner, sampler, reqs, prompt_len, [(tag, 1) for tag in step]).items():
+            got[tag][reqs[tag].done - 1] = row
+        n_replays += 1
+        runner.cache.check()
+    assert runner.graph_replays == n_replays
+    assert sorted(runner._graphs) == [1, 2, 4, 8, 64]
+    if dtype == torch.bfloat16:
+        rows_with_linear = {n for n, beside in launches if beside}
+        assert {n for n, _ in launches} >= {1, 2, 4, 8, 64}
+        # head size 64 and K = 2048: the attention of 1 to 4 rows takes the linear layer along; not so at head size 80
+        assert rows_with_linear == ({1, 2, 4} if sizes == "moondream2" else set()), rows_with_linear
+    cfg = SIZES[sizes]
+    weights = {k: v.double() for k, v in helpers.stored_weights(_folder(sizes)).items()}
+    for tag, req in reqs.items():
+        fed = req.done
+        expected = plain.forward(cfg, weights, req.ids[:fed - req.n_prefix], req.prefix).float()
+        places = sorted(got[tag])
+        assert places and places[-1] == fed - 1
+        actual = torch.stack([got[tag][p] for p in places])
+        helpers.assert_close(actual, expected[places], dtype, f"{sizes} sizes, graphs, request {tag}")

@@ -204,6 +204,42 @@ def test_a_bidirectional_block_goes_in_one_portion():
         sched.enqueue_request(GenerationRequest(2, [1], 1, prefix_embeds=torch.zeros(20, 8)))
 
 
+def test_several_blocks_in_one_request_are_each_kept_whole():
+    """A prompt with two blocks of given embeddings between text: ids with -1 where rows of ``prompt_embeds``
+    stand, ``blocks`` naming the ranges. Portions are cut so that no block is split: a portion that would end
+    inside a block ends at the block's start, whatever the page boundary says."""
+    ids = [1, 2, 3] + [-1] * 6 + [4, 5, 6, 7, 8] + [-1] * 5 + [9, 10]           # blocks [3, 9) and [14, 19)
+    rows = torch.arange(11 * 8, dtype=torch.float32).reshape(11, 8)
+    sched, runner = _scheduler(budget=8, n_pages=32)
+    sched.enqueue_request(GenerationRequest(0, ids, 2, prompt_embeds=rows, blocks=[(14, 19), (3, 9)]))
+    seen = []
+    step_entry = runner.step
+
+    def watching(entries):
+        seen.extend((e.start, len(e.tokens), list(e.bidirectional), None if e.embeds is None else e.embeds.clone())
+                    for e in entries if len(e.tokens) > 1)
+        return step_entry(entries)
+
+    runner.step = watching
+    (result,) = sched.run_until_done()
+    assert result.finish_reason == "length" and len(result.tokens) == 2
+    # budget 8, pages of 4: [0, 8) would split the first block -> [0, 3); [3, 11) is not cut back to the page
+    # boundary at 8, which lies inside the block; [11, 19) ends with the second block; the rest follows
+    assert [(start, n) for start, n, _b, _e in seen] == [(0, 3), (3, 8), (11, 8), (19, 2)]
+    assert [b for _s, _n, b, _e in seen] == [[], [(3, 9)], [(14, 19)], []]
+    assert torch.equal(seen[1][3], rows[:6]) and torch.equal(seen[2][3], rows[6:])
+    assert seen[0][3] is None and seen[3][3] is None
+    for bad, message in ((dict(blocks=[(3, 9), (8, 12)]), "not overlap"), (dict(blocks=[(20, 30)]), "inside the prompt"),
+                         (dict(blocks=[(4, 4)]), "at least one position"),
+                         (dict(prompt_embeds=rows[:10]), "10 rows for 11 places")):
+        options = dict(prompt_embeds=rows, blocks=[(3, 9)])
+        options.update(bad)
+        with pytest.raises(ValueError, match=message):
+            sched.enqueue_request(GenerationRequest(1, ids, 2, **options))
+    with pytest.raises(ValueError, match="does not fit in one step"):
+        sched.enqueue_request(GenerationRequest(2, ids, 2, prompt_embeds=rows, blocks=[(0, 12)]))
+
+
 def test_bad_requests_are_refused():
     sched, _ = _scheduler()
     for bad in (dict(max_new_tokens=0), dict(temperature=-1.0), dict(top_p=0.0), dict(top_p=1.5)):
@@ -309,11 +345,11 @@ def test_a_generated_prefix_is_fed_counted_and_returned():
 def test_a_generated_prefix_is_checked():
     from kestrel_amd.engine.types import GeneratedPrefix
 
-    with pytest.raises(ValueError, match="shorter"):
+    with pytest.raises(ValueError, match="leaves nothing to generate"):
         GenerationRequest(7, [1], 2, generated_prefix=GeneratedPrefix((10, 11)))
-    with pytest.raises(ValueError, match="same length"):
+    with pytest.raises(ValueError, match="one per token"):
         GenerationRequest(7, [1], 4, generated_prefix=GeneratedPrefix((10,), ()))
-    with pytest.raises(ValueError, match="return_logprobs"):
+    with pytest.raises(ValueError, match="must bring those of the tokens"):
         GenerationRequest(7, [1], 4, return_logprobs=True, generated_prefix=GeneratedPrefix((10,)))
     sched, _ = _scheduler()
     with pytest.raises(ValueError, match="generated_prefix.tokens: token id 70"):
