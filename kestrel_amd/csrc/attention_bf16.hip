@@ -430,16 +430,20 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_
 // (four waves per SIMD are all that a workgroup of 16 waves allows, two with the registers that
 // head size 128 needs; saying so keeps the compiler from trading loads in flight for an
 // occupancy the kernel cannot have. Workgroups of four waves, which many rows get, fit five to a
-// CU: 15.7k to 16.1k tok/s at batch 64; six spill registers and lose that again)
-template <int HD, int WAVES>
-__global__ void __launch_bounds__(KA_WAVE * WAVES) __attribute__((amdgpu_waves_per_eu(HD <= 64 ? (WAVES == 4 ? 5 : 4) : 2, HD <= 64 ? (WAVES == 4 ? 5 : 4) : 2)))
+// CU with tiles of 64 keys: 15.7k to 16.1k tok/s at batch 64; six spill registers and lose that again)
+constexpr int ad_waves_per_simd(int HD, int WAVES, int TP) { return HD > 64 ? 2 : (WAVES == 4 && TP <= 4 ? 5 : 4); }
+
+template <int HD, int WAVES, int TP>
+__global__ void __launch_bounds__(KA_WAVE * WAVES)
+    __attribute__((amdgpu_waves_per_eu(ad_waves_per_simd(HD, WAVES, TP), ad_waves_per_simd(HD, WAVES, TP))))
 attn_decode_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t* __restrict__ k_cache,
                    const bf16_t* __restrict__ v_cache, const int* __restrict__ block_table, int max_pages,
                    const int* __restrict__ token_row, const int* __restrict__ kv_lo,
                    const int* __restrict__ kv_hi, bf16_t* __restrict__ out, long out_row_stride, float scale,
                    int H, int Hkv, float* __restrict__ partial, DecodeFuse fz) {
-    attn_decode_body<HD, WAVES>(q, q_row_stride, k_cache, v_cache, block_table, max_pages, token_row, kv_lo, kv_hi, out,
-                                out_row_stride, scale, H, Hkv, partial, fz, blockIdx.x, blockIdx.y, blockIdx.z, gridDim.z);
+    attn_decode_body<HD, WAVES, false, TP>(q, q_row_stride, k_cache, v_cache, block_table, max_pages, token_row, kv_lo, kv_hi,
+                                           out, out_row_stride, scale, H, Hkv, partial, fz, blockIdx.x, blockIdx.y, blockIdx.z,
+                                           gridDim.z);
 }
 
 // ----------------------------------------------------------------------------------------------
@@ -722,17 +726,17 @@ static int decode_launch(const char* who, const void* q, long q_row_stride, cons
     KA_CHECK(waves == 4 || waves == 8 || waves == 16, "%s: waves must be 4, 8 or 16", who);
     if (hd > 64 && waves == 16) waves = 8;   // 16 waves leave 128 registers a lane: too few for a tile's loads (measured at head size 80: 26.4 against 23.6 us)
     dim3 grid(n, H, splits), block(KA_WAVE * waves);
-#define KA_AD(HDV, WV)                                                                                              \
-    hipLaunchKernelGGL((attn_decode_kernel<HDV, WV>), grid, block, 0, stream, (const bf16_t*)q, q_row_stride,      \
+#define KA_AD(HDV, WV, TPV)                                                                                         \
+    hipLaunchKernelGGL((attn_decode_kernel<HDV, WV, TPV>), grid, block, 0, stream, (const bf16_t*)q, q_row_stride, \
                        (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, max_pages, token_row, kv_lo,   \
                        kv_hi, (bf16_t*)out, out_row_stride, scale, H, Hkv, partial, fz)
 #define KA_AD_SMALL(HDV)                                                                                            \
     case HDV:                                                                                                       \
-        if (waves == 4) KA_AD(HDV, 4); else if (waves == 8) KA_AD(HDV, 8); else KA_AD(HDV, 16);                     \
+        if (waves == 4) KA_AD(HDV, 4, 4); else if (waves == 8) KA_AD(HDV, 8, 4); else KA_AD(HDV, 16, 4);            \
         break
 #define KA_AD_LARGE(HDV)                                                                                            \
     case HDV:                                                                                                       \
-        if (waves == 4) KA_AD(HDV, 4); else KA_AD(HDV, 8);                                                          \
+        if (waves == 4) KA_AD(HDV, 4, 4); else KA_AD(HDV, 8, 4);                                                    \
         break
     switch (hd) {
         KA_AD_SMALL(16); KA_AD_SMALL(32); KA_AD_SMALL(48); KA_AD_SMALL(64);

@@ -25,7 +25,7 @@ __device__ __forceinline__ void at_wave_sync() {
 // ----------------------------------------------------------------------------------------------
 // decode kernel
 // ----------------------------------------------------------------------------------------------
-constexpr int AD_TILE = 64;               // keys per wave tile
+constexpr int AD_TILE_PAGES = 4;          // pages of a wave's tile unless a kernel says otherwise (64 keys)
 constexpr int ad_lanes_per_key(int hd) { int l = 1; while (l * 8 < hd) l *= 2; return l; }
 
 // What the decode kernel needs to take over the rotary encoding and the cache write of the
@@ -91,12 +91,32 @@ __device__ __forceinline__ void at_rotated(const RotaryOperands& r, const Rotary
     }
 }
 
-// AHEAD: the keys of a wave's next tile are asked for before its current tile is worked on (32
-// registers more at head size 64): one trip to memory less per tile where a wave has more than one
-// tile and the kernel is a chain of trips (few rows), no gain where it streams (many rows).
+// How a row's keys are dealt out, page by page from the page that holds `lo` (keys below `lo` in it
+// are masked). The units are the parts of the row x the waves of a workgroup; a unit walks over
+// its keys in rounds of one tile (at most TP pages) each.
+// EVEN (workgroups of four waves: many rows, the launch streams keys and values): the pages are cut
+// evenly over the units, every unit gets a run of neighbouring pages, the first `rem` units one page
+// more than the others, and walks over its run in rounds of equal size: the waves of a workgroup
+// end together, whatever the number of pages.
+// Otherwise (eight or sixteen waves: few rows, a chain of trips to memory in which a round costs the
+// same whether its tile is full or not): whole tiles are dealt out in turn, unit u takes tiles u,
+// u + units, ..., so that no round is spent on a tile that is partly empty except the row's last (cut
+// evenly, 80 pages over sixteen waves are two rounds of 3 + 2 pages for every wave instead of a
+// second round for four of them: 21.8 against 20.9 us a launch at 8 rows of 1,280 keys).
+// Measured at 32 heads of 64, 8 and 64 rows, 1,024 to 1,280 keys: either way of dealing is within
+// 1 us (the run-to-run spread) of the other at tiles of 4 pages; tiles of 6 and 8 pages, which hold
+// a wave's pages in one round, are no faster at 1,040 to 1,280 keys and 1 us slower at 1,024 with
+// the arithmetic of a tile's empty part jumped over, 4 us slower with it masked; and the loads of
+// the empty part cannot be jumped over: under a condition they make the compiler wait for every
+// load in flight (137 against 105 us a launch at 64 rows). At 64 rows the launch reads at 5.0 TB/s,
+// what a copy of scattered 2 KB pieces reaches; a 17th page costs a wave a round of its own.
+//
+// AHEAD: the keys of a wave's next tile are asked for before its current tile is worked on (as
+// many registers more as a tile's keys take): one trip to memory less per tile where a wave has more
+// than one tile and the kernel is a chain of trips (few rows), no gain where it streams (many rows).
 // (A tile's values asked for together with its keys instead: slower, 11.8 against 11.2 us for the
 // attention of one row with eight waves.)
-template <int HD, int WAVES, bool AHEAD = false>
+template <int HD, int WAVES, bool AHEAD = false, int TP = AD_TILE_PAGES>
 __device__ __forceinline__ void
 attn_decode_body(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t* __restrict__ k_cache,
                  const bf16_t* __restrict__ v_cache, const int* __restrict__ block_table, int max_pages,
@@ -108,31 +128,50 @@ attn_decode_body(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t* 
     constexpr int CPK = HD / 8;            // 16-byte chunks of a key row
     constexpr int LPK = ad_lanes_per_key(HD);   // lanes per key row: the chunks, rounded up to a power of two
     constexpr int KPI = KA_WAVE / LPK;     // keys per load instruction
-    constexpr int KL = AD_TILE / KPI;      // key loads per lane and tile
+    constexpr int TILE = TP * AT_PAGE;     // keys of a full tile
+    static_assert(TILE % KPI == 0, "a tile is a whole number of key loads");
+    constexpr int KL = TILE / KPI;         // key loads per lane and tile
     constexpr int VU = (HD + 31) / 32;     // 16-byte value loads per lane and page (a lane takes channel u * 32 + lane / 2)
     // Where the head size is no power of two, the lanes past a key row's chunks, and past the
     // channels of a value page, ask for what another lane asks for and add nothing.
-    constexpr int TP = AD_TILE / AT_PAGE;  // pages of a tile
     constexpr int REC = HD + 2;            // floats of a partial result: m, l, o[HD]
-    __shared__ float ps[WAVES][AD_TILE];
+    __shared__ float ps[WAVES][TILE];
     __shared__ float merge[WAVES][REC];
     __shared__ int pages[AT_LDS_PAGES];
-    const int wave = threadIdx.x / KA_WAVE, lane = threadIdx.x % KA_WAVE;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / KA_WAVE), lane = threadIdx.x % KA_WAVE;
     const int kvh = h / (H / Hkv);
     const int row = token_row[t];
     const int lo = kv_lo ? kv_lo[t] : 0;
     const bool fused = fz.slots != nullptr && kv_hi[t] > 0;
     const int pos = kv_hi[t] - 1;                 // fused: the token's own position, whose key is not cached yet
     const int hi = fused ? pos : kv_hi[t];        // cached keys this token reads: [lo, hi)
-    const int lo_tile = lo & ~(AD_TILE - 1);      // tiles start on page boundaries; keys below lo are masked
-    const int chunk = ((hi - lo_tile + S - 1) / S + AD_TILE - 1) / AD_TILE * AD_TILE;
-    const int s_lo = lo_tile + split * chunk, s_hi = min(hi, s_lo + chunk);
+    // this unit's rounds: round r holds the keys [tile0, tile_hi) of round_keys(r) (a row without keys,
+    // hi <= lo, has no pages and no rounds: nothing of the cache is touched)
+    constexpr bool EVEN = WAVES == 4;
+    const int first_page = lo / AT_PAGE;
+    const int n_pages_live = hi > lo ? (hi - 1) / AT_PAGE - first_page + 1 : 0;
+    const int unit = split * WAVES + wave, units = S * WAVES;
+    int rounds, per, mine0, mine_hi;
+    if constexpr (EVEN) {
+        const int base = n_pages_live / units, rem = n_pages_live % units;
+        const int own = base + (unit < rem ? 1 : 0);
+        mine0 = first_page + unit * base + min(unit, rem);
+        rounds = (own + TP - 1) / TP;
+        per = rounds > 0 ? (own + rounds - 1) / rounds : 0;
+        mine_hi = min(hi, (mine0 + own) * AT_PAGE);       // keys of this unit end here
+    } else {
+        const int tiles = (n_pages_live + TP - 1) / TP;
+        rounds = tiles > unit ? (tiles - unit + units - 1) / units : 0;
+        per = TP;
+        mine0 = first_page + unit * TP;
+        mine_hi = hi;
+    }
     const int ks = lane / LPK, dg_lane = lane % LPK;
     const bool chunk_live = dg_lane < CPK;             // this lane holds a chunk of the key row
     const int dg = chunk_live ? dg_lane : 0;
     const float sl2 = scale * AT_LOG2E;
-    // this wave adds the token's own key and value: the last one, which has the fewest tiles where
-    // they do not divide over the waves
+    // this wave adds the token's own key and value: the last one, which is among those with the
+    // fewest keys where they do not divide over the waves
     const bool takes_new = fused && wave == WAVES - 1 && split == 0;
 
     // The operands of q (and, for the wave that takes them, of the token's own key and value) are
@@ -209,32 +248,54 @@ attn_decode_body(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t* 
         for (int u = 0; u < VU; ++u) acc[u] = (lane & 1) == 0 ? (float)vnew[u] : 0.f;
     }
 
-    // All key loads of a tile go out before any arithmetic, and none stands under a
-    // condition: a place outside [lo, s_hi) is moved to one inside and masked afterwards. The
-    // compiler can then wait for exactly the register it needs instead of for everything.
-    auto load_keys = [&](int tile0, bf16x8 (&dst)[KL]) {
+    // All key loads of a tile go out before any arithmetic, and none stands under a condition (a load
+    // under a branch makes the compiler wait for every load in flight: 137 against 105 us a launch at 64
+    // rows): a place outside the tile's keys [max(tile0, lo), tile_hi) is moved to one inside and masked
+    // afterwards (every page of a unit's run holds at least one key of [lo, hi), so there is one). A tile
+    // has room for TP pages and may hold fewer: what it does not hold is masked like any other place
+    // outside (jumping over its arithmetic, the same for all lanes, cuts the tile's straight run of
+    // instructions into pieces: 1,215 against 1,247 tok/s at one row).
+    auto load_keys = [&](int tile0, int tile_hi, bf16x8 (&dst)[KL]) {
 #pragma unroll
         for (int i = 0; i < KL; ++i) {
             int key = tile0 + i * KPI + ks;
-            int kc = max(min(key, s_hi - 1), lo);   // a place that holds data (pages below lo may be gone)
+            int kc = max(min(key, tile_hi - 1), lo);   // a place that holds data (pages below lo may be gone)
             int page = bt[kc / AT_PAGE];
             dst[i] = at_load8(k_cache + (((size_t)page * Hkv + kvh) * AT_PAGE + kc % AT_PAGE) * HD + dg * 8);
         }
     };
+    // round r of this unit: keys [tile0, tile_hi)
+    auto round_keys = [&](int r, int& tile0, int& tile_hi) {
+        const int page0 = mine0 + r * (EVEN ? per : units * TP);
+        tile0 = page0 * AT_PAGE;
+        tile_hi = min(mine_hi, (page0 + per) * AT_PAGE);
+    };
     bf16x8 kreg[KL], knext[AHEAD ? KL : 1];
     if constexpr (AHEAD) {
-        if (s_hi > lo) load_keys(s_lo + wave * AD_TILE, kreg);      // (a row without keys: nothing to clamp to)
+        if (rounds > 0) {
+            int t0, t1;
+            round_keys(0, t0, t1);
+            load_keys(t0, t1, kreg);
+        }
     }
-    for (int tile0 = s_lo + wave * AD_TILE; tile0 < s_hi; tile0 += WAVES * AD_TILE) {
-        if constexpr (AHEAD) load_keys(tile0 + WAVES * AD_TILE, knext);
-        else load_keys(tile0, kreg);
+    for (int r = 0; r < rounds; ++r) {
+        int tile0, tile_hi;
+        round_keys(r, tile0, tile_hi);
+        if constexpr (AHEAD) {
+            // (past the last round: the last round's keys once more, which nobody uses)
+            int n0, n1;
+            round_keys(min(r + 1, rounds - 1), n0, n1);
+            load_keys(n0, n1, knext);
+        } else {
+            load_keys(tile0, tile_hi, kreg);
+        }
         __builtin_amdgcn_sched_barrier(0);     // all of them, before the first is used
         float sc[KL];
         float mx = -INFINITY;
 #pragma unroll
         for (int i = 0; i < KL; ++i) {
             int key = tile0 + i * KPI + ks;
-            bool ok = key >= lo && key < s_hi;
+            bool ok = key >= lo && key < tile_hi;
             float dot = 0.f;
 #pragma unroll
             for (int j = 0; j < 8; ++j) dot = fmaf(qf[j], (float)kreg[i][j], dot);
@@ -243,20 +304,13 @@ attn_decode_body(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t* 
             mx = fmaxf(mx, sc[i]);
         }
         mx = ka_lanes_reduce<LPK, KA_WAVE>(mx, KaMax{});            // (the lanes of a key hold one value)
-        float m_new = fmaxf(m_i, mx);
-        if (m_new == -INFINITY) {              // a tile wholly below lo (wave-uniform)
-            if constexpr (AHEAD) {
-#pragma unroll
-                for (int i = 0; i < KL; ++i) kreg[i] = knext[i];
-            }
-            continue;
-        }
-        // the values: asked for as soon as the keys' registers are free, all at once and, like
-        // the keys, without a condition; the softmax below runs while they are on their way
+        float m_new = fmaxf(m_i, mx);                               // finite: the tile holds a key of [lo, hi)
+        // the values: asked for as soon as the keys' registers are free, all at once; the softmax
+        // below runs while they are on their way
         bf16x8 vreg[TP][VU];
 #pragma unroll
         for (int pg = 0; pg < TP; ++pg) {
-            int kc = max(min(tile0 + pg * AT_PAGE, s_hi - 1), lo);
+            int kc = max(min(tile0 + pg * AT_PAGE, tile_hi - 1), lo);
             int page = bt[kc / AT_PAGE];
 #pragma unroll
             for (int u = 0; u < VU; ++u) {
@@ -294,7 +348,7 @@ attn_decode_body(const bf16_t* __restrict__ q, long q_row_stride, const bf16_t* 
 #pragma unroll
                 for (int j = 0; j < 8; ++j) {
                     int key = first + j;                      // slots outside the data may hold anything
-                    float x = key >= lo && key < s_hi ? (float)vreg[pg][u][j] : 0.f;
+                    float x = key >= lo && key < tile_hi ? (float)vreg[pg][u][j] : 0.f;
                     sum = fmaf(pv[j], x, sum);
                 }
                 acc[u] += sum;

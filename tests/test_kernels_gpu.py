@@ -569,6 +569,59 @@ def test_attention_decode_kernel(shape):
     _close(_run_attention(windowed, "fast", 0.25), windowed.reference(0.25), bf)
 
 
+@pytest.mark.parametrize("waves", [4, 8, 16])
+@pytest.mark.parametrize("shape", [(4, 4, 64), (2, 1, 16), (6, 3, 48), (4, 2, 32), (2, 2, 80), (2, 1, 128)])
+def test_decode_attention_deals_out_every_page_once(shape, waves, monkeypatch):
+    """A row's pages are cut evenly over the four waves of a workgroup, or dealt out tile by tile to eight or
+    sixteen: every number of pages from none to more than waves x tile, contexts that end on a page's first
+    and last slot, a window whose start lies inside a page, at every wave count."""
+    from kestrel_amd.ops import fast
+
+    h, hkv, hd = shape
+    bf = torch.bfloat16
+    shape_of = fast.decode_shape
+    monkeypatch.setattr(fast, "decode_shape", lambda max_kv, workgroups=1: (shape_of(max_kv, workgroups)[0], waves))
+    for kv_lens in ([1, 15, 16, 17, 63, 64, 65, 81], [1040, 1041, 1279, 600, 2047, 1, 255, 513]):
+        case = PagedCase(kv_lens, [1] * len(kv_lens), h, hkv, hd, 16, bf, seed=31 + len(kv_lens))
+        _close(_run_attention(case, "fast", hd ** -0.5), case.reference(hd ** -0.5), bf)
+    for window in (1, 2, 16, 17, 33, 250):
+        windowed = PagedCase([300, 20, 129, 1041, 17, 16], [1] * 6, h, hkv, hd, 16, bf, seed=32, window=window)
+        _close(_run_attention(windowed, "fast", 0.25), windowed.reference(0.25), bf)
+
+
+def test_fused_decode_attention_with_a_window_of_one():
+    """A window of one position: the token reads no cached key at all, only its own, at positions on a
+    page's first slot (16, 32, 48: where the row's block table in LDS ends just before the token's page) and
+    elsewhere. The output is the token's own value, and nothing outside its slot of the cache is written."""
+    from kestrel_amd.ops import fast
+
+    h, hkv, hd, rot = 4, 2, 64, 32
+    bf = torch.bfloat16
+    kv_lens = [17, 33, 49, 18, 1, 64, 65]             # the token stands at kv - 1
+    case = PagedCase(kv_lens, [1] * len(kv_lens), h, hkv, hd, 16, bf, seed=33, window=1)
+    n = len(kv_lens)
+    torch.manual_seed(34)
+    qkv = torch.randn(n, (h + 2 * hkv) * hd).to(bf).to(DEV)
+    slots = torch.tensor([int(case.table[r, (kv - 1) // 16]) * 16 + (kv - 1) % 16 for r, kv in enumerate(kv_lens)],
+                         dtype=torch.int32, device=DEV)
+    table = plain.rotary_table(rot, 128, 10000.0, torch.float32).to(DEV)
+    k_f, v_f = case.k_cache.clone(), case.v_cache.clone()
+    out = torch.empty(n, h * hd, dtype=bf, device=DEV)
+    q_dim, kv_dim = h * hd, hkv * hd
+    for waves in (4, 16):
+        shape_of = fast.decode_shape
+        fast.decode_shape = lambda max_kv, workgroups=1, w=waves: (shape_of(max_kv, workgroups)[0], w)
+        try:
+            assert fast.attention_decode_bf16(qkv, k_f, v_f, case.table, case.token_row, case.kv_lo, case.kv_hi, out,
+                                              hd ** -0.5, h, hkv, hd, case.batch,
+                                              fuse=(qkv[:, q_dim:q_dim + kv_dim], qkv[:, q_dim + kv_dim:], table, slots))
+        finally:
+            fast.decode_shape = shape_of
+        v_new = qkv[:, q_dim + kv_dim:].view(n, hkv, hd)
+        expected = v_new.repeat_interleave(h // hkv, dim=1).reshape(n, h * hd)
+        assert torch.equal(out, expected)
+
+
 EDGE_HEADS = [(4, 4, 64), (4, 2, 80), (2, 1, 128), (6, 3, 48), (4, 1, 16), (2, 2, 96), (2, 2, 256)]
 
 
