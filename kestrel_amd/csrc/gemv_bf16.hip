@@ -107,18 +107,27 @@ skinny_split_kernel(SkinnyArgs p) {
         arow1[mb] = p.A[1] + (size_t)m * p.lda[1];
     }
 
+    // (a round's weights are all asked for before its activations: the weights come from HBM, the
+    // activations, which every workgroup reads, from L2)
     auto issue = [&](int slot, int round) {
 #pragma unroll
         for (int u = 0; u < UN; ++u) {
             // a block past the end reads the last one again and multiplies it with zeros
+            const int bc = min(wave + (round * UN + u) * WAVES, nb - 1);
+            const bool seg = bc >= nb1;
+            const int Ks = seg ? K1 : K0;
+            const int k = (seg ? bc - nb1 : bc) * SK_KBLOCK;
+            const bf16_t* wp = seg ? wrow1 : wrow0;
+            w[slot][u] = sk_load8_stream(wp + min(k + koff, Ks - 8));
+        }
+#pragma unroll
+        for (int u = 0; u < UN; ++u) {
             const int b = wave + (round * UN + u) * WAVES;
             const bool live = b < nb;
             const int bc = min(b, nb - 1);
             const bool seg = bc >= nb1;
             const int Ks = seg ? K1 : K0;
             const int k = (seg ? bc - nb1 : bc) * SK_KBLOCK;
-            const bf16_t* wp = seg ? wrow1 : wrow0;
-            w[slot][u] = sk_load8_stream(wp + min(k + koff, Ks - 8));
 #pragma unroll
             for (int mb = 0; mb < MB; ++mb) {
                 const bf16_t* ap = seg ? arow1[mb] : arow0[mb];

@@ -104,6 +104,40 @@ def test_decode_attention_that_allocates_nothing():
         torch.testing.assert_close(got.cpu().double(), case.reference(), atol=2e-2, rtol=2e-2)
 
 
+def test_it_allocates_nothing_and_runs_under_graph_capture():
+    """What gives the entry point its name: after a first call (which looks up the array's address on this
+    device) a call leaves the device's free memory as it was, and it can be recorded into a HIP graph (an
+    allocation inside a capture fails the capture). The graph is replayed several times with eager work of
+    the program's own between the replays, and every replay gives the eager call's bits."""
+    lib, no_alloc, _ = _library()
+    case = _Case([1500, 700, 33, 1024], 8, 2, 64, seed=44)
+    splits, waves = 4, 4
+    eager = torch.full((case.n, case.h * case.hd), float("nan"), dtype=torch.bfloat16, device=DEV)
+    tail = [None, None, 0, None, 0, None, None, None]
+    assert no_alloc(*case.common(eager, splits, waves), *tail, None) == 0, lib.ka_last_error().decode()
+    again = torch.full_like(eager, float("nan"))
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]
+    assert no_alloc(*case.common(again, splits, waves), *tail, None) == 0, lib.ka_last_error().decode()
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free_before, "the call changed the device's free memory"
+    assert torch.equal(again, eager)
+    replayed = torch.full_like(eager, float("nan"))
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        status = no_alloc(*case.common(replayed, splits, waves), *tail, ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    assert status == 0, lib.ka_last_error().decode()
+    other = _Case([90, 400], 4, 4, 64, seed=45)                 # eager work on the same static array between the replays
+    scratch_user = torch.empty(other.n, other.h * other.hd, dtype=torch.bfloat16, device=DEV)
+    for _ in range(3):
+        replayed.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(replayed, eager)
+        assert no_alloc(*other.common(scratch_user, splits, waves), *tail, None) == 0
+        torch.cuda.synchronize()
+
+
 def test_a_batch_beyond_the_static_array_is_refused():
     lib, no_alloc, _ = _library()
     case = _Case([40, 50], 4, 4, 64, seed=43)
