@@ -134,6 +134,12 @@ gemm_bf16_kernel(const bf16_t* __restrict__ A, long lda, const bf16_t* __restric
                 int n = n0 + wn * 32 * NT + a * 32 + q * 8 + lg * 4;
                 if (n >= N) continue;
                 float v[4];
+                if (ka_act_gated(act)) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) v[i] = acc[a][b][q * 4 + i] + (bias && n + i < N ? bias[n + i] : 0.f);
+                    ka_gated_store<true, 4>(out, out_dtype, ldo, m, n, N, v, act);
+                    continue;
+                }
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     float x = acc[a][b][q * 4 + i];
@@ -545,13 +551,20 @@ KA_API int ka_linear_tiled_bf16(const void* A, long lda, const void* W, long ldw
     KA_CHECK(M > 0 && N > 0 && K > 0 && K % 8 == 0, "ka_linear_tiled_bf16: M=%d N=%d K=%d (K must be a multiple of 8)", M, N, K);
     KA_CHECK(lda % 8 == 0 && ldw % 8 == 0 && lda >= K && ldw >= K, "ka_linear_tiled_bf16: row strides must be multiples of 8 and >= K");
     KA_CHECK(((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0), "ka_linear_tiled_bf16: operands must be 16-byte aligned");
-    KA_CHECK(ldo >= N, "ka_linear_tiled_bf16: output stride too small");
     KA_CHECK(ka_act_known(act), "ka_linear_tiled_bf16: unknown activation %d", act);
+    KA_CHECK(ldo >= ka_act_outputs(act, N), "ka_linear_tiled_bf16: output stride too small");
+    KA_CHECK(!ka_act_gated(act) || (N % 2 == 0 && !accumulate), "ka_linear_tiled_bf16: a gated linear needs an even N and no accumulation");
     KA_CHECK(out_dtype == KA_F32 || out_dtype == KA_BF16, "ka_linear_tiled_bf16: bad output type");
     KA_CHECK(!(accumulate && out_dtype != KA_F32), "ka_linear_tiled_bf16: accumulate needs an fp32 output");
     KA_CHECK((uintptr_t)out % 16 == 0, "ka_linear_tiled_bf16: output must be 16-byte aligned");
     int parts = config >= 1000000 ? config / 1000000 : 0;      // 0: chosen below
     config %= 1000000;
+    if (ka_act_gated(act) && config != 211 && config != 221) {
+        // the pairs of a gated linear meet in the epilogue of the tiles that are staged through registers (the
+        // large tiles write their outputs as whole rows through LDS, laid out for N columns)
+        config = (long)ka_cdiv(N, 128) * ka_cdiv(M, 128) >= 512 ? 221 : 211;
+        parts = 0;
+    }
     if (config == 0) {
         if (K % 64 == 0) {
             // Tiles of 128 x 128 read 64 flops' worth of operands per byte from L2, which is what

@@ -48,6 +48,13 @@ gemm_generic_kernel(const TA* __restrict__ A, long lda, const TW* __restrict__ W
     for (int i = 0; i < 4; ++i) {
         int m = m0 + ty * 4 + i;
         if (m >= M) continue;
+        if (ka_act_gated(act)) {           // pairs of neighbouring columns make one output
+            float v[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) v[j] = acc[i][j] + (bias && n0 + tx * 4 + j < N ? bias[n0 + tx * 4 + j] : 0.f);
+            ka_gated_store<false, 4>(out, sizeof(TOut) == 4 ? KA_F32 : KA_BF16, ldo, m, n0 + tx * 4, N, v, act);
+            continue;
+        }
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             int n = n0 + tx * 4 + j;
@@ -130,6 +137,13 @@ gemm_f32_kernel(const float* __restrict__ A, long lda, const float* __restrict__
     for (int i = 0; i < RM; ++i) {
         const int m = m0 + ty * RM + i;
         if (m >= M) continue;
+        if (ka_act_gated(act)) {
+            float v[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) v[j] = acc[i][j] + (bias && n0 + tx * 8 + j < N ? bias[n0 + tx * 8 + j] : 0.f);
+            ka_gated_store<false, 8>(out, KA_F32, ldo, m, n0 + tx * 8, N, v, act);
+            continue;
+        }
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
             const int n = n0 + tx * 8 + j;
@@ -201,8 +215,9 @@ KA_API int ka_linear_generic(const void* A, int a_dtype, long lda, const void* W
                              long ldw, const float* bias, void* out, int out_dtype, long ldo,
                              int M, int N, int K, int act, int accumulate, hipStream_t stream) {
     KA_CHECK(M >= 0 && N > 0 && K > 0, "ka_linear_generic: bad sizes M=%d N=%d K=%d", M, N, K);
-    KA_CHECK(lda >= K && ldw >= K && ldo >= N, "ka_linear_generic: strides too small");
     KA_CHECK(ka_act_known(act), "ka_linear_generic: unknown activation %d", act);
+    KA_CHECK(lda >= K && ldw >= K && ldo >= ka_act_outputs(act, N), "ka_linear_generic: strides too small");
+    KA_CHECK(!ka_act_gated(act) || (N % 2 == 0 && !accumulate), "ka_linear_generic: a gated linear needs an even N and no accumulation");
     KA_CHECK(!(accumulate && out_dtype != KA_F32), "ka_linear_generic: accumulate needs an fp32 output");
     KA_CHECK(ka_cdiv(M, GT) <= 65535, "ka_linear_generic: M=%d too large for one launch", M);
     if (M == 0) return 0;
@@ -219,7 +234,7 @@ KA_API int ka_linear_generic(const void* A, int a_dtype, long lda, const void* W
         KA_LAUNCH_CHECK();
         return 0;
     }
-    if (vectors && M <= GV_ROWS) {
+    if (vectors && M <= GV_ROWS && !ka_act_gated(act)) {      // (a wave per column there: the pair of a gate would meet nowhere)
         hipLaunchKernelGGL(gemv_f32_kernel, dim3(ka_cdiv(N, GV_WAVES)), dim3(GV_WAVES * KA_WAVE), 0, stream,
                            (const float*)A, lda, (const float*)W, ldw, bias, (float*)out, ldo, M, N, K, act, accumulate);
         KA_LAUNCH_CHECK();

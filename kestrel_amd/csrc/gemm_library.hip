@@ -166,13 +166,14 @@ KA_API int ka_linear_library_bf16(const void* A, long lda, const void* W, long l
                                   void* workspace, long workspace_bytes, hipStream_t stream) {
     const char* who = "ka_linear_library_bf16";
     KA_CHECK(M > 0 && N > 0 && K > 0, "%s: M=%d N=%d K=%d", who, M, N, K);
-    KA_CHECK(lda >= K && ldw >= K && ldo >= N, "%s: a row stride is smaller than its row", who);
+    KA_CHECK(lda >= K && ldw >= K && ldo >= ka_act_outputs(act, N), "%s: a row stride is smaller than its row", who);
     KA_CHECK((uintptr_t)A % 16 == 0 && (uintptr_t)W % 16 == 0 && (uintptr_t)out % 16 == 0, "%s: operands must be 16-byte aligned", who);
     KA_CHECK(ka_act_known(act), "%s: unknown activation %d", who, act);
     KA_CHECK(out_dtype == KA_F32 || out_dtype == KA_BF16, "%s: bad output type", who);
     KA_CHECK(!(accumulate && out_dtype != KA_F32), "%s: accumulate needs an fp32 output", who);
     KA_CHECK(workspace_bytes >= 0 && (workspace || workspace_bytes == 0), "%s: workspace missing", who);
     if (accumulate && act != KA_ACT_NONE) return 1;
+    if (ka_act_gated(act)) return 1;              // (the library has no epilogue that multiplies neighbouring columns)
     int device = -1;
     hipError_t e = hipGetDevice(&device);
     KA_CHECK(e == hipSuccess && device >= 0 && device < LT_MAX_DEVICES, "%s: no current device within the %d this library keeps a handle for", who, LT_MAX_DEVICES);

@@ -154,11 +154,23 @@ __device__ __forceinline__ float ka_gelu_tanh_fast(float x) {
 // the table of the Python face (ops/linear.py).
 enum KaAct : int { KA_ACT_NONE = 0, KA_ACT_GELU_TANH = 1, KA_ACT_RELU = 2, KA_ACT_SILU = 3, KA_ACT_COUNT = 4 };
 
-static inline bool ka_act_known(int act) { return act >= 0 && act < KA_ACT_COUNT; }
+// A gated linear layer (the first half of a feed-forward of the form act(x Wg^T) * (x Wu^T)): KA_ACT_GATED
+// added to an activation's code says that the rows of the weights come in pairs, row 2j the gate's and
+// row 2j + 1 the value's of output j (biases likewise), and that the epilogue writes
+// out[m][j] = act(sum 2j) * (sum 2j + 1): N / 2 outputs from N weight rows, in the same pass. Every
+// epilogue of this folder holds neighbouring columns in one thread, so the pair meets in registers
+// (ka_gated_store below). Not together with accumulation into the output.
+constexpr int KA_ACT_GATED = 0x100;
+
+__host__ __device__ __forceinline__ bool ka_act_gated(int act) { return (act & KA_ACT_GATED) != 0; }
+__host__ __device__ __forceinline__ int ka_act_base(int act) { return act & ~KA_ACT_GATED; }
+static inline bool ka_act_known(int act) { return ka_act_base(act) >= 0 && ka_act_base(act) < KA_ACT_COUNT; }
+// Columns of the output of a linear layer of N weight rows.
+static inline int ka_act_outputs(int act, int N) { return ka_act_gated(act) ? N / 2 : N; }
 
 // Library-exact forms: the 32-bit path.
 __device__ __forceinline__ float ka_activate(int act, float x) {
-    switch (act) {
+    switch (ka_act_base(act)) {
         case KA_ACT_GELU_TANH: return ka_gelu_tanh(x);
         case KA_ACT_RELU: return fmaxf(x, 0.f);
         case KA_ACT_SILU: return x / (1.0f + expf(-x));
@@ -168,11 +180,28 @@ __device__ __forceinline__ float ka_activate(int act, float x) {
 
 // On the hardware's exponential and reciprocal: the kernels that write bf16 activations.
 __device__ __forceinline__ float ka_activate_fast(int act, float x) {
-    switch (act) {
+    switch (ka_act_base(act)) {
         case KA_ACT_GELU_TANH: return ka_gelu_tanh_fast(x);
         case KA_ACT_RELU: return fmaxf(x, 0.f);
         case KA_ACT_SILU: return x * __fdividef(1.0f, 1.0f + __expf(-x));
         default: return x;
+    }
+}
+
+// The epilogue of a gated linear layer for the sums (biases added) of the weight rows n .. n + COUNT - 1 of
+// output row m, n even: out[m][(n + 2p) / 2] = act(v[2p]) * v[2p + 1] for every pair inside N. FAST: the
+// activations on the hardware's exponential (the kernels that write bf16), else the library's.
+template <bool FAST, int COUNT>
+__device__ __forceinline__ void ka_gated_store(void* out, int out_dtype, long ldo, int m, int n, int N, const float* v, int act) {
+    static_assert(COUNT % 2 == 0, "pairs");
+#pragma unroll
+    for (int p = 0; p < COUNT / 2; ++p) {
+        if (n + 2 * p + 1 >= N) continue;
+        const float g = FAST ? ka_activate_fast(act, v[2 * p]) : ka_activate(act, v[2 * p]);
+        const float y = g * v[2 * p + 1];
+        const size_t o = (size_t)m * ldo + (n + 2 * p) / 2;
+        if (out_dtype == KA_F32) reinterpret_cast<float*>(out)[o] = y;
+        else reinterpret_cast<bf16_t*>(out)[o] = (bf16_t)y;
     }
 }
 

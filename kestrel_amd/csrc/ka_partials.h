@@ -41,6 +41,12 @@ ka_partials_finish_kernel(const float* __restrict__ partial, int splits, const f
             for (int i = 0; i < 4 && n + i < N; ++i) s[i] += src[i];
         }
     }
+    if (ka_act_gated(act)) {
+        float v[4];
+        for (int i = 0; i < 4; ++i) v[i] = n + i < N ? s[i] + (bias ? bias[n + i] : 0.f) + (bias2 ? bias2[n + i] : 0.f) : 0.f;
+        ka_gated_store<true, 4>(out, out_dtype, ldo, m, n, N, v, act);
+        return;
+    }
     for (int i = 0; i < 4 && n + i < N; ++i) {
         float x = s[i] + (bias ? bias[n + i] : 0.f) + (bias2 ? bias2[n + i] : 0.f);
         if (act) x = ka_activate_fast(act, x);

@@ -126,6 +126,11 @@ __device__ __forceinline__ void sk_finish(const floatx4 (*red)[MB][KA_WAVE], con
         for (int w = 0; w < NW; ++w) s += red[w][mb][lane] + red[w][mb][lane + OTHER];
         const int m = mb * 16 + r;
         if (m >= M) continue;
+        if (ka_act_gated(tg.act)) {         // the four sums are two pairs of gate and value
+            const float v[4] = {s[0], s[1], s[2], s[3]};
+            ka_gated_store<true, 4>(tg.out, tg.out_dtype, tg.ldo, m, n, tg.N, v, tg.act);
+            continue;
+        }
         if (tg.act) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) s[i] = ka_activate_fast(tg.act, s[i]);
@@ -443,8 +448,9 @@ static inline bool persistent_bias_ok(const SkinnyTarget& t) {
 static inline int check_target(const char* who, const SkinnyTarget& t, int K) {
     KA_CHECK(t.W && t.out, "%s: weight or output missing", who);
     KA_CHECK(t.N > 0 && t.ldw % 8 == 0 && t.ldw >= K && (uintptr_t)t.W % 16 == 0, "%s: weight rows must be 16-byte aligned and >= K", who);
-    KA_CHECK(t.ldo >= t.N, "%s: output stride too small", who);
     KA_CHECK(ka_act_known(t.act), "%s: unknown activation %d", who, t.act);
+    KA_CHECK(t.ldo >= ka_act_outputs(t.act, t.N), "%s: output stride too small", who);
+    KA_CHECK(!ka_act_gated(t.act) || (t.N % 2 == 0 && !t.accumulate), "%s: a gated linear needs an even N and no accumulation", who);
     KA_CHECK(t.out_dtype == KA_F32 || t.out_dtype == KA_BF16, "%s: bad output type", who);
     KA_CHECK(!(t.accumulate && t.out_dtype != KA_F32), "%s: accumulate needs an fp32 output", who);
     return 0;

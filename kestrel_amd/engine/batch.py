@@ -63,7 +63,7 @@ class StepBatch:
     n_tokens: int
     n_rows: int
     token_ids: torch.Tensor             # int32 [tokens], -1 where an embedding is given
-    positions: torch.Tensor             # int32 [tokens]
+    positions: torch.Tensor             # int32 [tokens]: the token's place in its sequence (and in the cache)
     token_row: torch.Tensor             # int32 [tokens]
     kv_hi: torch.Tensor                 # int32 [tokens]
     row_slot: torch.Tensor              # int32 [rows]
@@ -79,6 +79,8 @@ class StepBatch:
     # (int32 [runs] first token, int32 [runs] count): the tokens cut into runs that fill one page of their row in
     # order, and runs of up to a page's worth of other tokens (for the kernels that write the cache by pages)
     page_runs: Optional[Tuple[torch.Tensor, torch.Tensor]] = None
+    # int32 [tokens, axes] where a position encoding of the model takes more than one number per token
+    position_axes: Optional[torch.Tensor] = None
     pending: Optional[torch.Tensor] = None        # int32 device table: an id <= -2 stands for pending[-2 - id]
     given_embeds: Optional[torch.Tensor] = None   # [m, dim]
     given_rows: Optional[torch.Tensor] = None     # int32 [m] token indices they go to

@@ -53,7 +53,9 @@ class StepEntry:
     ``kestrel/scheduler/scheduler.py:2289-2290``). ``want``: indices into ``tokens`` whose logits are returned.
     ``bidirectional``: position ranges ``[lo, hi)`` whose tokens see each other both ways
     (an image block); each must lie wholly inside this portion. ``start``: position of the
-    first token; ``None`` means right after what the request already holds.
+    first token; ``None`` means right after what the request already holds. ``positions``: for models
+    with a position encoding of several axes (``PositionEncoding.axes``), the numbers of every token,
+    ``[tokens, axes]``; ``None``: the place in the sequence on every axis.
     """
 
     slot: int
@@ -62,6 +64,7 @@ class StepEntry:
     embeds: Optional[torch.Tensor] = None
     bidirectional: Sequence[Tuple[int, int]] = ()
     start: Optional[int] = None
+    positions: Optional[Sequence[Sequence[int]]] = None
 
 
 def _align(n: int) -> int:
@@ -201,6 +204,8 @@ class ModelRunner:
         # so through ``query_tile()``): the step lists the blocks of each size, most keys first.
         tiles = getattr(model, "query_tiles", None)
         self.query_tiles: List[int] = sorted(tiles()) if callable(tiles) else []
+        axes = getattr(model, "position_axes", None)
+        self.position_axes: int = int(axes()) if callable(axes) else 1
 
     # ------------------------------------------------------------------ requests
     def admit(self, reserve_length: int = 0, portion: int = 1) -> int:
@@ -280,6 +285,12 @@ class ModelRunner:
             for w in e.want:
                 if not 0 <= int(w) < q:
                     raise refuse(f"wanted place {w} outside its {q} tokens")
+            if e.positions is not None:
+                if self.position_axes == 1:
+                    raise refuse("positions given, but the model's encodings take the place in the sequence")
+                given_axes = np.asarray(e.positions)
+                if given_axes.shape != (q, self.position_axes) or given_axes.dtype.kind not in "iu":
+                    raise refuse(f"positions must be integers of shape [{q}, {self.position_axes}]")
             starts.append(start)
             n_tokens += q
         if n_tokens > self.max_tokens_per_step:
@@ -305,6 +316,8 @@ class ModelRunner:
 
         n_groups = len(cache.groups)
         ids, positions, token_row, kv_hi = _Column(), _Column(), _Column(), _Column()
+        n_axes = self.position_axes
+        axes = _Column() if n_axes > 1 else None       # row-major [tokens, axes]
         # blocks of queries, per size: row, first token, most keys any of them sees
         blocks: Dict[int, List[Tuple[int, int, int]]] = {tile: [] for tile in self.query_tiles}
         logit_rows: List[int] = []
@@ -363,6 +376,11 @@ class ModelRunner:
                 positions.extend(np.arange(start, start + q, dtype=np.int64))
                 token_row.extend(np.full(q, r, dtype=np.int64))
             kv_hi.extend(hi)
+            if axes is not None:
+                if e.positions is not None:
+                    axes.extend(np.asarray(e.positions, dtype=np.int64).reshape(-1))
+                else:
+                    axes.extend(np.repeat(np.arange(start, start + q, dtype=np.int64), n_axes))
             for tile, listed in blocks.items():
                 if isinstance(hi, np.ndarray):
                     # most keys any query of a block sees: the blocks' maxima in one go
@@ -396,6 +414,8 @@ class ModelRunner:
             positions.append(0)
             token_row.append(r)
             kv_hi.append(0)
+            if axes is not None:
+                axes.extend([0] * n_axes)
             for listed in blocks.values():
                 listed.append((r, len(ids) - 1, 0))
             logit_rows.append(len(ids) - 1)
@@ -420,6 +440,8 @@ class ModelRunner:
             ("logit_slot", logit_slot),
             ("given_rows", given_rows), ("run_first", runs.first()), ("run_count", runs.count()),
         ]
+        if axes is not None:
+            sections.append(("position_axes", axes))
         for tile, listed in blocks.items():
             sections.append((f"qblk_row{tile}", [b[0] for b in listed]))
             sections.append((f"qblk_tok{tile}", [b[1] for b in listed]))
@@ -477,6 +499,7 @@ class ModelRunner:
             kv_len=view("kv_len"), logit_rows=view("logit_rows"), logit_slot=view("logit_slot"), groups=groups,
             workspace=workspace or self.workspace,
             query_blocks={tile: (view(f"qblk_row{tile}"), view(f"qblk_tok{tile}")) for tile in blocks},
+            position_axes=view("position_axes").view(n_tokens, n_axes) if axes is not None else None,
             pending=self.pending, given_embeds=given_embeds, given_rows=view("given_rows") if given else None, max_q=max_q, max_kv=max_kv,
             decode_only=max_q == 1, causal_only=causal_only, wants_every_token=logit_rows == list(range(n_tokens)),
             page_runs=(view("run_first"), view("run_count")),
@@ -563,7 +586,7 @@ class ModelRunner:
         cache, plan = self.cache, self.model.plan
         limit = self.max_tokens_per_step if prompt_tokens is None else min(prompt_tokens, self.max_tokens_per_step)
         rows = max(cache.max_requests, 1)
-        per_token = 8 + 2 * len(cache.groups) + 2 * max(len(self.query_tiles), 1)
+        per_token = 8 + 2 * len(cache.groups) + 2 * max(len(self.query_tiles), 1) + self.position_axes
         ints = per_token * (limit + rows) + rows * (8 + len(cache.groups) * (self._pages_cap + 4)) + 4096
         if self._meta_device is None or self._meta_device.numel() < ints:
             self._meta_device = torch.empty(ints, dtype=torch.int32, device=self.device)

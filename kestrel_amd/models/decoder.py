@@ -24,6 +24,7 @@ class DecoderModel:
         self.plan = plan
         self.blocks: List[Block] = [Block(layer) for layer in plan.layers]
         self.final_norm = build_part("norm", plan.final_norm)
+        self.position = build_part("position", plan.position) if plan.position is not None else None
         for index, entry in enumerate(plan.schedule):
             if not 0 <= entry.layer < len(self.blocks):
                 raise ValueError(f"schedule entry {index} names layer {entry.layer}, the plan has {len(self.blocks)}")
@@ -47,6 +48,9 @@ class DecoderModel:
             out.update(block.params())
         for local, pspec in self.final_norm.params().items():
             out[plan.names[f"final_norm.{local}"]] = pspec
+        if self.position is not None:
+            for local, pspec in self.position.params().items():
+                out[plan.names[f"position.{local}"]] = pspec
         if not plan.tied_head:
             out[plan.names["head.weight"]] = ParamSpec((plan.vocab_size, plan.dim), "matrix", "normal")
         if plan.head_bias:
@@ -61,6 +65,8 @@ class DecoderModel:
             block.bind(tensors, dtype, device)
         self.final_norm.bind({k: tensors[plan.names[f"final_norm.{k}"]] for k in self.final_norm.params()}, dtype,
                              device)
+        if self.position is not None:
+            self.position.bind({k: tensors[plan.names[f"position.{k}"]] for k in self.position.params()}, dtype, device)
         self.head_weight = self.embedding if plan.tied_head else tensors[plan.names["head.weight"]].to(device).contiguous()
         if plan.head_bias:
             self.head_bias = tensors[plan.names["head.bias"]].to(device=device, dtype=torch.float32).contiguous()
@@ -73,6 +79,11 @@ class DecoderModel:
             mixer = self.blocks[entry.layer].mixer
             needs.append((mixer.cache_spec(), mixer.state_spec(), entry.reads_cache_of))
         return needs
+
+    def position_axes(self) -> int:
+        """The most numbers any position encoding of the model (its own, or a mixer's) needs per token."""
+        parts = [self.position] + [getattr(block.mixer, "position", None) for block in self.blocks]
+        return max([1] + [int(getattr(part, "axes", 1)) for part in parts if part is not None])
 
     def query_tiles(self):
         """Sizes of blocks of queries that the mixers' kernels want listed with a step."""
@@ -97,6 +108,8 @@ class DecoderModel:
         core.embed(self.embedding, batch.token_ids, x, batch.pending, plan.embedding_scale)
         if batch.given_embeds is not None:
             core.scatter_rows(batch.given_embeds, batch.given_rows, x)
+        if self.position is not None:
+            self.position.add_to_embeddings(x, batch)
         handed = None      # the next block's first norm of x, where a block's last launch has computed it
         for index, entry in enumerate(plan.schedule):
             after = plan.schedule[index + 1] if index + 1 < len(plan.schedule) else None

@@ -246,7 +246,10 @@ def linear_generic(a: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.T
     m, k = a.shape
     n = weight.shape[0]
     _need(weight.dim() == 2 and weight.shape[1] == k, f"linear: weight {tuple(weight.shape)} does not match K={k}")
-    _need(out.dim() == 2 and tuple(out.shape) == (m, n), f"linear: out {tuple(out.shape)} is not [{m}, {n}]")
+    gated = bool(act & 0x100)          # (ops.linear.ACT_GATED: pairs of weight rows make one output)
+    _need(not gated or (n % 2 == 0 and not accumulate), "linear: a gated linear needs an even number of weight rows and no accumulation")
+    n_out = n // 2 if gated else n
+    _need(out.dim() == 2 and tuple(out.shape) == (m, n_out), f"linear: out {tuple(out.shape)} is not [{m}, {n_out}]")
     _need(a.stride(1) == 1 and weight.stride(1) == 1 and out.stride(1) == 1, "linear: rows must be contiguous")
     _need(bias is None or (bias.dtype == torch.float32 and bias.numel() == n and bias.is_contiguous()),
           "linear: bias must be fp32 [N]")

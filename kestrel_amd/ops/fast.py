@@ -117,6 +117,8 @@ def chip_sizes(device=None) -> ChipSizes:
     return _chips[index]
 
 
+ACT_GATED = 0x100                  # (ops.linear.ACT_GATED)
+
 _lib = None
 _scratch: Dict[int, torch.Tensor] = {}
 _OUT_CODE = {torch.float32: KA_F32, torch.bfloat16: KA_BF16}
@@ -235,8 +237,10 @@ def _bias_ok(bias: Optional[torch.Tensor], n: int) -> bool:
     return bias is None or (bias.dtype == torch.float32 and bias.numel() == n and bias.is_contiguous())
 
 
-def _out_ok(out: torch.Tensor, m: int, n: int) -> bool:
-    return (out.dtype in _OUT_CODE and tuple(out.shape) == (m, n) and out.stride(1) == 1 and out.data_ptr() % 16 == 0)
+def _out_ok(out: torch.Tensor, m: int, n: int, act: int = 0) -> bool:
+    """``out`` is ``[m, columns]`` of a linear of ``n`` weight rows (half of them if ``act`` says gated)."""
+    n_out = n // 2 if act & ACT_GATED else n
+    return (out.dtype in _OUT_CODE and tuple(out.shape) == (m, n_out) and out.stride(1) == 1 and out.data_ptr() % 16 == 0)
 
 
 def linear_bf16(a, weight, bias, out, act, accumulate) -> bool:
@@ -247,7 +251,9 @@ def linear_bf16(a, weight, bias, out, act, accumulate) -> bool:
     if k % 8 or not _operand_ok(a, k) or not _operand_ok(weight, k) or out.dtype not in _OUT_CODE \
             or out.data_ptr() % 16 or out.stride(1) != 1:
         return False
-    if tuple(out.shape) != (m, n):
+    if act & ACT_GATED and (n % 2 or accumulate):
+        raise KernelError("linear: a gated linear needs an even number of weight rows and no accumulation")
+    if tuple(out.shape) != (m, n // 2 if act & ACT_GATED else n):
         raise KernelError(f"linear: shapes a {tuple(a.shape)}, weight {tuple(weight.shape)}, out {tuple(out.shape)}")
     if not _bias_ok(bias, n):
         raise KernelError("linear: bias must be fp32 [N]")
@@ -323,8 +329,8 @@ def linear_two_outputs(a, wa, ba, out_a, act_a, wb, bb, out_b, act_b) -> bool:
     na, nb = wa.shape[0], wb.shape[0]
     if not (0 < m <= SKINNY_MAX_ROWS) or k % 8:
         return False
-    if not (_operand_ok(a, k) and _operand_ok(wa, k) and _operand_ok(wb, k) and _out_ok(out_a, m, na)
-            and _out_ok(out_b, m, nb) and _bias_ok(ba, na) and _bias_ok(bb, nb)):
+    if not (_operand_ok(a, k) and _operand_ok(wa, k) and _operand_ok(wb, k) and _out_ok(out_a, m, na, act_a)
+            and _out_ok(out_b, m, nb, act_b) and _bias_ok(ba, na) and _bias_ok(bb, nb)):
         return False
     _check(lib().ka_linear_skinny_fused(
         a.data_ptr(), a.stride(0), k, None, 0, 0, None, 0, None,
@@ -349,11 +355,11 @@ def layernorm_linear(x, gamma, beta, eps, wa, ba, out_a, act_a, wb=None, bb=None
     if beta is not None and (beta.dtype != torch.float32 or beta.numel() != k or beta.data_ptr() % 16):
         return False
     na = wa.shape[0]
-    if not (_operand_ok(wa, k) and _out_ok(out_a, m, na) and _bias_ok(ba, na)):
+    if not (_operand_ok(wa, k) and _out_ok(out_a, m, na, act_a) and _bias_ok(ba, na)):
         return False
     two = wb is not None
     nb = wb.shape[0] if two else 0
-    if two and not (_operand_ok(wb, k) and _out_ok(out_b, m, nb) and _bias_ok(bb, nb)):
+    if two and not (_operand_ok(wb, k) and _out_ok(out_b, m, nb, act_b) and _bias_ok(bb, nb)):
         return False
     if m * (k + 8) * 2 > 96 * 1024:
         return False
@@ -436,7 +442,7 @@ def _side_linear_ok(job) -> bool:
         return False
     m, k = a.shape
     n = w.shape[0]
-    if k % 8 or not (_operand_ok(a, k) and _operand_ok(w, k) and _out_ok(out, m, n) and _bias_ok(job.bias, n)):
+    if k % 8 or not (_operand_ok(a, k) and _operand_ok(w, k) and _out_ok(out, m, n, int(job.act)) and _bias_ok(job.bias, n)):
         return False
     return job.bias is None or (n % 4 == 0 and job.bias.data_ptr() % 16 == 0)
 

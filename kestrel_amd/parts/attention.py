@@ -63,6 +63,9 @@ class PagedAttention(Mixer):
         if self.spec.bias:
             self.qkv_bias = tensors["qkv.bias"].to(device=device, dtype=torch.float32).contiguous()
             self.proj_bias = tensors["proj.bias"].to(device=device, dtype=torch.float32).contiguous()
+        if int(getattr(self.position, "axes", 1)) != 1:
+            raise ValueError(f"attention rotates by a token's place in the sequence; the position encoding "
+                             f"{getattr(spec.position, 'kind', '?')!r} takes {self.position.axes} numbers per token")
         rotation = self.position.rotation(device)
         if rotation is None and callable(getattr(self.position, "table", None)) and self.position.table(device) is not None:
             raise ValueError(f"the position encoding {getattr(spec.position, 'kind', '?')!r} holds a table but offers no "

@@ -54,12 +54,26 @@ class Rotation:
 
 
 class PositionEncoding(Part):
-    """What a mixer needs to encode positions. An encoding that turns pairs of channels by angles
-    that grow with the position offers ``rotation``; one that offers nothing is applied nowhere
-    inside attention (order then comes from elsewhere, or from nowhere)."""
+    """How positions are encoded, inside a mixer (``AttentionSpec.position``) or once for the whole
+    model (``ModelPlan.position``). An encoding that turns pairs of channels by angles that grow with
+    the position offers ``rotation``; one that adds something to the embeddings before the first block
+    overrides ``add_to_embeddings``; one that offers neither is applied nowhere (order then comes from
+    elsewhere, or from nowhere).
+
+    ``axes``: how many numbers say where a token stands. 1: its place in the sequence, which every
+    step carries as ``StepBatch.positions`` ``[tokens]``. More (rows and columns of an image patch, time):
+    the step then also carries ``StepBatch.position_axes`` ``[tokens, axes]``, taken from
+    ``StepEntry.positions`` where an entry gives them and else the place in the sequence on every axis."""
+
+    axes: int = 1
 
     def rotation(self, device: torch.device) -> Optional[Rotation]:
         return None
+
+    def add_to_embeddings(self, x: torch.Tensor, batch) -> None:
+        """Model-level encodings: add the encoding of every token's position into the fp32 rows ``x``
+        ``[tokens, dim]`` in place (``batch.positions``, ``batch.position_axes``). Under replayed graphs
+        (``batch.decode_only``) this must neither synchronise nor allocate."""
 
 
 @dataclass

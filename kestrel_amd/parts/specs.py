@@ -154,6 +154,10 @@ class ModelPlan:
     embedding_scale: float = 1.0
     logit_scale: float = 1.0
     logit_softcap: Optional[float] = None
+    # a position encoding of the whole model (a specification whose part is registered as a position
+    # encoding): its ``add_to_embeddings`` runs on the embedded tokens before the first block; its tensors
+    # are named by ``names["position.<local name>"]``. ``None``: positions are the mixers' business.
+    position: Optional[object] = None
 
     def describe(self) -> Dict[str, object]:
         return {"architecture": self.architecture, "layers": len(self.layers), "schedule": len(self.schedule),

@@ -166,6 +166,74 @@ def test_every_activation_in_every_linear_kernel(name, code):
     _close(out, _ACTIVATE[code](h @ w.double().T), bf, scale=2)
 
 
+def _gated_case(fn, m, n, k, a_dtype, w_dtype, out_dtype, code, seed=0):
+    """``fn(a, weight_pairs, bias_pairs, out, act)`` against ``act(a Wg^T + bg) * (a Wu^T + bu)`` in float64; the
+    output is poisoned first, so a column the kernel leaves out shows."""
+    from kestrel_amd.ops.linear import pair_rows
+
+    torch.manual_seed(seed)
+    a = torch.randn(m, k).to(a_dtype).to(DEV)
+    gate, value = ((torch.randn(n, k) / k ** 0.5).to(w_dtype).to(DEV) for _ in range(2))
+    gate_bias, value_bias = torch.randn(n).to(DEV), torch.randn(n).to(DEV)
+    out = torch.full((m, n), float("nan"), dtype=out_dtype, device=DEV)
+    fn(a, pair_rows(gate, value), pair_rows(gate_bias, value_bias), out, code)
+    ref = _ACTIVATE[code](a.double() @ gate.double().T + gate_bias.double()) * (a.double() @ value.double().T + value_bias.double())
+    worst = torch.float32 if (a_dtype == w_dtype == out_dtype == torch.float32) else torch.bfloat16
+    _close(out, ref, worst, scale=3)
+
+
+@pytest.mark.parametrize("name,code", [("silu", 3), ("gelu_tanh", 1), ("none", 0)])
+def test_a_gated_linear_in_every_kernel_family(name, code):
+    """``out = act(gate) * value`` as an epilogue option of the linear kernels (weight rows in pairs): the plain
+    fp32 kernels, the weight-streaming ones (persistent, split, wide, behind a LayerNorm prologue, as the second
+    of two targets), the tiled one with and without the vendor library asked first (which has no such
+    epilogue and declines)."""
+    from kestrel_amd.ops import core, fast
+    from kestrel_amd.ops.linear import ACT_GATED, linear_gated, pair_rows
+
+    bf, f32 = torch.bfloat16, torch.float32
+    for m, n, k in ((3, 37, 36), (19, 77, 130), (200, 136, 264), (130, 65, 333)):       # few rows, the tiled fp32 form, odd sizes
+        _gated_case(linear_gated, m, n, k, f32, f32, f32, code)
+    _gated_case(linear_gated, 9, 40, 64, bf, f32, bf, code)                            # mixed types: the plain kernel
+    for library in (True, False):
+        fast.LIBRARY_LINEAR, was = library, fast.LIBRARY_LINEAR
+        try:
+            for m, n, k in ((1, 24, 64), (8, 1024, 2048), (16, 515, 520), (40, 2050, 2048), (64, 512, 10240), (200, 333, 520),
+                            (520, 1024, 2048), (2048, 512, 1024)):
+                _gated_case(linear_gated, m, n, k, bf, bf, bf, code)
+        finally:
+            fast.LIBRARY_LINEAR = was
+    for mode in (0, 2):                                      # the split kernel, then the wide one wherever it can run
+        fast.set_skinny_persistent(0 if mode == 0 else 1)
+        fast.set_skinny_wide(mode)
+        try:
+            _gated_case(linear_gated, 12, 258, 3000, bf, bf, bf, code)
+            _gated_case(linear_gated, 40, 130, 1000, bf, bf, f32, code)
+        finally:
+            fast.set_skinny_persistent(1)
+            fast.set_skinny_wide(1)
+    # behind the LayerNorm prologue, as the second of two targets (the first plain): one launch
+    torch.manual_seed(7)
+    x = (torch.randn(5, 264) * 2).to(DEV)
+    gamma, beta = (1 + 0.1 * torch.randn(264)).to(DEV), (0.1 * torch.randn(264)).to(DEV)
+    w_plain = (torch.randn(72, 264) / 16).bfloat16().to(DEV)
+    gate, value = ((torch.randn(40, 264) / 16).bfloat16().to(DEV) for _ in range(2))
+    out_plain = torch.empty(5, 72, dtype=bf, device=DEV)
+    out_gated = torch.full((5, 40), float("nan"), dtype=bf, device=DEV)
+    assert fast.layernorm_linear(x, gamma, beta, 1e-5, w_plain, None, out_plain, 0, pair_rows(gate, value), None, out_gated,
+                                 code | ACT_GATED)
+    h = F.layer_norm(x.double(), (264,), gamma.double(), beta.double(), 1e-5).to(bf).double()
+    _close(out_plain, h @ w_plain.double().T, bf, scale=2)
+    _close(out_gated, _ACTIVATE[code](h @ gate.double().T) * (h @ value.double().T), bf, scale=3)
+    # what cannot be: an odd number of weight rows, accumulation
+    from kestrel_amd.ops.core import KernelError
+    with pytest.raises((KernelError, ValueError), match="even"):
+        linear_gated(torch.zeros(4, 64, device=DEV), torch.zeros(7, 64, device=DEV), None, torch.zeros(4, 3, device=DEV), code)
+    with pytest.raises((KernelError, ValueError), match="accumulation"):
+        core.linear_generic(torch.zeros(4, 64, device=DEV), torch.zeros(8, 64, device=DEV), None, torch.zeros(4, 4, device=DEV),
+                            code | ACT_GATED, True)
+
+
 @pytest.mark.parametrize("persistent,wide", [(1, 0), (0, 0), (1, 2)])
 @pytest.mark.parametrize("shape", [(1, 48, 64), (8, 2048, 2048), (5, 100, 200), (16, 6144, 2048), (33, 77, 8192),
                                    (64, 51200, 512), (17, 2048, 8192), (3, 16, 8), (9, 20000, 1032), (40, 4100, 2048),

@@ -602,6 +602,210 @@ def test_constants_around_the_stack():
         runner.release(slot)
 
 
+@dataclass(frozen=True)
+class GatedSpec:
+    kind: str
+    dim: int
+    hidden_dim: int
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+def test_a_gated_feed_forward_as_a_part(dtype):
+    """Another feed-forward, defined here: ``down(silu(x Wg^T) * (x Wu^T))``, three matrices without biases. It
+    binds gate and value as one matrix of row pairs and offers its stages like the dense one, so the product
+    of the pair is taken in the epilogue of whatever kernel runs its first linear: the prompt's tiled kernel,
+    and in decode steps the launch that also normalises and projects q|k|v (one launch for norm + q|k|v + gate
+    and value, one for attention, one for both last linears). A tiny Moondream plan with it in every layer
+    against a plain computation; prompt portions, then tokens one by one, eagerly and replayed."""
+    from dataclasses import replace
+
+    from kestrel_amd.config import get_spec
+    from kestrel_amd.engine.loading import make_runner
+    from kestrel_amd.engine.step import StepEntry
+    from kestrel_amd.models import DecoderModel
+    from kestrel_amd.ops.linear import ACT_GATED, activation_code, linear, linear_gated, pair_rows
+    from kestrel_amd.parts import FeedForward, ParamSpec, register_feed_forward
+
+    class GatedFeedForward(FeedForward):
+        def params(self):
+            d, f = self.spec.dim, self.spec.hidden_dim
+            return {"gate.weight": ParamSpec((f, d)), "up.weight": ParamSpec((f, d)), "down.weight": ParamSpec((d, f))}
+
+        def bind(self, tensors, dtype, device):
+            self.dtype = dtype
+            self.pairs = pair_rows(tensors["gate.weight"].to(device), tensors["up.weight"].to(device))
+            self.down = tensors["down.weight"].to(device).contiguous()
+            self.act = activation_code("silu")
+
+        def input_projection(self):
+            return self.pairs, None, self.spec.hidden_dim, self.act | ACT_GATED
+
+        def output_projection(self):
+            return self.down, None
+
+        def forward(self, h, batch, residual):
+            hidden = batch.workspace.get("toy.gated_hidden", (h.shape[0], self.spec.hidden_dim), self.dtype)
+            linear_gated(h, self.pairs, None, hidden, self.act)
+            linear(hidden, self.down, None, residual, accumulate=True)
+
+    register_feed_forward("toy_gated", GatedFeedForward)
+    name = "D"
+    cfg = helpers.flat_config(name)
+    hidden_dim = 72
+    spec = get_spec("moondream2")
+    base = spec.build_plan(spec.read_config(helpers.CONFIGS[name]))
+    layers = []
+    for index, layer in enumerate(base.layers):
+        names = {k: v for k, v in layer.names.items() if not k.startswith("feed_forward.")}
+        names.update({f"feed_forward.{part}.weight": f"text.blocks.{index}.glu.{part}.weight" for part in ("gate", "up", "down")})
+        layers.append(replace(layer, feed_forward=GatedSpec("toy_gated", cfg["dim"], hidden_dim), names=names))
+    model = DecoderModel(replace(base, layers=tuple(layers)))
+    gen = torch.Generator().manual_seed(61)
+    stored = helpers.stored_weights(helpers.model_dir(name))
+    weights = {}
+    for tensor_name, pspec in model.params().items():
+        if tensor_name in stored:
+            weights[tensor_name] = stored[tensor_name].float()
+        else:
+            weights[tensor_name] = (0.3 * torch.randn(pspec.shape, generator=gen)).to(dtype).float()
+    model.bind({k: v.to(dtype) if v.dim() == 2 else v for k, v in weights.items()}, dtype, DEV)
+
+    ids = helpers.random_ids(62, 45, cfg["vocab_size"])
+    w = {k: v.double() for k, v in weights.items()}
+    x = w["text.wte"][torch.tensor(ids)]
+    positions = torch.arange(len(ids))
+    allowed = plain.visibility(positions, None)
+    table = plain.rotary_table(plain.rotary_dim_of(cfg), len(ids), float(cfg["rope_theta"]))
+    for index in range(cfg["n_layers"]):
+        prefix = f"text.blocks.{index}."
+        xn = plain.layer_norm(x, w[prefix + "ln.weight"], w[prefix + "ln.bias"], plain.eps_of(cfg))
+        gated = torch.nn.functional.silu(xn @ w[prefix + "glu.gate.weight"].T) * (xn @ w[prefix + "glu.up.weight"].T)
+        x = x + plain.attention(xn, w, prefix, cfg, positions, allowed, table) + gated @ w[prefix + "glu.down.weight"].T
+    expected = plain.head(x, w, cfg)
+    for graphs in (False, True):
+        runner = make_runner(model, 16, 8, 2, enable_graphs=graphs)
+        slot = runner.admit()
+        got = [runner.step([StepEntry(slot, ids[:21], want=list(range(21)))]).clone(),
+               runner.step([StepEntry(slot, ids[21:30], want=list(range(9)))]).clone()]
+        got += [runner.step([StepEntry(slot, [t], want=[0])]).clone() for t in ids[30:]]
+        assert (runner.graph_replays > 0) == graphs
+        helpers.assert_close(torch.cat(got), expected, dtype, f"a gated feed-forward, graphs={graphs}")
+        runner.release(slot)
+    if dtype == torch.bfloat16:
+        # the decode steps took the three-launch form: the gated linear rode in the launch of norm + q|k|v, or
+        # (a few rows whose attention leaves the chip idle) in the attention launch
+        from kestrel_amd.ops import fast
+        rode = []
+        first_launch, attention_launch = fast.layernorm_linear, fast.attention_decode_bf16
+
+        def watched_first(*args, **kwargs):
+            done = first_launch(*args, **kwargs)
+            rode.append(done and len(args) > 11 and args[11])
+            return done
+
+        def watched_attention(*args, **kwargs):
+            done = attention_launch(*args, **kwargs)
+            rode.append(done and kwargs.get("beside") is not None and kwargs["beside"].act)
+            return done
+
+        fast.layernorm_linear, fast.attention_decode_bf16 = watched_first, watched_attention
+        try:
+            runner = make_runner(model, 16, 8, 2)
+            slot = runner.admit()
+            runner.step([StepEntry(slot, ids[:5])])
+            runner.step([StepEntry(slot, ids[5:6], want=[0])])
+        finally:
+            fast.layernorm_linear, fast.attention_decode_bf16 = first_launch, attention_launch
+        # (both steps have few rows: the prompt's five tokens take the same three launches a layer)
+        assert rode.count(activation_code("silu") | ACT_GATED) == 2 * cfg["n_layers"], rode
+
+
+@dataclass(frozen=True)
+class GridPositionSpec:
+    kind: str
+    dim: int
+    rows: int
+    columns: int
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+def test_a_position_encoding_of_the_whole_model_over_two_axes(dtype):
+    """Another position encoding, defined here: two learned tables, one per axis (row and column), whose
+    vectors are added to the embeddings before the first block. It says ``axes = 2``; the step then carries
+    two numbers per token: what an entry gives (an image's patches as a grid), else the place in the
+    sequence on both axes (text, decoded tokens). A tiny Moondream plan with it (the attention keeps its
+    rotation by the place in the sequence) against the plain model fed with embeddings that have the
+    position vectors added by hand; a prompt in portions, then tokens one by one, eagerly and replayed."""
+    from dataclasses import replace
+
+    from kestrel_amd.config import get_spec
+    from kestrel_amd.engine.loading import make_runner
+    from kestrel_amd.engine.step import StepEntry, StepRefused
+    from kestrel_amd.models import DecoderModel
+    from kestrel_amd.parts import ParamSpec, PositionEncoding, register_position
+
+    class GridPosition(PositionEncoding):
+        axes = 2
+
+        def params(self):
+            return {"rows": ParamSpec((self.spec.rows, self.spec.dim), "matrix", "normal"),
+                    "columns": ParamSpec((self.spec.columns, self.spec.dim), "matrix", "normal")}
+
+        def bind(self, tensors, dtype, device):
+            self.rows, self.columns = tensors["rows"].to(device).float(), tensors["columns"].to(device).float()
+
+        def add_to_embeddings(self, x, batch):
+            at = batch.position_axes.long()
+            x += self.rows[at[:, 0]] + self.columns[at[:, 1]]
+
+    register_position("toy_grid", GridPosition)
+    spec = get_spec("moondream2")
+    cfg = helpers.flat_config("E")
+    base = spec.build_plan(spec.read_config(helpers.TINY_E))
+    plan = replace(base, position=GridPositionSpec("toy_grid", cfg["dim"], 64, 64),
+                   names={**base.names, "position.rows": "pos.rows", "position.columns": "pos.columns"})
+    model = DecoderModel(plan)
+    assert model.position_axes() == 2
+    stored = helpers.stored_weights(helpers.model_dir("E"))
+    gen = torch.Generator().manual_seed(51)
+    weights = {k: v.float() for k, v in stored.items()}
+    weights["pos.rows"] = 0.5 * torch.randn(64, cfg["dim"], generator=gen)
+    weights["pos.columns"] = 0.5 * torch.randn(64, cfg["dim"], generator=gen)
+    weights = {k: v.to(dtype).float() for k, v in weights.items()}          # what both sides compute with
+    assert set(model.params()) == set(weights)
+    model.bind({k: v.to(dtype) if v.dim() == 2 else v for k, v in weights.items()}, dtype, DEV)
+    # 6 text ids, a grid of 3 x 4 patches (given embeddings, numbered by row and column), 9 text ids, then decoding
+    ids_a, ids_b = helpers.random_ids(52, 6, cfg["vocab_size"]), helpers.random_ids(53, 9 + 6, cfg["vocab_size"])
+    patches = torch.randn(12, cfg["dim"], generator=gen)
+    grid = [(10 + r, 20 + c) for r in range(3) for c in range(4)]
+    numbers = [(p, p) for p in range(6)] + grid + [(p, p) for p in range(18, 18 + len(ids_b))]
+    table = weights[plan.names["embedding"]].double()
+    embedded = torch.cat([table[ids_a], patches.double(), table[ids_b]])
+    embedded = embedded + torch.stack([weights["pos.rows"][r].double() + weights["pos.columns"][c].double() for r, c in numbers])
+    block_of = [-1] * 6 + [0] * 12 + [-1] * len(ids_b)
+    expected = plain.forward(cfg, {k: v.double() for k, v in weights.items()}, [], prefix_embeds=embedded, block_ids=block_of)
+    for graphs in (False, True):
+        runner = make_runner(model, 16, 8, 2, enable_graphs=graphs)
+        slot = runner.admit()
+        with pytest.raises(StepRefused, match=r"shape \[2, 2\]"):
+            runner.step([StepEntry(slot, ids_a[:2], positions=[(0, 0, 0), (1, 1, 1)])])
+        got = [runner.step([StepEntry(slot, ids_a[:4], want=[0, 1, 2, 3])]).clone()]
+        # the rest of the first text and the whole grid in one portion: positions given for all of its tokens
+        got.append(runner.step([StepEntry(slot, ids_a[4:] + [-1] * 12, want=list(range(14)), embeds=patches.to(DEV),
+                                          bidirectional=[(6, 18)], positions=[(4, 4), (5, 5)] + grid)]).clone())
+        got.append(runner.step([StepEntry(slot, ids_b[:9], want=list(range(9)))]).clone())
+        got += [runner.step([StepEntry(slot, [t], want=[0])]).clone() for t in ids_b[9:]]
+        assert (runner.graph_replays > 0) == graphs
+        helpers.assert_close(torch.cat(got), expected, dtype, f"a two-axis position encoding, graphs={graphs}")
+        runner.release(slot)
+    # an encoding of several axes cannot stand inside attention, which turns by the place in the sequence
+    from kestrel_amd.parts import AttentionSpec, build_part
+
+    mixer = build_part("mixer", AttentionSpec("attention", 32, 2, 2, 16, GridPositionSpec("toy_grid", 32, 4, 4)))
+    with pytest.raises(ValueError, match="takes 2 numbers per token"):
+        mixer.bind({name: torch.zeros(p.shape) for name, p in mixer.params().items()}, torch.float32, DEV)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
 def test_a_windowed_layer_beside_a_full_one(dtype):
     """The second layer of a tiny Moondream plan is given a window of 24 keys: its keys and values
