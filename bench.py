@@ -6,13 +6,14 @@ prefix embeddings and text ids) through the engine's step function with greedy s
 on the GPU. The model has the layer sizes of the Moondream 2 text decoder with seeded
 random weights N(0, 0.02) in bf16; inputs are synthetic. Besides ``value`` (decoded tokens
 a second) the line carries a 2,048-token prefill, the decode step's HBM roofline and
-decode throughput at batch 1 and 64. ``--peaks`` adds what this GPU reaches on a plain read stream
-and on a loop of matrix instructions beside the nominal peaks.
+decode throughput at batch 1 and 64. Beside the nominal peaks the line names what this GPU reaches on a plain
+read stream and on a loop of matrix instructions (``peak_measured``; ``--no-peaks`` leaves that out).
 
 ``--workload waves256`` and ``--workload mixed48`` (the latter meant for ``--sizes phi2``) measure
 the whole engine instead: a model folder is written with seeded random weights, loaded through the
 loader, and requests go through ``InferenceEngine`` (scheduler, sampler, paged cache under
-pressure); the line then reports generated tokens a second.
+pressure); the line then reports generated tokens a second. With ``--check N`` (meant for ``--layers 2``) the first N
+greedy requests of such a run are compared, token by token, with the plain implementation under ``tests/``.
 """
 
 from __future__ import annotations
@@ -182,7 +183,7 @@ def time_prefill(net, typed, tokens, repeats=8):
     prefix = min(typed.prefix_attn, tokens - 1)
     embeds = torch.randn(prefix, typed.dim, generator=gen).to(net.device)
     ids = torch.randint(0, typed.vocab_size, (tokens - prefix,), generator=gen).tolist()
-    best = None
+    times = []
     for i in range(repeats + 1):
         slot = runner.admit()
         entry = StepEntry(slot, [-1] * prefix + ids, want=[tokens - 1], embeds=embeds,
@@ -194,8 +195,9 @@ def time_prefill(net, typed, tokens, repeats=8):
         elapsed = time.perf_counter() - started
         runner.release(slot)
         if i > 0:                      # the first run warms up
-            best = elapsed if best is None else min(best, elapsed)
-    return best
+            times.append(elapsed)
+    times.sort()
+    return times[len(times) // 2], times[0]          # the median of the runs, and the best of them
 
 
 def write_model_folder(sizes: dict, layers: int, seed: int) -> str:
@@ -207,6 +209,37 @@ def write_model_folder(sizes: dict, layers: int, seed: int) -> str:
     folder = tempfile.mkdtemp(prefix="kestrel_amd_bench_")
     write_random_model(folder, {"text": dict(sizes, n_layers=layers)}, seed, InitRecipe(std=0.02))
     return folder
+
+
+def check_greedy(args, sizes: dict, folder: str, greedy: dict, results, prefix) -> int:
+    """``--check N``: the first N greedy requests of a workload against the plain implementation under ``tests/``
+    (float64, whole sequences, no cache): every token the engine generated must be the plain model's choice
+    after the engine's own earlier tokens, up to what the precision leaves of a near tie (twice the bound the
+    tests put on a bf16 logit: 3 % of the row's spread + 1 % of the value). Returns how many were compared;
+    raises if a token is not."""
+    if args.check <= 0:
+        return 0
+    from safetensors.torch import load_file
+
+    from tests.plain import moondream_plain as plain
+
+    weights = {k: v.double() for k, v in load_file(os.path.join(folder, "model.safetensors")).items()}
+    cfg = dict(sizes, n_layers=args.layers)
+    done = 0
+    for index in sorted(greedy)[:args.check]:
+        ids, tokens = greedy[index], results[index].tokens
+        logits = plain.forward(cfg, weights, list(ids) + tokens[:-1], prefix)
+        first = (0 if prefix is None else prefix.shape[0]) + len(ids) - 1
+        for i, token in enumerate(tokens):
+            row = logits[first + i]
+            gap, allowed = float(row.max() - row[token]), 2 * float(0.03 * row.std() + 0.01 * row.max().abs())
+            if args.dtype == "fp32":
+                allowed = 1e-4
+            if gap > allowed:
+                raise AssertionError(f"request {index}: token {i} is {token}, the plain implementation prefers "
+                                     f"{int(row.argmax())} by {gap:.3g} (allowed {allowed:.3g})")
+        done += 1
+    return done
 
 
 def run_workload(args, sizes: dict) -> dict:
@@ -242,12 +275,19 @@ def run_workload(args, sizes: dict) -> dict:
         vocab, dim = sizes["vocab_size"], sizes["dim"]
         prefix = torch.randn(730, dim, generator=torch.Generator().manual_seed(seed)).to("cuda:0") if waves else None
 
+        greedy = {}                    # index of a timed greedy request -> its prompt ids
+
         def submit(i):
             if waves:
                 ids = [rng.randrange(0, vocab) for _ in range(rng.randint(32, 128))]
                 options = dict(temperature=1.0, top_p=1.0, seed=i) if i % 2 else {}
+                if not options and i < 1000:
+                    greedy[i] = ids
                 return engine.submit_sync(ids, max_new_tokens=n_new, prefix_embeds=prefix, stop_ids=(), **options)
             ids = [rng.randrange(0, vocab) for _ in range(rng.randint(64, 1536))]
+            if i < args.check:             # (to be compared with the plain implementation: these decode greedily)
+                greedy[i] = ids
+                return engine.submit_sync(ids, max_new_tokens=n_new, stop_ids=())
             return engine.submit_sync(ids, max_new_tokens=n_new, temperature=0.7, top_p=1.0, seed=i, stop_ids=())
 
         for future in [submit(1000 + i) for i in range(8 if waves else 4)]:      # warm-up: graphs, workspaces
@@ -264,6 +304,7 @@ def run_workload(args, sizes: dict) -> dict:
         elapsed = time.perf_counter() - started
         steps = engine.scheduler.steps - steps_before
         pages = engine.runner.cache.n_pages
+        checked = check_greedy(args, sizes, folder, greedy, results, None if prefix is None else prefix.cpu())
     finally:
         engine.shutdown_sync()
         shutil.rmtree(folder, ignore_errors=True)
@@ -284,7 +325,7 @@ def run_workload(args, sizes: dict) -> dict:
                    "kv_cache_pages": pages, "page_size": PAGE_SIZE, "parallelism": "single-gpu"},
         "seconds": round(elapsed, 3), "generated_tokens": generated, "prompt_tokens": prompt,
         "all_tokens_per_second": round((generated + prompt) / elapsed, 1),
-        "finish_reasons": sorted({r.finish_reason for r in results}),
+        "finish_reasons": sorted({r.finish_reason for r in results}), "checked_against_plain": checked,
         "setup_seconds": {"write_folder": round(written, 1), "load": round(loaded, 1)},
     }
 
@@ -302,8 +343,11 @@ def main() -> int:
     parser.add_argument("--prefill-tokens", type=int, default=PREFILL_TOKENS, help="length of the timed prompt")
     parser.add_argument("--skip-points", action="store_true", help="only the default batch (no batch 1 / 64, no prefill)")
     parser.add_argument("--only-prefill", action="store_true", help="only the 2,048-token prefill (for profiling)")
-    parser.add_argument("--peaks", action="store_true",
-                        help="also measure a plain read stream and a loop of matrix instructions on this GPU and report against them")
+    parser.add_argument("--peaks", action=argparse.BooleanOptionalAction, default=True,
+                        help="also measure a plain read stream and a loop of matrix instructions on this GPU and report "
+                             "against them (about 0.1 s; --no-peaks leaves it out)")
+    parser.add_argument("--check", type=int, default=0,
+                        help="with --workload: compare this many greedy requests with the plain implementation (for --layers 2)")
     parser.add_argument("--workload", default="decode", choices=["decode", "waves256", "mixed48"],
                         help="decode: the benchmark's decode step (default); the others run requests through InferenceEngine")
     parser.add_argument("--max-batch-size", type=int, default=None, help="for the workloads through the entry point")
@@ -338,8 +382,9 @@ def main() -> int:
     weights = model_bytes(net, size)
 
     if args.only_prefill:
-        seconds = time_prefill(net, typed, args.prefill_tokens)
-        print(json.dumps({"prefill_ms": round(seconds * 1e3, 3), "tokens": args.prefill_tokens, "dtype": args.dtype}))
+        seconds, best = time_prefill(net, typed, args.prefill_tokens)
+        print(json.dumps({"prefill_ms": round(seconds * 1e3, 3), "best_ms": round(best * 1e3, 3), "tokens": args.prefill_tokens,
+                          "dtype": args.dtype}))
         return 0
     elapsed, kv_bytes = time_decode(net, typed, args.batch, args.context, args.steps, args.warmup)
     ms_per_step = elapsed / args.steps * 1e3
@@ -362,15 +407,20 @@ def main() -> int:
                      "frac": round(achieved / PEAK_HBM, 4)},
     }
     if not args.skip_points:
-        seconds = time_prefill(net, typed, args.prefill_tokens)
+        seconds, best = time_prefill(net, typed, args.prefill_tokens)         # the median of eight runs, and the best
         flops = prefill_flops(typed, args.prefill_tokens, min(typed.prefix_attn, args.prefill_tokens - 1))
         record["prefill"] = {"value": round(args.prefill_tokens / seconds, 1), "tokens": args.prefill_tokens,
-                             "ms": round(seconds * 1e3, 3), "frac": round(flops / seconds / PEAK_FLOPS[args.dtype], 4)}
-        points = {}
+                             "ms": round(seconds * 1e3, 3), "frac": round(flops / seconds / PEAK_FLOPS[args.dtype], 4),
+                             "best_ms": round(best * 1e3, 3)}
+        points, detail = {}, {}
         for batch, steps in ((1, args.steps), (64, max(16, args.steps // 4))):
-            e, _ = time_decode(net, typed, batch, args.context, steps, min(args.warmup, 4))
+            e, kv = time_decode(net, typed, batch, args.context, steps, min(args.warmup, 4))
             points[f"decode_b{batch}"] = round(batch * steps / e, 1)
+            moved = weights + kv * (size / 2) + batch * typed.dim * size
+            detail[f"decode_b{batch}"] = {"ms_per_step": round(e / steps * 1e3, 4), "steps": steps,
+                                          "frac": round(moved / (e / steps) / PEAK_HBM, 4)}
         record["points"] = points
+        record["points_detail"] = detail
     if args.peaks:
         from kestrel_amd.ops import core
 

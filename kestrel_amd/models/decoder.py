@@ -92,12 +92,11 @@ class DecoderModel:
     def _head_with_norm(self, x, batch, logits) -> bool:
         """A few decoded rows, every one of them wanted, in order: the head's launch normalises them itself
         (one launch less a step)."""
-        if self.dtype != torch.bfloat16 or not batch.decode_only or not getattr(batch, "wants_every_token", False) \
-                or getattr(self.final_norm.spec, "kind", None) != "layernorm":
+        ln = self.final_norm.layernorm_operands()
+        if self.dtype != torch.bfloat16 or not batch.decode_only or not getattr(batch, "wants_every_token", False) or ln is None:
             return False
         from ..ops import fast
-        norm = self.final_norm
-        return fast.layernorm_linear(x, norm.weight, norm.bias, norm.spec.eps, self.head_weight, self.head_bias, logits, 0)
+        return fast.layernorm_linear(x, *ln, self.head_weight, self.head_bias, logits, 0)
 
     # ------------------------------------------------------------------ forward
     def forward(self, batch, caches: List[LayerCache]) -> torch.Tensor:

@@ -38,6 +38,14 @@ class Norm(Part):
         """Normalise fp32 rows of ``x`` (all, or those in ``rows``) into ``out``."""
         raise NotImplementedError
 
+    def layernorm_operands(self):
+        """Optional. A norm that computes ``(x - mean) / sqrt(var + eps) * weight + bias`` over the last axis
+        says so here: ``(weight fp32 [dim], bias fp32 [dim] or None, eps)``. The linear kernels that can
+        normalise their input rows themselves, or the rows they have just finished, then take the norm
+        into their launch (a block's first norm in decode steps, the final norm before the head).
+        ``None`` (the default): the norm is always run through ``forward``, in a launch of its own."""
+        return None
+
 
 @dataclass(frozen=True)
 class Rotation:

@@ -35,18 +35,18 @@ def _parallel_few_rows(block: "Block", x, batch, cache, normed, then, handed) ->
     beside = None
     if normed is not None:
         fused = fast.linear_two_outputs(normed, m_in[0], m_in[1], projected, 0, f_in[0], f_in[1], hidden, f_in[3])
-    if not fused and fast.FUSE_LAYERNORM_PROLOGUE and getattr(norm.spec, "kind", None) == "layernorm":
+    ln = norm.layernorm_operands()            # (a norm of another form is run through its own forward below)
+    if not fused and fast.FUSE_LAYERNORM_PROLOGUE and ln is not None:
         # the feed-forward's first linear goes into the mixer's launch where the mixer takes it (the
         # launch of the mixer's first linear then leaves the normalised rows for it), else into the
         # launch of the mixer's first linear
         h = ws.get("block.h", tuple(x.shape), block.dtype)
         job = SideLinear(h, f_in[0], f_in[1], hidden, f_in[3])
         if block.mixer.takes_beside(job, batch, cache) and \
-                fast.layernorm_linear(x, norm.weight, norm.bias, norm.spec.eps, m_in[0], m_in[1], projected, 0, store=h):
+                fast.layernorm_linear(x, *ln, m_in[0], m_in[1], projected, 0, store=h):
             fused, beside = True, job
         else:
-            fused = fast.layernorm_linear(x, norm.weight, norm.bias, norm.spec.eps, m_in[0], m_in[1], projected, 0,
-                                          f_in[0], f_in[1], hidden, f_in[3])
+            fused = fast.layernorm_linear(x, *ln, m_in[0], m_in[1], projected, 0, f_in[0], f_in[1], hidden, f_in[3])
     if not fused:
         h = ws.get("block.h", tuple(x.shape), block.dtype)
         norm.forward(x, h)
@@ -61,10 +61,11 @@ def _parallel_few_rows(block: "Block", x, batch, cache, normed, then, handed) ->
     # rows of 2560, which leave the prologue's kernel no registers for a third strip of weights in flight, from
     # 5 rows on: 3 to 4 %).
     handing = n > fast.SKINNY_LN_MAX_ROWS or fast.pair_finishes_rows(n, x.shape[1])
-    if then is not None and handing and getattr(then.spec, "kind", None) == "layernorm":
+    then_ln = then.layernorm_operands() if then is not None and handing else None
+    if then_ln is not None:
         rows = ws.get("block.handed", tuple(x.shape), block.dtype)
         if fast.linear_pair_accumulate(mixed, m_out[0], m_out[1], hidden, f_out[0], f_out[1], x,
-                                       then_norm=(then.weight, then.bias, then.spec.eps, rows)):
+                                       then_norm=(*then_ln, rows)):
             handed.append(rows)
             return True
     if not fast.linear_pair_accumulate(mixed, m_out[0], m_out[1], hidden, f_out[0], f_out[1], x):

@@ -37,5 +37,8 @@ class LayerNorm(Norm):
     def forward(self, x, out, rows=None) -> None:
         core.layernorm(x, self.weight, self.bias, self.spec.eps, out, rows)
 
+    def layernorm_operands(self):
+        return self.weight, self.bias, float(self.spec.eps)
+
 
 register_norm("layernorm", LayerNorm)

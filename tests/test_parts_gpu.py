@@ -720,6 +720,69 @@ def test_a_gated_feed_forward_as_a_part(dtype):
         assert rode.count(activation_code("silu") | ACT_GATED) == 2 * cfg["n_layers"], rode
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
+def test_another_norm_as_a_part(dtype):
+    """Another norm, defined here: ``x / sqrt(mean(x^2) + eps) * weight`` (no mean taken off, no shift), in every
+    block and before the head of a tiny Moondream plan. It does not claim to be a LayerNorm
+    (``layernorm_operands`` stays ``None``), so no kernel takes it into its launch: blocks and head run it through
+    its ``forward``, also in decode steps and under replayed graphs. Against a plain computation."""
+    from dataclasses import replace
+
+    from kestrel_amd.config import get_spec
+    from kestrel_amd.engine.loading import make_runner
+    from kestrel_amd.engine.step import StepEntry
+    from kestrel_amd.models import DecoderModel
+    from kestrel_amd.parts import Norm, NormSpec, ParamSpec, register_norm
+
+    class RootMeanSquare(Norm):
+        def params(self):
+            return {"weight": ParamSpec((self.spec.dim,), "vector", "gain")}
+
+        def bind(self, tensors, dtype, device):
+            self.weight = tensors["weight"].to(device=device, dtype=torch.float32)
+
+        def forward(self, x, out, rows=None):
+            picked = x if rows is None else x[rows.long()]
+            out.copy_(picked * torch.rsqrt(picked.pow(2).mean(dim=-1, keepdim=True) + self.spec.eps) * self.weight)
+
+    register_norm("toy_rms", RootMeanSquare)
+    name = "D"
+    cfg = helpers.flat_config(name)
+    spec = get_spec("moondream2")
+    base = spec.build_plan(spec.read_config(helpers.CONFIGS[name]))
+    rms = NormSpec("toy_rms", cfg["dim"], 1e-5, bias=False)
+    layers = tuple(replace(layer, norm=rms, names={k: v for k, v in layer.names.items() if k != "norm.bias"})
+                   for layer in base.layers)
+    plan = replace(base, layers=layers, final_norm=rms, names={k: v for k, v in base.names.items() if k != "final_norm.bias"})
+    model = DecoderModel(plan)
+    weights = {k: v.float() for k, v in helpers.stored_weights(helpers.model_dir(name)).items() if k in model.params()}
+    assert set(weights) == set(model.params())
+    model.bind({k: v.to(dtype) if v.dim() == 2 else v for k, v in weights.items()}, dtype, DEV)
+
+    def rms_norm(x, weight):
+        return x / torch.sqrt(x.pow(2).mean(dim=-1, keepdim=True) + 1e-5) * weight
+
+    ids = helpers.random_ids(71, 40, cfg["vocab_size"])
+    w = {k: v.double() for k, v in weights.items()}
+    x = w["text.wte"][torch.tensor(ids)]
+    positions = torch.arange(len(ids))
+    allowed = plain.visibility(positions, None)
+    table = plain.rotary_table(plain.rotary_dim_of(cfg), len(ids), float(cfg["rope_theta"]))
+    for index in range(cfg["n_layers"]):
+        prefix = f"text.blocks.{index}."
+        xn = rms_norm(x, w[prefix + "ln.weight"])
+        x = x + plain.attention(xn, w, prefix, cfg, positions, allowed, table) + plain.mlp(xn, w, prefix)
+    expected = plain.linear(rms_norm(x, w["text.post_ln.weight"]), w["text.lm_head.weight"], w["text.lm_head.bias"])
+    for graphs in (False, True):
+        runner = make_runner(model, 16, 8, 2, enable_graphs=graphs)
+        slot = runner.admit()
+        got = [runner.step([StepEntry(slot, ids[:26], want=list(range(26)))]).clone()]
+        got += [runner.step([StepEntry(slot, [t], want=[0])]).clone() for t in ids[26:]]
+        assert (runner.graph_replays > 0) == graphs
+        helpers.assert_close(torch.cat(got), expected, dtype, f"another norm, graphs={graphs}")
+        runner.release(slot)
+
+
 @dataclass(frozen=True)
 class GridPositionSpec:
     kind: str
