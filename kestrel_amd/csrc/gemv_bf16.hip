@@ -378,7 +378,8 @@ KA_API void ka_skinny_set_wide(int enabled) { sk_wide_enabled = enabled; }
 template <int PER, int MB, bool HALF, bool LN>
 static int launch_persistent_one(int grid, size_t dyn, int strips, hipStream_t stream, const SkinnyArgs& args) {
     // two strips ahead where one workgroup has a CU (and its registers) to itself (three, which the
-    // registers would still hold, were measured slower: 6.56k against 6.72k tok/s at batch 8)
+    // registers would still hold, were measured slower: 6.56k against 6.72k tok/s at batch 8; for five
+    // k-blocks a wave, K = 2560, likewise: 523 against 537 tok/s at one row)
     constexpr int DEPTH = LN && PER <= 4 ? 3 : 2;
     if (dyn > 0) {
         static size_t reserved = 0;
@@ -399,7 +400,13 @@ static int launch_persistent_per(int per, int grid, size_t dyn, int strips, hipS
     if (per <= 1) return launch_persistent_one<1, MB, HALF, LN>(grid, dyn, strips, stream, args);
     if (per <= 2) return launch_persistent_one<2, MB, HALF, LN>(grid, dyn, strips, stream, args);
     if (per <= 4) return launch_persistent_one<4, MB, HALF, LN>(grid, dyn, strips, stream, args);
-    if constexpr (MB == 1) return launch_persistent_one<8, MB, HALF, LN>(grid, dyn, strips, stream, args);
+    if constexpr (MB == 1) {
+        // (a wave's k-blocks beyond K are loaded from inside and multiplied with zeros: a K of 2560, five blocks
+        // a wave, took 26.6 us in the form for eight where the form for five takes its share of them)
+        if (per <= 5) return launch_persistent_one<5, MB, HALF, LN>(grid, dyn, strips, stream, args);
+        if (per <= 6) return launch_persistent_one<6, MB, HALF, LN>(grid, dyn, strips, stream, args);
+        return launch_persistent_one<8, MB, HALF, LN>(grid, dyn, strips, stream, args);
+    }
     return 1;
 }
 
