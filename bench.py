@@ -263,10 +263,11 @@ def run_workload(args, sizes: dict) -> dict:
     n_requests, n_new = (256, 128) if waves else (48, 128)
     if waves:
         cfg = RuntimeConfig(model_path=folder, dtype=args.dtype, max_batch_size=args.max_batch_size or 64,
-                            kv_cache_bytes=60 * 10 ** 9 * args.layers // sizes["n_layers"], max_seq_len=2048, seed=seed)
+                            kv_cache_bytes=60 * 10 ** 9 * args.layers // sizes["n_layers"], max_seq_len=2048, seed=seed,
+                            tune_linears=args.tune_linears)
     else:
         cfg = RuntimeConfig(model_path=folder, dtype=args.dtype, max_batch_size=args.max_batch_size or 48,
-                            max_num_batched_tokens=512, max_seq_len=2048, seed=seed)
+                            max_num_batched_tokens=512, max_seq_len=2048, seed=seed, tune_linears=args.tune_linears)
     started = time.perf_counter()
     engine = InferenceEngine.create_sync(cfg)
     loaded = time.perf_counter() - started
@@ -346,6 +347,8 @@ def main() -> int:
     parser.add_argument("--peaks", action=argparse.BooleanOptionalAction, default=True,
                         help="also measure a plain read stream and a loop of matrix instructions on this GPU and report "
                              "against them (about 0.1 s; --no-peaks leaves it out)")
+    parser.add_argument("--tune-linears", type=int, default=0,
+                        help="with --workload: RuntimeConfig.tune_linears (time the vendor library's algorithms at warm-up)")
     parser.add_argument("--check", type=int, default=0,
                         help="with --workload: compare this many greedy requests with the plain implementation (for --layers 2)")
     parser.add_argument("--workload", default="decode", choices=["decode", "waves256", "mixed48"],

@@ -32,6 +32,9 @@ def _add_runtime_options(parser: argparse.ArgumentParser) -> None:
                         help="2: launch a step before the previous step's tokens have reached the host")
     parser.add_argument("--no-warmup", action="store_true",
                         help="do not capture the decode graphs and make scratch memory and plans at start")
+    parser.add_argument("--tune-linears", type=int, default=0,
+                        help="at warm-up, time the vendor library's algorithms for the prompt's linears (this many products "
+                             "each) once per bucket of rows and keep the fastest; 0: the first the library names")
     parser.add_argument("--log-level", default="WARNING", choices=["DEBUG", "INFO", "WARNING", "ERROR"],
                         help="what the engine's logger reports on stderr (INFO: load, pool size, warm-up)")
 
@@ -61,7 +64,7 @@ def _generate(args) -> int:
                         kv_cache_pages=args.kv_cache_pages, kv_cache_bytes=args.kv_cache_bytes,
                         max_num_batched_tokens=args.max_num_batched_tokens,
                         seed=args.seed, enable_graphs=not args.disable_graphs, pipeline_depth=args.pipeline_depth,
-                        warmup=not args.no_warmup)
+                        warmup=not args.no_warmup, tune_linears=args.tune_linears)
     engine = InferenceEngine.create_sync(cfg)
     try:
         if args.random_prompts:

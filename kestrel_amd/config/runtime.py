@@ -46,6 +46,9 @@ class RuntimeConfig:
     ``warmup``: make everything at start that steps would otherwise make when they first need it (the
     graph of every bucket of decode rows, scratch buffers, the plans of the prompt's linears), as
     the reference does before ``create`` returns (``kestrel/engine/core.py:458-484``).
+    ``tune_linears``: with ``warmup``, the linears of prompt steps that go through the vendor library time the
+    algorithms it offers (that many products each) once per bucket of rows and keep the fastest; 0: the first
+    the library names. Which algorithm wins can differ from start to start, and with it the last bits of a result.
     """
 
     model_path: Union[str, Path, None] = None
@@ -63,6 +66,7 @@ class RuntimeConfig:
     seed: int = 0
     max_seq_len: Optional[int] = None
     warmup: bool = True
+    tune_linears: int = 0
 
     def __post_init__(self) -> None:
         self.dtype = parse_dtype(self.dtype)
@@ -80,6 +84,8 @@ class RuntimeConfig:
             raise ValueError("give one of kv_cache_pages, kv_cache_tokens and kv_cache_bytes")
         if self.max_num_batched_tokens <= 0:
             raise ValueError("max_num_batched_tokens must be a positive integer")
+        if self.tune_linears < 0:
+            raise ValueError("tune_linears must be zero or a positive number of timed products")
         if self.pipeline_depth not in (1, 2):
             raise ValueError("pipeline_depth must be 1 or 2")
         if self.max_seq_len is not None and self.max_seq_len <= 0:

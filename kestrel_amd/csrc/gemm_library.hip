@@ -26,6 +26,7 @@
 #include <map>
 #include <mutex>
 #include <tuple>
+#include <vector>
 
 namespace {
 
@@ -39,6 +40,7 @@ struct Plan {
     hipblasLtMatmulAlgo_t algo;
     bool usable = false;
     bool every_count = true;       // false once the library has refused the algorithm for a row count of the bucket
+    std::vector<hipblasLtMatmulAlgo_t> candidates;     // what the heuristic named, until the plan has been tuned
     int rows_set = 0;              // the row count the layouts of a and out stand at
     unsigned long used = 0;        // the call that used the plan last
 };
@@ -50,7 +52,8 @@ using Key = std::tuple<int, int, int, int, long, long, long, int, int, int, int,
 std::mutex g_lock;
 hipblasLtHandle_t g_handle[LT_MAX_DEVICES];
 std::map<Key, Plan> g_plans;
-unsigned long g_calls = 0, g_heuristic_calls = 0, g_evicted = 0;
+unsigned long g_calls = 0, g_heuristic_calls = 0, g_evicted = 0, g_tuned = 0, g_tuned_other = 0;
+int g_tune_runs = 0;               // > 0: a new plan times the heuristic's candidates on its first call (ka_linear_library_set_tuning)
 
 bool epilogue_of(int act, bool bias, hipblasLtEpilogue_t* epilogue) {
     switch (act) {
@@ -122,10 +125,11 @@ Plan make_plan(hipblasLtHandle_t handle, int rows, int N, int K, long lda, long 
                  hipblasLtMatmulAlgoGetHeuristic(handle, plan.desc, plan.w, plan.a, plan.out, plan.out, preference,
                                                  LT_CANDIDATES, candidates, &n) == HIPBLAS_STATUS_SUCCESS;
             if (ok) {
-                for (int i = 0; i < n && !plan.usable; ++i) {
+                for (int i = 0; i < n; ++i) {
                     if (candidates[i].state != HIPBLAS_STATUS_SUCCESS || candidates[i].workspaceSize > workspace_bytes) continue;
-                    plan.algo = candidates[i].algo;
+                    if (!plan.usable) plan.algo = candidates[i].algo;
                     plan.usable = true;
+                    plan.candidates.push_back(candidates[i].algo);
                 }
             }
             hipblasLtMatmulPreferenceDestroy(preference);
@@ -143,6 +147,49 @@ Plan* plan_for(hipblasLtHandle_t handle, const Key& key, int rows, int N, int K,
     }
     found->second.used = ++g_calls;
     return &found->second;
+}
+
+// Times every algorithm the heuristic named for this plan on the operands of the call at hand and keeps the
+// fastest (the first named is the fastest at most sizes, but not at all: q|k|v of 2048 x 6144 at 1,318 rows
+// 34.6 against 42.7 us). Only while tuning is switched on, which the engine does during its warm-up: the
+// products are run several times over (a sum into the output is added several times), so the operands must
+// be ones whose content nobody needs, and the stream must not be capturing. The stream is waited for.
+void tune(hipblasLtHandle_t handle, Plan* plan, const float* alpha, const float* beta, const void* W, const void* A, void* out,
+          void* workspace, size_t workspace_bytes, hipStream_t stream) {
+    std::vector<hipblasLtMatmulAlgo_t> candidates;
+    candidates.swap(plan->candidates);                  // (whatever happens, the plan is not tuned twice)
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (candidates.size() < 2 || hipStreamIsCapturing(stream, &capturing) != hipSuccess || capturing != hipStreamCaptureStatusNone) return;
+    hipEvent_t start = nullptr, stop = nullptr;
+    if (hipEventCreate(&start) != hipSuccess || hipEventCreate(&stop) != hipSuccess) {
+        if (start) hipEventDestroy(start);
+        return;
+    }
+    float best = 0.f;
+    int best_index = -1;
+    for (size_t i = 0; i < candidates.size(); ++i) {
+        auto run = [&]() {
+            return hipblasLtMatmul(handle, plan->desc, alpha, W, plan->w, A, plan->a, beta, out, plan->out, out, plan->out,
+                                   &candidates[i], workspace, workspace_bytes, stream) == HIPBLAS_STATUS_SUCCESS;
+        };
+        if (!run()) continue;                           // (once untimed: the kernel's code is loaded)
+        bool ok = hipEventRecord(start, stream) == hipSuccess;
+        for (int r = 0; r < g_tune_runs && ok; ++r) ok = run();
+        float ms = 0.f;
+        ok = ok && hipEventRecord(stop, stream) == hipSuccess && hipEventSynchronize(stop) == hipSuccess &&
+             hipEventElapsedTime(&ms, start, stop) == hipSuccess;
+        if (ok && (best_index < 0 || ms < best)) {
+            best = ms;
+            best_index = (int)i;
+        }
+    }
+    hipEventDestroy(start);
+    hipEventDestroy(stop);
+    if (best_index >= 0) {
+        plan->algo = candidates[best_index];
+        ++g_tuned;
+        if (best_index > 0) ++g_tuned_other;
+    }
 }
 
 // The layouts of a plan's A and out at M rows (they are made at the bucket's edge).
@@ -201,6 +248,8 @@ KA_API int ka_linear_library_bf16(const void* A, long lda, const void* W, long l
             hipblasStatus_t s = hipblasLtMatmulDescSetAttribute(plan->desc, HIPBLASLT_MATMUL_DESC_BIAS_POINTER, &bias, sizeof(bias));
             KA_CHECK(s == HIPBLAS_STATUS_SUCCESS, "%s: cannot set the bias (status %d)", who, (int)s);
         }
+        if (g_tune_runs > 0 && !plan->candidates.empty())
+            tune(g_handle[device], plan, &alpha, &beta, W, A, out, workspace, (size_t)workspace_bytes, stream);
         hipblasStatus_t s = hipblasLtMatmul(g_handle[device], plan->desc, &alpha, W, plan->w, A, plan->a, &beta, out, plan->out,
                                             out, plan->out, &plan->algo, workspace, (size_t)workspace_bytes, stream);
         if (s == HIPBLAS_STATUS_SUCCESS) return 0;
@@ -214,10 +263,20 @@ KA_API int ka_linear_library_bf16(const void* A, long lda, const void* W, long l
 }
 
 // For measurements and tests: how many plans are kept, how often the heuristic was asked, how many
-// plans had to make room.
-KA_API void ka_linear_library_stats(long* plans, long* heuristic_calls, long* evicted) {
+// plans had to make room, how many were tuned and how many of those took another algorithm than the first named.
+KA_API void ka_linear_library_stats(long* plans, long* heuristic_calls, long* evicted, long* tuned, long* tuned_other) {
     std::lock_guard<std::mutex> hold(g_lock);
     if (plans) *plans = (long)g_plans.size();
     if (heuristic_calls) *heuristic_calls = (long)g_heuristic_calls;
     if (evicted) *evicted = (long)g_evicted;
+    if (tuned) *tuned = (long)g_tuned;
+    if (tuned_other) *tuned_other = (long)g_tuned_other;
+}
+
+// `runs` > 0: from now on a plan's first call times the algorithms the heuristic named, `runs` products each, on
+// that call's operands and keeps the fastest (see `tune`: only for operands whose content nobody needs: a
+// warm-up). 0: plans take the first algorithm named (the default).
+KA_API void ka_linear_library_set_tuning(int runs) {
+    std::lock_guard<std::mutex> hold(g_lock);
+    g_tune_runs = runs > 0 ? runs : 0;
 }

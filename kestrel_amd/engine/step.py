@@ -566,14 +566,16 @@ class ModelRunner:
 
     # ------------------------------------------------------------------ everything made at start
     @torch.inference_mode()
-    def prepare(self, prompt_tokens: Optional[int] = None, wanted_rows: int = 1) -> Dict[str, float]:
+    def prepare(self, prompt_tokens: Optional[int] = None, wanted_rows: int = 1, tune_linears: int = 0) -> Dict[str, float]:
         """Make now what steps would otherwise make when they first need it, with live requests
         waiting (``kestrel/runtime/decode_graph.py:70-93``, ``kestrel/models/moondream/runtime.py:886-888``,
         ``kestrel/engine/core.py:458-484``): the kernels' scratch buffers, the graph of every bucket of
         decode rows (captured on padding rows), the metadata buffer at its largest, and the scratch
         tensors and vendor-library plans of prompt steps, by running prompts of ids 0 of every
         multiple of 64 tokens up to ``prompt_tokens`` (default: the step's token limit) through a slot
-        that is given back. No request may be live. Returns what was done and how long it took."""
+        that is given back. ``tune_linears`` > 0: the vendor-library linears of these prompts time the algorithms
+        the library offers, that many products each, and keep the fastest per bucket of rows. No request may be
+        live. Returns what was done and how long it took."""
         if self.held:
             raise RuntimeError("prepare() runs before the first request is admitted")
         import time
@@ -603,14 +605,22 @@ class ModelRunner:
         if self.model.dtype != torch.bfloat16:
             sizes = sizes[:1] + ([64] if fits > 64 else [])      # no library plans on the 32-bit path
         prompt_started = time.perf_counter()
-        for tokens in sizes:
-            if not cache.can_admit(tokens, tokens):
-                continue
-            slot = self.admit(tokens, tokens)
-            try:
-                self.step([StepEntry(slot, np.zeros(tokens, dtype=np.int64), want=list(range(min(tokens, wanted_rows, rows))))])
-            finally:
-                self.release(slot)
+        tuning = tune_linears > 0 and self.model.dtype == torch.bfloat16
+        if tuning:
+            fast.set_library_tuning(tune_linears)      # (the plans made by these prompts time their candidates)
+        try:
+            for tokens in sizes:
+                if not cache.can_admit(tokens, tokens):
+                    continue
+                slot = self.admit(tokens, tokens)
+                try:
+                    self.step([StepEntry(slot, np.zeros(tokens, dtype=np.int64), want=list(range(min(tokens, wanted_rows, rows))))])
+                finally:
+                    self.release(slot)
+        finally:
+            if tuning:
+                fast.set_library_tuning(0)
+                done.update({f"library_{k}": v for k, v in fast.library_stats().items()})
         torch.cuda.synchronize(self.device)
         done["prompt_steps"] = len(sizes)
         done["prompt_s"] = time.perf_counter() - prompt_started

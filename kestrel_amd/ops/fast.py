@@ -133,7 +133,9 @@ def lib():
             fn.argtypes = argtypes
             fn.restype = _c_int
         handle.ka_last_error.restype = ctypes.c_char_p
-        handle.ka_linear_library_stats.argtypes = [ctypes.POINTER(ctypes.c_long)] * 3
+        handle.ka_linear_library_stats.argtypes = [ctypes.POINTER(ctypes.c_long)] * 5
+        handle.ka_linear_library_set_tuning.argtypes = [_c_int]
+        handle.ka_linear_library_set_tuning.restype = None
         handle.ka_linear_library_stats.restype = None
         handle.ka_skinny_set_persistent.argtypes = [_c_int]
         handle.ka_skinny_set_persistent.restype = None
@@ -221,11 +223,19 @@ def prepare(device: torch.device) -> int:
 
 def library_stats() -> Dict[str, int]:
     """Plans the vendor-library linears keep, how often the library's heuristic was asked for an
-    algorithm, and how many plans had to make room (all since the process started)."""
+    algorithm, how many plans had to make room, how many were tuned and how many of those took another
+    algorithm than the first named (all since the process started)."""
     handle = lib()
-    values = [ctypes.c_long(0) for _ in range(3)]
+    values = [ctypes.c_long(0) for _ in range(5)]
     handle.ka_linear_library_stats(*[ctypes.byref(v) for v in values])
-    return dict(zip(("plans", "heuristic_calls", "evicted"), (int(v.value) for v in values)))
+    return dict(zip(("plans", "heuristic_calls", "evicted", "tuned", "tuned_other"), (int(v.value) for v in values)))
+
+
+def set_library_tuning(runs: int) -> None:
+    """``runs`` > 0: a plan of the vendor-library linears that is made from now on times, at its first call, every
+    algorithm the library's heuristic named (``runs`` products each, on that call's operands, whose content is
+    run over several times: a warm-up's) and keeps the fastest. 0 (the default): the first named."""
+    lib().ka_linear_library_set_tuning(int(runs))
 
 
 def _operand_ok(t: torch.Tensor, k: int) -> bool:

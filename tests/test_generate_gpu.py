@@ -510,3 +510,26 @@ def test_a_prompt_with_two_blocks_of_given_embeddings(dtype):
     causal = plain.forward(cfg, weights, [], prefix_embeds=torch.cat(embedded), block_ids=[-1] * len(ids))[-1]
     assert float((causal - logits[len(ids) - 1]).abs().max()) > 1e-3
     helpers.assert_greedy_follows(cfg, weights, other, beside.tokens, slack, f"beside the blocks, {dtype}")
+
+
+def test_linears_tuned_at_warm_up_give_the_same_tokens():
+    """``tune_linears``: the warm-up's prompts time the vendor library's algorithms for every bucket of rows and keep
+    the fastest. Whatever it picks, generation stays the plain implementation's (prompts long enough for their
+    linears to go through the library: more than 64 rows)."""
+    from kestrel_amd.ops import fast
+
+    name = "D"
+    cfg = helpers.flat_config(name)
+    weights = helpers.stored_weights(helpers.model_dir(name))
+    before = fast.library_stats()
+    engine = _engine(name, "bfloat16", max_num_batched_tokens=192, kv_cache_pages=64, tune_linears=2)
+    try:
+        after = fast.library_stats()
+        assert after["tuned"] > before["tuned"], (before, after)
+        prompts = [helpers.random_ids(2000 + i, n, cfg["vocab_size"]) for i, n in enumerate((150, 70, 9))]
+        results = engine.generate_batch_sync(prompts, max_new_tokens=8, stop_ids=())
+        assert fast.library_stats()["tuned"] == after["tuned"], "nothing is timed once the warm-up is over"
+    finally:
+        engine.shutdown_sync()
+    for prompt, result in zip(prompts, results):
+        helpers.assert_greedy_follows(cfg, weights, prompt, result.tokens, 5e-2, "tuned linears")
