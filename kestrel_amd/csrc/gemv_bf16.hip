@@ -406,13 +406,19 @@ static int launch_persistent_per(int per, int grid, size_t dyn, int strips, hipS
         if (per <= 5) return launch_persistent_one<5, MB, HALF, LN>(grid, dyn, strips, stream, args);
         if (per <= 6) return launch_persistent_one<6, MB, HALF, LN>(grid, dyn, strips, stream, args);
         return launch_persistent_one<8, MB, HALF, LN>(grid, dyn, strips, stream, args);
+    } else {
+        if (per <= 5) return launch_persistent_one<5, MB, HALF, LN>(grid, dyn, strips, stream, args);
     }
     return 1;
 }
 
+// Most k-blocks a wave keeps activations for when there are more than 16 rows of them: K up to 2560 (at 64 rows
+// the form for five blocks fills a lane's 256 registers and spills five of them).
+constexpr int SP_MAX_PER_MANY_ROWS = 5;
+
 static bool persistent_fits(int M, int kblocks, const SkinnyArgs& args) {
     const int per = ka_cdiv(kblocks, SP_WAVES);
-    return per <= (M <= 16 ? SP_MAX_PER : 4) && persistent_bias_ok(args.a) && persistent_bias_ok(args.b);
+    return per <= (M <= 16 ? SP_MAX_PER : SP_MAX_PER_MANY_ROWS) && persistent_bias_ok(args.a) && persistent_bias_ok(args.b);
 }
 
 static int launch_persistent(int strips, int M, int kblocks, bool ln, size_t dyn, hipStream_t stream,
