@@ -178,7 +178,8 @@ def time_prefill(net, typed, tokens, repeats=8):
     from kestrel_amd.engine.loading import make_runner
     from kestrel_amd.engine.step import StepEntry
 
-    runner = make_runner(net, PAGE_SIZE, -(-tokens // PAGE_SIZE) + 1, 1, max_tokens_per_step=tokens)
+    # (as the engine runs it: a step short enough for the host's launches to take longer than its kernels is a replayed graph)
+    runner = make_runner(net, PAGE_SIZE, -(-tokens // PAGE_SIZE) + 1, 1, max_tokens_per_step=tokens, enable_graphs=True)
     gen = torch.Generator().manual_seed(SEED + 1)
     prefix = min(typed.prefix_attn, tokens - 1)
     embeds = torch.randn(prefix, typed.dim, generator=gen).to(net.device)

@@ -68,11 +68,13 @@ KA_API int ka_adjust_logits(float* logits, long count, float scale, float cap, h
     return 0;
 }
 
-// out[rows[i], :] = src[i, :] (given embeddings spliced into the stream).
+// out[rows[i], :] = src[i, :] (given embeddings spliced into the stream); a negative row: nothing
+// (the unused end of a list of fixed length).
 template <typename T>
 __global__ void scatter_rows_kernel(const T* __restrict__ src, const int* __restrict__ rows,
                                     float* __restrict__ out, int dim) {
     int i = blockIdx.x;
+    if (rows[i] < 0) return;
     const T* s = src + (size_t)i * dim;
     float* dst = out + (size_t)rows[i] * dim;
     for (int d = threadIdx.x; d < dim; d += blockDim.x) dst[d] = ka_to_float(s[d]);

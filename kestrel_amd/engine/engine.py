@@ -202,8 +202,9 @@ class InferenceEngine:
             # graphs, scratch memory and plans now, not in the middle of the first steps that need them
             done = self.runner.prepare(cfg.max_num_batched_tokens, wanted_rows=cfg.max_batch_size, tune_linears=cfg.tune_linears)
             sampler.reserve(cfg.max_batch_size)
-            _LOGGER.info("warm-up: %d decode graphs captured in %.2f s, %d prompt steps in %.2f s, %.0f MiB of kernel scratch",
-                         int(done.get("graphs", 0)), done.get("capture_s", 0.0), int(done.get("prompt_steps", 0)),
+            _LOGGER.info("warm-up: %d decode graphs and %d graphs of other steps captured in %.2f s, %d prompt steps in %.2f s, "
+                         "%.0f MiB of kernel scratch",
+                         int(done.get("graphs", 0)), int(done.get("step_graphs", 0)), done.get("capture_s", 0.0), int(done.get("prompt_steps", 0)),
                          done.get("prompt_s", 0.0), done.get("kernel_scratch_bytes", 0) / float(1 << 20))
             if "library_tuned" in done:
                 _LOGGER.info("warm-up: %d plans of the vendor library timed, %d of them took another algorithm than the first named",

@@ -13,6 +13,13 @@ size bucket (1, 2, 4, 8, 16, 32, 48, ... as in ``kestrel/runtime/decode_graph.py
 metadata lives at fixed addresses, rows that pad the bucket see no keys and write nothing. A graph
 is captured, and run once before that, on padding rows alone: no live request is touched by
 anything but the replays, so a mixer that keeps state is advanced once a step.
+
+Steps of any other shape (a prompt portion, alone or beside decoded tokens) of up to
+``MIXED_GRAPH_MAX_TOKENS`` tokens are replayed as well where every part of the model allows it
+(``Part.replays_every_step``), one graph per bucket of tokens and of rows: launching a layer's kernels
+one by one costs the host about 0.13 ms, which is more than the kernels of a short portion take.
+Their layout is fixed by the bucket (``ModelRunner.build_batch`` with ``pad_tokens``); longer steps, and
+steps that want more logits than the largest bucket of rows, are launched kernel by kernel.
 """
 
 from __future__ import annotations
@@ -82,6 +89,26 @@ def graph_buckets(max_batch: int) -> List[int]:
     return sorted(sizes)
 
 
+# Steps of any shape are captured up to this many tokens: beyond, a step's kernels take longer than the
+# host needs to launch them one by one, and a graph would gain nothing.
+MIXED_GRAPH_MAX_TOKENS = 1024
+
+
+def mixed_graph_buckets(max_tokens: int) -> List[int]:
+    """Token counts that steps of any shape are captured for: 16, 32, every multiple of 64 up to 512, every
+    multiple of 128 up to ``MIXED_GRAPH_MAX_TOKENS``, and the step's token limit itself where that is less."""
+    top = max(1, min(int(max_tokens), MIXED_GRAPH_MAX_TOKENS))
+    sizes = {size for size in (16, 32, *range(64, 513, 64), *range(640, MIXED_GRAPH_MAX_TOKENS + 1, 128)) if size <= top}
+    sizes.add(top)
+    return sorted(sizes)
+
+
+def mixed_graph_rows(max_requests: int) -> List[int]:
+    """Numbers of rows (requests, and wanted places) that steps of any shape are captured for."""
+    top = max(1, int(max_requests))
+    return sorted({min(8, top), min(64, top), top})
+
+
 class _Column:
     """The int32 values of one section of a step's metadata, gathered piece by piece: lists from
     rows of a few tokens, arrays from prompt portions (thousands of tokens, which are never
@@ -115,13 +142,14 @@ class _Column:
 
 
 class _GraphState:
-    """A captured decode step of one bucket size: its metadata, scratch and graph."""
+    """A captured step of one bucket size: its metadata, scratch and graph."""
 
     def __init__(self, device: torch.device) -> None:
         self.workspace = Workspace(device)
         self.meta: Optional[torch.Tensor] = None
         self.graph: Optional[torch.cuda.CUDAGraph] = None
         self.logits: Optional[torch.Tensor] = None
+        self.given: Optional[torch.Tensor] = None      # steps of any shape: where given embeddings are copied to
 
 
 class _PageRuns:
@@ -197,6 +225,14 @@ class ModelRunner:
         self._graphs: Dict[int, _GraphState] = {}
         self._pages_cap = -(-model.plan.max_positions // cache.page_size)
         self.graph_replays = 0
+        # steps of any shape (prompt portions, beside decoded tokens or not) are replayed too, if every
+        # part of the model can be (``Part.replays_every_step``): per bucket of tokens and of rows
+        every = getattr(model, "replays_every_step", None)
+        self.mixed_graphs = bool(enable_graphs and callable(every) and every())
+        self._mixed_tokens = mixed_graph_buckets(max_tokens_per_step)
+        self._mixed_rows = mixed_graph_rows(cache.max_requests)
+        self._mixed: Dict[Tuple[int, int], _GraphState] = {}      # (tokens, rows) -> the captured step
+        self.mixed_graph_replays = 0
         self.logit_slots: Optional[torch.Tensor] = None     # of the last step: the slot per row of logits, on the device
         # the latest sampled token of every request slot, written by the sampling kernels
         self.pending = torch.zeros(max(1, cache.max_requests), dtype=torch.int32, device=device)
@@ -298,13 +334,22 @@ class ModelRunner:
         return starts
 
     def build_batch(self, entries: Sequence[StepEntry], pad_rows: int = 0, fixed_pages: int = 0,
-                    meta: Optional[torch.Tensor] = None, workspace: Optional[Workspace] = None) -> StepBatch:
+                    meta: Optional[torch.Tensor] = None, workspace: Optional[Workspace] = None,
+                    pad_tokens: int = 0) -> StepBatch:
         """Checks the entries, backs their positions with pages and lays the metadata out.
 
         ``pad_rows`` > number of entries adds rows of one token that see no keys and write
         nothing; ``fixed_pages`` fixes the width of the block tables; ``meta`` is the device
         buffer the metadata is copied into. With all three the layout depends on ``pad_rows``
         alone, which is what a captured graph needs.
+
+        ``pad_tokens`` > 0 (with ``pad_rows`` and ``fixed_pages``) lays out a step of any shape so that the
+        layout depends on ``pad_tokens`` and ``pad_rows`` alone: ``pad_rows + 1`` rows, of which those
+        behind the entries hold no token and the last holds the tokens that fill the step up to
+        ``pad_tokens`` (they see no keys and write nothing); ``pad_rows`` wanted places (those behind
+        the entries' name token 0, for nobody); as many places for given rows as tokens (-1 behind
+        the entries'); the lists of runs and of blocks of queries at the most entries any such step
+        can have (runs without tokens and blocks without queries behind the step's own).
         """
         cache, plan = self.cache, self.model.plan
         ps = cache.page_size
@@ -408,7 +453,39 @@ class ModelRunner:
                 if kv_lo[g] is not None:
                     kv_lo[g].extend(cache.window_start(g, p) for p in range(start, start + q))
         n_real = len(entries)
-        for r in range(n_real, pad_rows):          # rows that only fill the bucket
+        n_wanted = len(logit_rows)
+        if pad_tokens:
+            n_live = len(ids)
+            if n_live > pad_tokens or n_real > pad_rows or n_wanted > pad_rows or not fixed_pages:
+                raise ValueError(f"{n_live} tokens of {n_real} rows with {n_wanted} wanted places do not fit a step "
+                                 f"laid out for {pad_tokens} tokens and {pad_rows} rows")
+            fill = pad_tokens - n_live
+            cu_q.extend([n_live] * (pad_rows - n_real))            # rows without a token
+            kv_len.extend([0] * (pad_rows - n_real))
+            row_slot.extend([-1] * (pad_rows - n_real))
+            if fill:                                               # the last row: what fills the step up
+                zeros = np.zeros(fill, dtype=np.int64)
+                runs.add(n_live, 0, fill)
+                ids.extend(zeros)
+                positions.extend(zeros)
+                token_row.extend(np.full(fill, pad_rows, dtype=np.int64))
+                kv_hi.extend(zeros)
+                if axes is not None:
+                    axes.extend(np.zeros(fill * n_axes, dtype=np.int64))
+                for tile, listed in blocks.items():
+                    listed.extend((pad_rows, n_live + first, 0) for first in range(0, fill, tile))
+                for g in range(n_groups):
+                    slots[g].extend(np.full(fill, -1, dtype=np.int64))
+                    if kv_lo[g] is not None:
+                        kv_lo[g].extend(zeros)
+            cu_q.append(pad_tokens)
+            kv_len.append(0)
+            row_slot.append(-1)
+            logit_rows.extend([0] * (pad_rows - n_wanted))
+            logit_slot.extend([-1] * (pad_rows - n_wanted))
+            given_rows = given_rows + [-1] * (pad_tokens - len(given_rows))
+            pad_rows += 1                                          # (the last row is one of the step's rows)
+        for r in range(n_real, 0 if pad_tokens else pad_rows):     # rows that only fill the bucket, a token each
             runs.add(len(ids), 0, 1)
             ids.append(0)
             positions.append(0)
@@ -433,12 +510,21 @@ class ModelRunner:
         # the blocks that see the most keys first: a launch then ends with short ones
         for listed in blocks.values():
             listed.sort(key=lambda b: -b[2])
+        run_first, run_count = runs.first(), runs.count()
+        if pad_tokens:
+            # every row with tokens has at most one block that is not full, and at most two runs that are no whole page
+            most_runs = pad_tokens // ps + 2 * n_rows
+            run_first = run_first + [0] * (most_runs - len(run_first))
+            run_count = run_count + [0] * (most_runs - len(run_count))
+            for tile, listed in blocks.items():
+                # (a block of the last row that starts behind its last token: no query in it is live)
+                listed.extend([(n_rows - 1, pad_tokens, 0)] * (pad_tokens // tile + n_rows - len(listed)))
         # one packed int32 buffer, every section starting on a 16-byte boundary
         sections: List[Tuple[str, object]] = [
             ("ids", ids), ("positions", positions), ("token_row", token_row), ("kv_hi", kv_hi),
             ("row_slot", row_slot), ("cu_q", cu_q), ("kv_len", kv_len), ("logit_rows", logit_rows),
             ("logit_slot", logit_slot),
-            ("given_rows", given_rows), ("run_first", runs.first()), ("run_count", runs.count()),
+            ("given_rows", given_rows), ("run_first", run_first), ("run_count", run_count),
         ]
         if axes is not None:
             sections.append(("position_axes", axes))
@@ -449,13 +535,12 @@ class ModelRunner:
             sections.append((f"slots{g}", slots[g]))
             if kv_lo[g] is not None:
                 sections.append((f"kv_lo{g}", kv_lo[g]))
-            flat: List[int] = []
-            for e in entries:
+            tables = np.zeros((n_rows, max_pages), dtype=np.int32)     # (rows without a request: page 0, never read)
+            for r, e in enumerate(entries):
                 table = cache.block_table(g, e.slot)
-                flat.extend(table)
-                flat.extend([-1] * (max_pages - len(table)))
-            flat.extend([0] * (max_pages * (n_rows - n_real)))
-            sections.append((f"table{g}", flat))
+                tables[r, :len(table)] = table
+                tables[r, len(table):] = -1
+            sections.append((f"table{g}", tables.reshape(-1)))
         offsets: Dict[str, Tuple[int, int]] = {}
         total = 0
         for name, values in sections:
@@ -500,8 +585,9 @@ class ModelRunner:
             workspace=workspace or self.workspace,
             query_blocks={tile: (view(f"qblk_row{tile}"), view(f"qblk_tok{tile}")) for tile in blocks},
             position_axes=view("position_axes").view(n_tokens, n_axes) if axes is not None else None,
-            pending=self.pending, given_embeds=given_embeds, given_rows=view("given_rows") if given else None, max_q=max_q, max_kv=max_kv,
-            decode_only=max_q == 1, causal_only=causal_only, wants_every_token=logit_rows == list(range(n_tokens)),
+            pending=self.pending, given_embeds=given_embeds, given_rows=view("given_rows") if given or pad_tokens else None,
+            max_q=max_q, max_kv=max_kv, decode_only=max_q == 1 and not pad_tokens, causal_only=causal_only and not pad_tokens,
+            wants_every_token=not pad_tokens and logit_rows == list(range(n_tokens)),
             page_runs=(view("run_first"), view("run_count")),
             host={"starts": starts, "q_lens": [len(e.tokens) for e in entries], "kv_len": kv_len, "meta_ints": total},
         )
@@ -555,6 +641,62 @@ class ModelRunner:
             state.graph = graph
         return state
 
+    def _mixed_bucket(self, entries: Sequence[StepEntry]) -> Optional[Tuple[int, int]]:
+        """``(tokens, rows)`` of the captured layout that a step of any shape fits in, or ``None``."""
+        if not self.mixed_graphs:
+            return None
+        try:
+            n_tokens = sum(len(e.tokens) for e in entries)
+            n_wanted = sum(len(e.want) for e in entries)
+        except TypeError:
+            return None                  # (``_check_entries`` names what is odd: the eager path)
+        n_rows = max(len(entries), n_wanted)
+        if n_tokens > self._mixed_tokens[-1] or n_rows > self._mixed_rows[-1]:
+            return None
+        return (next(t for t in self._mixed_tokens if t >= n_tokens), next(r for r in self._mixed_rows if r >= n_rows))
+
+    def _capture_mixed(self, tokens: int, rows: int) -> _GraphState:
+        """The graph of a step of up to ``tokens`` tokens of up to ``rows`` requests, made if it is not
+        there yet: as for decode steps, on tokens that belong to no request."""
+        state = self._mixed.get((tokens, rows))
+        if state is None:
+            state = self._mixed[(tokens, rows)] = _GraphState(self.device)
+        if state.graph is None:
+            layout = dict(pad_rows=rows, pad_tokens=tokens, fixed_pages=self._pages_cap)
+            probe = self.build_batch([], **layout)
+            state.meta = torch.empty(probe.host["meta_ints"], dtype=torch.int32, device=self.device)
+            state.given = torch.zeros(tokens, self.model.plan.dim, dtype=torch.float32, device=self.device)
+            blank = self.build_batch([], meta=state.meta, workspace=state.workspace, **layout)
+            blank.max_kv = self.model.plan.max_positions       # (kernels that size themselves by the longest row)
+            blank.given_embeds = state.given
+            current = torch.cuda.current_stream()
+            side = torch.cuda.Stream()
+            side.wait_stream(current)
+            with torch.cuda.stream(side):          # first run outside capture: every buffer comes into being
+                self.model.forward(blank, self.layer_caches)
+            current.wait_stream(side)
+            torch.cuda.synchronize()
+            state.workspace.freeze()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                state.logits = self.model.forward(blank, self.layer_caches)
+            state.graph = graph
+        return state
+
+    def _step_mixed(self, entries: Sequence[StepEntry], tokens: int, rows: int) -> Tuple[torch.Tensor, List[int]]:
+        if (tokens, rows) not in self._mixed:
+            self._check_entries(entries)           # (no graph is made for a step that is refused)
+        state = self._capture_mixed(tokens, rows)
+        batch = self.build_batch(entries, pad_rows=rows, pad_tokens=tokens, fixed_pages=self._pages_cap, meta=state.meta,
+                                 workspace=state.workspace)
+        if batch.given_embeds is not None:
+            state.given[:batch.given_embeds.shape[0]].copy_(batch.given_embeds)
+        state.graph.replay()
+        self.mixed_graph_replays += 1
+        wanted = sum(len(e.want) for e in entries)
+        self.logit_slots = batch.logit_slot[:wanted]
+        return state.logits[:wanted], batch.host["starts"]
+
     def _step_graph(self, entries: Sequence[StepEntry], bucket: int) -> torch.Tensor:
         state = self._capture(bucket)
         batch = self.build_batch(entries, pad_rows=bucket, fixed_pages=self._pages_cap, meta=state.meta,
@@ -570,7 +712,8 @@ class ModelRunner:
         """Make now what steps would otherwise make when they first need it, with live requests
         waiting (``kestrel/runtime/decode_graph.py:70-93``, ``kestrel/models/moondream/runtime.py:886-888``,
         ``kestrel/engine/core.py:458-484``): the kernels' scratch buffers, the graph of every bucket of
-        decode rows (captured on padding rows), the metadata buffer at its largest, and the scratch
+        decode rows and, where steps of any shape are replayed, of every bucket of tokens and rows up to
+        ``prompt_tokens`` (captured on padding rows), the metadata buffer at its largest, and the scratch
         tensors and vendor-library plans of prompt steps, by running prompts of ids 0 of every
         multiple of 64 tokens up to ``prompt_tokens`` (default: the step's token limit) through a slot
         that is given back. ``tune_linears`` > 0: the vendor-library linears of these prompts time the algorithms
@@ -592,10 +735,31 @@ class ModelRunner:
         ints = per_token * (limit + rows) + rows * (8 + len(cache.groups) * (self._pages_cap + 4)) + 4096
         if self._meta_device is None or self._meta_device.numel() < ints:
             self._meta_device = torch.empty(ints, dtype=torch.int32, device=self.device)
+        # (plans of the vendor library made from here on, by the runs before a capture or by the prompts below,
+        # time their candidates)
+        tuning = tune_linears > 0 and self.model.dtype == torch.bfloat16
+        if tuning:
+            fast.set_library_tuning(tune_linears)
+        try:
+            return self._prepare(done, started, limit, rows, wanted_rows)
+        finally:
+            if tuning:
+                fast.set_library_tuning(0)
+                done.update({f"library_{k}": v for k, v in fast.library_stats().items()})
+
+    def _prepare(self, done: Dict[str, float], started: float, limit: int, rows: int, wanted_rows: int) -> Dict[str, float]:
+        import time
+
+        cache, plan = self.cache, self.model.plan
         if self.enable_graphs:
             for bucket in self._buckets:
                 self._capture(bucket)
             done["graphs"] = len(self._buckets)
+            if self.mixed_graphs:
+                shapes = [(t, r) for t in self._mixed_tokens if t <= max(limit, self._mixed_tokens[0]) for r in self._mixed_rows]
+                for tokens, rows_here in shapes:
+                    self._capture_mixed(tokens, rows_here)
+                done["step_graphs"] = len(shapes)
             done["capture_s"] = time.perf_counter() - started
         # prompts: the largest first (every scratch tensor at its largest), then one per bucket of rows of
         # the vendor library's plans, the smallest (64 tokens: the kernels of few rows) last
@@ -605,22 +769,14 @@ class ModelRunner:
         if self.model.dtype != torch.bfloat16:
             sizes = sizes[:1] + ([64] if fits > 64 else [])      # no library plans on the 32-bit path
         prompt_started = time.perf_counter()
-        tuning = tune_linears > 0 and self.model.dtype == torch.bfloat16
-        if tuning:
-            fast.set_library_tuning(tune_linears)      # (the plans made by these prompts time their candidates)
-        try:
-            for tokens in sizes:
-                if not cache.can_admit(tokens, tokens):
-                    continue
-                slot = self.admit(tokens, tokens)
-                try:
-                    self.step([StepEntry(slot, np.zeros(tokens, dtype=np.int64), want=list(range(min(tokens, wanted_rows, rows))))])
-                finally:
-                    self.release(slot)
-        finally:
-            if tuning:
-                fast.set_library_tuning(0)
-                done.update({f"library_{k}": v for k, v in fast.library_stats().items()})
+        for tokens in sizes:
+            if not cache.can_admit(tokens, tokens):
+                continue
+            slot = self.admit(tokens, tokens)
+            try:
+                self.step([StepEntry(slot, np.zeros(tokens, dtype=np.int64), want=list(range(min(tokens, wanted_rows, rows))))])
+            finally:
+                self.release(slot)
         torch.cuda.synchronize(self.device)
         done["prompt_steps"] = len(sizes)
         done["prompt_s"] = time.perf_counter() - prompt_started
@@ -637,9 +793,12 @@ class ModelRunner:
         if not entries:
             raise ValueError("a step needs at least one entry")
         bucket = self._graph_bucket(entries)
+        mixed = self._mixed_bucket(entries) if bucket is None else None
         if bucket is not None:
             logits = self._step_graph(entries, bucket)
             starts = [self.held[e.slot] for e in entries]
+        elif mixed is not None:
+            logits, starts = self._step_mixed(entries, *mixed)
         else:
             batch = self.build_batch(entries)
             logits = self.model.forward(batch, self.layer_caches)

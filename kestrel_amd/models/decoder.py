@@ -85,6 +85,14 @@ class DecoderModel:
         parts = [self.position] + [getattr(block.mixer, "position", None) for block in self.blocks]
         return max([1] + [int(getattr(part, "axes", 1)) for part in parts if part is not None])
 
+    def replays_every_step(self) -> bool:
+        """Whether steps of every shape may be captured and replayed: every part of the model says so
+        (``Part.replays_every_step``)."""
+        parts = [self.final_norm, self.position]
+        for block in self.blocks:
+            parts += list(block.parts().values()) + [getattr(block.mixer, "position", None)]
+        return all(bool(getattr(part, "replays_every_step", False)) for part in parts if part is not None)
+
     def query_tiles(self):
         """Sizes of blocks of queries that the mixers' kernels want listed with a step."""
         return {tile for tile in (block.mixer.query_tile() for block in self.blocks) if tile}

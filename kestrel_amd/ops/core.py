@@ -70,7 +70,15 @@ def _check(status: int, handle=None) -> None:
         raise KernelError(handle.ka_last_error().decode())
 
 
+# torch's own short way to the current stream's handle (what its compiled kernels call before a launch);
+# `torch.cuda.current_stream()` builds a Python object per call: 2.8 us against 0.07 us, some 170 times a step
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
 def stream_ptr() -> int:
+    """The handle of the current stream of the current device."""
+    if _raw_stream is not None:
+        return _raw_stream(torch.cuda.current_device())
     return torch.cuda.current_stream().cuda_stream
 
 
@@ -175,7 +183,8 @@ def adjust_logits(logits: torch.Tensor, scale: float = 1.0, softcap: Optional[fl
 
 
 def scatter_rows(src: torch.Tensor, rows: torch.Tensor, out: torch.Tensor) -> None:
-    """``out[rows[i]] = src[i]`` in fp32 (given embeddings spliced into the stream)."""
+    """``out[rows[i]] = src[i]`` in fp32 (given embeddings spliced into the stream); a negative ``rows[i]``
+    is passed over."""
     _dev(src, rows, out)
     m, dim = src.shape
     _need(out.dim() == 2 and out.shape[1] == dim and out.dtype == torch.float32 and out.is_contiguous(),

@@ -30,6 +30,8 @@ class PagedAttention(Mixer):
     the input) is refused when the weights are bound, not silently turned the rotary way.
     """
 
+    replays_every_step = True
+
     def __init__(self, spec: AttentionSpec) -> None:
         super().__init__(spec)
         if spec.n_heads % spec.n_kv_heads:

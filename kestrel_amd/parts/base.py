@@ -22,6 +22,14 @@ from .specs import CacheSpec, ParamSpec, StateSpec
 class Part:
     """Common face of every part."""
 
+    # Whether steps of every shape (prompt portions beside decoded tokens), not only those of one token per
+    # request, may be captured with this part in them and replayed: its ``forward`` then neither
+    # synchronises nor allocates outside ``batch.workspace`` for any batch, takes from the host side of the
+    # batch nothing but its sizes, and passes over what pads a captured step: rows without a request
+    # (``row_slot`` -1, possibly without tokens) and tokens that see no keys and are cached nowhere
+    # (``kv_hi`` 0, slot -1). A model is replayed that way only if all of its parts say so.
+    replays_every_step: bool = False
+
     def __init__(self, spec) -> None:
         self.spec = spec
 

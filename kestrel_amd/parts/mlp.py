@@ -18,6 +18,8 @@ class DenseFeedForward(FeedForward):
     tanh approximation ``layers.py:30-31``, ``fc2``).
     """
 
+    replays_every_step = True
+
     def __init__(self, spec: DenseFeedForwardSpec) -> None:
         super().__init__(spec)
         self.act = activation_code(spec.activation)

@@ -18,6 +18,8 @@ class LayerNorm(Norm):
     eps; the modules are ``nn.LayerNorm(dim)``, ``text.py:311,359``).
     """
 
+    replays_every_step = True
+
     def __init__(self, spec: NormSpec) -> None:
         super().__init__(spec)
         self.weight: Optional[torch.Tensor] = None

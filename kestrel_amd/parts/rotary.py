@@ -18,6 +18,8 @@ class NeoxRotary(PositionEncoding):
     (``kestrel/models/moondream/rope.py:6-32``; applied at ``text.py:123-125``).
     """
 
+    replays_every_step = True
+
     def __init__(self, spec: PositionSpec) -> None:
         super().__init__(spec)
         if spec.rotary_dim % 2:
@@ -44,6 +46,8 @@ class NeoxRotary(PositionEncoding):
 
 class NoPosition(PositionEncoding):
     """Encodes nothing (a mixer whose order comes from elsewhere)."""
+
+    replays_every_step = True
 
 
 register_position("rotary_neox", NeoxRotary)

@@ -430,6 +430,8 @@ def test_everything_is_made_at_start(dtype, caplog):
         runner = engine.runner
         assert sorted(runner._graphs) == graph_buckets(6) == [1, 2, 4, 6]
         assert all(state.graph is not None for state in runner._graphs.values())
+        assert sorted(runner._mixed) == [(16, 6), (32, 6), (64, 6)]         # steps of any shape, up to the token limit of 64
+        assert all(state.graph is not None for state in runner._mixed.values())
         assert not runner.held and runner.cache.free_slots == runner.cache.max_requests
         first = engine.generate_sync(helpers.random_ids(1800, 9, cfg["vocab_size"]), max_new_tokens=4, stop_ids=())
         assert len(first.tokens) == 4
@@ -448,7 +450,7 @@ def test_everything_is_made_at_start(dtype, caplog):
     finally:
         engine.shutdown_sync()
     text = caplog.text
-    assert "warm-up: 4 decode graphs captured" in text and "cache pool: 60 pages" in text and "loaded" in text
+    assert "warm-up: 4 decode graphs and 3 graphs of other steps captured" in text and "cache pool: 60 pages" in text and "loaded" in text
     assert "refused at the door" in text and "outside the vocabulary" in text
 
 
