@@ -229,3 +229,54 @@ def test_replayed_decode_graphs_at_real_layer_sizes(sizes, dtype, monkeypatch):
         assert places and places[-1] == fed - 1
         actual = torch.stack([got[tag][p] for p in places])
         helpers.assert_close(actual, expected[places], dtype, f"{sizes} sizes, graphs, request {tag}")
+
+
+# ----------------------------------------------------------------------------------------------------
+# prompt portions replayed as HIP graphs, the vendor library's kernels among the captured
+# ----------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("sizes", ["moondream2", "phi2"])
+def test_replayed_prompt_portions_at_real_layer_sizes(sizes):
+    """What serving runs on short prompts and on portions beside decoded tokens: the graph of a bucket of
+    tokens, whose linears of more than 64 rows are the vendor library's kernels. Each graph here is replayed
+    three to five times on other tokens, with replays of other graphs and decode steps between them, and every
+    replay's logits are compared with the plain implementation (a node that a replay would run differently
+    from the capture shows as a replay that is wrong)."""
+    from kestrel_amd.engine.loading import load_model, make_runner
+    from tests.test_mixed_graphs_gpu import replay_last_places
+
+    cfg = SIZES[sizes]
+    vocab = cfg["vocab_size"]
+    lengths = {"a": 700, "b": 610, "c": 333, "d": 129}
+    reqs = {tag: Request(tag, helpers.random_ids(1600 + i, n, vocab)) for i, (tag, n) in enumerate(lengths.items())}
+    steps = [
+        [("a", 200)],                                   # 256
+        [("a", 1), ("b", 180)],                         # 256, a decoded token beside
+        [("a", 1), ("b", 1)],                           # a decode step
+        [("a", 100), ("b", 1), ("c", 20)],              # 128
+        [("a", 190), ("b", 60)],                        # 256
+        [("a", 1), ("b", 1), ("c", 1)],
+        [("a", 90), ("b", 30), ("c", 2)],               # 128
+        [("a", 117), ("b", 120), ("c", 10)],            # 256
+        [("b", 100), ("c", 15), ("d", 3)],              # 128
+        [("b", 117), ("c", 130)],                       # 256
+        [("c", 100), ("d", 26)],                        # 128
+        [("c", 55), ("d", 100)],                        # 192
+    ]
+    fed = {}
+    for step in steps:
+        for tag, count in step:
+            fed[tag] = fed.get(tag, 0) + count
+    assert fed == lengths
+    net = load_model(_folder(sizes), torch.bfloat16, torch.device("cuda:0"))
+    pages = sum(-(-n // 16) for n in lengths.values()) + 2
+    runner = make_runner(net, 16, pages, 4, max_tokens_per_step=512, enable_graphs=True)
+    helpers.poison_cache(runner)
+    got = replay_last_places(runner, reqs, steps, wanted=1)
+    assert runner.graph_replays == 2 and runner.mixed_graph_replays == len(steps) - 2
+    assert sorted(runner._mixed) == [(128, 4), (192, 4), (256, 4)]
+    weights = {k: v.double() for k, v in helpers.stored_weights(_folder(sizes)).items()}
+    for tag, req in reqs.items():
+        expected = plain.forward(cfg, weights, req.ids, None).float()
+        places = sorted(got[tag])
+        helpers.assert_close(torch.stack([got[tag][p] for p in places]), expected[places], torch.bfloat16,
+                             f"{sizes} sizes, replayed portions, request {tag}")
