@@ -27,11 +27,11 @@ def _add_runtime_options(parser: argparse.ArgumentParser) -> None:
     parser.add_argument("--kv-cache-bytes", type=int, default=None, help="size the cache pool by a byte budget instead")
     parser.add_argument("--max-num-batched-tokens", type=int, default=2048)
     parser.add_argument("--seed", type=int, default=0)
-    parser.add_argument("--disable-graphs", action="store_true", help="do not replay decode steps as HIP graphs")
+    parser.add_argument("--disable-graphs", action="store_true", help="do not replay steps as HIP graphs")
     parser.add_argument("--pipeline-depth", type=int, default=2, choices=(1, 2),
                         help="2: launch a step before the previous step's tokens have reached the host")
     parser.add_argument("--no-warmup", action="store_true",
-                        help="do not capture the decode graphs and make scratch memory and plans at start")
+                        help="do not capture the graphs and make scratch memory and plans at start")
     parser.add_argument("--tune-linears", type=int, default=0,
                         help="at warm-up, time the vendor library's algorithms for the prompt's linears (this many products "
                              "each) once per bucket of rows and keep the fastest; 0: the first the library names")

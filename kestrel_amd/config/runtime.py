@@ -39,12 +39,12 @@ class RuntimeConfig:
     none of them, for ``max_batch_size`` full contexts. A pool that does not fit in the device's
     free memory is refused at start with a ``MemoryError``.
     ``max_num_batched_tokens``: token budget of one step (prompt portions are cut to it).
-    ``enable_graphs``: replay decode-only steps as captured HIP graphs.
+    ``enable_graphs``: replay decode-only steps, and every other step of up to 1,024 tokens, as captured HIP graphs.
     ``pipeline_depth``: 2 launches a step before the tokens of the one before have reached
     the host (``kestrel/scheduler/pipeline.py:49-65``); 1 reads every step first.
     ``seed``: base of the sampling generator.
     ``warmup``: make everything at start that steps would otherwise make when they first need it (the
-    graph of every bucket of decode rows, scratch buffers, the plans of the prompt's linears), as
+    graph of every bucket of decode rows and of tokens, scratch buffers, the plans of the prompt's linears), as
     the reference does before ``create`` returns (``kestrel/engine/core.py:458-484``).
     ``tune_linears``: with ``warmup``, the linears of prompt steps that go through the vendor library time the
     algorithms it offers (that many products each) once per bucket of rows and keep the fastest; 0: the first
