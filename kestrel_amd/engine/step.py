@@ -149,7 +149,6 @@ class _GraphState:
         self.meta: Optional[torch.Tensor] = None
         self.graph: Optional[torch.cuda.CUDAGraph] = None
         self.logits: Optional[torch.Tensor] = None
-        self.given: Optional[torch.Tensor] = None      # steps of any shape: where given embeddings are copied to
 
 
 class _PageRuns:
@@ -232,6 +231,8 @@ class ModelRunner:
         self._mixed_tokens = mixed_graph_buckets(max_tokens_per_step)
         self._mixed_rows = mixed_graph_rows(cache.max_requests)
         self._mixed: Dict[Tuple[int, int], _GraphState] = {}      # (tokens, rows) -> the captured step
+        self._mixed_workspace: Optional[Workspace] = None         # their scratch tensors, shared
+        self._mixed_given: Optional[torch.Tensor] = None          # where given embeddings are copied to before a replay
         self.mixed_graph_replays = 0
         self.logit_slots: Optional[torch.Tensor] = None     # of the last step: the slot per row of logits, on the device
         # the latest sampled token of every request slot, written by the sampling kernels
@@ -627,13 +628,7 @@ class ModelRunner:
             # the decode attention kernel cuts a row's keys by the longest context of the batch: a
             # graph must cut the same way on every replay, so it is captured for the longest possible
             blank.max_kv = self.model.plan.max_positions
-            current = torch.cuda.current_stream()
-            side = torch.cuda.Stream()
-            side.wait_stream(current)
-            with torch.cuda.stream(side):          # first run outside capture: every buffer comes into being
-                self.model.forward(blank, self.layer_caches)
-            current.wait_stream(side)
-            torch.cuda.synchronize()
+            self._run_aside(blank)
             state.workspace.freeze()
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph):
@@ -655,28 +650,58 @@ class ModelRunner:
             return None
         return (next(t for t in self._mixed_tokens if t >= n_tokens), next(r for r in self._mixed_rows if r >= n_rows))
 
+    def _blank_step(self, tokens: int, rows: int, meta: Optional[torch.Tensor], workspace: Optional[Workspace] = None) -> StepBatch:
+        """A step of the layout ``(tokens, rows)`` whose tokens belong to no request."""
+        blank = self.build_batch([], pad_rows=rows, pad_tokens=tokens, fixed_pages=self._pages_cap, meta=meta,
+                                 workspace=workspace or self._mixed_workspace)
+        blank.max_kv = self.model.plan.max_positions       # (kernels that size themselves by the longest row)
+        blank.given_embeds = self._mixed_given[:tokens]
+        return blank
+
+    def _run_aside(self, batch: StepBatch) -> None:
+        """A run outside any capture, on a stream of its own: every buffer and plan that the run needs comes into being."""
+        current = torch.cuda.current_stream()
+        side = torch.cuda.Stream()
+        side.wait_stream(current)
+        with torch.cuda.stream(side):
+            self.model.forward(batch, self.layer_caches)
+        current.wait_stream(side)
+        torch.cuda.synchronize()
+
     def _capture_mixed(self, tokens: int, rows: int) -> _GraphState:
         """The graph of a step of up to ``tokens`` tokens of up to ``rows`` requests, made if it is not
-        there yet: as for decode steps, on tokens that belong to no request."""
+        there yet: as for decode steps, on tokens that belong to no request. All these graphs run one
+        after the other on one stream and share one set of scratch tensors: before the first of them
+        is captured, every bucket of tokens (at the most rows) and of rows (at the most tokens) is run
+        once, kernel by kernel, largest first, which brings every tensor that any of them asks for to
+        the size that serves them all. (Which tensors a step asks for depends on its number of tokens:
+        the kernels of few rows have scratch tensors of their own.)"""
+        if self._mixed_workspace is None:
+            self._mixed_workspace = Workspace(self.device)
+            self._mixed_given = torch.zeros(self._mixed_tokens[-1], self.model.plan.dim, dtype=torch.float32, device=self.device)
+            shapes = [(t, self._mixed_rows[-1]) for t in reversed(self._mixed_tokens)]
+            shapes += [(self._mixed_tokens[-1], r) for r in reversed(self._mixed_rows[:-1])]
+            for shape in shapes:
+                self._run_aside(self._blank_step(*shape, None))
+            self._mixed_workspace.freeze()
         state = self._mixed.get((tokens, rows))
         if state is None:
             state = self._mixed[(tokens, rows)] = _GraphState(self.device)
+            state.workspace = self._mixed_workspace
         if state.graph is None:
-            layout = dict(pad_rows=rows, pad_tokens=tokens, fixed_pages=self._pages_cap)
-            probe = self.build_batch([], **layout)
+            probe = self.build_batch([], pad_rows=rows, pad_tokens=tokens, fixed_pages=self._pages_cap)
             state.meta = torch.empty(probe.host["meta_ints"], dtype=torch.int32, device=self.device)
-            state.given = torch.zeros(tokens, self.model.plan.dim, dtype=torch.float32, device=self.device)
-            blank = self.build_batch([], meta=state.meta, workspace=state.workspace, **layout)
-            blank.max_kv = self.model.plan.max_positions       # (kernels that size themselves by the longest row)
-            blank.given_embeds = state.given
-            current = torch.cuda.current_stream()
-            side = torch.cuda.Stream()
-            side.wait_stream(current)
-            with torch.cuda.stream(side):          # first run outside capture: every buffer comes into being
-                self.model.forward(blank, self.layer_caches)
-            current.wait_stream(side)
-            torch.cuda.synchronize()
-            state.workspace.freeze()
+            try:
+                blank = self._blank_step(tokens, rows, state.meta, state.workspace)
+                self._run_aside(blank)             # (the vendor library's plans for this number of rows)
+            except RuntimeError as error:
+                if "after freeze()" not in str(error):
+                    raise
+                # a layout that asks for a tensor none of the runs above has made: scratch tensors of its own
+                state.workspace = Workspace(self.device)
+                blank = self._blank_step(tokens, rows, state.meta, state.workspace)
+                self._run_aside(blank)
+                state.workspace.freeze()
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph):
                 state.logits = self.model.forward(blank, self.layer_caches)
@@ -690,7 +715,7 @@ class ModelRunner:
         batch = self.build_batch(entries, pad_rows=rows, pad_tokens=tokens, fixed_pages=self._pages_cap, meta=state.meta,
                                  workspace=state.workspace)
         if batch.given_embeds is not None:
-            state.given[:batch.given_embeds.shape[0]].copy_(batch.given_embeds)
+            self._mixed_given[:batch.given_embeds.shape[0]].copy_(batch.given_embeds)
         state.graph.replay()
         self.mixed_graph_replays += 1
         wanted = sum(len(e.want) for e in entries)
@@ -707,7 +732,7 @@ class ModelRunner:
         return state.logits[:len(entries)]
 
     # ------------------------------------------------------------------ everything made at start
-    @torch.inference_mode()
+    @torch.no_grad()
     def prepare(self, prompt_tokens: Optional[int] = None, wanted_rows: int = 1, tune_linears: int = 0) -> Dict[str, float]:
         """Make now what steps would otherwise make when they first need it, with live requests
         waiting (``kestrel/runtime/decode_graph.py:70-93``, ``kestrel/models/moondream/runtime.py:886-888``,
@@ -784,7 +809,10 @@ class ModelRunner:
         return done
 
     # ------------------------------------------------------------------ the step
-    @torch.inference_mode()
+    # (no_grad, not inference_mode: at a graph capture torch makes tensors of its own, the random
+    # generator's state, which a later capture by the caller, outside inference mode, has to update:
+    # tensors made inside inference mode would refuse that)
+    @torch.no_grad()
     def step(self, entries: Sequence[StepEntry]) -> torch.Tensor:
         """Run the entries as one batch. Returns fp32 logits ``[wanted, vocab]`` in the order of
         the entries and of their ``want``; the tensor is scratch memory and is overwritten by

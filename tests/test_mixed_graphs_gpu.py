@@ -113,6 +113,8 @@ def test_replayed_steps_of_any_shape_match_the_plain_implementation(name, dtype)
     decode_steps = sum(1 for step in steps if all(count == 1 for _tag, count in step))
     assert runner.graph_replays == decode_steps and runner.mixed_graph_replays == len(steps) - decode_steps
     assert sorted(runner._mixed) == [(16, 4), (32, 4), (64, 4), (128, 4)]
+    # the graphs run one after the other and share their scratch tensors
+    assert all(state.workspace is runner._mixed_workspace for state in runner._mixed.values())
     _check(name, dtype, reqs, got)
     assert runner.cache.groups[0].pool.free_count == 18
 
