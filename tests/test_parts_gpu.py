@@ -871,12 +871,15 @@ def test_a_position_encoding_of_the_whole_model_over_two_axes(dtype):
         mixer.bind({name: torch.zeros(p.shape) for name, p in mixer.params().items()}, torch.float32, DEV)
 
 
+@pytest.mark.parametrize("graphs", [False, True], ids=["launched", "replayed"])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["fp32", "bf16"])
-def test_a_windowed_layer_beside_a_full_one(dtype):
+def test_a_windowed_layer_beside_a_full_one(dtype, graphs):
     """The second layer of a tiny Moondream plan is given a window of 24 keys: its keys and values
     live in a group with a pool of its own, which gives pages back as the window passes them, while
     the first layer keeps all keys. Two requests in portions and single tokens, against the plain
-    model with the window in the second layer's mask."""
+    model with the window in the second layer's mask. Replayed: every step is a graph (of decode rows or
+    of a bucket of tokens), whose padding tokens have a window's start of their own; only the last place
+    of every portion is wanted then."""
     from dataclasses import replace
 
     from kestrel_amd.config import get_spec
@@ -892,7 +895,7 @@ def test_a_windowed_layer_beside_a_full_one(dtype):
     model = DecoderModel(replace(plan, layers=tuple(layers)))
     stored = helpers.stored_weights(helpers.model_dir(name))
     model.bind(dict(stored), dtype, DEV)
-    runner = make_runner(model, 16, 12, 2)
+    runner = make_runner(model, 16, 12, 2, enable_graphs=graphs)
     assert len(runner.cache.groups) == 2 and [g.spec.window for g in runner.cache.groups] == [None, window]
     helpers.poison_cache(runner)
     cfg = helpers.flat_config(name)
@@ -909,7 +912,12 @@ def test_a_windowed_layer_beside_a_full_one(dtype):
         return out
 
     runner.step = step_and_count
-    got = helpers.replay(runner, reqs, steps, poison=True)
+    if graphs:
+        from tests.test_mixed_graphs_gpu import replay_last_places
+        places = replay_last_places(runner, reqs, steps, wanted=1)
+        assert runner.mixed_graph_replays == 3 and runner.graph_replays == len(steps) - 3
+    else:
+        got = helpers.replay(runner, reqs, steps, poison=True)
     # the windowed group never holds more than the window and a portion's worth of pages per request
     assert max(held) <= 2 * (-(-(window + 37) // 16) + 1) and held[-1] <= -(-window // 16) + 1
     assert all(g.pool.free_count == runner.cache.n_pages for g in runner.cache.groups)
@@ -923,4 +931,9 @@ def test_a_windowed_layer_beside_a_full_one(dtype):
         table = plain.rotary_table(plain.rotary_dim_of(cfg), n, cfg["rope_theta"])
         x = plain.block(x, w, 0, cfg, positions, causal, table)
         x = plain.block(x, w, 1, cfg, positions, near, table)
-        helpers.assert_close(got[tag], plain.head(x, w, cfg), dtype, f"windowed layer, request {tag}")
+        expected = plain.head(x, w, cfg)
+        if graphs:
+            at = sorted(places[tag])
+            helpers.assert_close(torch.stack([places[tag][p] for p in at]), expected[at], dtype, f"windowed layer replayed, request {tag}")
+        else:
+            helpers.assert_close(got[tag], expected, dtype, f"windowed layer, request {tag}")
