@@ -39,7 +39,7 @@ class RuntimeConfig:
     none of them, for ``max_batch_size`` full contexts. A pool that does not fit in the device's
     free memory is refused at start with a ``MemoryError``.
     ``max_num_batched_tokens``: token budget of one step (prompt portions are cut to it).
-    ``enable_graphs``: replay decode-only steps, and every other step of up to 1,024 tokens, as captured HIP graphs.
+    ``enable_graphs``: replay decode-only steps, and every other step of up to 2,048 tokens, as captured HIP graphs.
     ``pipeline_depth``: 2 launches a step before the tokens of the one before have reached
     the host (``kestrel/scheduler/pipeline.py:49-65``); 1 reads every step first.
     ``seed``: base of the sampling generator.
