@@ -280,3 +280,34 @@ def test_replayed_prompt_portions_at_real_layer_sizes(sizes):
         places = sorted(got[tag])
         helpers.assert_close(torch.stack([got[tag][p] for p in places]), expected[places], torch.bfloat16,
                              f"{sizes} sizes, replayed portions, request {tag}")
+
+
+def test_a_whole_prompt_replayed_three_times_at_real_layer_sizes():
+    """The graph of the largest bucket (2,048 tokens), in which the vendor library runs its kernels for many rows
+    (among them one that cuts the work of all tiles evenly over the compute units and sums the pieces through
+    scratch memory): three prompts of about 2,000 tokens, the first with a block of given embeddings, each a
+    replay of that one graph, decode steps between them; the last place of each against the plain implementation."""
+    from kestrel_amd.engine.loading import load_model, make_runner
+    from tests.test_mixed_graphs_gpu import replay_last_places
+
+    sizes = "moondream2"
+    cfg = SIZES[sizes]
+    vocab, n_prefix = cfg["vocab_size"], cfg["prefix_attn"]
+    prefix = torch.randn(n_prefix, cfg["dim"], generator=torch.Generator().manual_seed(79))
+    reqs = {"a": Request("a", helpers.random_ids(1700, 1955 - n_prefix, vocab), prefix),
+            "b": Request("b", helpers.random_ids(1701, 1993, vocab)),
+            "c": Request("c", helpers.random_ids(1702, 2043, vocab))}
+    steps = [[("a", 1950)], [("a", 1)], [("b", 1990), ("a", 1)], [("a", 1), ("b", 1)], [("c", 2040), ("a", 1), ("b", 1)],
+             [("a", 1), ("b", 1), ("c", 1)], [("c", 1)], [("c", 1)]]
+    net = load_model(_folder(sizes), torch.bfloat16, torch.device("cuda:0"))
+    runner = make_runner(net, 16, 3 * 129, 4, max_tokens_per_step=2048, enable_graphs=True)
+    helpers.poison_cache(runner)
+    got = replay_last_places(runner, reqs, steps, wanted=1, poison=False)
+    assert all(r.done == r.length for r in reqs.values())
+    assert sorted(runner._mixed) == [(2048, 4)] and runner.mixed_graph_replays == 3 and runner.graph_replays == 5
+    weights = {k: v.double() for k, v in helpers.stored_weights(_folder(sizes)).items()}
+    for tag, req in reqs.items():
+        expected = plain.forward(cfg, weights, req.ids, req.prefix).float()
+        places = sorted(got[tag])
+        helpers.assert_close(torch.stack([got[tag][p] for p in places]), expected[places], torch.bfloat16,
+                             f"{sizes} sizes, a whole prompt replayed, request {tag}")
