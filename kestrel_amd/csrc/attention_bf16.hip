@@ -96,6 +96,9 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_
     const int kvh = h / (H / Hkv);
     const int row = qblk_row[blk];
     const int tok_end = cu_q[row + 1];
+    // A block that starts behind its row's last token holds no query (the unused end of a list of
+    // blocks of fixed length, as a captured step has it): nothing to do, and nothing more to look up.
+    if (qblk_tok[blk] >= tok_end) return;
     int t[QB], tq[QB], hi[QB], lo[QB];
     bool q_valid[QB];
     int wave_hi = 0, wave_lo = 0x7fffffff;
