@@ -618,7 +618,8 @@ def test_a_gated_feed_forward_as_a_part(dtype):
     of the pair is taken in the epilogue of whatever kernel runs its first linear: the prompt's tiled kernel,
     and in decode steps the launch that also normalises and projects q|k|v (one launch for norm + q|k|v + gate
     and value, one for attention, one for both last linears). A tiny Moondream plan with it in every layer
-    against a plain computation; prompt portions, then tokens one by one, eagerly and replayed."""
+    against a plain computation; prompt portions, then tokens one by one, eagerly and replayed; then prompt portions
+    replayed as well, which the part allows by saying ``replays_every_step``."""
     from dataclasses import replace
 
     from kestrel_amd.config import get_spec
@@ -629,6 +630,8 @@ def test_a_gated_feed_forward_as_a_part(dtype):
     from kestrel_amd.parts import FeedForward, ParamSpec, register_feed_forward
 
     class GatedFeedForward(FeedForward):
+        replays_every_step = True      # (its scratch comes from the batch's workspace, and it asks the host side of a batch nothing)
+
         def params(self):
             d, f = self.spec.dim, self.spec.hidden_dim
             return {"gate.weight": ParamSpec((f, d)), "up.weight": ParamSpec((f, d)), "down.weight": ParamSpec((d, f))}
@@ -693,6 +696,15 @@ def test_a_gated_feed_forward_as_a_part(dtype):
         assert (runner.graph_replays > 0) == graphs
         helpers.assert_close(torch.cat(got), expected, dtype, f"a gated feed-forward, graphs={graphs}")
         runner.release(slot)
+    # the part says it can be replayed in steps of any shape, the parts around it do too: portions of a prompt of which
+    # the scheduler's places are wanted go through the graph of their bucket of tokens
+    runner = make_runner(model, 16, 8, 2, enable_graphs=True)
+    assert runner.mixed_graphs
+    slot = runner.admit()
+    got = [runner.step([StepEntry(slot, ids[:21], want=[20])]).clone(), runner.step([StepEntry(slot, ids[21:30], want=[7, 8])]).clone()]
+    assert runner.mixed_graph_replays == 2 and sorted(runner._mixed) == [(16, 2), (32, 2)]
+    helpers.assert_close(torch.cat(got), expected[[20, 28, 29]], dtype, "a gated feed-forward in replayed prompt steps")
+    runner.release(slot)
     if dtype == torch.bfloat16:
         # the decode steps took the three-launch form: the gated linear rode in the launch of norm + q|k|v, or
         # (a few rows whose attention leaves the chip idle) in the attention launch
