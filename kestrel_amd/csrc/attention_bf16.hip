@@ -433,8 +433,13 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_
 // (four waves per SIMD are all that a workgroup of 16 waves allows, two with the registers that
 // head size 128 needs; saying so keeps the compiler from trading loads in flight for an
 // occupancy the kernel cannot have. Workgroups of four waves, which many rows get, fit five to a
-// CU with tiles of 64 keys: 15.7k to 16.1k tok/s at batch 64; six spill registers and lose that again)
-constexpr int ad_waves_per_simd(int HD, int WAVES, int TP) { return HD > 64 ? 2 : (WAVES == 4 && TP <= 4 ? 5 : 4); }
+// CU with tiles of 64 keys: 15.7k to 16.1k tok/s at batch 64. With tiles of 32 keys they need 56
+// registers a lane and fit eight to a CU: the 2,048 workgroups of 64 rows x 32 heads then run all at
+// once instead of in a round of 1,280 and one of 768: 17.8k -> 18.0k tok/s at batch 64, 15.9k -> 16.5k
+// at 48, 11.9k -> 12.8k at 24, measured at 1,024 keys a row.)
+constexpr int ad_waves_per_simd(int HD, int WAVES, int TP) { return HD > 64 ? 2 : (WAVES == 4 && TP <= 2 ? 8 : WAVES == 4 && TP <= 4 ? 5 : 4); }
+constexpr int AD_SMALL_TILE_PAGES = 2;
+constexpr int AD_SMALL_TILE_MAX_PAGES = 128;   // rows of up to this many pages get the small tiles
 
 template <int HD, int WAVES, int TP>
 __global__ void __launch_bounds__(KA_WAVE * WAVES)
@@ -729,13 +734,22 @@ static int decode_launch(const char* who, const void* q, long q_row_stride, cons
     KA_CHECK(waves == 4 || waves == 8 || waves == 16, "%s: waves must be 4, 8 or 16", who);
     if (hd > 64 && waves == 16) waves = 8;   // 16 waves leave 128 registers a lane: too few for a tile's loads (measured at head size 80: 26.4 against 23.6 us)
     dim3 grid(n, H, splits), block(KA_WAVE * waves);
+    // Workgroups of four waves that the chip holds all at once when eight of them share a CU (and that are not
+    // so few that most CUs would hold one or none: then the larger tile's loads in flight count for more):
+    // tiles of two pages (see ad_waves_per_simd).
+    const long groups = (long)n * H * splits;
+    const int cus = ka_compute_units();
+    // (Rows of up to 2,048 keys, going by the width of the block table: behind 4,096 keys a row the larger tile
+    // came out 2 to 3 % ahead at 24 and 32 rows, level at 48 and 64.)
+    const bool small_tiles = waves == 4 && hd <= 64 && max_pages <= AD_SMALL_TILE_MAX_PAGES && groups * 2 >= 3L * cus && groups <= 8L * cus;
 #define KA_AD(HDV, WV, TPV)                                                                                         \
     hipLaunchKernelGGL((attn_decode_kernel<HDV, WV, TPV>), grid, block, 0, stream, (const bf16_t*)q, q_row_stride, \
                        (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, max_pages, token_row, kv_lo,   \
                        kv_hi, (bf16_t*)out, out_row_stride, scale, H, Hkv, partial, fz)
 #define KA_AD_SMALL(HDV)                                                                                            \
     case HDV:                                                                                                       \
-        if (waves == 4) KA_AD(HDV, 4, 4); else if (waves == 8) KA_AD(HDV, 8, 4); else KA_AD(HDV, 16, 4);            \
+        if (small_tiles) KA_AD(HDV, 4, AD_SMALL_TILE_PAGES); else if (waves == 4) KA_AD(HDV, 4, 4);                \
+        else if (waves == 8) KA_AD(HDV, 8, 4); else KA_AD(HDV, 16, 4);                                              \
         break
 #define KA_AD_LARGE(HDV)                                                                                            \
     case HDV:                                                                                                       \

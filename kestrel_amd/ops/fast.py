@@ -88,6 +88,9 @@ WIDE_FLOATS = 8 << 20              # 32 MB of partial sums for the wide skinny k
 _wide_scratch = {}
 # Keys of one row a workgroup of the decode attention kernel takes before the row is split.
 DECODE_KEYS_PER_WORKGROUP = 4096
+# Longest row for which workgroups of four waves run with tiles of 32 keys, eight to a CU (the kernel goes by the
+# width of the block table: 128 pages).
+DECODE_SMALL_TILE_KEYS = 2048
 
 
 class ChipSizes(NamedTuple):
@@ -100,9 +103,12 @@ class ChipSizes(NamedTuple):
     # for an output projection + second feed-forward linear of 2048 outputs)
     skinny_target_waves: int
     # waves of the decode attention kernel that the chip holds at once (16 per compute unit: four per
-    # SIMD at the registers the kernel needs), and its workgroups of four waves (five per compute unit)
+    # SIMD at the registers the kernel needs), its workgroups of four waves (five per compute unit), and
+    # its workgroups of four waves with tiles of two pages, which the kernel takes where all of them then
+    # fit on the chip at once (eight per compute unit)
     decode_wave_slots: int
     decode_four_wave_places: int
+    decode_small_tile_places: int
 
 
 _chips: Dict[int, ChipSizes] = {}
@@ -113,7 +119,7 @@ def chip_sizes(device=None) -> ChipSizes:
     index = torch.cuda.current_device() if device is None else _device_index(device)
     if index not in _chips:
         units = int(torch.cuda.get_device_properties(index).multi_processor_count)
-        _chips[index] = ChipSizes(units, 8 * units, 16 * units, 5 * units)
+        _chips[index] = ChipSizes(units, 8 * units, 16 * units, 5 * units, 8 * units)
     return _chips[index]
 
 
@@ -417,24 +423,36 @@ def rope_cache_bf16(qkv, positions, slots, table, k_cache, v_cache, n_heads, n_k
     return True
 
 
-def decode_shape(max_kv: int, workgroups: int = 1):
+def decode_shape(max_kv: int, workgroups: int = 1, head_dim: int = 64):
     """``(splits, waves)`` of the decode attention kernel: a workgroup of up to 16 waves takes a
     64-key tile per wave and round; rows longer than 4096 keys are cut into parts whose sums
     a second kernel merges (cutting the keys of a few short rows further, to put more CUs to
-    work, was measured and changes nothing: 0.887 ms a step at batch 1 either way). With many workgroups (rows x heads) each gets fewer waves, so that
-    they all fit on the chip at once (measured at 1024 keys: 16 waves up to 256 workgroups, 8 up to
-    512, 4 beyond: workgroups of four waves fit five to a CU; 8 again where those of four would end
-    in a round that leaves much of the chip idle)."""
+    work, was measured and changes nothing: 0.887 ms a step at batch 1 either way). With many
+    workgroups (rows x heads) each gets fewer waves, so that they all fit on the chip at once.
+    Head sizes up to 64 (measured at 32 heads and 1,024 keys): 16 waves up to 256 workgroups, 4
+    beyond, which the kernel runs with tiles of 32 keys, eight workgroups to a CU, while the chip
+    holds them all at once (four waves against eight: 6.70k against 6.53k tok/s at 9 rows, 10.6k
+    against 10.4k at 16, 12.8k against 11.9k at 24, 16.5k against 15.9k at 48, 18.0k against 16.5k at
+    64; rows of up to 2,048 keys: behind 4,096 keys the larger tile is 2 to 3 % ahead at 24 and 32
+    rows). Larger head sizes, whose registers leave a CU eight waves, and longer rows: 16 waves up to
+    256 workgroups, 8 up to 512, 4 beyond. Workgroups of four waves with tiles of 64 keys fit five to a CU; where they
+    would end in a round that leaves much of the chip idle, eight waves again."""
     chip = chip_sizes()
     splits = max(1, -(-max_kv // DECODE_KEYS_PER_WORKGROUP))
     tiles = -(-max_kv // (64 * splits))
     waves = 4 if tiles <= 4 else 8 if tiles <= 8 else 16
     groups = workgroups * splits
-    fit = 16 if groups <= chip.decode_wave_slots // 16 else 8 if groups <= chip.decode_wave_slots // 8 else 4
-    if fit == 4:
+    if groups <= chip.decode_wave_slots // 16:
+        fit = 16
+    elif head_dim <= 64 and groups <= chip.decode_small_tile_places and max_kv <= DECODE_SMALL_TILE_KEYS:
+        fit = 4
+    elif groups <= chip.decode_wave_slots // 8:
+        fit = 8
+    else:
         # workgroups of four waves run in rounds of as many as the chip has places for; where the last round
         # would leave much of the chip idle, workgroups of eight waves come out better (48 rows x 32 heads are
         # 1.2 rounds of the one, 3 rounds of the other: 14.9k against 15.2k tok/s)
+        fit = 4
         rounds = -(-groups // chip.decode_four_wave_places)
         if groups < 0.7 * rounds * chip.decode_four_wave_places:
             fit = 8
@@ -462,7 +480,7 @@ def attention_decode_takes(job, n: int, n_heads: int, head_dim: int, page_size: 
     rows whose attention leaves most of the chip idle."""
     if not ATTENTION_TAKES_LINEAR or n == 0 or not _side_linear_ok(job) or job.a.shape[0] != n:
         return False
-    splits = decode_shape(max_kv, n * n_heads)[0]
+    splits = decode_shape(max_kv, n * n_heads, head_dim)[0]
     return bool(lib().ka_attention_decode_beside_supported(n, n_heads, splits, head_dim, page_size, job.a.shape[1]))
 
 
@@ -482,7 +500,7 @@ def attention_decode_bf16(q, k_cache, v_cache, block_table, token_row, kv_lo, kv
         return False
     if beside is not None and not attention_decode_takes(beside, n, n_heads, head_dim, page_size, batch.max_kv):
         return False
-    splits, waves = decode_shape(batch.max_kv, n * n_heads)
+    splits, waves = decode_shape(batch.max_kv, n * n_heads, head_dim)
     partial = scratch(q.device)
     if n * n_heads * splits * (head_dim + 2) > partial.numel():
         return False

@@ -638,17 +638,18 @@ def test_attention_decode_kernel(shape):
 
 
 @pytest.mark.parametrize("waves", [4, 8, 16])
-@pytest.mark.parametrize("shape", [(4, 4, 64), (2, 1, 16), (6, 3, 48), (4, 2, 32), (2, 2, 80), (2, 1, 128)])
+@pytest.mark.parametrize("shape", [(4, 4, 64), (2, 1, 16), (6, 3, 48), (4, 2, 32), (2, 2, 80), (2, 1, 128), (64, 8, 64), (48, 48, 32)])
 def test_decode_attention_deals_out_every_page_once(shape, waves, monkeypatch):
     """A row's pages are cut evenly over the four waves of a workgroup, or dealt out tile by tile to eight or
     sixteen: every number of pages from none to more than waves x tile, contexts that end on a page's first
-    and last slot, a window whose start lies inside a page, at every wave count."""
+    and last slot, a window whose start lies inside a page, at every wave count. With 48 or 64 heads the rows
+    here make a few hundred workgroups, which at four waves run with tiles of two pages instead of four."""
     from kestrel_amd.ops import fast
 
     h, hkv, hd = shape
     bf = torch.bfloat16
     shape_of = fast.decode_shape
-    monkeypatch.setattr(fast, "decode_shape", lambda max_kv, workgroups=1: (shape_of(max_kv, workgroups)[0], waves))
+    monkeypatch.setattr(fast, "decode_shape", lambda max_kv, workgroups=1, head_dim=64: (shape_of(max_kv, workgroups, head_dim)[0], waves))
     for kv_lens in ([1, 15, 16, 17, 63, 64, 65, 81], [1040, 1041, 1279, 600, 2047, 1, 255, 513]):
         case = PagedCase(kv_lens, [1] * len(kv_lens), h, hkv, hd, 16, bf, seed=31 + len(kv_lens))
         _close(_run_attention(case, "fast", hd ** -0.5), case.reference(hd ** -0.5), bf)
@@ -678,7 +679,7 @@ def test_fused_decode_attention_with_a_window_of_one():
     q_dim, kv_dim = h * hd, hkv * hd
     for waves in (4, 16):
         shape_of = fast.decode_shape
-        fast.decode_shape = lambda max_kv, workgroups=1, w=waves: (shape_of(max_kv, workgroups)[0], w)
+        fast.decode_shape = lambda max_kv, workgroups=1, head_dim=64, w=waves: (shape_of(max_kv, workgroups, head_dim)[0], w)
         try:
             assert fast.attention_decode_bf16(qkv, k_f, v_f, case.table, case.token_row, case.kv_lo, case.kv_hi, out,
                                               hd ** -0.5, h, hkv, hd, case.batch,
@@ -1115,7 +1116,7 @@ def test_decode_attention_with_a_linear_layer_beside_it(shape, keys_per_workgrou
     bf = torch.bfloat16
     monkeypatch.setattr(fast, "DECODE_KEYS_PER_WORKGROUP", keys_per_workgroup)
     shape_of = fast.decode_shape
-    monkeypatch.setattr(fast, "decode_shape", lambda max_kv, workgroups=1: (shape_of(max_kv, workgroups)[0], 8))
+    monkeypatch.setattr(fast, "decode_shape", lambda max_kv, workgroups=1, head_dim=64: (shape_of(max_kv, workgroups, head_dim)[0], 8))
     for kv_lens in ([1024, 16, 17, 300, 1], [700], [1000, 64, 65, 129, 2, 5, 33, 48]):
         # (as many rows as leave attention within the quarter of a 256-CU chip's places that the launch takes)
         kv_lens = kv_lens[:max(1, 128 // (h * shape_of(max(kv_lens))[0]))]
