@@ -430,14 +430,18 @@ attn_prefill_kernel(const bf16_t* __restrict__ q, long q_row_stride, const bf16_
 // ----------------------------------------------------------------------------------------------
 // decode kernel (its body: ka_attention_decode.h)
 // ----------------------------------------------------------------------------------------------
-// (four waves per SIMD are all that a workgroup of 16 waves allows, two with the registers that
-// head size 128 needs; saying so keeps the compiler from trading loads in flight for an
-// occupancy the kernel cannot have. Workgroups of four waves, which many rows get, fit five to a
+// (four waves per SIMD are all that a workgroup of 16 waves allows; head sizes of 80 to 128 fit four
+// a SIMD as well, in 120 to 124 registers (112: three; it would spill two), larger ones two; saying so
+// keeps the compiler from trading loads in flight for an occupancy the kernel cannot have. Head size
+// 80 at two a SIMD, as it was: 4.62k against 4.89k tok/s at batch 12, 6.75k against 7.32k at 24, 8.80k
+// against 9.72k at 48, 9.79k against 9.98k at 64, at 32 layers of Phi-2's sizes. Workgroups of four waves, which many rows get, fit five to a
 // CU with tiles of 64 keys: 15.7k to 16.1k tok/s at batch 64. With tiles of 32 keys they need 56
 // registers a lane and fit eight to a CU: the 2,048 workgroups of 64 rows x 32 heads then run all at
 // once instead of in a round of 1,280 and one of 768: 17.8k -> 18.0k tok/s at batch 64, 15.9k -> 16.5k
 // at 48, 11.9k -> 12.8k at 24, measured at 1,024 keys a row.)
-constexpr int ad_waves_per_simd(int HD, int WAVES, int TP) { return HD > 64 ? 2 : (WAVES == 4 && TP <= 2 ? 8 : WAVES == 4 && TP <= 4 ? 5 : 4); }
+constexpr int ad_waves_per_simd(int HD, int WAVES, int TP) {
+    return HD > 128 ? 2 : HD > 64 ? (HD > 96 && HD < 128 ? 3 : 4) : (WAVES == 4 && TP <= 2 ? 8 : WAVES == 4 && TP <= 4 ? 5 : 4);
+}
 constexpr int AD_SMALL_TILE_PAGES = 2;
 constexpr int AD_SMALL_TILE_MAX_PAGES = 128;   // rows of up to this many pages get the small tiles
 
@@ -732,7 +736,7 @@ static int decode_launch(const char* who, const void* q, long q_row_stride, cons
                      partial_floats, k_new, v_new, new_stride, table, rot, slots, k_cache_w, v_cache_w, &fz))
         return -1;
     KA_CHECK(waves == 4 || waves == 8 || waves == 16, "%s: waves must be 4, 8 or 16", who);
-    if (hd > 64 && waves == 16) waves = 8;   // 16 waves leave 128 registers a lane: too few for a tile's loads (measured at head size 80: 26.4 against 23.6 us)
+    if (hd > 64 && waves == 16) waves = 8;   // measured at head size 80: 16 waves 26.4 against 23.6 us at two waves per SIMD; at four a SIMD 3.80k against 3.84k tok/s at batch 8
     dim3 grid(n, H, splits), block(KA_WAVE * waves);
     // Workgroups of four waves that the chip holds all at once when eight of them share a CU (and that are not
     // so few that most CUs would hold one or none: then the larger tile's loads in flight count for more):
