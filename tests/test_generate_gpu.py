@@ -535,3 +535,63 @@ def test_linears_tuned_at_warm_up_give_the_same_tokens():
         engine.shutdown_sync()
     for prompt, result in zip(prompts, results):
         helpers.assert_greedy_follows(cfg, weights, prompt, result.tokens, 5e-2, "tuned linears")
+
+
+@pytest.mark.parametrize("name,dtype", [("D", "bfloat16"), ("B", "float32")])
+def test_a_random_stream_of_requests_leaves_nothing_behind(name, dtype):
+    """Sixty requests in bursts, drawn at random: prompts of 1 to 150 ids (some behind a block of given
+    embeddings), 1 to 20 new tokens, stop ids that occur or do not, greedy or sampled, in a pool so small
+    that requests wait for pages, with a token budget of 32 so that prompts go in portions beside the
+    decoded tokens of others; every step is a replayed graph. The greedy ones are the plain
+    implementation's tokens as far as they go; a stop id ends a request where it first occurs; at the
+    end every page and every slot is back."""
+    import random
+    import time
+
+    cfg = helpers.flat_config(name)
+    weights = helpers.stored_weights(helpers.model_dir(name))
+    rng = random.Random(2024)
+    n_prefix = cfg["prefix_attn"]
+    engine = _engine(name, dtype, max_batch_size=4, kv_cache_pages=26, max_num_batched_tokens=32, enable_graphs=True,
+                     pipeline_depth=2)
+    slack = 1e-4 if dtype == "float32" else 5e-2
+    submitted = []
+    try:
+        for burst in range(4):
+            for _ in range(15):
+                ids = helpers.random_ids(rng.randrange(10 ** 6), rng.randint(1, 150), cfg["vocab_size"])
+                rows = None
+                if n_prefix and n_prefix <= 32 and rng.random() < 0.3:
+                    rows = torch.randn(n_prefix, cfg["dim"], generator=torch.Generator().manual_seed(rng.randrange(10 ** 6)))
+                greedy = rng.random() < 0.6
+                stops = tuple(rng.randrange(cfg["vocab_size"]) for _ in range(rng.choice((0, 0, 3, 40))))
+                options = dict(max_new_tokens=rng.randint(1, 20), stop_ids=stops)
+                if not greedy:
+                    options.update(temperature=rng.choice((0.7, 1.3)), top_p=rng.choice((1.0, 0.8)), seed=rng.randrange(1000))
+                if rows is not None:
+                    options.update(prefix_embeds=rows)
+                submitted.append((ids, rows, greedy, stops, options["max_new_tokens"], engine.submit_sync(ids, **options)))
+            time.sleep(0.02 * burst)
+        results = [entry[-1].result(timeout=180) for entry in submitted]
+        runner = engine.runner
+        assert runner.mixed_graph_replays > 0 and runner.graph_replays > 0
+        assert not runner.held and runner.cache.free_slots == runner.cache.max_requests
+        assert all(g.pool.free_count == runner.cache.n_pages for g in runner.cache.groups)
+        runner.cache.check()
+    finally:
+        engine.shutdown_sync()
+    checked = 0
+    for (ids, rows, greedy, stops, n_new, _future), result in zip(submitted, results):
+        assert result.finish_reason in ("stop", "length"), result.finish_reason
+        tokens = list(result.tokens)
+        assert 1 <= len(tokens) <= n_new and all(0 <= t < cfg["vocab_size"] for t in tokens)
+        assert not any(t in stops for t in tokens[:-1]), "a stop id ends the request where it first occurs"
+        if result.finish_reason == "stop":
+            assert tokens[-1] in stops
+        else:
+            assert len(tokens) == n_new and tokens[-1] not in stops
+        if greedy and checked < 12:
+            helpers.assert_greedy_follows(cfg, weights, ids, tokens, slack, f"a random stream, tiny {name} {dtype}",
+                                          prefix_embeds=rows)
+            checked += 1
+    assert checked == 12

@@ -470,3 +470,22 @@ def test_graph_buckets_follow_the_reference_rule():
     assert graph_buckets(33) == [1, 2, 4, 8, 16, 32, 33]
     assert graph_buckets(64) == [1, 2, 4, 8, 16, 32, 48, 64]
     assert graph_buckets(100) == [1, 2, 4, 8, 16, 32, 48, 64, 80, 96, 100]
+
+
+def test_buckets_of_steps_of_any_shape():
+    """Token counts and numbers of rows that steps other than decode steps are captured for: fine where a step is
+    short, in steps of 128 further up, never beyond the step's token limit or 2,048 tokens."""
+    from kestrel_amd.engine.step import MIXED_GRAPH_MAX_TOKENS, mixed_graph_buckets, mixed_graph_rows
+
+    assert MIXED_GRAPH_MAX_TOKENS == 2048
+    assert mixed_graph_buckets(1) == [1] and mixed_graph_buckets(16) == [16] and mixed_graph_buckets(40) == [16, 32, 40]
+    assert mixed_graph_buckets(512) == [16, 32, 64, 128, 192, 256, 320, 384, 448, 512]
+    assert mixed_graph_buckets(700) == [16, 32, 64, 128, 192, 256, 320, 384, 448, 512, 640, 700]
+    top = mixed_graph_buckets(10 ** 6)
+    assert top == mixed_graph_buckets(2048) and top[-1] == 2048 and top[-3:] == [1792, 1920, 2048]
+    for tokens in range(1, 2049):
+        bucket = next(b for b in top if b >= tokens)
+        # never more than 127 tokens that fill a step up, and from 16 tokens on fewer than the step's own
+        assert bucket - tokens < 128 and (tokens < 16 or bucket < 2 * tokens), (tokens, bucket)
+    assert mixed_graph_rows(1) == [1] and mixed_graph_rows(6) == [6] and mixed_graph_rows(8) == [8]
+    assert mixed_graph_rows(64) == [8, 64] and mixed_graph_rows(300) == [8, 64, 300]
