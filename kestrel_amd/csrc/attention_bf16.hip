@@ -64,7 +64,10 @@ constexpr int ap_max_table(int hd) {
 // fit in 256 registers up to head size 64 (the prompt attention of 2,048 tokens: 63 to 48 us a
 // layer); beyond that they would take a SIMD's registers for one wave, which was measured far
 // slower than one block and two waves (head size 80: 98 against 63 us, 128: 267 against 139 us).
-constexpr int ap_waves_per_simd(int hd, int qb) { return qb == 1 ? (hd <= 96 ? 2 : 1) : (hd <= 64 ? 2 : 1); }
+// One block fits two waves a SIMD up to head size 128 (204 registers; told that one wave is enough
+// the compiler spread out over 280: 124 against 107 to 111 us at head size 128, 94 against 73 to 77
+// at 112, a prompt of 2,048 tokens with 32 heads).
+constexpr int ap_waves_per_simd(int hd, int qb) { return qb == 1 ? (hd <= 128 ? 2 : 1) : (hd <= 64 ? 2 : 1); }
 
 // QB blocks of 32 queries per workgroup: every tile of keys and values that a wave fetches serves
 // QB tiles of scores (the fetches, their addresses and the block table look-ups are shared).
