@@ -595,3 +595,113 @@ def test_a_random_stream_of_requests_leaves_nothing_behind(name, dtype):
                                           prefix_embeds=rows)
             checked += 1
     assert checked == 12
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_whole_architecture_registered_in_a_test(dtype, tmp_path, request):
+    """Another architecture, made up here and registered under a name of its own: configuration keys of its
+    own, blocks that run mixer and feed-forward one after the other from two norms without shifts, attention
+    without biases over grouped kv heads with every channel rotated, a ReLU feed-forward, a final norm, a head
+    tied to an embedding table that is scaled on the way in, capped logits, and a schedule that runs its middle
+    layer twice (each run with a cache of its own). Nothing of the package is edited: the registry, the
+    random-weights writer, the loader, the cache manager, the scheduler and the entry point take it from its
+    ``config.json``; greedy generation, with graphs and prompts cut into portions, follows a plain computation
+    written here."""
+    from dataclasses import dataclass
+
+    from kestrel_amd import InferenceEngine, RuntimeConfig
+    from kestrel_amd.config.registry import ModelSpec, register
+    from kestrel_amd.parts.specs import (AttentionSpec, DenseFeedForwardSpec, LayerSpec, ModelPlan, NormSpec, PositionSpec,
+                                         ScheduleEntry)
+    from kestrel_amd.weights import InitRecipe, write_random_model
+
+    @dataclass(frozen=True)
+    class StackConfig:
+        width: int
+        depth: int
+        heads: int
+        kv_heads: int
+        head: int
+        inner: int
+        vocab: int
+        positions: int
+        theta: float
+        eps: float
+        cap: float
+
+    def read_config(config):
+        keys = ("width", "depth", "heads", "kv_heads", "head", "inner", "vocab", "positions", "theta", "eps", "cap")
+        missing = [k for k in keys if k not in config]
+        if missing:
+            raise ValueError(f"config.json: keys missing: {missing}")
+        return StackConfig(**{k: config[k] for k in keys})
+
+    def build_plan(cfg):
+        position = PositionSpec("rotary_neox", cfg.head, cfg.theta, cfg.positions)
+        layers = []
+        for i in range(cfg.depth):
+            p = f"stack.{i}."
+            layers.append(LayerSpec(
+                arrangement="sequential", norm=NormSpec("layernorm", cfg.width, cfg.eps, bias=False),
+                norm2=NormSpec("layernorm", cfg.width, cfg.eps, bias=False),
+                mixer=AttentionSpec("attention", cfg.width, cfg.heads, cfg.kv_heads, cfg.head, position, bias=False),
+                feed_forward=DenseFeedForwardSpec("dense", cfg.width, cfg.inner, "relu", bias=False),
+                names={"norm.weight": p + "n1", "norm2.weight": p + "n2", "mixer.qkv.weight": p + "qkv", "mixer.proj.weight": p + "o",
+                       "feed_forward.fc1.weight": p + "up", "feed_forward.fc2.weight": p + "down"}))
+        order = [0] + [i for i in range(1, cfg.depth - 1) for _ in range(2)] + [cfg.depth - 1]
+        return ModelPlan(architecture="toy_stack", vocab_size=cfg.vocab, dim=cfg.width, max_positions=cfg.positions,
+                         layers=tuple(layers), schedule=tuple(ScheduleEntry(i) for i in order),
+                         final_norm=NormSpec("layernorm", cfg.width, cfg.eps, bias=False), head_bias=False, tied_head=True,
+                         names={"embedding": "table", "final_norm.weight": "last_norm"}, eos_token_ids=(1,),
+                         embedding_scale=float(cfg.width) ** 0.5, logit_softcap=cfg.cap)
+
+    from kestrel_amd.config import registry
+
+    register(ModelSpec(name="toy_stack", read_config=read_config, build_plan=build_plan))
+    request.addfinalizer(lambda: registry._REGISTRY.pop("toy_stack", None))       # (other tests list the registered names)
+    config = {"model": "toy_stack", "width": 96, "depth": 3, "heads": 6, "kv_heads": 2, "head": 16, "inner": 136, "vocab": 257,
+              "positions": 160, "theta": 777.0, "eps": 1e-4, "cap": 12.0}
+    folder = str(tmp_path / "toy_stack")
+    write_random_model(folder, config, seed=9, recipe=InitRecipe(std=0.08, gain_std=0.1))
+    weights = {k: v.double() for k, v in helpers.stored_weights(folder).items()}
+    assert sorted(weights)[:3] == ["last_norm", "stack.0.down", "stack.0.n1"] and "table" in weights
+
+    def logits_of(ids):
+        cfg = read_config(config)
+        n = len(ids)
+        x = weights["table"][torch.tensor(ids)] * cfg.width ** 0.5
+        positions = torch.arange(n)
+        allowed = plain.visibility(positions, None)
+        table = plain.rotary_table(cfg.head, n, cfg.theta)
+        zero = torch.zeros(cfg.width, dtype=torch.float64)
+        for i in (0, 1, 1, 2):
+            p = f"stack.{i}."
+            h = plain.layer_norm(x, weights[p + "n1"], zero, cfg.eps)
+            q, k, v = plain.linear(h, weights[p + "qkv"], None).split([cfg.heads * cfg.head, cfg.kv_heads * cfg.head, cfg.kv_heads * cfg.head], dim=-1)
+            q = plain.apply_rotary(q.reshape(n, cfg.heads, cfg.head), positions, table)
+            k = plain.apply_rotary(k.reshape(n, cfg.kv_heads, cfg.head), positions, table)
+            mixed = plain.attention_core(q, k, v.reshape(n, cfg.kv_heads, cfg.head), allowed, cfg.head ** -0.5)
+            x = x + plain.linear(mixed.reshape(n, -1), weights[p + "o"], None)
+            h = plain.layer_norm(x, weights[p + "n2"], zero, cfg.eps)
+            x = x + plain.linear(torch.relu(plain.linear(h, weights[p + "up"], None)), weights[p + "down"], None)
+        out = plain.linear(plain.layer_norm(x, weights["last_norm"], zero, cfg.eps), weights["table"], None)
+        return cfg.cap * torch.tanh(out / cfg.cap)
+
+    engine = InferenceEngine.create_sync(RuntimeConfig(model_path=folder, dtype=dtype, max_batch_size=3, kv_cache_pages=40,
+                                                       max_num_batched_tokens=32))
+    try:
+        assert engine.runner.model.plan.architecture == "toy_stack" and len(engine.runner.layer_caches) == 4
+        prompts = [helpers.random_ids(2100 + i, n, 257) for i, n in enumerate((7, 45, 70))]
+        results = engine.generate_batch_sync(prompts, max_new_tokens=10, stop_ids=())
+        assert engine.runner.mixed_graph_replays > 0 and engine.runner.graph_replays > 0
+    finally:
+        engine.shutdown_sync()
+    slack = 1e-4 if dtype == "float32" else 5e-2
+    for prompt, result in zip(prompts, results):
+        tokens = list(result.tokens)
+        assert len(tokens) == 10
+        rows = logits_of(prompt + tokens[:-1])
+        for i, token in enumerate(tokens):
+            row = rows[len(prompt) - 1 + i]
+            gap = float(row.max() - row[token])
+            assert gap <= slack, f"toy_stack {dtype}: token {i} is {token}, the plain computation gives {int(row.argmax())} ({gap:.3g} better)"
